@@ -1,0 +1,248 @@
+/*
+ * tcbnn_hip.h — C ABI of the MI355X (gfx950) binarized-network inference path.
+ *
+ * Every entry point replaces one piece of the CUDA reference's bit-matmul /
+ * bit-convolution inference path (pnnl/TCBNN).  The citation on each
+ * declaration names the reference function or method whose behaviour the
+ * entry point reproduces.  The reference fuses its layers into one persistent
+ * cooperative kernel (imagenet_resnet.cu:34-125); here every layer is one
+ * stream-ordered launch, so a network is a host loop over *_forward calls on
+ * one stream.
+ *
+ * Conventions
+ *   - All data pointers are DEVICE pointers unless the name ends in _host.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).
+ *   - Return value: 0 on success, a negative TCBNN_E* code otherwise.  No
+ *     entry point ever calls exit(); tcbnn_last_error() returns a message for
+ *     the calling thread.  (The reference prints and exits, utility.h:57-92;
+ *     the C++ layer classes layered above this ABI keep that behaviour.)
+ *   - Bit convention (kernel.cuh:168, param.h:60): bit = 1 <=> value >= 0
+ *     (resp. >= threshold) <=> "+1"; element e of a group of 32 is bit (31-e)
+ *     of its uint32 ("MSB first"); pad bits are 0 in both operands and the
+ *     true K / Cin enters  K - 2*popc(a xor w).
+ *
+ * Engine layouts (device memory)
+ *   FC activations   : uint32 [B][KW128]          KW128 = 4*ceil(K/128) words per row
+ *   conv activations : uint32 [H][W][B][CW]       CW    = ceil(C/32) words per (pixel,image)
+ *   FC-ready conv out: uint32 [B][OH*OW*CW128]    feature order (y, x, c), c padded to 128
+ *                                                 (kernel.cuh:798-808)
+ *   packed weights   : uint32 [NPAD32][KWTOT]     one row per output neuron/channel,
+ *                                                 FC: KWTOT = KW128; conv: KWTOT = R*S*CW,
+ *                                                 K index = (r*S+s)*32*CW + c; rows >= N are 0
+ *   residual tensors : int32  [P][Q][B][O]        true channel count, no 128-padding
+ *   fp32 stem input  : float  [B][3][H][W]        (kernel.cuh:620-625)
+ * The reference's own tile-contiguous "FMT" layouts ([.../8][.../128][8][4],
+ * kernel.cuh:170,222,650-660,798-815) are produced / consumed by the
+ * *_to_reference_fmt / *_from_reference_fmt converters below.
+ */
+#ifndef TCBNN_HIP_H
+#define TCBNN_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TCBNN_OK 0
+#define TCBNN_EINVAL (-1)   /* bad shape / flag combination                  */
+#define TCBNN_ENULL (-2)    /* required pointer is NULL (utility.h:84-92)    */
+#define TCBNN_EHIP (-3)     /* HIP runtime error (utility.h:57-81)           */
+#define TCBNN_EUNSUPPORTED (-4)
+
+/* Inner-product engines.  AUTO picks per shape. */
+#define TCBNN_VARIANT_AUTO 0
+#define TCBNN_VARIANT_POPC 1      /* v_xor_b32 + v_bcnt_u32_b32 on the VALU   */
+#define TCBNN_VARIANT_MFMA_I8 2   /* +-1 unpacked to int8, v_mfma_i32_32x32x32_i8 */
+#define TCBNN_VARIANT_MFMA_F4 3   /* +-1 unpacked to FP4 E2M1, v_mfma_f32_32x32x64_f8f6f4 (exact: |sum| < 2^24) */
+
+/* ------------------------------------------------------------------ misc */
+int tcbnn_abi_version(void);
+/* Message of the last failing call on this thread ("" if none). */
+const char* tcbnn_last_error(void);
+/* Process-wide default for TCBNN_VARIANT_AUTO (also read once from the
+ * environment variable TCBNN_VARIANT = popc | mfma_i8 | mfma_f4). */
+int tcbnn_set_default_variant(int variant);
+int tcbnn_get_default_variant(void);
+
+/* ------------------------------------------------------------ geometry */
+/* Derived conv geometry, identical in both reference conv constructors
+ * (param.h:719-728, 897-906):
+ *   pad = padding ? ((((H + s - H%s)/s - 1)*s + R - H)/2) : 0
+ *   buf = padding ? ceil(H/s) : (H-R)/s + 1 ;  out = ceil(buf/pool)          */
+int tcbnn_conv_pad(int in_size, int filter, int stride, int padding);
+int tcbnn_conv_out(int in_size, int filter, int stride, int padding, int pool);
+
+/* Word counts of the engine layouts above. */
+size_t tcbnn_fc_act_words(int batch, int features);                    /* B*KW128          */
+size_t tcbnn_conv_act_words(int height, int width, int batch, int ch); /* H*W*B*CW         */
+size_t tcbnn_fc_weight_words(int in_features, int out_features);       /* NPAD32*KW128     */
+size_t tcbnn_conv_filter_words(int r, int s, int in_ch, int out_ch);   /* NPAD32*R*S*CW    */
+size_t tcbnn_inconv_filter_words(int r, int s, int in_ch, int out_ch); /* R*S*OPAD32*4     */
+
+/* ------------------------------------------------- one-time weight packing */
+/* fp32 [K][N] (param.h:58-59) -> packed [NPAD32][KW128].  Replaces
+ * PackFcWeight128FMT (param.h:44-63). */
+int tcbnn_pack_fc_weight(const float* weight_kn, uint32_t* packed, int in_features,
+                         int out_features, void* stream);
+/* fp32 HWIO [R][S][C][O] (param.h:573-574) -> packed [OPAD32][R*S][CW].  Replaces
+ * PackFiltersByInChannels128FMT (param.h:560-581). */
+int tcbnn_pack_conv_filter(const float* filter_hwio, uint32_t* packed, int r, int s, int in_ch,
+                           int out_ch, void* stream);
+/* fp32 HWIO [R][S][3][O] -> sign-mask table uint32 [R*S][OPAD32][4]: entry c<3 is
+ * 0 if the weight is >= 0 and 0x80000000 otherwise (the bit the first layer
+ * flips on the fp32 input, kernel.cuh:636-638).  Replaces
+ * PackFiltersByOutChannels32 (param.h:613-632). */
+int tcbnn_pack_inconv_filter(const float* filter_hwio, uint32_t* packed, int r, int s, int in_ch,
+                             int out_ch, void* stream);
+/* fp32 +-1 matrix rows -> packed rows, MSB first: out[row][k/32].  `rows` x `k`
+ * row-major input with leading dimension `ld`; k_words words are written per
+ * row (zero padded).  Replaces BMMA_toBit32Row (tensorcore_kernel.cu:87-97). */
+int tcbnn_pack_rows(const float* src, uint32_t* packed, int rows, int k, int ld, int k_words,
+                    void* stream);
+/* fp32 [K][N] -> packed [N][k_words] (each column contiguous along K).  Replaces
+ * BMMA_toBit32Col (tensorcore_kernel.cu:74-84). */
+int tcbnn_pack_cols(const float* src, uint32_t* packed, int k, int n, int k_words, void* stream);
+/* fp32 +-1 NHWC [B][H][W][C] -> packed [H][W][B][CW].  Replaces BTC_bin_input
+ * (bmma_kernel.cu:73-98). */
+int tcbnn_pack_conv_input_nhwc(const float* src, uint32_t* packed, int batch, int height,
+                               int width, int ch, void* stream);
+
+/* ------------------------------------------------------------ layer forward */
+/* In128LayerFMT (kernel.cuh:153-172), descriptor fields of In128LayerParam
+ * (param.h:210-218): fp32 [B][K] -> sign bits, FC activation layout. */
+typedef struct tcbnn_in128_desc {
+    const float* input;   /* [input_height][input_width] */
+    uint32_t* output;     /* [B][KW128] */
+    int input_height;     /* batch */
+    int input_width;      /* features */
+} tcbnn_in128_desc;
+int tcbnn_in128_forward(const tcbnn_in128_desc* d, void* stream);
+
+/* Fc128LayerFMT (kernel.cuh:174-226), fields of Fc128LayerParam (param.h:362-384):
+ * bit[b][n] = ((float)K - 2*(float)popc(a_b xor w_n) >= bn[n]). */
+typedef struct tcbnn_fc128_desc {
+    const uint32_t* input;   /* [B][KW128(input_width)] */
+    const uint32_t* weight;  /* tcbnn_pack_fc_weight output */
+    const float* bn;         /* [weight_width] thresholds */
+    uint32_t* output;        /* [B][KW128(weight_width)] */
+    int input_height;        /* batch */
+    int input_width;         /* K */
+    int weight_width;        /* N */
+    int variant;             /* TCBNN_VARIANT_* */
+    int32_t* workspace;      /* optional int32 [B][NPAD32] for split-K; may be NULL */
+    size_t workspace_words;
+} tcbnn_fc128_desc;
+int tcbnn_fc128_forward(const tcbnn_fc128_desc* d, void* stream);
+
+/* Out128LayerFMT (kernel.cuh:230-280), fields of Out128LayerParam (param.h:506-530):
+ * y[b][n] = ((float)K - (float)popc*2.0f)*bn_scale[n] + bn_bias[n], fp32 row major. */
+typedef struct tcbnn_out128_desc {
+    const uint32_t* input;
+    const uint32_t* weight;
+    const float* bn_scale;
+    const float* bn_bias;
+    float* output;           /* [B][weight_width] */
+    int input_height, input_width, weight_width;
+    int variant;
+} tcbnn_out128_desc;
+int tcbnn_out128_forward(const tcbnn_out128_desc* d, void* stream);
+
+/* InConv128LayerFMT (kernel.cuh:578-672), fields of InConv128LayerParam
+ * (param.h:841-869).  fp32 NCHW 3-channel input, +-1 filters, fp32 adds in the
+ * reference order  acc += ((+-f0) + (+-f1)) + (+-f2)  per in-frame tap in (r,s)
+ * raster order; bit = !((float)acc < bn[o]); OR-pool; residual = (int)acc.
+ * save_residual requires pool 1x1 (the reference index by*output_width+bx,
+ * kernel.cuh:666, is only meaningful then). */
+typedef struct tcbnn_inconv128_desc {
+    const float* input;        /* [batch][3][input_height][input_width] */
+    const uint32_t* filter;    /* tcbnn_pack_inconv_filter output */
+    const float* bn;           /* [output_channels] */
+    uint32_t* output;          /* [OH][OW][B][CW(output_channels)] */
+    int32_t* output_residual;  /* [P][Q][B][O] or NULL */
+    int input_height, input_width, input_channels;
+    int filter_height, filter_width;
+    int output_channels, batch;
+    int stride_height, stride_width;
+    int padding;               /* bool */
+    int pool_height, pool_width;
+    int save_residual;         /* bool */
+} tcbnn_inconv128_desc;
+int tcbnn_inconv128_forward(const tcbnn_inconv128_desc* d, void* stream);
+
+/* Conv128LayerFMT (kernel.cuh:676-827), fields of Conv128LayerParam (param.h:1028-1064).
+ *   res = Cin*R*S - exclude*Cin - 2*popc                      (kernel.cuh:766-768)
+ *   if inject_residual && o < residual_channels:
+ *        res += residual_pool ? max_{i,j in {0,1}} Rin[2y+i][2x+j][b][o] : Rin[y][x][b][o]
+ *                                                              (kernel.cuh:770-794)
+ *   bit = !((float)res < bn[o]); OR over the pool window      (kernel.cuh:795-816)
+ *   if save_residual: Rout[y][x][b][o] = res                  (kernel.cuh:818-824)
+ * Channels o >= input_residual_channels of the source read as 0 (the reference
+ * gets the same effect from its zero-filled 128-channel padding, param.h:979-980).
+ * save_residual / inject_residual require pool 1x1, residual_pool requires the
+ * source to be exactly twice the output size (as the reference indexing assumes). */
+typedef struct tcbnn_conv128_desc {
+    const uint32_t* input;         /* [H][W][B][CW(input_channels)] */
+    const uint32_t* filter;        /* tcbnn_pack_conv_filter output */
+    const float* bn;               /* [output_channels] */
+    uint32_t* output;              /* [OH][OW][B][CW(O)], or FC-ready if ahead_fc */
+    const int32_t* input_residual; /* [Hr][Wr][B][input_residual_channels] or NULL */
+    int32_t* output_residual;      /* [P][Q][B][O] or NULL */
+    int input_height, input_width, input_channels;
+    int filter_height, filter_width;
+    int output_channels, batch;
+    int stride_height, stride_width;
+    int padding;
+    int pool_height, pool_width;
+    int ahead_fc, save_residual, inject_residual;
+    int residual_channels;         /* inject only into o < residual_channels */
+    int residual_pool;
+    int input_residual_channels;   /* channel count (stride) of the source tensor */
+    int variant;
+} tcbnn_conv128_desc;
+int tcbnn_conv128_forward(const tcbnn_conv128_desc* d, void* stream);
+
+/* ------------------------------------------------ standalone GEMM / conv */
+/* C[m][n] = K - 2*popc(A[m,:] xor B[n,:]), int32 row major [M][N].  A: [M][K/32],
+ * B: [N][K/32] (each column of the logical K x N matrix contiguous along K);
+ * K % 32 == 0.  Replaces BMMAS / BMMAS_new (tensorcore_kernel.cu:305-356). */
+int tcbnn_bmm(const uint32_t* a, const uint32_t* b, int32_t* c, int m, int n, int k, int variant,
+              void* stream);
+/* out[b][p][q][o] = Cin*R*S - exclude*Cin - 2*popc  (bmma_kernel.cu:154-159), int32
+ * [N][P][Q][O] (the layout BTC_trans_output produces, bmma_kernel.cu:247-263).
+ * input: [H][W][B][CW]; filter: tcbnn_pack_conv_filter output.  Replaces
+ * BTC_Conv2d_balance[_128] (bmma_kernel.cu:101-165, 326-392). */
+int tcbnn_bconv(const uint32_t* input, const uint32_t* filter, int32_t* output, int batch,
+                int height, int width, int in_ch, int out_ch, int r, int s, int stride_h,
+                int stride_w, int pad_h, int pad_w, int out_h, int out_w, int variant,
+                void* stream);
+
+/* -------------------------------------------------- unpack / interop */
+/* bits -> +-1.0f, [B][N] row major.  Replaces UnPackFcOutput128FMT (param.h:87-104). */
+int tcbnn_unpack_fc_output(const uint32_t* packed, float* out, int batch, int features,
+                           void* stream);
+/* bits -> +-1.0f, NHWC [B][H][W][C].  Replaces UnpackConvOutput32FMT (param.h:661-688). */
+int tcbnn_unpack_conv_output(const uint32_t* packed, float* out, int height, int width, int ch,
+                             int batch, void* stream);
+/* Engine FC activation layout <-> reference [ceil(B/8)][ceil(K/128)][8][4] tiles
+ * (kernel.cuh:170,222-223).  fmt holds PAD8(B)*ceil(K/128)*4 words. */
+int tcbnn_fc_to_reference_fmt(const uint32_t* packed, uint32_t* fmt, int batch, int features,
+                              void* stream);
+int tcbnn_fc_from_reference_fmt(const uint32_t* fmt, uint32_t* packed, int batch, int features,
+                                void* stream);
+/* Engine conv activation layout <-> reference [H][W][PAD8(B)/8][ceil(C/128)][8][4]
+ * (kernel.cuh:650-660, 811-815). */
+int tcbnn_conv_to_reference_fmt(const uint32_t* packed, uint32_t* fmt, int height, int width,
+                                int batch, int ch, void* stream);
+int tcbnn_conv_from_reference_fmt(const uint32_t* fmt, uint32_t* packed, int height, int width,
+                                  int batch, int ch, void* stream);
+/* Engine residual [P][Q][B][O] -> reference [P][Q][PAD8(B)][PAD128(O)] with zero
+ * fill (kernel.cuh:666-668, 820-823). */
+int tcbnn_residual_to_reference(const int32_t* res, int32_t* ref, int height, int width,
+                                int batch, int ch, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TCBNN_HIP_H */

@@ -1,0 +1,10 @@
+// Matrix-core variants of the implicit GEMM (placeholder until the MFMA kernels land).
+#include "common.h"
+
+namespace tcbnn {
+int launch_bgemm_mfma(const BgemmParams& p, int variant, hipStream_t stream) {
+    (void)p;
+    (void)stream;
+    return fail(TCBNN_EUNSUPPORTED, "MFMA variant %d is not built", variant);
+}
+}  // namespace tcbnn

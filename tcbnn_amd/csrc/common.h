@@ -1,0 +1,87 @@
+// Shared host/device helpers of the gfx950 BNN inference library.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <string>
+
+#include "../../include/tcbnn_hip.h"
+
+namespace tcbnn {
+
+// STEPn / PADn of the reference (utility.h:33-45).
+__host__ __device__ constexpr inline int step32(int x) { return (x + 31) >> 5; }
+__host__ __device__ constexpr inline int step128(int x) { return (x + 127) >> 7; }
+__host__ __device__ constexpr inline int pad8(int x) { return ((x + 7) >> 3) << 3; }
+__host__ __device__ constexpr inline int pad32(int x) { return step32(x) << 5; }
+__host__ __device__ constexpr inline int pad128(int x) { return step128(x) << 7; }
+// words per FC activation / weight row
+__host__ __device__ constexpr inline int kw128(int k) { return 4 * step128(k); }
+
+int fail(int code, const char* fmt, ...);
+int check_hip(hipError_t e, const char* what);
+int resolve_variant(int requested);
+
+#define TCBNN_REQUIRE(cond, ...)                                  \
+    do {                                                          \
+        if (!(cond)) return ::tcbnn::fail(TCBNN_EINVAL, __VA_ARGS__); \
+    } while (0)
+#define TCBNN_NOTNULL(p)                                                              \
+    do {                                                                              \
+        if ((p) == nullptr) return ::tcbnn::fail(TCBNN_ENULL, "NULL pointer: %s", #p); \
+    } while (0)
+#define TCBNN_LAUNCH_CHECK(name)                                      \
+    do {                                                              \
+        int rc__ = ::tcbnn::check_hip(hipGetLastError(), name);       \
+        if (rc__) return rc__;                                        \
+    } while (0)
+
+// ---------------------------------------------------------------------------
+// Implicit-GEMM problem shared by the FC, Out, Conv, bmm and bconv entry points.
+// Rows of the GEMM are (pre-pool output pixel, image); columns are output
+// neurons/channels; K runs over (filter tap, input-channel word).
+// ---------------------------------------------------------------------------
+enum EpilogueMode : int {
+    EPI_THRESH = 0,  // threshold -> bit, OR over the pool window, packed store
+    EPI_AFFINE = 1,  // (K - 2c)*scale + bias -> fp32
+    EPI_RAW = 2,     // +-1 dot product -> int32
+};
+
+struct BgemmParams {
+    const uint32_t* act;  // [H][W][B][cw]
+    const uint32_t* wgt;  // [npad32][taps*cw]
+    int H, W, B, cw;      // input geometry, words per (pixel, image)
+    int R, S, stride_h, stride_w, pad_h, pad_w;
+    int PH, PW;           // conv output size before pooling
+    int pool_h, pool_w;
+    int OH, OW;           // after pooling
+    int N;                // true number of output columns
+    int k_tap;            // true K per tap (Cin, or K for FC)
+    int mode;
+    int nan_bit;          // bit emitted when the threshold compare is unordered
+    // EPI_THRESH
+    const float* bn;
+    uint32_t* out_bits;
+    long long bits_pix_stride, bits_b_stride;  // in words, indexed by pooled pixel
+    int bits_row_words;  // words per (pixel, image) row; those past ceil(N/32) are written as 0
+    // EPI_AFFINE
+    const float* bn_scale;
+    const float* bn_bias;
+    float* out_f32;  // [B][N]
+    // EPI_RAW
+    int32_t* out_i32;
+    long long raw_pix_stride, raw_b_stride;  // in ints, indexed by pre-pool pixel
+    // residuals (pool 1x1 only)
+    const int32_t* res_in;
+    int res_in_ch;     // channel stride of the source
+    int res_limit;     // inject only into n < res_limit
+    int res_pool;      // 2x2 max over a source twice the output size
+    int32_t* res_out;  // [PH][PW][B][N]
+};
+
+int launch_bgemm_popc(const BgemmParams& p, hipStream_t stream);
+int launch_bgemm_mfma(const BgemmParams& p, int variant, hipStream_t stream);
+int validate_bgemm(const BgemmParams& p);
+
+}  // namespace tcbnn

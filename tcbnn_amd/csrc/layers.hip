@@ -1,0 +1,289 @@
+// C-ABI entry points of the bit-matmul / bit-convolution layers: descriptor
+// validation and translation into the implicit-GEMM problem.
+#include <stdarg.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <atomic>
+
+#include "common.h"
+
+namespace tcbnn {
+
+static thread_local char g_err[512] = "";
+static std::atomic<int> g_default_variant{-1};
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int check_hip(hipError_t e, const char* what) {
+    if (e == hipSuccess) return TCBNN_OK;
+    return fail(TCBNN_EHIP, "%s failed: %s", what, hipGetErrorString(e));
+}
+
+static int variant_from_env() {
+    const char* v = getenv("TCBNN_VARIANT");
+    if (v == nullptr) return TCBNN_VARIANT_POPC;
+    if (!strcmp(v, "popc")) return TCBNN_VARIANT_POPC;
+    if (!strcmp(v, "mfma_i8")) return TCBNN_VARIANT_MFMA_I8;
+    if (!strcmp(v, "mfma_f4")) return TCBNN_VARIANT_MFMA_F4;
+    return TCBNN_VARIANT_POPC;
+}
+
+int resolve_variant(int requested) {
+    if (requested != TCBNN_VARIANT_AUTO) return requested;
+    int v = g_default_variant.load();
+    if (v < 0) {
+        v = variant_from_env();
+        g_default_variant.store(v);
+    }
+    return v;
+}
+
+static int run_bgemm(const BgemmParams& p, int variant, hipStream_t stream) {
+    const int v = resolve_variant(variant);
+    switch (v) {
+        case TCBNN_VARIANT_POPC:
+            return launch_bgemm_popc(p, stream);
+        case TCBNN_VARIANT_MFMA_I8:
+        case TCBNN_VARIANT_MFMA_F4:
+            return launch_bgemm_mfma(p, v, stream);
+        default:
+            return fail(TCBNN_EINVAL, "unknown variant %d", v);
+    }
+}
+
+static BgemmParams fc_problem(const uint32_t* input, const uint32_t* weight, int batch, int k,
+                              int n) {
+    BgemmParams p;
+    memset(&p, 0, sizeof(p));
+    p.act = input;
+    p.wgt = weight;
+    p.H = p.W = 1;
+    p.B = batch;
+    p.cw = kw128(k);
+    p.R = p.S = 1;
+    p.stride_h = p.stride_w = 1;
+    p.PH = p.PW = p.OH = p.OW = 1;
+    p.pool_h = p.pool_w = 1;
+    p.N = n;
+    p.k_tap = k;
+    return p;
+}
+
+}  // namespace tcbnn
+
+using namespace tcbnn;
+
+extern "C" {
+
+int tcbnn_abi_version(void) { return 1; }
+const char* tcbnn_last_error(void) { return g_err; }
+
+int tcbnn_set_default_variant(int variant) {
+    TCBNN_REQUIRE(variant >= TCBNN_VARIANT_POPC && variant <= TCBNN_VARIANT_MFMA_F4,
+                  "set_default_variant: unknown variant %d", variant);
+    g_default_variant.store(variant);
+    return TCBNN_OK;
+}
+int tcbnn_get_default_variant(void) { return resolve_variant(TCBNN_VARIANT_AUTO); }
+
+int tcbnn_conv_pad(int in_size, int filter, int stride, int padding) {
+    if (!padding || stride <= 0) return 0;
+    return (((in_size + stride - (in_size % stride)) / stride - 1) * stride + filter - in_size) / 2;
+}
+int tcbnn_conv_out(int in_size, int filter, int stride, int padding, int pool) {
+    if (stride <= 0 || pool <= 0) return 0;
+    const int buf = padding ? (in_size + stride - 1) / stride : (in_size - filter) / stride + 1;
+    return (buf + pool - 1) / pool;
+}
+
+size_t tcbnn_fc_act_words(int batch, int features) { return (size_t)batch * kw128(features); }
+size_t tcbnn_conv_act_words(int height, int width, int batch, int ch) {
+    return (size_t)height * width * batch * step32(ch);
+}
+size_t tcbnn_fc_weight_words(int in_features, int out_features) {
+    return (size_t)pad32(out_features) * kw128(in_features);
+}
+size_t tcbnn_conv_filter_words(int r, int s, int in_ch, int out_ch) {
+    return (size_t)pad32(out_ch) * r * s * step32(in_ch);
+}
+size_t tcbnn_inconv_filter_words(int r, int s, int in_ch, int out_ch) {
+    (void)in_ch;
+    return (size_t)r * s * pad32(out_ch) * 4;
+}
+
+int tcbnn_fc128_forward(const tcbnn_fc128_desc* d, void* stream) {
+    TCBNN_NOTNULL(d);
+    TCBNN_NOTNULL(d->input);
+    TCBNN_NOTNULL(d->weight);
+    TCBNN_NOTNULL(d->bn);
+    TCBNN_NOTNULL(d->output);
+    TCBNN_REQUIRE(d->input_height > 0 && d->input_width > 0 && d->weight_width > 0,
+                  "fc128: bad shape");
+    BgemmParams p = fc_problem(d->input, d->weight, d->input_height, d->input_width,
+                               d->weight_width);
+    p.mode = EPI_THRESH;
+    p.nan_bit = 0;  // kernel.cuh:210-213 uses >=, false when unordered
+    p.bn = d->bn;
+    p.out_bits = d->output;
+    p.bits_pix_stride = 0;
+    p.bits_b_stride = kw128(d->weight_width);
+    p.bits_row_words = kw128(d->weight_width);
+    return run_bgemm(p, d->variant, (hipStream_t)stream);
+}
+
+int tcbnn_out128_forward(const tcbnn_out128_desc* d, void* stream) {
+    TCBNN_NOTNULL(d);
+    TCBNN_NOTNULL(d->input);
+    TCBNN_NOTNULL(d->weight);
+    TCBNN_NOTNULL(d->bn_scale);
+    TCBNN_NOTNULL(d->bn_bias);
+    TCBNN_NOTNULL(d->output);
+    TCBNN_REQUIRE(d->input_height > 0 && d->input_width > 0 && d->weight_width > 0,
+                  "out128: bad shape");
+    BgemmParams p = fc_problem(d->input, d->weight, d->input_height, d->input_width,
+                               d->weight_width);
+    p.mode = EPI_AFFINE;
+    p.bn_scale = d->bn_scale;
+    p.bn_bias = d->bn_bias;
+    p.out_f32 = d->output;
+    return run_bgemm(p, d->variant, (hipStream_t)stream);
+}
+
+int tcbnn_conv128_forward(const tcbnn_conv128_desc* d, void* stream) {
+    TCBNN_NOTNULL(d);
+    TCBNN_NOTNULL(d->input);
+    TCBNN_NOTNULL(d->filter);
+    TCBNN_NOTNULL(d->bn);
+    TCBNN_NOTNULL(d->output);
+    TCBNN_REQUIRE(d->input_height > 0 && d->input_width > 0 && d->batch > 0 &&
+                      d->input_channels > 0 && d->output_channels > 0 && d->filter_height > 0 &&
+                      d->filter_width > 0 && d->stride_height > 0 && d->stride_width > 0 &&
+                      d->pool_height > 0 && d->pool_width > 0,
+                  "conv128: bad shape");
+    BgemmParams p;
+    memset(&p, 0, sizeof(p));
+    p.act = d->input;
+    p.wgt = d->filter;
+    p.H = d->input_height;
+    p.W = d->input_width;
+    p.B = d->batch;
+    p.cw = step32(d->input_channels);
+    p.R = d->filter_height;
+    p.S = d->filter_width;
+    p.stride_h = d->stride_height;
+    p.stride_w = d->stride_width;
+    p.pad_h = tcbnn_conv_pad(p.H, p.R, p.stride_h, d->padding);
+    p.pad_w = tcbnn_conv_pad(p.W, p.S, p.stride_w, d->padding);
+    p.PH = tcbnn_conv_out(p.H, p.R, p.stride_h, d->padding, 1);
+    p.PW = tcbnn_conv_out(p.W, p.S, p.stride_w, d->padding, 1);
+    TCBNN_REQUIRE(p.PH > 0 && p.PW > 0, "conv128: empty output");
+    p.pool_h = d->pool_height;
+    p.pool_w = d->pool_width;
+    p.OH = (p.PH + p.pool_h - 1) / p.pool_h;
+    p.OW = (p.PW + p.pool_w - 1) / p.pool_w;
+    p.N = d->output_channels;
+    p.k_tap = d->input_channels;
+    p.mode = EPI_THRESH;
+    p.nan_bit = 1;  // kernel.cuh:795-796: (res < bn) ? 0 : 1
+    p.bn = d->bn;
+    p.out_bits = d->output;
+    const int ow = step32(p.N);
+    if (d->ahead_fc) {
+        const int ow128 = kw128(p.N);
+        p.bits_pix_stride = ow128;
+        p.bits_b_stride = (long long)p.OH * p.OW * ow128;
+        p.bits_row_words = ow128;
+    } else {
+        p.bits_pix_stride = (long long)p.B * ow;
+        p.bits_b_stride = ow;
+        p.bits_row_words = ow;
+    }
+    if (d->inject_residual) {
+        TCBNN_NOTNULL(d->input_residual);
+        TCBNN_REQUIRE(d->input_residual_channels > 0, "conv128: input_residual_channels unset");
+        TCBNN_REQUIRE(d->residual_channels >= 0, "conv128: negative residual_channels");
+        p.res_in = d->input_residual;
+        p.res_in_ch = d->input_residual_channels;
+        p.res_limit = d->residual_channels;
+        p.res_pool = d->residual_pool ? 1 : 0;
+    }
+    if (d->save_residual) {
+        TCBNN_NOTNULL(d->output_residual);
+        p.res_out = d->output_residual;
+    }
+    return run_bgemm(p, d->variant, (hipStream_t)stream);
+}
+
+int tcbnn_bmm(const uint32_t* a, const uint32_t* b, int32_t* c, int m, int n, int k, int variant,
+              void* stream) {
+    TCBNN_NOTNULL(a);
+    TCBNN_NOTNULL(b);
+    TCBNN_NOTNULL(c);
+    TCBNN_REQUIRE(m > 0 && n > 0 && k > 0, "bmm: empty dimension");
+    TCBNN_REQUIRE(k % 32 == 0, "bmm: K must be a multiple of 32");
+    TCBNN_REQUIRE(n % 32 == 0, "bmm: N must be a multiple of 32 (B holds one packed row per column)");
+    BgemmParams p;
+    memset(&p, 0, sizeof(p));
+    p.act = a;
+    p.wgt = b;
+    p.H = p.W = 1;
+    p.B = m;
+    p.cw = k / 32;
+    p.R = p.S = 1;
+    p.stride_h = p.stride_w = 1;
+    p.PH = p.PW = p.OH = p.OW = 1;
+    p.pool_h = p.pool_w = 1;
+    p.N = n;
+    p.k_tap = k;
+    p.mode = EPI_RAW;
+    p.out_i32 = c;
+    p.raw_pix_stride = 0;
+    p.raw_b_stride = n;
+    return run_bgemm(p, variant, (hipStream_t)stream);
+}
+
+int tcbnn_bconv(const uint32_t* input, const uint32_t* filter, int32_t* output, int batch,
+                int height, int width, int in_ch, int out_ch, int r, int s, int stride_h,
+                int stride_w, int pad_h, int pad_w, int out_h, int out_w, int variant,
+                void* stream) {
+    TCBNN_NOTNULL(input);
+    TCBNN_NOTNULL(filter);
+    TCBNN_NOTNULL(output);
+    TCBNN_REQUIRE(batch > 0 && height > 0 && width > 0 && in_ch > 0 && out_ch > 0 && r > 0 &&
+                      s > 0 && stride_h > 0 && stride_w > 0 && out_h > 0 && out_w > 0 &&
+                      pad_h >= 0 && pad_w >= 0,
+                  "bconv: bad shape");
+    BgemmParams p;
+    memset(&p, 0, sizeof(p));
+    p.act = input;
+    p.wgt = filter;
+    p.H = height;
+    p.W = width;
+    p.B = batch;
+    p.cw = step32(in_ch);
+    p.R = r;
+    p.S = s;
+    p.stride_h = stride_h;
+    p.stride_w = stride_w;
+    p.pad_h = pad_h;
+    p.pad_w = pad_w;
+    p.PH = p.OH = out_h;
+    p.PW = p.OW = out_w;
+    p.pool_h = p.pool_w = 1;
+    p.N = out_ch;
+    p.k_tap = in_ch;
+    p.mode = EPI_RAW;
+    p.out_i32 = output;
+    p.raw_pix_stride = out_ch;
+    p.raw_b_stride = (long long)out_h * out_w * out_ch;
+    return run_bgemm(p, variant, (hipStream_t)stream);
+}
+
+}  // extern "C"

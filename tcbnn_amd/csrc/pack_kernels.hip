@@ -1,0 +1,326 @@
+// Binarise / pack / unpack / layout-conversion kernels (HBM-bound byte work).
+// Packing rule everywhere: bit = (value >= 0), element e of a 32-group is bit
+// (31 - e) of its word, pad bits are 0 (kernel.cuh:165-170, param.h:58-61).
+#include "common.h"
+
+namespace tcbnn {
+namespace {
+
+constexpr int kThreads = 256;
+
+inline unsigned blocks_for(long long n, int per_block = kThreads) {
+    long long b = (n + per_block - 1) / per_block;
+    if (b < 1) b = 1;
+    return (unsigned)b;
+}
+
+// One wave binarises 64 consecutive elements of one row with a ballot:
+// a fully coalesced 256-byte read yields two MSB-first words.
+// src element (row, k) at src[row*row_stride + k*k_stride].
+__global__ __launch_bounds__(kThreads) void pack_rows_kernel(const float* __restrict__ src,
+                                                             uint32_t* __restrict__ dst,
+                                                             long long rows, int k,
+                                                             long long row_stride,
+                                                             long long k_stride, int k_words) {
+    const int lane = threadIdx.x & 63;
+    const long long wave = ((long long)blockIdx.x * kThreads + threadIdx.x) >> 6;
+    const int segs = (k_words + 1) >> 1;  // 64-element segments per row
+    if (wave >= rows * segs) return;
+    const long long row = wave / segs;
+    const int seg = (int)(wave - row * segs);
+    const int kk = seg * 64 + lane;
+    const float f = kk < k ? src[row * row_stride + kk * k_stride] : -1.0f;
+    const unsigned long long m = __ballot(f >= 0.0f);
+    if (lane == 0) {
+        dst[row * k_words + 2 * seg] = __brev((unsigned)(m & 0xffffffffull));
+        if (2 * seg + 1 < k_words) dst[row * k_words + 2 * seg + 1] = __brev((unsigned)(m >> 32));
+    }
+}
+
+// HWIO fp32 filter -> [opad32][R*S][cw]; one thread per output word.
+__global__ void pack_conv_filter_kernel(const float* __restrict__ f, uint32_t* __restrict__ dst,
+                                        int taps, int in_ch, int out_ch, int cw, int opad) {
+    const long long idx = (long long)blockIdx.x * kThreads + threadIdx.x;
+    if (idx >= (long long)opad * taps * cw) return;
+    const int w = (int)(idx % cw);
+    const int t = (int)((idx / cw) % taps);
+    const int o = (int)(idx / ((long long)cw * taps));
+    uint32_t word = 0;
+    if (o < out_ch) {
+        for (int e = 0; e < 32; ++e) {
+            const int c = w * 32 + e;
+            if (c < in_ch && f[((size_t)t * in_ch + c) * out_ch + o] >= 0.0f) word |= 1u << (31 - e);
+        }
+    }
+    dst[idx] = word;
+}
+
+// HWIO fp32 [R*S][C<=4][O] -> sign masks [R*S][opad32][4].
+__global__ void pack_inconv_filter_kernel(const float* __restrict__ f, uint32_t* __restrict__ dst,
+                                          int taps, int in_ch, int out_ch, int opad) {
+    const long long idx = (long long)blockIdx.x * kThreads + threadIdx.x;
+    if (idx >= (long long)taps * opad * 4) return;
+    const int c = (int)(idx & 3);
+    const int o = (int)((idx >> 2) % opad);
+    const int t = (int)((idx >> 2) / opad);
+    uint32_t m = 0;
+    // padded channels / outputs behave like the reference's -1.0f fill (param.h:626-627)
+    if (c < in_ch) {
+        const float v = o < out_ch ? f[((size_t)t * in_ch + c) * out_ch + o] : -1.0f;
+        m = v >= 0.0f ? 0u : 0x80000000u;
+    }
+    dst[idx] = m;
+}
+
+// NHWC fp32 -> [H][W][B][cw]; one thread per output word.
+__global__ void pack_conv_input_nhwc_kernel(const float* __restrict__ src,
+                                            uint32_t* __restrict__ dst, int batch, int height,
+                                            int width, int ch, int cw) {
+    const long long idx = (long long)blockIdx.x * kThreads + threadIdx.x;
+    const long long total = (long long)height * width * batch * cw;
+    if (idx >= total) return;
+    const int w = (int)(idx % cw);
+    const int b = (int)((idx / cw) % batch);
+    const long long pix = idx / ((long long)cw * batch);
+    const float* s = src + ((size_t)b * height * width + pix) * ch + w * 32;
+    uint32_t word = 0;
+    for (int e = 0; e < 32 && w * 32 + e < ch; ++e)
+        if (s[e] >= 0.0f) word |= 1u << (31 - e);
+    dst[idx] = word;
+}
+
+__global__ void unpack_fc_kernel(const uint32_t* __restrict__ packed, float* __restrict__ out,
+                                 int batch, int features, int kw) {
+    const long long idx = (long long)blockIdx.x * kThreads + threadIdx.x;
+    if (idx >= (long long)batch * features) return;
+    const int k = (int)(idx % features);
+    const long long b = idx / features;
+    const uint32_t w = packed[b * kw + (k >> 5)];
+    out[idx] = 2.0f * (float)((w >> (31 - (k & 31))) & 1u) - 1.0f;
+}
+
+__global__ void unpack_conv_kernel(const uint32_t* __restrict__ packed, float* __restrict__ out,
+                                   int height, int width, int ch, int batch, int cw) {
+    const long long idx = (long long)blockIdx.x * kThreads + threadIdx.x;  // NHWC index
+    const long long total = (long long)batch * height * width * ch;
+    if (idx >= total) return;
+    const int c = (int)(idx % ch);
+    const long long pix = (idx / ch) % ((long long)height * width);
+    const long long b = idx / ((long long)ch * height * width);
+    const uint32_t w = packed[(pix * batch + b) * cw + (c >> 5)];
+    out[idx] = 2.0f * (float)((w >> (31 - (c & 31))) & 1u) - 1.0f;
+}
+
+// engine rows [rows][row_words] <-> reference tiles [groups][ceil(rows/8)][row128][8][4]
+// where `groups` is the number of leading (pixel) blocks, each holding `rows` rows.
+// to_fmt != 0: fmt is written (zero where the engine has no word); else packed is written.
+__global__ void fmt_convert_kernel(uint32_t* __restrict__ packed, uint32_t* __restrict__ fmt,
+                                   long long groups, int rows, int row_words, int row128,
+                                   int to_fmt) {
+    const int rows8 = (rows + 7) >> 3;
+    const long long per_group = (long long)rows8 * row128 * 32;
+    const long long idx = (long long)blockIdx.x * kThreads + threadIdx.x;  // fmt index
+    if (idx >= groups * per_group) return;
+    const long long g = idx / per_group;
+    const int rem = (int)(idx - g * per_group);
+    const int w = rem & 3;
+    const int r = (rem >> 2) & 7;
+    const int tile = rem >> 5;
+    const int kc = tile % row128;
+    const int rt = tile / row128;
+    const int row = rt * 8 + r;
+    const int word = kc * 4 + w;
+    const bool has = row < rows && word < row_words;
+    const long long pidx = (g * rows + row) * row_words + word;
+    if (to_fmt)
+        fmt[idx] = has ? packed[pidx] : 0u;
+    else if (has)
+        packed[pidx] = fmt[idx];
+}
+
+__global__ void residual_to_reference_kernel(const int32_t* __restrict__ res,
+                                             int32_t* __restrict__ ref, long long pixels,
+                                             int batch, int ch, int b8, int c128) {
+    const long long idx = (long long)blockIdx.x * kThreads + threadIdx.x;
+    if (idx >= pixels * b8 * c128) return;
+    const int c = (int)(idx % c128);
+    const int b = (int)((idx / c128) % b8);
+    const long long pix = idx / ((long long)c128 * b8);
+    ref[idx] = (b < batch && c < ch) ? res[(pix * batch + b) * ch + c] : 0;
+}
+
+}  // namespace
+}  // namespace tcbnn
+
+using namespace tcbnn;
+
+extern "C" {
+
+int tcbnn_pack_rows(const float* src, uint32_t* packed, int rows, int k, int ld, int k_words,
+                    void* stream) {
+    TCBNN_NOTNULL(src);
+    TCBNN_NOTNULL(packed);
+    TCBNN_REQUIRE(rows > 0 && k > 0 && ld >= k && k_words >= step32(k), "pack_rows: bad shape");
+    const long long waves = (long long)rows * ((k_words + 1) / 2);
+    hipLaunchKernelGGL(pack_rows_kernel, dim3(blocks_for(waves * 64)), dim3(kThreads), 0,
+                       (hipStream_t)stream, src, packed, (long long)rows, k, (long long)ld, 1LL,
+                       k_words);
+    TCBNN_LAUNCH_CHECK("pack_rows_kernel");
+    return TCBNN_OK;
+}
+
+int tcbnn_pack_cols(const float* src, uint32_t* packed, int k, int n, int k_words, void* stream) {
+    TCBNN_NOTNULL(src);
+    TCBNN_NOTNULL(packed);
+    TCBNN_REQUIRE(k > 0 && n > 0 && k_words >= step32(k), "pack_cols: bad shape");
+    const long long waves = (long long)n * ((k_words + 1) / 2);
+    hipLaunchKernelGGL(pack_rows_kernel, dim3(blocks_for(waves * 64)), dim3(kThreads), 0,
+                       (hipStream_t)stream, src, packed, (long long)n, k, 1LL, (long long)n,
+                       k_words);
+    TCBNN_LAUNCH_CHECK("pack_cols_kernel");
+    return TCBNN_OK;
+}
+
+int tcbnn_pack_fc_weight(const float* weight_kn, uint32_t* packed, int in_features,
+                         int out_features, void* stream) {
+    TCBNN_NOTNULL(weight_kn);
+    TCBNN_NOTNULL(packed);
+    TCBNN_REQUIRE(in_features > 0 && out_features > 0, "pack_fc_weight: bad shape");
+    const int kw = kw128(in_features);
+    const int npad = pad32(out_features);
+    if (int rc = check_hip(hipMemsetAsync(packed, 0, (size_t)npad * kw * 4, (hipStream_t)stream),
+                           "hipMemsetAsync"))
+        return rc;
+    return tcbnn_pack_cols(weight_kn, packed, in_features, out_features, kw, stream);
+}
+
+int tcbnn_pack_conv_filter(const float* filter_hwio, uint32_t* packed, int r, int s, int in_ch,
+                           int out_ch, void* stream) {
+    TCBNN_NOTNULL(filter_hwio);
+    TCBNN_NOTNULL(packed);
+    TCBNN_REQUIRE(r > 0 && s > 0 && in_ch > 0 && out_ch > 0, "pack_conv_filter: bad shape");
+    const int cw = step32(in_ch), opad = pad32(out_ch);
+    const long long total = (long long)opad * r * s * cw;
+    hipLaunchKernelGGL(pack_conv_filter_kernel, dim3(blocks_for(total)), dim3(kThreads), 0,
+                       (hipStream_t)stream, filter_hwio, packed, r * s, in_ch, out_ch, cw, opad);
+    TCBNN_LAUNCH_CHECK("pack_conv_filter_kernel");
+    return TCBNN_OK;
+}
+
+int tcbnn_pack_inconv_filter(const float* filter_hwio, uint32_t* packed, int r, int s, int in_ch,
+                             int out_ch, void* stream) {
+    TCBNN_NOTNULL(filter_hwio);
+    TCBNN_NOTNULL(packed);
+    TCBNN_REQUIRE(r > 0 && s > 0 && out_ch > 0, "pack_inconv_filter: bad shape");
+    TCBNN_REQUIRE(in_ch == 3, "first-layer convolution has 3 input channels (kernel.cuh:620-625)");
+    const int opad = pad32(out_ch);
+    const long long total = (long long)r * s * opad * 4;
+    hipLaunchKernelGGL(pack_inconv_filter_kernel, dim3(blocks_for(total)), dim3(kThreads), 0,
+                       (hipStream_t)stream, filter_hwio, packed, r * s, in_ch, out_ch, opad);
+    TCBNN_LAUNCH_CHECK("pack_inconv_filter_kernel");
+    return TCBNN_OK;
+}
+
+int tcbnn_pack_conv_input_nhwc(const float* src, uint32_t* packed, int batch, int height,
+                               int width, int ch, void* stream) {
+    TCBNN_NOTNULL(src);
+    TCBNN_NOTNULL(packed);
+    TCBNN_REQUIRE(batch > 0 && height > 0 && width > 0 && ch > 0, "pack_conv_input: bad shape");
+    const int cw = step32(ch);
+    const long long total = (long long)height * width * batch * cw;
+    hipLaunchKernelGGL(pack_conv_input_nhwc_kernel, dim3(blocks_for(total)), dim3(kThreads), 0,
+                       (hipStream_t)stream, src, packed, batch, height, width, ch, cw);
+    TCBNN_LAUNCH_CHECK("pack_conv_input_nhwc_kernel");
+    return TCBNN_OK;
+}
+
+int tcbnn_in128_forward(const tcbnn_in128_desc* d, void* stream) {
+    TCBNN_NOTNULL(d);
+    TCBNN_NOTNULL(d->input);
+    TCBNN_NOTNULL(d->output);
+    TCBNN_REQUIRE(d->input_height > 0 && d->input_width > 0, "in128: bad shape");
+    return tcbnn_pack_rows(d->input, d->output, d->input_height, d->input_width, d->input_width,
+                           kw128(d->input_width), stream);
+}
+
+int tcbnn_unpack_fc_output(const uint32_t* packed, float* out, int batch, int features,
+                           void* stream) {
+    TCBNN_NOTNULL(packed);
+    TCBNN_NOTNULL(out);
+    TCBNN_REQUIRE(batch > 0 && features > 0, "unpack_fc: bad shape");
+    hipLaunchKernelGGL(unpack_fc_kernel, dim3(blocks_for((long long)batch * features)),
+                       dim3(kThreads), 0, (hipStream_t)stream, packed, out, batch, features,
+                       kw128(features));
+    TCBNN_LAUNCH_CHECK("unpack_fc_kernel");
+    return TCBNN_OK;
+}
+
+int tcbnn_unpack_conv_output(const uint32_t* packed, float* out, int height, int width, int ch,
+                             int batch, void* stream) {
+    TCBNN_NOTNULL(packed);
+    TCBNN_NOTNULL(out);
+    TCBNN_REQUIRE(batch > 0 && height > 0 && width > 0 && ch > 0, "unpack_conv: bad shape");
+    const long long total = (long long)batch * height * width * ch;
+    hipLaunchKernelGGL(unpack_conv_kernel, dim3(blocks_for(total)), dim3(kThreads), 0,
+                       (hipStream_t)stream, packed, out, height, width, ch, batch, step32(ch));
+    TCBNN_LAUNCH_CHECK("unpack_conv_kernel");
+    return TCBNN_OK;
+}
+
+static int fmt_convert(uint32_t* packed, uint32_t* fmt, long long groups, int rows, int row_words,
+                       int row128, int to_fmt, void* stream) {
+    const long long total = groups * ((rows + 7) / 8) * row128 * 32;
+    hipLaunchKernelGGL(fmt_convert_kernel, dim3(blocks_for(total)), dim3(kThreads), 0,
+                       (hipStream_t)stream, packed, fmt, groups, rows, row_words, row128, to_fmt);
+    TCBNN_LAUNCH_CHECK("fmt_convert_kernel");
+    return TCBNN_OK;
+}
+
+int tcbnn_fc_to_reference_fmt(const uint32_t* packed, uint32_t* fmt, int batch, int features,
+                              void* stream) {
+    TCBNN_NOTNULL(packed);
+    TCBNN_NOTNULL(fmt);
+    TCBNN_REQUIRE(batch > 0 && features > 0, "fc_to_reference_fmt: bad shape");
+    return fmt_convert(const_cast<uint32_t*>(packed), fmt, 1, batch, kw128(features),
+                       step128(features), 1, stream);
+}
+int tcbnn_fc_from_reference_fmt(const uint32_t* fmt, uint32_t* packed, int batch, int features,
+                                void* stream) {
+    TCBNN_NOTNULL(packed);
+    TCBNN_NOTNULL(fmt);
+    TCBNN_REQUIRE(batch > 0 && features > 0, "fc_from_reference_fmt: bad shape");
+    return fmt_convert(packed, const_cast<uint32_t*>(fmt), 1, batch, kw128(features),
+                       step128(features), 0, stream);
+}
+int tcbnn_conv_to_reference_fmt(const uint32_t* packed, uint32_t* fmt, int height, int width,
+                                int batch, int ch, void* stream) {
+    TCBNN_NOTNULL(packed);
+    TCBNN_NOTNULL(fmt);
+    TCBNN_REQUIRE(batch > 0 && height > 0 && width > 0 && ch > 0, "conv_to_reference_fmt: bad shape");
+    return fmt_convert(const_cast<uint32_t*>(packed), fmt, (long long)height * width, batch,
+                       step32(ch), step128(ch), 1, stream);
+}
+int tcbnn_conv_from_reference_fmt(const uint32_t* fmt, uint32_t* packed, int height, int width,
+                                  int batch, int ch, void* stream) {
+    TCBNN_NOTNULL(packed);
+    TCBNN_NOTNULL(fmt);
+    TCBNN_REQUIRE(batch > 0 && height > 0 && width > 0 && ch > 0,
+                  "conv_from_reference_fmt: bad shape");
+    return fmt_convert(packed, const_cast<uint32_t*>(fmt), (long long)height * width, batch,
+                       step32(ch), step128(ch), 0, stream);
+}
+
+int tcbnn_residual_to_reference(const int32_t* res, int32_t* ref, int height, int width, int batch,
+                                int ch, void* stream) {
+    TCBNN_NOTNULL(res);
+    TCBNN_NOTNULL(ref);
+    TCBNN_REQUIRE(batch > 0 && height > 0 && width > 0 && ch > 0, "residual_to_reference: bad shape");
+    const long long pixels = (long long)height * width;
+    const long long total = pixels * pad8(batch) * pad128(ch);
+    hipLaunchKernelGGL(residual_to_reference_kernel, dim3(blocks_for(total)), dim3(kThreads), 0,
+                       (hipStream_t)stream, res, ref, pixels, batch, ch, pad8(batch), pad128(ch));
+    TCBNN_LAUNCH_CHECK("residual_to_reference_kernel");
+    return TCBNN_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,491 @@
+"""Python host mirror of the reference's layer objects (param.h:115-1065).
+
+Same class names, constructor arguments, public field names and method names as
+In128LayerParam / Fc128LayerParam / Out128LayerParam / InConv128LayerParam /
+Conv128LayerParam.  Differences forced by the redesign:
+  * `initialize` takes a weight source with a `launch_array(n)` method (the
+    reference reads a FILE* with launch_array, utility.h:188-196) and returns self;
+  * each layer has `forward(stream=None)` — one stream-ordered launch — in place of
+    the device function called inside the reference's cooperative network kernel;
+  * `download_output()` returns the packed activations in the reference's
+    tile-contiguous layout (what the reference's download_output() yields);
+    `download_packed()` returns the engine layout.
+All compute goes through the C ABI of libtcbnn_hip.so.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import _lib
+from ._lib import lib, check
+from .device import DeviceBuffer
+
+
+def STEP8(x):
+    return (x + 7) >> 3
+
+
+def STEP32(x):
+    return (x + 31) >> 5
+
+
+def STEP128(x):
+    return (x + 127) >> 7
+
+
+def PAD8(x):
+    return STEP8(x) << 3
+
+
+def PAD32(x):
+    return STEP32(x) << 5
+
+
+def PAD128(x):
+    return STEP128(x) << 7
+
+
+class ArrayWeights:
+    """Weight source over in-memory arrays, consumed strictly in order like the
+    reference's weight file (utility.h:188-196)."""
+
+    def __init__(self, arrays):
+        self._flat = np.concatenate([np.asarray(a, dtype=np.float32).ravel() for a in arrays]) \
+            if arrays else np.zeros(0, np.float32)
+        self._pos = 0
+
+    def launch_array(self, size):
+        if self._pos + size > self._flat.size:
+            raise _lib.TcbnnError("weight source exhausted: need %d more values" % size)
+        out = self._flat[self._pos:self._pos + size]
+        self._pos += size
+        return out
+
+
+class TextWeightFile:
+    """Text file of floats separated by white space and/or commas (the reference's .csv)."""
+
+    def __init__(self, path):
+        with open(path) as f:
+            txt = f.read().replace(",", " ")
+        self._src = ArrayWeights([np.array(txt.split(), dtype=np.float32)])
+
+    def launch_array(self, size):
+        return self._src.launch_array(size)
+
+
+def _stream_handle(stream):
+    return stream.handle if stream is not None else None
+
+
+def _residual_buffer(nbytes, channels, height, width):
+    buf = DeviceBuffer(nbytes)
+    buf.channels, buf.height, buf.width = channels, height, width
+    return buf
+
+
+class In128LayerParam:
+    """param.h:115-222; forward = In128LayerFMT (kernel.cuh:153-172)."""
+
+    def __init__(self, name, input_height, input_width):
+        self.name = name
+        self.input_height = self.output_height = input_height
+        self.input_width = self.output_width = input_width
+        self.input_gpu = self.output_gpu = None
+
+    def output_bit_size(self):
+        return PAD8(self.output_height) * STEP128(self.output_width)
+
+    def output_bit_bytes(self):
+        return self.output_bit_size() * 16
+
+    def initialize(self, input):
+        if input is None:
+            raise _lib.TcbnnError("Error: NULL pointer (input)")
+        x = np.ascontiguousarray(input, dtype=np.float32).reshape(self.input_height, self.input_width)
+        self.input_gpu = DeviceBuffer.from_numpy(x)
+        self.output_gpu = DeviceBuffer(4 * lib.tcbnn_fc_act_words(self.output_height, self.output_width))
+        return self
+
+    def set_input(self, input):
+        self.input_gpu.upload(np.ascontiguousarray(input, dtype=np.float32))
+
+    def get_output_gpu(self):
+        return self.output_gpu
+
+    def forward(self, stream=None):
+        d = _lib.In128Desc(self.input_gpu.ptr, self.output_gpu.ptr, self.input_height, self.input_width)
+        check(lib.tcbnn_in128_forward(C.byref(d), _stream_handle(stream)))
+
+    def download_packed(self):
+        return self.output_gpu.to_numpy(np.uint32, (self.output_height, 4 * STEP128(self.output_width)))
+
+    def download_output(self):
+        return _fc_download_fmt(self.output_gpu, self.output_height, self.output_width)
+
+    def download_full_output(self):
+        return _fc_download_full(self.output_gpu, self.output_height, self.output_width)
+
+    def release(self):
+        for b in (self.input_gpu, self.output_gpu):
+            if b is not None:
+                b.free()
+        self.input_gpu = self.output_gpu = None
+
+
+def _fc_download_fmt(buf, batch, features):
+    words = PAD8(batch) * STEP128(features) * 4
+    tmp = DeviceBuffer(4 * words)
+    check(lib.tcbnn_fc_to_reference_fmt(buf.ptr, tmp.ptr, batch, features, None))
+    _lib.device_synchronize()
+    return tmp.to_numpy(np.uint32, (words,))
+
+
+def _fc_download_full(buf, batch, features):
+    tmp = DeviceBuffer(4 * batch * features)
+    check(lib.tcbnn_unpack_fc_output(buf.ptr, tmp.ptr, batch, features, None))
+    _lib.device_synchronize()
+    return tmp.to_numpy(np.float32, (batch, features))
+
+
+class Fc128LayerParam:
+    """param.h:224-385; forward = Fc128LayerFMT (kernel.cuh:174-226)."""
+
+    def __init__(self, name, input_height, input_width, weight_width, variant=_lib.VARIANT_AUTO):
+        self.name = name
+        self.weight_height, self.weight_width = input_width, weight_width
+        self.input_height, self.input_width = input_height, input_width
+        self.output_height, self.output_width = input_height, weight_width
+        self.bn_width = weight_width
+        self.variant = variant
+        self.weight = self.bn = None
+        self.weight_gpu = self.bn_gpu = self.output_gpu = self.input_gpu = None
+
+    def weight_size(self):
+        return self.weight_height * self.weight_width
+
+    def bn_size(self):
+        return self.bn_width
+
+    def output_bit_size(self):
+        return PAD8(self.output_height) * STEP128(self.output_width)
+
+    def set_input_gpu(self, input_gpu):
+        self.input_gpu = input_gpu
+
+    def initialize(self, config_file, prev_layer_gpu):
+        self.weight = np.array(config_file.launch_array(self.weight_size()), dtype=np.float32)
+        self.weight_gpu = DeviceBuffer(4 * lib.tcbnn_fc_weight_words(self.weight_height, self.weight_width))
+        wf = DeviceBuffer.from_numpy(self.weight)
+        check(lib.tcbnn_pack_fc_weight(wf.ptr, self.weight_gpu.ptr, self.weight_height, self.weight_width, None))
+        _lib.device_synchronize()
+        wf.free()
+        self.bn = np.array(config_file.launch_array(self.bn_size()), dtype=np.float32)
+        self.bn_gpu = DeviceBuffer.from_numpy(self.bn)
+        self.output_gpu = DeviceBuffer(4 * lib.tcbnn_fc_act_words(self.output_height, self.output_width))
+        self.set_input_gpu(prev_layer_gpu)
+        if self.input_gpu is None:
+            raise _lib.TcbnnError("Error: NULL pointer (input_gpu)")
+        return self
+
+    def get_output_gpu(self):
+        return self.output_gpu
+
+    def forward(self, stream=None):
+        d = _lib.Fc128Desc(self.input_gpu.ptr, self.weight_gpu.ptr, self.bn_gpu.ptr, self.output_gpu.ptr,
+                           self.input_height, self.input_width, self.weight_width, self.variant, None, 0)
+        check(lib.tcbnn_fc128_forward(C.byref(d), _stream_handle(stream)))
+
+    def download_packed(self):
+        return self.output_gpu.to_numpy(np.uint32, (self.output_height, 4 * STEP128(self.output_width)))
+
+    def download_output(self):
+        return _fc_download_fmt(self.output_gpu, self.output_height, self.output_width)
+
+    def download_full_output(self):
+        return _fc_download_full(self.output_gpu, self.output_height, self.output_width)
+
+    def release(self):
+        for b in (self.weight_gpu, self.bn_gpu, self.output_gpu):
+            if b is not None:
+                b.free()
+        self.weight_gpu = self.bn_gpu = self.output_gpu = None
+
+
+class Out128LayerParam:
+    """param.h:388-531; forward = Out128LayerFMT (kernel.cuh:230-280)."""
+
+    def __init__(self, name, input_height, input_width, weight_width, variant=_lib.VARIANT_AUTO):
+        self.name = name
+        self.input_height, self.input_width = input_height, input_width
+        self.weight_height, self.weight_width = input_width, weight_width
+        self.output_height, self.output_width = input_height, weight_width
+        self.variant = variant
+        self.weight = self.bn_scale = self.bn_bias = None
+        self.weight_gpu = self.bn_scale_gpu = self.bn_bias_gpu = self.output_gpu = self.input_gpu = None
+
+    def weight_size(self):
+        return self.weight_height * self.weight_width
+
+    def bn_size(self):
+        return self.output_width
+
+    def set_input_gpu(self, input_gpu):
+        self.input_gpu = input_gpu
+
+    def initialize(self, config_file, prev_layer_gpu):
+        self.weight = np.array(config_file.launch_array(self.weight_size()), dtype=np.float32)
+        self.weight_gpu = DeviceBuffer(4 * lib.tcbnn_fc_weight_words(self.weight_height, self.weight_width))
+        wf = DeviceBuffer.from_numpy(self.weight)
+        check(lib.tcbnn_pack_fc_weight(wf.ptr, self.weight_gpu.ptr, self.weight_height, self.weight_width, None))
+        _lib.device_synchronize()
+        wf.free()
+        self.bn_scale = np.array(config_file.launch_array(self.bn_size()), dtype=np.float32)
+        self.bn_scale_gpu = DeviceBuffer.from_numpy(self.bn_scale)
+        self.bn_bias = np.array(config_file.launch_array(self.bn_size()), dtype=np.float32)
+        self.bn_bias_gpu = DeviceBuffer.from_numpy(self.bn_bias)
+        self.output_gpu = DeviceBuffer.zeros(4 * self.output_height * self.output_width)
+        self.set_input_gpu(prev_layer_gpu)
+        if self.input_gpu is None:
+            raise _lib.TcbnnError("Error: NULL pointer (input_gpu)")
+        return self
+
+    def get_output_gpu(self):
+        return self.output_gpu
+
+    def forward(self, stream=None):
+        d = _lib.Out128Desc(self.input_gpu.ptr, self.weight_gpu.ptr, self.bn_scale_gpu.ptr,
+                            self.bn_bias_gpu.ptr, self.output_gpu.ptr, self.input_height,
+                            self.input_width, self.weight_width, self.variant)
+        check(lib.tcbnn_out128_forward(C.byref(d), _stream_handle(stream)))
+
+    def download_output(self):
+        return self.output_gpu.to_numpy(np.float32, (self.output_height, self.output_width))
+
+    def release(self):
+        for b in (self.weight_gpu, self.bn_scale_gpu, self.bn_bias_gpu, self.output_gpu):
+            if b is not None:
+                b.free()
+        self.weight_gpu = self.bn_scale_gpu = self.bn_bias_gpu = self.output_gpu = None
+
+
+class _ConvGeometry:
+    """Derived geometry shared by both conv constructors (param.h:719-728, 897-906)."""
+
+    def _derive(self):
+        self.pad_h = lib.tcbnn_conv_pad(self.input_height, self.filter_height, self.stride_height, int(self.padding))
+        self.pad_w = lib.tcbnn_conv_pad(self.input_width, self.filter_width, self.stride_width, int(self.padding))
+        self.buf_height = lib.tcbnn_conv_out(self.input_height, self.filter_height, self.stride_height, int(self.padding), 1)
+        self.buf_width = lib.tcbnn_conv_out(self.input_width, self.filter_width, self.stride_width, int(self.padding), 1)
+        self.output_height = lib.tcbnn_conv_out(self.input_height, self.filter_height, self.stride_height,
+                                                int(self.padding), self.pool_height)
+        self.output_width = lib.tcbnn_conv_out(self.input_width, self.filter_width, self.stride_width,
+                                               int(self.padding), self.pool_width)
+
+    def filter_size(self):
+        return self.output_channels * self.input_channels * self.filter_height * self.filter_width
+
+    def bn_size(self):
+        return self.output_channels
+
+    def output_bit_size(self):
+        return STEP128(self.output_channels) * self.output_height * self.output_width * PAD8(self.batch)
+
+    def residual_size(self):
+        return PAD128(self.output_channels) * PAD8(self.batch) * self.output_height * self.output_width
+
+    def get_output_gpu(self):
+        return self.output_gpu
+
+    def get_output_residual_gpu(self):
+        return self.output_residual_gpu
+
+    def download_residual(self):
+        """Saved residual in the engine layout int32 [P][Q][B][O]."""
+        return self.output_residual_gpu.to_numpy(
+            np.int32, (self.buf_height, self.buf_width, self.batch, self.output_channels))
+
+    def download_residual_reference(self):
+        """Saved residual in the reference layout int32 [P][Q][PAD8(B)][PAD128(O)]."""
+        shape = (self.buf_height, self.buf_width, PAD8(self.batch), PAD128(self.output_channels))
+        tmp = DeviceBuffer(4 * int(np.prod(shape)))
+        check(lib.tcbnn_residual_to_reference(self.output_residual_gpu.ptr, tmp.ptr, self.buf_height,
+                                              self.buf_width, self.batch, self.output_channels, None))
+        _lib.device_synchronize()
+        return tmp.to_numpy(np.int32, shape)
+
+    def _is_fc_ready(self):
+        return bool(getattr(self, "ahead_fc", False))
+
+    def download_packed(self):
+        if self._is_fc_ready():
+            return self.output_gpu.to_numpy(
+                np.uint32, (self.batch, self.output_height * self.output_width * 4 * STEP128(self.output_channels)))
+        return self.output_gpu.to_numpy(
+            np.uint32, (self.output_height, self.output_width, self.batch, STEP32(self.output_channels)))
+
+    def download_output(self):
+        if self._is_fc_ready():
+            feats = self.output_height * self.output_width * PAD128(self.output_channels)
+            return _fc_download_fmt(self.output_gpu, self.batch, feats)
+        words = self.output_bit_size() * 4
+        tmp = DeviceBuffer(4 * words)
+        check(lib.tcbnn_conv_to_reference_fmt(self.output_gpu.ptr, tmp.ptr, self.output_height,
+                                              self.output_width, self.batch, self.output_channels, None))
+        _lib.device_synchronize()
+        return tmp.to_numpy(np.uint32, (words,))
+
+    def download_full_output(self):
+        """+-1.0f, NHWC [B][OH][OW][O] (UnpackConvOutput32FMT, param.h:661-688)."""
+        if self._is_fc_ready():
+            feats = self.output_height * self.output_width * PAD128(self.output_channels)
+            full = _fc_download_full(self.output_gpu, self.batch, feats)
+            full = full.reshape(self.batch, self.output_height, self.output_width, PAD128(self.output_channels))
+            return np.ascontiguousarray(full[..., :self.output_channels])
+        shape = (self.batch, self.output_height, self.output_width, self.output_channels)
+        tmp = DeviceBuffer(4 * int(np.prod(shape)))
+        check(lib.tcbnn_unpack_conv_output(self.output_gpu.ptr, tmp.ptr, self.output_height, self.output_width,
+                                           self.output_channels, self.batch, None))
+        _lib.device_synchronize()
+        return tmp.to_numpy(np.float32, shape)
+
+
+class InConv128LayerParam(_ConvGeometry):
+    """param.h:701-870; forward = InConv128LayerFMT (kernel.cuh:578-672)."""
+
+    def __init__(self, name, input_height, input_width, filter_height, filter_width, input_channels,
+                 output_channels, batch, stride_height=1, stride_width=1, padding=True, pool_height=1,
+                 pool_width=1, save_residual=False):
+        self.name = name
+        self.input_height, self.input_width = input_height, input_width
+        self.filter_height, self.filter_width = filter_height, filter_width
+        self.input_channels, self.output_channels, self.batch = input_channels, output_channels, batch
+        self.stride_height, self.stride_width = stride_height, stride_width
+        self.padding, self.pool_height, self.pool_width = padding, pool_height, pool_width
+        self.save_residual = save_residual
+        self.filter = self.bn = None
+        self.input_gpu = self.filter_gpu = self.bn_gpu = self.output_gpu = self.output_residual_gpu = None
+        self._derive()
+
+    def input_size(self):
+        return self.input_channels * self.input_height * self.input_width * self.batch
+
+    def initialize(self, input, config_file):
+        if input is None:
+            raise _lib.TcbnnError("Error: NULL pointer (input)")
+        x = np.ascontiguousarray(input, dtype=np.float32)
+        assert x.size == self.input_size(), (x.size, self.input_size())
+        self.input_gpu = DeviceBuffer.from_numpy(x)
+        self.filter = np.array(config_file.launch_array(self.filter_size()), dtype=np.float32)
+        self.filter_gpu = DeviceBuffer(4 * lib.tcbnn_inconv_filter_words(
+            self.filter_height, self.filter_width, self.input_channels, self.output_channels))
+        ff = DeviceBuffer.from_numpy(self.filter)
+        check(lib.tcbnn_pack_inconv_filter(ff.ptr, self.filter_gpu.ptr, self.filter_height, self.filter_width,
+                                           self.input_channels, self.output_channels, None))
+        _lib.device_synchronize()
+        ff.free()
+        self.bn = np.array(config_file.launch_array(self.bn_size()), dtype=np.float32)
+        self.bn_gpu = DeviceBuffer.from_numpy(self.bn)
+        self.output_gpu = DeviceBuffer(4 * lib.tcbnn_conv_act_words(
+            self.output_height, self.output_width, self.batch, self.output_channels))
+        if self.save_residual:
+            self.output_residual_gpu = _residual_buffer(
+                4 * self.buf_height * self.buf_width * self.batch * self.output_channels,
+                self.output_channels, self.buf_height, self.buf_width)
+        return self
+
+    def set_input(self, input):
+        self.input_gpu.upload(np.ascontiguousarray(input, dtype=np.float32))
+
+    def forward(self, stream=None):
+        d = _lib.InConv128Desc(
+            self.input_gpu.ptr, self.filter_gpu.ptr, self.bn_gpu.ptr, self.output_gpu.ptr,
+            self.output_residual_gpu.ptr if self.output_residual_gpu is not None else None,
+            self.input_height, self.input_width, self.input_channels, self.filter_height, self.filter_width,
+            self.output_channels, self.batch, self.stride_height, self.stride_width, int(self.padding),
+            self.pool_height, self.pool_width, int(self.save_residual))
+        check(lib.tcbnn_inconv128_forward(C.byref(d), _stream_handle(stream)))
+
+    def release(self):
+        for b in (self.input_gpu, self.filter_gpu, self.bn_gpu, self.output_gpu, self.output_residual_gpu):
+            if b is not None:
+                b.free()
+        self.input_gpu = self.filter_gpu = self.bn_gpu = self.output_gpu = self.output_residual_gpu = None
+
+
+class Conv128LayerParam(_ConvGeometry):
+    """param.h:872-1065; forward = Conv128LayerFMT (kernel.cuh:676-827)."""
+
+    def __init__(self, name, input_height, input_width, filter_height, filter_width, input_channels,
+                 output_channels, batch, stride_height=1, stride_width=1, padding=True, pool_height=1,
+                 pool_width=1, ahead_fc=False, save_residual=False, inject_residual=False,
+                 residual_channels=0, residual_pool=False, variant=_lib.VARIANT_AUTO):
+        self.name = name
+        self.input_height, self.input_width = input_height, input_width
+        self.filter_height, self.filter_width = filter_height, filter_width
+        self.input_channels, self.output_channels, self.batch = input_channels, output_channels, batch
+        self.stride_height, self.stride_width = stride_height, stride_width
+        self.padding, self.pool_height, self.pool_width = padding, pool_height, pool_width
+        self.ahead_fc, self.save_residual, self.inject_residual = ahead_fc, save_residual, inject_residual
+        self.residual_channels, self.residual_pool = residual_channels, residual_pool
+        self.variant = variant
+        self.filter = self.bn = None
+        self.input_gpu = self.filter_gpu = self.bn_gpu = self.output_gpu = None
+        self.output_residual_gpu = self.input_residual_gpu = None
+        self._derive()
+
+    def set_input_gpu(self, input_gpu):
+        self.input_gpu = input_gpu
+
+    def set_input_residual_gpu(self, input_residual_gpu):
+        self.input_residual_gpu = input_residual_gpu
+
+    def initialize(self, config_file, prev_layer_gpu, input_residual_gpu=None):
+        self.filter = np.array(config_file.launch_array(self.filter_size()), dtype=np.float32)
+        self.filter_gpu = DeviceBuffer(4 * lib.tcbnn_conv_filter_words(
+            self.filter_height, self.filter_width, self.input_channels, self.output_channels))
+        ff = DeviceBuffer.from_numpy(self.filter)
+        check(lib.tcbnn_pack_conv_filter(ff.ptr, self.filter_gpu.ptr, self.filter_height, self.filter_width,
+                                         self.input_channels, self.output_channels, None))
+        _lib.device_synchronize()
+        ff.free()
+        self.bn = np.array(config_file.launch_array(self.bn_size()), dtype=np.float32)
+        self.bn_gpu = DeviceBuffer.from_numpy(self.bn)
+        if self.ahead_fc:
+            words = lib.tcbnn_fc_act_words(
+                self.batch, self.output_height * self.output_width * PAD128(self.output_channels))
+        else:
+            words = lib.tcbnn_conv_act_words(self.output_height, self.output_width, self.batch,
+                                             self.output_channels)
+        self.output_gpu = DeviceBuffer(4 * words)
+        self.set_input_gpu(prev_layer_gpu)
+        if self.save_residual:
+            self.output_residual_gpu = _residual_buffer(
+                4 * self.buf_height * self.buf_width * self.batch * self.output_channels,
+                self.output_channels, self.buf_height, self.buf_width)
+        if self.inject_residual:
+            self.set_input_residual_gpu(input_residual_gpu)
+            if self.input_residual_gpu is None:
+                raise _lib.TcbnnError("Error: NULL pointer (input_residual_gpu)")
+        if self.input_gpu is None:
+            raise _lib.TcbnnError("Error: NULL pointer (input_gpu)")
+        return self
+
+    def forward(self, stream=None):
+        rin = self.input_residual_gpu if self.inject_residual else None
+        d = _lib.Conv128Desc(
+            self.input_gpu.ptr, self.filter_gpu.ptr, self.bn_gpu.ptr, self.output_gpu.ptr,
+            rin.ptr if rin is not None else None,
+            self.output_residual_gpu.ptr if self.output_residual_gpu is not None else None,
+            self.input_height, self.input_width, self.input_channels, self.filter_height, self.filter_width,
+            self.output_channels, self.batch, self.stride_height, self.stride_width, int(self.padding),
+            self.pool_height, self.pool_width, int(self.ahead_fc), int(self.save_residual),
+            int(self.inject_residual), self.residual_channels, int(self.residual_pool),
+            rin.channels if rin is not None else 0, self.variant)
+        check(lib.tcbnn_conv128_forward(C.byref(d), _stream_handle(stream)))
+
+    def release(self):
+        for b in (self.filter_gpu, self.bn_gpu, self.output_gpu, self.output_residual_gpu):
+            if b is not None:
+                b.free()
+        self.filter_gpu = self.bn_gpu = self.output_gpu = self.output_residual_gpu = None

@@ -1,0 +1,80 @@
+"""CPU-side checks of the drop-in boundary: the C-ABI library loads and exports every symbol the
+header declares; host-only entry points (geometry, sizes, error reporting) behave."""
+import os
+import re
+
+import pytest
+
+from tests import refmath as rm
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    txt = open(os.path.join(ROOT, "include", "tcbnn_hip.h")).read()
+    txt = re.sub(r"/\*.*?\*/", "", txt, flags=re.S)
+    return sorted(set(re.findall(r"\b(tcbnn_[a-z0-9_]+)\s*\(", txt)))
+
+
+def test_library_exports_every_declared_symbol():
+    from tcbnn_amd import _lib
+    syms = _declared_symbols()
+    assert len(syms) >= 30
+    for s in syms:
+        assert hasattr(_lib.lib, s), "libtcbnn_hip.so does not export %s" % s
+    assert sorted(_lib.ABI) == syms, "Python binding table and header disagree"
+    assert _lib.lib.tcbnn_abi_version() == 1
+
+
+def test_geometry_entry_points_match_reference_formulas():
+    from tcbnn_amd import _lib
+    for h in range(1, 40):
+        for s in (1, 2, 4):
+            for r in (1, 3, 7, 11):
+                for pool in (1, 2):
+                    pad, buf, out = rm.conv_pad_out(h, r, s, True, pool)
+                    assert _lib.lib.tcbnn_conv_pad(h, r, s, 1) == pad
+                    assert _lib.lib.tcbnn_conv_out(h, r, s, 1, pool) == out
+                    assert _lib.lib.tcbnn_conv_pad(h, r, s, 0) == 0
+
+
+def test_size_helpers():
+    from tcbnn_amd import _lib
+    L = _lib.lib
+    assert L.tcbnn_fc_act_words(8192, 784) == 8192 * 28
+    assert L.tcbnn_conv_act_words(56, 56, 256, 64) == 56 * 56 * 256 * 2
+    assert L.tcbnn_fc_weight_words(784, 10) == 32 * 28
+    assert L.tcbnn_conv_filter_words(3, 3, 64, 64) == 64 * 9 * 2
+    assert L.tcbnn_inconv_filter_words(7, 7, 3, 64) == 49 * 64 * 4
+
+
+def test_errors_are_codes_not_exits():
+    from tcbnn_amd import _lib
+    L = _lib.lib
+    assert L.tcbnn_fc128_forward(None, None) == -2
+    assert b"NULL" in L.tcbnn_last_error()
+    d = _lib.Fc128Desc(1, 1, 1, 1, 0, 128, 128, 0, None, 0)  # batch 0; never launches
+    assert L.tcbnn_fc128_forward(d, None) == -1
+    assert L.tcbnn_bmm(1, 1, 1, 8, 8, 100, 1, None) == -1  # K not a multiple of 32
+    assert L.tcbnn_set_default_variant(99) == -1
+    with pytest.raises(_lib.TcbnnError):
+        _lib.check(-1)
+
+
+def test_network_specs_match_reference_wiring():
+    from tcbnn_amd import nets
+    spec = nets.imagenet_resnet_spec(batch=256)
+    assert len(spec) == 19
+    by = {L["name"]: L for L in spec}
+    assert by["Conv1"]["stride"] == 4 and by["Conv1"]["save_residual"]
+    assert by["L2B1C2"]["residual_pool"] and by["L2B1C2"]["res_src"] == "L1B2C2"
+    assert by["L3B1C2"]["residual_channels"] == 128 and by["L4B1C2"]["residual_channels"] == 256
+    assert by["L1B2C2"]["residual_channels"] == 128 and by["L4B2C2"]["ahead_fc"]
+    assert by["Fc1"]["inp"] == 7 * 7 * 512
+    bops, flops = nets.binary_ops(spec)
+    assert abs(bops / 256 / 1e9 - 3.379) < 0.01  # binary ops per image
+    assert abs(flops / 1e9 - 15.1) < 0.1
+    bops, _ = nets.binary_ops(nets.mnist_mlp_spec(8192))
+    assert abs(bops / 1e9 - 47.68) < 0.05
+    bops, _ = nets.binary_ops(nets.cifar10_vgg_spec(256))
+    assert abs(bops / 1e9 - 314.1) < 0.5

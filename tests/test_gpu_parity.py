@@ -1,0 +1,338 @@
+"""Parity of the HIP path (through the C ABI) with the CPU oracle: bit-exact for popcount
+accumulators, packed activations and int32 residuals; fp32 logits to 1e-5 relative (they are in
+fact bit-identical: multiply and add are separately rounded on both sides)."""
+import numpy as np
+import pytest
+
+from oracle import orc
+from oracle import nets as orc_nets
+from tests import gpuops, refmath as rm
+
+pytestmark = pytest.mark.gpu
+
+VARIANTS = ["popc"]
+
+
+def rng(seed):
+    return np.random.default_rng(seed)
+
+
+def _variant(gpu, name):
+    return gpu.VARIANTS[name]
+
+
+# --------------------------------------------------------------------------- standalone GEMM
+@pytest.mark.parametrize("variant", VARIANTS)
+@pytest.mark.parametrize("m,n,k", [(1024, 1024, 1024), (8, 32, 32), (100, 64, 96), (77, 160, 1056),
+                                   (300, 32, 4096), (64, 32, 64)])
+def test_bmm(gpu, variant, m, n, k):
+    r = rng(m + n + k)
+    a = r.integers(0, 2 ** 32, size=(m, k // 32), dtype=np.uint64).astype(np.uint32)
+    b = r.integers(0, 2 ** 32, size=(n, k // 32), dtype=np.uint64).astype(np.uint32)
+    got = gpuops.bmm(a, b, m, n, k, _variant(gpu, variant))
+    np.testing.assert_array_equal(got, orc.bmm(a, b, k))
+
+
+# --------------------------------------------------------------------------- In / Fc / Out layers
+@pytest.mark.parametrize("b,k", [(8, 784), (100, 128), (8192, 784), (3, 1000)])
+def test_in128(gpu, b, k):
+    x = rng(b + k).standard_normal((b, k)).astype(np.float32)
+    x[0, :3] = [0.0, -0.0, 1e-30]
+    layer = gpu.In128LayerParam("Fin", b, k).initialize(x)
+    layer.forward()
+    want = orc.in128(x)
+    np.testing.assert_array_equal(layer.download_packed(), want)
+    np.testing.assert_array_equal(layer.download_output(), orc.fc_to_fmt(want, b, k))
+    np.testing.assert_array_equal(layer.download_full_output(), np.where(x >= 0, 1.0, -1.0))
+    layer.release()
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+@pytest.mark.parametrize("b,k,n", [(8, 128, 128), (64, 784, 1024), (100, 1024, 1024), (13, 300, 100),
+                                   (256, 2048, 160), (130, 25088, 64), (1000, 1024, 32)])
+def test_fc128(gpu, variant, b, k, n):
+    r = rng(b + k + n)
+    x = r.standard_normal((b, k)).astype(np.float32)
+    w = rm.pm1(r, (k, n))
+    bn = r.normal(0, np.sqrt(k), n).astype(np.float32)
+    wl = orc.pack_fc_weight(w)
+    _, acc = orc.fc128(orc.in128(x), wl, bn, k, n, want_acc=True)
+    bn[: min(n, 8)] = (k - 2 * acc)[0, : min(n, 8)]  # exact ties
+    want = orc.fc128(orc.in128(x), wl, bn, k, n)
+    inp = gpuops.in128(x)
+    wbuf = gpuops.pack_fc_weight(w)
+    out = gpuops.fc128(inp, wbuf, bn, b, k, n, _variant(gpu, variant))
+    got = out.to_numpy(np.uint32, (b, orc.kw128(n)))
+    np.testing.assert_array_equal(got, want)
+    # packed weights agree with the oracle's packing (rows >= N are zero)
+    wg = wbuf.to_numpy(np.uint32, (((n + 31) // 32) * 32, orc.kw128(k)))
+    np.testing.assert_array_equal(wg[:n], wl)
+    assert not wg[n:].any()
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+def test_fc128_nan_threshold(gpu, variant):
+    r = rng(3)
+    x = r.standard_normal((8, 128)).astype(np.float32)
+    w = rm.pm1(r, (128, 32))
+    bn = np.full(32, np.nan, np.float32)
+    out = gpuops.fc128(gpuops.in128(x), gpuops.pack_fc_weight(w), bn, 8, 128, 32, _variant(gpu, variant))
+    assert not out.to_numpy(np.uint32, (8, 4)).any()
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+@pytest.mark.parametrize("b,k,n", [(8, 1024, 10), (256, 512, 1000), (70, 300, 33), (8192, 1024, 10)])
+def test_out128(gpu, variant, b, k, n):
+    r = rng(b + k + n)
+    x = r.standard_normal((b, k)).astype(np.float32)
+    w = rm.pm1(r, (k, n))
+    scale = r.normal(1, 0.1, n).astype(np.float32)
+    bias = r.normal(0, 1, n).astype(np.float32)
+    want = orc.out128(orc.in128(x), orc.pack_fc_weight(w), scale, bias, k, n)
+    got = gpuops.out128(gpuops.in128(x), gpuops.pack_fc_weight(w), scale, bias, b, k, n, _variant(gpu, variant))
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=0)  # tolerance stated by the target
+    np.testing.assert_array_equal(got, want)  # and in fact bit-identical
+
+
+# --------------------------------------------------------------------------- standalone conv
+SWEEP = [(32, 128), (16, 256), (8, 512), (56, 64), (28, 128), (14, 256), (7, 512)]
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+@pytest.mark.parametrize("h,c", SWEEP)
+def test_bconv_sweep_shapes(gpu, variant, h, c):
+    """The 3x3 stride-1 pad-1 sweep shapes at a batch the CPU oracle finishes in seconds."""
+    b = 8 if h > 16 else 24
+    r = rng(h + c)
+    x = rm.pm1(r, (b, h, h, c))
+    f = rm.pm1(r, (3, 3, c, c))
+    pad, buf, _ = orc.conv_geometry(h, 3, 1)
+    want = orc.bconv(orc.pack_conv_input_nhwc(x), orc.pack_conv_filter(f), c, c, 3, 3, 1, pad, buf, buf)
+    inp, filt = gpuops.pack_conv_input(x), gpuops.pack_conv_filter(f)
+    np.testing.assert_array_equal(inp.to_numpy(np.uint32, (h, h, b, c // 32)), orc.pack_conv_input_nhwc(x))
+    got = gpuops.bconv(inp, filt, b, h, h, c, c, 3, 3, 1, pad, buf, buf, _variant(gpu, variant))
+    np.testing.assert_array_equal(got, want)
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+@pytest.mark.parametrize("b,h,cin,cout,R,stride", [(70, 9, 32, 16, 3, 2), (3, 12, 160, 40, 5, 2),
+                                                   (130, 6, 96, 24, 1, 2), (5, 16, 64, 8, 7, 4),
+                                                   (260, 5, 256, 64, 3, 1)])
+def test_bconv_odd_shapes(gpu, variant, b, h, cin, cout, R, stride):
+    r = rng(b + h + cin)
+    x = rm.pm1(r, (b, h, h, cin))
+    f = rm.pm1(r, (R, R, cin, cout))
+    pad, buf, _ = orc.conv_geometry(h, R, stride)
+    want = orc.bconv(orc.pack_conv_input_nhwc(x), orc.pack_conv_filter(f), cin, cout, R, R, stride, pad, buf, buf)
+    got = gpuops.bconv(gpuops.pack_conv_input(x), gpuops.pack_conv_filter(f), b, h, h, cin, cout, R, R, stride,
+                       pad, buf, buf, _variant(gpu, variant))
+    np.testing.assert_array_equal(got, want)
+
+
+# --------------------------------------------------------------------------- Conv128 layer
+class _PackedSource:
+    """Stands in for the previous layer: a device buffer holding packed activations."""
+
+    def __init__(self, packed):
+        self.buf = gpuops.dev(packed)
+
+
+def _run_conv_layer(gpu, variant, x, f, bn, stride=1, pool=1, ahead_fc=False, save_residual=False,
+                    inject_residual=False, residual_channels=0, residual_pool=False, res_in=None):
+    b, h, w, cin = x.shape
+    R, S, _, cout = f.shape
+    layer = gpu.Conv128LayerParam("C", h, w, R, S, cin, cout, b, stride, stride, True, pool, pool, ahead_fc,
+                                  save_residual, inject_residual, residual_channels, residual_pool,
+                                  variant=_variant(gpu, variant))
+    src = gpuops.pack_conv_input(x)
+    rbuf = None
+    if inject_residual:
+        rbuf = gpuops.dev(res_in.astype(np.int32))
+        rbuf.channels = res_in.shape[-1]
+    layer.initialize(gpu.ArrayWeights([f, bn]), src, rbuf)
+    layer.output_gpu.fill(0xCD)  # every output word must be written by the call
+    layer.forward()
+    layer.forward()  # idempotent: a second run on the same objects gives the same result
+    gpuops.sync()
+    return layer
+
+
+CONV_CASES = [
+    # b, h, cin, cout, stride, pool, ahead_fc
+    (8, 8, 128, 128, 1, 1, False), (70, 8, 128, 128, 1, 2, False), (8, 7, 64, 96, 1, 2, False),
+    (130, 12, 64, 128, 2, 1, False), (8, 9, 256, 32, 1, 3, False), (24, 4, 512, 512, 1, 2, True),
+    (8, 4, 64, 160, 1, 2, True), (256, 7, 128, 64, 1, 1, False),
+]
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+@pytest.mark.parametrize("b,h,cin,cout,stride,pool,ahead_fc", CONV_CASES)
+def test_conv128_layer(gpu, variant, b, h, cin, cout, stride, pool, ahead_fc):
+    r = rng(b + h + cin + cout + pool)
+    x = rm.pm1(r, (b, h, h, cin))
+    f = rm.pm1(r, (3, 3, cin, cout))
+    bn = r.normal(0, np.sqrt(9 * cin), cout).astype(np.float32)
+    inp, filt = orc.pack_conv_input_nhwc(x), orc.pack_conv_filter(f)
+    _, res = orc.conv128(inp, filt, bn, cin, cout, 3, 3, stride, True, 1, save_residual=True)
+    bn[:4] = res[0, 0, 0, :4]  # ties on a border pixel
+    want, _ = orc.conv128(inp, filt, bn, cin, cout, 3, 3, stride, True, pool, ahead_fc)
+    layer = _run_conv_layer(gpu, variant, x, f, bn, stride, pool, ahead_fc)
+    np.testing.assert_array_equal(layer.download_packed(), want)
+    # what the reference's download_output() would return (tile-contiguous layout)
+    oh = layer.output_height
+    if ahead_fc:
+        want_fmt = orc.fc_to_fmt(want, b, oh * oh * orc.pad128(cout))
+    else:
+        want_fmt = orc.conv_to_fmt(want, cout)
+    np.testing.assert_array_equal(layer.download_output(), want_fmt)
+    full = layer.download_full_output()
+    assert full.shape == (b, oh, oh, cout)
+    if not ahead_fc:
+        np.testing.assert_array_equal(full, np.transpose(orc.unpack_bits(want, cout), (2, 0, 1, 3)))
+    layer.release()
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+def test_conv128_residual_modes(gpu, variant):
+    r = rng(41)
+    b, h, cin, cout = 72, 6, 64, 96
+    x = rm.pm1(r, (b, h, h, cin))
+    f = rm.pm1(r, (3, 3, cin, cout))
+    bn = r.normal(0, 20, cout).astype(np.float32)
+    inp, filt = orc.pack_conv_input_nhwc(x), orc.pack_conv_filter(f)
+
+    layer = _run_conv_layer(gpu, variant, x, f, bn, save_residual=True)
+    want, wres = orc.conv128(inp, filt, bn, cin, cout, 3, 3, save_residual=True)
+    np.testing.assert_array_equal(layer.download_packed(), want)
+    np.testing.assert_array_equal(layer.download_residual(), wres)
+    np.testing.assert_array_equal(layer.download_residual_reference(), orc.residual_to_reference(wres))
+    layer.release()
+
+    src = r.integers(-300, 300, size=(h, h, b, 64)).astype(np.int32)
+    layer = _run_conv_layer(gpu, variant, x, f, bn, save_residual=True, inject_residual=True,
+                            residual_channels=80, res_in=src)
+    want, wres = orc.conv128(inp, filt, bn, cin, cout, 3, 3, save_residual=True, inject_residual=True,
+                             residual_channels=80, res_in=src)
+    np.testing.assert_array_equal(layer.download_packed(), want)
+    np.testing.assert_array_equal(layer.download_residual(), wres)
+    layer.release()
+
+    src2 = r.integers(-300, 300, size=(2 * h, 2 * h, b, 96)).astype(np.int32)
+    layer = _run_conv_layer(gpu, variant, x, f, bn, save_residual=True, inject_residual=True,
+                            residual_channels=48, residual_pool=True, res_in=src2)
+    want, wres = orc.conv128(inp, filt, bn, cin, cout, 3, 3, save_residual=True, inject_residual=True,
+                             residual_channels=48, residual_pool=True, res_in=src2)
+    np.testing.assert_array_equal(layer.download_packed(), want)
+    np.testing.assert_array_equal(layer.download_residual(), wres)
+    layer.release()
+
+
+def test_conv128_rejects_residual_with_pooling(gpu):
+    x = rm.pm1(rng(1), (8, 4, 4, 64))
+    f = rm.pm1(rng(2), (3, 3, 64, 32))
+    layer = gpu.Conv128LayerParam("C", 4, 4, 3, 3, 64, 32, 8, 1, 1, True, 2, 2, False, True)
+    layer.initialize(gpu.ArrayWeights([f, np.zeros(32, np.float32)]), gpuops.pack_conv_input(x))
+    with pytest.raises(gpu.TcbnnError):
+        layer.forward()
+
+
+# --------------------------------------------------------------------------- first layer
+@pytest.mark.parametrize("b,h,R,stride,cout,pool,save", [(8, 32, 3, 1, 128, 1, False), (5, 20, 7, 4, 64, 1, True),
+                                                         (70, 12, 3, 1, 32, 2, False), (3, 13, 5, 2, 96, 1, True),
+                                                         (2, 224, 7, 4, 64, 1, True)])
+def test_inconv128_layer(gpu, b, h, R, stride, cout, pool, save):
+    r = rng(b + h + R + cout)
+    x = r.standard_normal((b, 3, h, h)).astype(np.float32)
+    f = rm.pm1(r, (R, R, 3, cout))
+    bn = r.normal(0, np.sqrt(3 * R * R), cout).astype(np.float32)
+    want, wres = orc.inconv128(x, f, bn, stride, True, pool, save)
+    layer = gpu.InConv128LayerParam("Conv1", h, h, R, R, 3, cout, b, stride, stride, True, pool, pool, save)
+    layer.initialize(x, gpu.ArrayWeights([f, bn]))
+    layer.forward()
+    gpuops.sync()
+    np.testing.assert_array_equal(layer.download_packed(), want)
+    np.testing.assert_array_equal(layer.download_output(), orc.conv_to_fmt(want, cout))
+    if save:
+        np.testing.assert_array_equal(layer.download_residual(), wres)
+    layer.release()
+
+
+def test_inconv128_presigned_input_is_exact_integer_conv(gpu):
+    """The config's 'input binarized by sign' variant: +-1.0f input, sums are exact integers."""
+    r = rng(5)
+    b, h, cout = 8, 32, 128
+    xs = rm.pm1(r, (b, 3, h, h))
+    f = rm.pm1(r, (3, 3, 3, cout))
+    want = rm.xcorr_pm1(np.transpose(xs, (0, 2, 3, 1)), f, 1, 1, 1, h, h)
+    layer = gpu.InConv128LayerParam("Conv1", h, h, 3, 3, 3, cout, b, 1, 1, True, 1, 1, True)
+    layer.initialize(xs, gpu.ArrayWeights([f, np.zeros(cout, np.float32)]))
+    layer.forward()
+    gpuops.sync()
+    np.testing.assert_array_equal(np.transpose(layer.download_residual(), (2, 0, 1, 3)), want)
+    layer.release()
+
+
+# --------------------------------------------------------------------------- whole networks
+def _compare_network(gpu, spec, seed, variant):
+    weights = gpu.synthetic_weights(spec, seed)
+    x = gpu.synthetic_input(spec, seed)
+    want = orc_nets.run(spec, weights, x)
+    net = gpu.Network(spec, weights, x, variant=_variant(gpu, variant))
+    net.forward()
+    logits = net.logits()
+    for L in spec:
+        layer = net.layers[L["name"]]
+        w = want[L["name"]]
+        if L["kind"] == "out":
+            np.testing.assert_allclose(logits, w["out"], rtol=1e-5, atol=0)
+            np.testing.assert_array_equal(logits, w["out"])
+        else:
+            got = layer.download_packed()
+            np.testing.assert_array_equal(got, w["out"].reshape(got.shape), err_msg=L["name"])
+            if w.get("res") is not None:
+                np.testing.assert_array_equal(layer.download_residual(), w["res"], err_msg=L["name"])
+    # second forward on the same objects: identical logits (no stale-bit accumulation)
+    net.forward()
+    np.testing.assert_array_equal(net.logits(), logits)
+    net.release()
+    return logits
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+def test_mnist_mlp_full_batch(gpu, variant):
+    from tcbnn_amd import nets
+    _compare_network(gpu, nets.mnist_mlp_spec(batch=8192), 1, variant)
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+def test_cifar10_vgg(gpu, variant):
+    from tcbnn_amd import nets
+    _compare_network(gpu, nets.cifar10_vgg_spec(batch=16), 2, variant)
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+def test_imagenet_resnet18(gpu, variant):
+    from tcbnn_amd import nets
+    _compare_network(gpu, nets.imagenet_resnet_spec(batch=8), 3, variant)
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+def test_imagenet_resnet18_batch256_properties(gpu, variant):
+    """Full configured size: images are independent, so the first 8 images of a batch-256 run
+    must reproduce the batch-8 run (which the oracle checks above) bit for bit."""
+    from tcbnn_amd import nets
+    spec256, spec8 = nets.imagenet_resnet_spec(batch=256), nets.imagenet_resnet_spec(batch=8)
+    weights = gpu.synthetic_weights(spec256, 3)
+    x = gpu.synthetic_input(spec256, 3)
+    net = gpu.Network(spec256, weights, x, variant=_variant(gpu, variant))
+    net.forward()
+    big = net.logits()
+    net.release()
+    net8 = gpu.Network(spec8, weights, x[:8], variant=_variant(gpu, variant))
+    net8.forward()
+    small = net8.logits()
+    net8.release()
+    assert np.isfinite(big).all()
+    np.testing.assert_array_equal(big[:8], small)
+    want = orc_nets.run(spec8, weights, x[:8])["Fout"]["out"]
+    np.testing.assert_allclose(small, want, rtol=1e-5, atol=0)
