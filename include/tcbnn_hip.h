@@ -21,15 +21,16 @@
  *     of its uint32 ("MSB first"); pad bits are 0 in both operands and the
  *     true K / Cin enters  K - 2*popc(a xor w).
  *
- * Engine layouts (device memory)
- *   FC activations   : uint32 [B][KW128]          KW128 = 4*ceil(K/128) words per row
- *   conv activations : uint32 [H][W][B][CW]       CW    = ceil(C/32) words per (pixel,image)
- *   FC-ready conv out: uint32 [B][OH*OW*CW128]    feature order (y, x, c), c padded to 128
- *                                                 (kernel.cuh:798-808)
+ * Engine layouts (device memory).  The batch index is innermost everywhere, so a
+ * wavefront whose lanes are 64 consecutive images reads and writes contiguous runs:
+ *   FC activations   : uint32 [KW128][B]          KW128 = 4*ceil(K/128) words per image
+ *   conv activations : uint32 [H][W][CW][B]       CW    = ceil(C/32) words per (pixel,image)
+ *   FC-ready conv out: uint32 [OH*OW*CW128][B]    feature order (y, x, c), c padded to 128
+ *                                                 (kernel.cuh:798-808): an FC activation
  *   packed weights   : uint32 [NPAD32][KWTOT]     one row per output neuron/channel,
  *                                                 FC: KWTOT = KW128; conv: KWTOT = R*S*CW,
  *                                                 K index = (r*S+s)*32*CW + c; rows >= N are 0
- *   residual tensors : int32  [P][Q][B][O]        true channel count, no 128-padding
+ *   residual tensors : int32  [P][Q][O][B]        true channel count, no 128-padding
  *   fp32 stem input  : float  [B][3][H][W]        (kernel.cuh:620-625)
  * The reference's own tile-contiguous "FMT" layouts ([.../8][.../128][8][4],
  * kernel.cuh:170,222,650-660,798-815) are produced / consumed by the
@@ -96,15 +97,16 @@ int tcbnn_pack_conv_filter(const float* filter_hwio, uint32_t* packed, int r, in
  * PackFiltersByOutChannels32 (param.h:613-632). */
 int tcbnn_pack_inconv_filter(const float* filter_hwio, uint32_t* packed, int r, int s, int in_ch,
                              int out_ch, void* stream);
-/* fp32 +-1 matrix rows -> packed rows, MSB first: out[row][k/32].  `rows` x `k`
- * row-major input with leading dimension `ld`; k_words words are written per
- * row (zero padded).  Replaces BMMA_toBit32Row (tensorcore_kernel.cu:87-97). */
+/* fp32 +-1 matrix rows -> packed activation matrix, MSB first, batch (row) innermost:
+ * out[k/32][row].  `rows` x `k` row-major input with leading dimension `ld`; k_words
+ * words are written per row (zero padded).  Replaces BMMA_toBit32Row
+ * (tensorcore_kernel.cu:87-97). */
 int tcbnn_pack_rows(const float* src, uint32_t* packed, int rows, int k, int ld, int k_words,
                     void* stream);
 /* fp32 [K][N] -> packed [N][k_words] (each column contiguous along K).  Replaces
  * BMMA_toBit32Col (tensorcore_kernel.cu:74-84). */
 int tcbnn_pack_cols(const float* src, uint32_t* packed, int k, int n, int k_words, void* stream);
-/* fp32 +-1 NHWC [B][H][W][C] -> packed [H][W][B][CW].  Replaces BTC_bin_input
+/* fp32 +-1 NHWC [B][H][W][C] -> packed [H][W][CW][B].  Replaces BTC_bin_input
  * (bmma_kernel.cu:73-98). */
 int tcbnn_pack_conv_input_nhwc(const float* src, uint32_t* packed, int batch, int height,
                                int width, int ch, void* stream);
@@ -114,7 +116,7 @@ int tcbnn_pack_conv_input_nhwc(const float* src, uint32_t* packed, int batch, in
  * (param.h:210-218): fp32 [B][K] -> sign bits, FC activation layout. */
 typedef struct tcbnn_in128_desc {
     const float* input;   /* [input_height][input_width] */
-    uint32_t* output;     /* [B][KW128] */
+    uint32_t* output;     /* [KW128][B] */
     int input_height;     /* batch */
     int input_width;      /* features */
 } tcbnn_in128_desc;
@@ -123,15 +125,16 @@ int tcbnn_in128_forward(const tcbnn_in128_desc* d, void* stream);
 /* Fc128LayerFMT (kernel.cuh:174-226), fields of Fc128LayerParam (param.h:362-384):
  * bit[b][n] = ((float)K - 2*(float)popc(a_b xor w_n) >= bn[n]). */
 typedef struct tcbnn_fc128_desc {
-    const uint32_t* input;   /* [B][KW128(input_width)] */
+    const uint32_t* input;   /* [KW128(input_width)][B] */
     const uint32_t* weight;  /* tcbnn_pack_fc_weight output */
     const float* bn;         /* [weight_width] thresholds */
-    uint32_t* output;        /* [B][KW128(weight_width)] */
+    uint32_t* output;        /* [KW128(weight_width)][B] */
     int input_height;        /* batch */
     int input_width;         /* K */
     int weight_width;        /* N */
     int variant;             /* TCBNN_VARIANT_* */
-    int32_t* workspace;      /* optional int32 [B][NPAD32] for split-K; may be NULL */
+    int32_t* workspace;      /* optional int32 [NPAD32][B] scratch: lets small-batch layers
+                                split K over workgroups; NULL = never split */
     size_t workspace_words;
 } tcbnn_fc128_desc;
 int tcbnn_fc128_forward(const tcbnn_fc128_desc* d, void* stream);
@@ -159,8 +162,8 @@ typedef struct tcbnn_inconv128_desc {
     const float* input;        /* [batch][3][input_height][input_width] */
     const uint32_t* filter;    /* tcbnn_pack_inconv_filter output */
     const float* bn;           /* [output_channels] */
-    uint32_t* output;          /* [OH][OW][B][CW(output_channels)] */
-    int32_t* output_residual;  /* [P][Q][B][O] or NULL */
+    uint32_t* output;          /* [OH][OW][CW(output_channels)][B] */
+    int32_t* output_residual;  /* [P][Q][O][B] or NULL */
     int input_height, input_width, input_channels;
     int filter_height, filter_width;
     int output_channels, batch;
@@ -183,12 +186,12 @@ int tcbnn_inconv128_forward(const tcbnn_inconv128_desc* d, void* stream);
  * save_residual / inject_residual require pool 1x1, residual_pool requires the
  * source to be exactly twice the output size (as the reference indexing assumes). */
 typedef struct tcbnn_conv128_desc {
-    const uint32_t* input;         /* [H][W][B][CW(input_channels)] */
+    const uint32_t* input;         /* [H][W][CW(input_channels)][B] */
     const uint32_t* filter;        /* tcbnn_pack_conv_filter output */
     const float* bn;               /* [output_channels] */
-    uint32_t* output;              /* [OH][OW][B][CW(O)], or FC-ready if ahead_fc */
-    const int32_t* input_residual; /* [Hr][Wr][B][input_residual_channels] or NULL */
-    int32_t* output_residual;      /* [P][Q][B][O] or NULL */
+    uint32_t* output;              /* [OH][OW][CW(O)][B]; ahead_fc: [OH][OW][CW128(O)][B] */
+    const int32_t* input_residual; /* [Hr][Wr][input_residual_channels][B] or NULL */
+    int32_t* output_residual;      /* [P][Q][O][B] or NULL */
     int input_height, input_width, input_channels;
     int filter_height, filter_width;
     int output_channels, batch;
@@ -198,20 +201,29 @@ typedef struct tcbnn_conv128_desc {
     int ahead_fc, save_residual, inject_residual;
     int residual_channels;         /* inject only into o < residual_channels */
     int residual_pool;
-    int input_residual_channels;   /* channel count (stride) of the source tensor */
+    int input_residual_channels;   /* channel count of the source tensor */
     int variant;
 } tcbnn_conv128_desc;
 int tcbnn_conv128_forward(const tcbnn_conv128_desc* d, void* stream);
 
+/* Name of the device kernel (as a profiler lists it, template arguments included) that
+ * tcbnn_conv128_forward / tcbnn_fc128_forward would launch for this descriptor; no
+ * launch happens and no pointer is dereferenced.  No counterpart in the reference
+ * (its layers are inlined device functions of one network kernel); used to match
+ * per-launch timings with profiler output. */
+int tcbnn_conv128_kernel_name(const tcbnn_conv128_desc* d, char* buf, size_t len);
+int tcbnn_fc128_kernel_name(const tcbnn_fc128_desc* d, char* buf, size_t len);
+
 /* ------------------------------------------------ standalone GEMM / conv */
-/* C[m][n] = K - 2*popc(A[m,:] xor B[n,:]), int32 row major [M][N].  A: [M][K/32],
- * B: [N][K/32] (each column of the logical K x N matrix contiguous along K);
- * K % 32 == 0.  Replaces BMMAS / BMMAS_new (tensorcore_kernel.cu:305-356). */
+/* C[m][n] = K - 2*popc(A[m,:] xor B[n,:]), int32 row major [M][N].  A: [K/32][M]
+ * (tcbnn_pack_rows output), B: [N][K/32] (tcbnn_pack_cols output: each column of the
+ * logical K x N matrix contiguous along K); K % 32 == 0, N % 32 == 0.  Replaces
+ * BMMAS / BMMAS_new (tensorcore_kernel.cu:305-356). */
 int tcbnn_bmm(const uint32_t* a, const uint32_t* b, int32_t* c, int m, int n, int k, int variant,
               void* stream);
 /* out[b][p][q][o] = Cin*R*S - exclude*Cin - 2*popc  (bmma_kernel.cu:154-159), int32
  * [N][P][Q][O] (the layout BTC_trans_output produces, bmma_kernel.cu:247-263).
- * input: [H][W][B][CW]; filter: tcbnn_pack_conv_filter output.  Replaces
+ * input: [H][W][CW][B]; filter: tcbnn_pack_conv_filter output.  Replaces
  * BTC_Conv2d_balance[_128] (bmma_kernel.cu:101-165, 326-392). */
 int tcbnn_bconv(const uint32_t* input, const uint32_t* filter, int32_t* output, int batch,
                 int height, int width, int in_ch, int out_ch, int r, int s, int stride_h,
@@ -237,7 +249,7 @@ int tcbnn_conv_to_reference_fmt(const uint32_t* packed, uint32_t* fmt, int heigh
                                 int batch, int ch, void* stream);
 int tcbnn_conv_from_reference_fmt(const uint32_t* fmt, uint32_t* packed, int height, int width,
                                   int batch, int ch, void* stream);
-/* Engine residual [P][Q][B][O] -> reference [P][Q][PAD8(B)][PAD128(O)] with zero
+/* Engine residual [P][Q][O][B] -> reference [P][Q][PAD8(B)][PAD128(O)] with zero
  * fill (kernel.cuh:666-668, 820-823). */
 int tcbnn_residual_to_reference(const int32_t* res, int32_t* ref, int height, int width,
                                 int batch, int ch, void* stream);

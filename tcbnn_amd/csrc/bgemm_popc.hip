@@ -5,8 +5,9 @@
 //   lane            = one image b of a batch tile; a wave holds RPL batch tiles of 64
 //                     images (RPL rows per lane) that all sit on the SAME output pixel,
 //                     so the zero-padding predicate of a filter tap is wave-uniform
-//                     (a scalar branch) and the activation load of a tap is one
-//                     coalesced run of 64*cw words.
+//                     (a scalar branch) and, with the batch-innermost activation layout
+//                     [H][W][cw][B], every activation word load is one contiguous
+//                     256-byte run.
 //   workgroup       = 4 waves (4 different (pixel, batch-tile) rows) x one tile of 32
 //                     output channels.  The weights of that channel tile are staged
 //                     once in LDS as [k-chunk][32 channels][CH words]; every lane reads
@@ -16,9 +17,14 @@
 //                     32 +-1 multiply-accumulates.
 //   epilogue        = in-lane: the lane owns all 32 channel sums of its row, so
 //                     threshold -> bit -> shift/or builds the packed output word with
-//                     no ballot, no LDS round trip and no atomics.  Pool windows are a
-//                     sequential loop in the same lane (OR of the words), so every
-//                     output word is written exactly once and re-runs are idempotent.
+//                     no ballot, no LDS round trip and no atomics; residual tensors are
+//                     [P][Q][O][B], so each channel's residual load/store is again one
+//                     contiguous run across the wave.  Pool windows are a sequential
+//                     loop in the same lane (OR of the words), so every output word is
+//                     written exactly once and re-runs are idempotent.
+//   split-K         = FC-shaped problems with few rows split K over blockIdx; partial
+//                     popcounts are atomically added into an int32 workspace and a small
+//                     finishing kernel applies the epilogue.
 //
 // Semantics follow Fc128LayerFMT / Out128LayerFMT / Conv128LayerFMT
 // (kernel.cuh:174-280, 676-827) and BMMAS / BTC_Conv2d_balance
@@ -49,17 +55,36 @@ struct WordVec<1> {
     using type = uint32_t;
 };
 
-__device__ __forceinline__ int xpopc(uint4 a, uint4 w) {
-    return __popc(a.x ^ w.x) + __popc(a.y ^ w.y) + __popc(a.z ^ w.z) + __popc(a.w ^ w.w);
+__device__ __forceinline__ int xpopc(const uint32_t* a, uint4 w) {
+    return __popc(a[0] ^ w.x) + __popc(a[1] ^ w.y) + __popc(a[2] ^ w.z) + __popc(a[3] ^ w.w);
 }
-__device__ __forceinline__ int xpopc(uint2 a, uint2 w) {
-    return __popc(a.x ^ w.x) + __popc(a.y ^ w.y);
+__device__ __forceinline__ int xpopc(const uint32_t* a, uint2 w) {
+    return __popc(a[0] ^ w.x) + __popc(a[1] ^ w.y);
 }
-__device__ __forceinline__ int xpopc(uint32_t a, uint32_t w) { return __popc(a ^ w); }
+__device__ __forceinline__ int xpopc(const uint32_t* a, uint32_t w) { return __popc(a[0] ^ w); }
 
-template <int RPL, int CH>
-__global__ __launch_bounds__(kThreads) void bgemm_popc_kernel(const BgemmParams p, int n_tiles,
-                                                              int row_waves, int b_tiles) {
+// Threshold compare of the reference: conv layers emit (res < bn) ? 0 : 1
+// (kernel.cuh:795-796), FC layers emit (res >= bn) (kernel.cuh:210-213); the two differ
+// only when bn is NaN.
+__device__ __forceinline__ uint32_t thresh_bit(int res, float thr, int nan_bit) {
+    const float rf = (float)res;
+    return nan_bit ? (rf < thr ? 0u : 1u) : (rf >= thr ? 1u : 0u);
+}
+
+// Epilogue selected at compile time so that each instance only keeps its own operands live.
+enum KernelMode : int {
+    KM_THRESH = 0,      // threshold + pack (+ pooling)
+    KM_THRESH_RES = 1,  // threshold + pack with residual inject and/or save
+    KM_AFFINE = 2,      // fp32 affine output
+    KM_RAW = 3,         // int32 dot products
+    KM_PARTIAL = 4,     // split-K partial popcounts -> workspace
+};
+
+// register budget: 32*RPL accumulators + operands; keep as many waves per SIMD as that allows
+template <int RPL, int CH, int KM>
+__global__ __launch_bounds__(kThreads)
+    __attribute__((amdgpu_waves_per_eu(RPL == 1 ? 4 : (RPL == 2 ? 3 : 2)))) void bgemm_popc_kernel(
+        const BgemmParams p, int n_tiles, int row_waves, int b_tiles, int row_blocks) {
     using V = typename WordVec<CH>::type;
     __shared__ __attribute__((aligned(16))) uint32_t lds_w[kLdsWords];
 
@@ -67,14 +92,21 @@ __global__ __launch_bounds__(kThreads) void bgemm_popc_kernel(const BgemmParams 
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int nt = blockIdx.x % n_tiles;
-    const int rw = (blockIdx.x / n_tiles) * kWavesPerBlock + wave;
+    const int rb = (blockIdx.x / n_tiles) % row_blocks;
+    const int ks = blockIdx.x / (n_tiles * row_blocks);  // K split index
+    const int rw = rb * kWavesPerBlock + wave;
     const bool active = rw < row_waves;
 
     const int cw_chunks = p.cw / CH;
     const int taps = p.R * p.S;
-    const int nq = taps * cw_chunks;           // k-chunks in total
-    const int kw_tot = taps * p.cw;            // words per weight row
+    const int nq_all = taps * cw_chunks;  // k-chunks in total
+    const int kw_tot = taps * p.cw;       // words per weight row
     constexpr int kQB = kLdsWords / (kNTile * CH);  // chunks per staging block
+    // this block's K range (the whole K unless split)
+    const int q_per = (nq_all + p.ksplit - 1) / p.ksplit;
+    const int q_begin = ks * q_per;
+    const int q_end = min(nq_all, q_begin + q_per);
+    const int nq = q_end - q_begin;
     const bool single_block = nq <= kQB;
 
     const int opix = active ? rw / b_tiles : 0;  // pooled output pixel
@@ -90,7 +122,7 @@ __global__ __launch_bounds__(kThreads) void bgemm_popc_kernel(const BgemmParams 
     }
 
     auto stage_weights = [&](int q0) {
-        const int cnt = min(kQB, nq - q0);
+        const int cnt = min(kQB, q_end - q0);
         const int blk_words = cnt * CH;  // words per weight row in this block
         const uint32_t* wrow = p.wgt + (size_t)nt * kNTile * kw_tot + (size_t)q0 * CH;
         for (int idx = tid; idx < blk_words * kNTile; idx += kThreads) {
@@ -100,8 +132,8 @@ __global__ __launch_bounds__(kThreads) void bgemm_popc_kernel(const BgemmParams 
         }
     };
 
-    if (single_block) {
-        stage_weights(0);
+    if (single_block && nq > 0) {
+        stage_weights(q_begin);
         __syncthreads();
     }
 
@@ -109,6 +141,7 @@ __global__ __launch_bounds__(kThreads) void bgemm_popc_kernel(const BgemmParams 
 #pragma unroll
     for (int r = 0; r < RPL; ++r) outword[r] = 0;
 
+    const int n0 = nt * kNTile;
     const int pool_n = p.pool_h * p.pool_w;
     for (int pp = 0; pp < pool_n; ++pp) {
         const int y = oy * p.pool_h + pp / p.pool_w;
@@ -125,25 +158,28 @@ __global__ __launch_bounds__(kThreads) void bgemm_popc_kernel(const BgemmParams 
         int exclude = 0;
 
         // running (tap row, tap col, chunk) counters: no integer division in the loop
-        int tr = 0, ts = 0, kc = 0;
-        for (int q0 = 0; q0 < nq; q0 += kQB) {
+        int tr = (q_begin / cw_chunks) / p.S, ts = (q_begin / cw_chunks) % p.S,
+            kc = q_begin % cw_chunks;
+        for (int q0 = q_begin; q0 < q_end; q0 += kQB) {
             if (!single_block) {
                 __syncthreads();
                 stage_weights(q0);
                 __syncthreads();
             }
-            const int cnt = min(kQB, nq - q0);
+            const int cnt = min(kQB, q_end - q0);
             for (int ql = 0; ql < cnt; ++ql) {
                 const int ay = ay0 + tr, ax = ax0 + ts;
                 const bool in_frame = ay >= 0 && ay < p.H && ax >= 0 && ax < p.W;
                 if (valid) {
                     if (in_frame) {
-                        V a[RPL];
-                        const size_t pix = (size_t)(ay * p.W + ax) * p.B;
+                        uint32_t a[RPL][CH];
+                        const uint32_t* src =
+                            p.act + ((size_t)(ay * p.W + ax) * p.cw + kc * CH) * p.B;
 #pragma unroll
-                        for (int r = 0; r < RPL; ++r)
-                            a[r] = *reinterpret_cast<const V*>(p.act + (pix + bload[r]) * p.cw +
-                                                               kc * CH);
+                        for (int j = 0; j < CH; ++j)
+#pragma unroll
+                            for (int r = 0; r < RPL; ++r)
+                                a[r][j] = src[(size_t)j * p.B + bload[r]];
                         const V* wl = reinterpret_cast<const V*>(lds_w) + ql * kNTile;
 #pragma unroll
                         for (int n = 0; n < kNTile; ++n) {
@@ -168,62 +204,63 @@ __global__ __launch_bounds__(kThreads) void bgemm_popc_kernel(const BgemmParams 
         if (!valid) continue;
 
         // ---------------- epilogue for pre-pool pixel (y, x) ----------------
+        if constexpr (KM == KM_PARTIAL) {  // partial popcounts only; the finishing kernel does the rest
+#pragma unroll
+            for (int r = 0; r < RPL; ++r) {
+                if (brow[r] >= p.B) continue;
+#pragma unroll
+                for (int n = 0; n < kNTile; ++n)
+                    atomicAdd(p.workspace + (size_t)(n0 + n) * p.B + brow[r], acc[r][n]);
+            }
+            continue;
+        }
+
         const int base = p.k_tap * taps - exclude * p.k_tap;
-        const int n0 = nt * kNTile;
+        const size_t pix = (size_t)y * p.PW + x;
 #pragma unroll
         for (int r = 0; r < RPL; ++r) {
             if (brow[r] >= p.B) continue;
             const int b = brow[r];
-            int res[kNTile];
+            if constexpr (KM == KM_THRESH || KM == KM_THRESH_RES) {
+                uint32_t word = 0;
+                int rv[kNTile];
+                if constexpr (KM == KM_THRESH_RES) {
+                    // all residual loads first (one contiguous run per channel across the
+                    // wave), so they are in flight together before any store is issued
+                    const int32_t* __restrict__ rin = p.res_in;
 #pragma unroll
-            for (int n = 0; n < kNTile; ++n) res[n] = base - 2 * acc[r][n];
-
-            if (p.res_in != nullptr) {
-#pragma unroll
-                for (int n = 0; n < kNTile; ++n) {
-                    const int ch = n0 + n;
-                    if (ch < p.res_limit && ch < p.res_in_ch) {
-                        int v;
-                        if (p.res_pool) {
-                            const int rw2 = 2 * p.PW;
-                            v = INT_MIN;
-#pragma unroll
-                            for (int i = 0; i < 2; ++i)
-#pragma unroll
-                                for (int j = 0; j < 2; ++j)
-                                    v = max(v, p.res_in[(((size_t)(2 * y + i) * rw2 + (2 * x + j)) *
-                                                             p.B +
-                                                         b) *
-                                                            p.res_in_ch +
-                                                        ch]);
-                        } else {
-                            v = p.res_in[(((size_t)y * p.PW + x) * p.B + b) * p.res_in_ch + ch];
+                    for (int n = 0; n < kNTile; ++n) {
+                        const int ch = n0 + n;
+                        int v = 0;
+                        if (rin != nullptr && ch < p.res_limit && ch < p.res_in_ch && ch < p.N) {
+                            if (p.res_pool) {
+                                const size_t rw2 = 2 * (size_t)p.PW;
+                                const int32_t* s00 =
+                                    rin + (((size_t)(2 * y) * rw2 + 2 * x) * p.res_in_ch + ch) * p.B + b;
+                                const size_t dx = (size_t)p.res_in_ch * p.B, dy = rw2 * dx;
+                                v = max(max(s00[0], s00[dx]), max(s00[dy], s00[dy + dx]));
+                            } else {
+                                v = rin[(pix * p.res_in_ch + ch) * p.B + b];
+                            }
                         }
-                        res[n] += v;
+                        rv[n] = v;
                     }
                 }
-            }
-
-            if (p.mode == EPI_THRESH) {
-                uint32_t word = 0;
+                const float* __restrict__ bn = p.bn;
+                int32_t* __restrict__ rout = p.res_out;
 #pragma unroll
                 for (int n = 0; n < kNTile; ++n) {
                     const int ch = n0 + n;
-                    if (ch < p.N) {
-                        const float rf = (float)res[n];
-                        const float thr = p.bn[ch];
-                        const bool bit = p.nan_bit ? !(rf < thr) : (rf >= thr);
-                        word |= (bit ? 1u : 0u) << (31 - n);
+                    if (ch >= p.N) continue;  // (no break: the loop must stay fully unrolled)
+                    int res = base - 2 * acc[r][n];
+                    if constexpr (KM == KM_THRESH_RES) {
+                        res += rv[n];
+                        if (rout != nullptr) rout[(pix * p.N + ch) * p.B + b] = res;
                     }
+                    word |= thresh_bit(res, bn[ch], p.nan_bit) << (31 - n);
                 }
                 outword[r] |= word;
-                if (p.res_out != nullptr) {
-                    int32_t* dst = p.res_out + (((size_t)y * p.PW + x) * p.B + b) * p.N;
-#pragma unroll
-                    for (int n = 0; n < kNTile; ++n)
-                        if (n0 + n < p.N) dst[n0 + n] = res[n];
-                }
-            } else if (p.mode == EPI_AFFINE) {
+            } else if constexpr (KM == KM_AFFINE) {
                 float* dst = p.out_f32 + (size_t)b * p.N;
 #pragma unroll
                 for (int n = 0; n < kNTile; ++n) {
@@ -235,49 +272,128 @@ __global__ __launch_bounds__(kThreads) void bgemm_popc_kernel(const BgemmParams 
                         dst[ch] = __fadd_rn(__fmul_rn(d, p.bn_scale[ch]), p.bn_bias[ch]);
                     }
                 }
-            } else {  // EPI_RAW
-                int32_t* dst = p.out_i32 + ((size_t)y * p.PW + x) * p.raw_pix_stride +
-                               (size_t)b * p.raw_b_stride;
+            } else if constexpr (KM == KM_RAW) {
+                int32_t* dst = p.out_i32 + pix * p.raw_pix_stride + (size_t)b * p.raw_b_stride;
 #pragma unroll
                 for (int n = 0; n < kNTile; ++n)
-                    if (n0 + n < p.N) dst[n0 + n] = res[n];
+                    if (n0 + n < p.N) dst[n0 + n] = base - 2 * acc[r][n];
             }
         }
     }
 
-    if (p.mode == EPI_THRESH && active) {
+    if ((KM == KM_THRESH || KM == KM_THRESH_RES) && active) {
 #pragma unroll
         for (int r = 0; r < RPL; ++r)
             if (brow[r] < p.B) {
-                uint32_t* dst = p.out_bits + (size_t)opix * p.bits_pix_stride +
-                                (size_t)brow[r] * p.bits_b_stride;
-                dst[nt] = outword[r];
-                if (nt == n_tiles - 1)  // zero the row's padding words
-                    for (int w = n_tiles; w < p.bits_row_words; ++w) dst[w] = 0;
+                uint32_t* dst = p.out_bits + (size_t)opix * p.bits_pix_stride + brow[r];
+                dst[(size_t)nt * p.B] = outword[r];
+                if (nt == n_tiles - 1)  // zero the pixel's padding words
+                    for (int w = n_tiles; w < p.bits_row_words; ++w) dst[(size_t)w * p.B] = 0;
             }
     }
 }
 
-template <int RPL, int CH>
+// ---- split-K helpers: workspace int32 [npad32][B] of popcounts -----------------------
+__global__ void splitk_clear_kernel(int32_t* ws, size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) ws[i] = 0;
+}
+
+__global__ __launch_bounds__(256) void splitk_finish_kernel(const BgemmParams p, int n_tiles) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= (size_t)n_tiles * p.B) return;
+    const int b = (int)(i % p.B);
+    const int nt = (int)(i / p.B);
+    const int n0 = nt * kNTile;
+    if (p.mode == EPI_THRESH) {
+        uint32_t word = 0;
+        for (int n = 0; n < kNTile && n0 + n < p.N; ++n) {
+            const int res = p.k_tap - 2 * p.workspace[(size_t)(n0 + n) * p.B + b];
+            word |= thresh_bit(res, p.bn[n0 + n], p.nan_bit) << (31 - n);
+        }
+        p.out_bits[(size_t)nt * p.B + b] = word;
+        if (nt == n_tiles - 1)
+            for (int w = n_tiles; w < p.bits_row_words; ++w) p.out_bits[(size_t)w * p.B + b] = 0;
+    } else if (p.mode == EPI_AFFINE) {
+        for (int n = 0; n < kNTile && n0 + n < p.N; ++n) {
+            const float d = (float)p.k_tap - (float)p.workspace[(size_t)(n0 + n) * p.B + b] * 2.0f;
+            p.out_f32[(size_t)b * p.N + n0 + n] =
+                __fadd_rn(__fmul_rn(d, p.bn_scale[n0 + n]), p.bn_bias[n0 + n]);
+        }
+    } else {
+        for (int n = 0; n < kNTile && n0 + n < p.N; ++n)
+            p.out_i32[(size_t)b * p.raw_b_stride + n0 + n] =
+                p.k_tap - 2 * p.workspace[(size_t)(n0 + n) * p.B + b];
+    }
+}
+
+int rows_per_lane(const BgemmParams& p) {
+    // as many 64-image tiles per lane as the batch holds, but never so many that the
+    // launch no longer fills the chip
+    const long long pix = (long long)p.OH * p.OW;
+    const int n_tiles = (p.N + kNTile - 1) / kNTile;
+    for (int rpl = 4; rpl > 1; rpl >>= 1) {
+        if (p.B <= 64 * (rpl / 2)) continue;
+        const long long waves = pix * ((p.B + 64 * rpl - 1) / (64 * rpl)) * n_tiles * p.ksplit;
+        if (waves >= 2048) return rpl;
+    }
+    return 1;
+}
+
+template <int RPL, int CH, int KM>
 int launch_t(const BgemmParams& p, hipStream_t stream) {
     const int n_tiles = (p.N + kNTile - 1) / kNTile;
     const int b_tiles = (p.B + 64 * RPL - 1) / (64 * RPL);
     const long long row_waves = (long long)p.OH * p.OW * b_tiles;
-    const long long blocks = (row_waves + kWavesPerBlock - 1) / kWavesPerBlock * n_tiles;
+    const long long row_blocks = (row_waves + kWavesPerBlock - 1) / kWavesPerBlock;
+    const long long blocks = row_blocks * n_tiles * p.ksplit;
     if (blocks <= 0 || blocks > 0x7fffffffLL) return fail(TCBNN_EINVAL, "bgemm grid too large");
-    hipLaunchKernelGGL((bgemm_popc_kernel<RPL, CH>), dim3((unsigned)blocks), dim3(kThreads), 0,
-                       stream, p, n_tiles, (int)row_waves, b_tiles);
+    hipLaunchKernelGGL((bgemm_popc_kernel<RPL, CH, KM>), dim3((unsigned)blocks), dim3(kThreads), 0,
+                       stream, p, n_tiles, (int)row_waves, b_tiles, (int)row_blocks);
     TCBNN_LAUNCH_CHECK("bgemm_popc_kernel");
     return TCBNN_OK;
 }
 
+int kernel_mode(const BgemmParams& p) {
+    if (p.ksplit > 1) return KM_PARTIAL;
+    if (p.mode == EPI_AFFINE) return KM_AFFINE;
+    if (p.mode == EPI_RAW) return KM_RAW;
+    return (p.res_in != nullptr || p.res_out != nullptr) ? KM_THRESH_RES : KM_THRESH;
+}
+
+template <int RPL, int CH>
+int launch_m(const BgemmParams& p, hipStream_t stream) {
+    switch (kernel_mode(p)) {
+        case KM_THRESH:
+            return launch_t<RPL, CH, KM_THRESH>(p, stream);
+        case KM_THRESH_RES:
+            return launch_t<RPL, CH, KM_THRESH_RES>(p, stream);
+        case KM_AFFINE:
+            return launch_t<RPL, CH, KM_AFFINE>(p, stream);
+        case KM_RAW:
+            return launch_t<RPL, CH, KM_RAW>(p, stream);
+        default:
+            return launch_t<RPL, CH, KM_PARTIAL>(p, stream);
+    }
+}
+
 template <int CH>
 int launch_r(const BgemmParams& p, hipStream_t stream) {
-    // rows per lane: as many 64-image tiles of the batch as there are, up to 4
-    if (p.B > 128) return launch_t<4, CH>(p, stream);
-    if (p.B > 64) return launch_t<2, CH>(p, stream);
-    return launch_t<1, CH>(p, stream);
+    if constexpr (CH == 1) {  // odd word counts are rare: one instance
+        return launch_m<1, CH>(p, stream);
+    } else {
+        switch (rows_per_lane(p)) {
+            case 4:
+                return launch_m<4, CH>(p, stream);
+            case 2:
+                return launch_m<2, CH>(p, stream);
+            default:
+                return launch_m<1, CH>(p, stream);
+        }
+    }
 }
+
+int chunk_words(const BgemmParams& p) { return p.cw % 4 == 0 ? 4 : (p.cw % 2 == 0 ? 2 : 1); }
 
 }  // namespace
 
@@ -309,11 +425,62 @@ int validate_bgemm(const BgemmParams& p) {
     return TCBNN_OK;
 }
 
-int launch_bgemm_popc(const BgemmParams& p, hipStream_t stream) {
-    if (int rc = validate_bgemm(p)) return rc;
-    if (p.cw % 4 == 0) return launch_r<4>(p, stream);
-    if (p.cw % 2 == 0) return launch_r<2>(p, stream);
-    return launch_r<1>(p, stream);
+int choose_ksplit(const BgemmParams& p) {
+    // only FC-shaped problems (one pixel, one tap) with a workspace are split
+    if (p.workspace == nullptr || p.PH * p.PW != 1 || p.R * p.S != 1 || p.res_in || p.res_out)
+        return 1;
+    const int n_tiles = (p.N + kNTile - 1) / kNTile;
+    const long long waves = (long long)((p.B + 63) / 64) * n_tiles;
+    const int chunks = p.cw / chunk_words(p);
+    int ks = (int)(2048 / waves);
+    ks = min(ks, chunks / 8);
+    return ks < 2 ? 1 : min(ks, 64);
+}
+
+int launch_splitk_clear(const BgemmParams& p, hipStream_t stream) {
+    const size_t n = (size_t)pad32(p.N) * p.B;
+    hipLaunchKernelGGL(splitk_clear_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream,
+                       p.workspace, n);
+    TCBNN_LAUNCH_CHECK("splitk_clear_kernel");
+    return TCBNN_OK;
+}
+
+int launch_splitk_finish(const BgemmParams& p, hipStream_t stream) {
+    const int n_tiles = (p.N + kNTile - 1) / kNTile;
+    const size_t n = (size_t)n_tiles * p.B;
+    hipLaunchKernelGGL(splitk_finish_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream,
+                       p, n_tiles);
+    TCBNN_LAUNCH_CHECK("splitk_finish_kernel");
+    return TCBNN_OK;
+}
+
+void bgemm_popc_kernel_name(const BgemmParams& p, char* buf, size_t len) {
+    BgemmParams q = p;
+    q.ksplit = choose_ksplit(p);
+    const int ch = chunk_words(q);
+    snprintf(buf, len, "bgemm_popc_kernel<%d, %d, %d>", ch == 1 ? 1 : rows_per_lane(q), ch, kernel_mode(q));
+}
+
+int launch_bgemm_popc(const BgemmParams& p_in, hipStream_t stream) {
+    if (int rc = validate_bgemm(p_in)) return rc;
+    BgemmParams p = p_in;
+    p.ksplit = choose_ksplit(p);
+    if (p.ksplit > 1)
+        if (int rc = launch_splitk_clear(p, stream)) return rc;
+    int rc;
+    switch (chunk_words(p)) {
+        case 4:
+            rc = launch_r<4>(p, stream);
+            break;
+        case 2:
+            rc = launch_r<2>(p, stream);
+            break;
+        default:
+            rc = launch_r<1>(p, stream);
+    }
+    if (rc) return rc;
+    if (p.ksplit > 1) return launch_splitk_finish(p, stream);
+    return TCBNN_OK;
 }
 
 }  // namespace tcbnn

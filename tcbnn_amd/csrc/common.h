@@ -41,15 +41,21 @@ int resolve_variant(int requested);
 // Implicit-GEMM problem shared by the FC, Out, Conv, bmm and bconv entry points.
 // Rows of the GEMM are (pre-pool output pixel, image); columns are output
 // neurons/channels; K runs over (filter tap, input-channel word).
+//
+// Device layouts (batch innermost, so that lane = image makes every activation,
+// residual and output access one contiguous run):
+//   activations  uint32 [H][W][cw][B]
+//   weights      uint32 [npad32][taps*cw]
+//   residuals    int32  [P][Q][O][B]
 // ---------------------------------------------------------------------------
 enum EpilogueMode : int {
     EPI_THRESH = 0,  // threshold -> bit, OR over the pool window, packed store
-    EPI_AFFINE = 1,  // (K - 2c)*scale + bias -> fp32
+    EPI_AFFINE = 1,  // (K - 2c)*scale + bias -> fp32 [B][N]
     EPI_RAW = 2,     // +-1 dot product -> int32
 };
 
 struct BgemmParams {
-    const uint32_t* act;  // [H][W][B][cw]
+    const uint32_t* act;  // [H][W][cw][B]
     const uint32_t* wgt;  // [npad32][taps*cw]
     int H, W, B, cw;      // input geometry, words per (pixel, image)
     int R, S, stride_h, stride_w, pad_h, pad_w;
@@ -60,28 +66,40 @@ struct BgemmParams {
     int k_tap;            // true K per tap (Cin, or K for FC)
     int mode;
     int nan_bit;          // bit emitted when the threshold compare is unordered
-    // EPI_THRESH
+    // EPI_THRESH: word (pooled pixel, word w, image b) at out_bits[pix*bits_pix_stride + w*B + b]
     const float* bn;
     uint32_t* out_bits;
-    long long bits_pix_stride, bits_b_stride;  // in words, indexed by pooled pixel
-    int bits_row_words;  // words per (pixel, image) row; those past ceil(N/32) are written as 0
+    long long bits_pix_stride;
+    int bits_row_words;  // words per pixel; those past ceil(N/32) are written as 0
     // EPI_AFFINE
     const float* bn_scale;
     const float* bn_bias;
     float* out_f32;  // [B][N]
-    // EPI_RAW
+    // EPI_RAW: out_i32[pix*raw_pix_stride + b*raw_b_stride + n], indexed by pre-pool pixel
     int32_t* out_i32;
-    long long raw_pix_stride, raw_b_stride;  // in ints, indexed by pre-pool pixel
+    long long raw_pix_stride, raw_b_stride;
     // residuals (pool 1x1 only)
-    const int32_t* res_in;
-    int res_in_ch;     // channel stride of the source
-    int res_limit;     // inject only into n < res_limit
-    int res_pool;      // 2x2 max over a source twice the output size
-    int32_t* res_out;  // [PH][PW][B][N]
+    const int32_t* res_in;  // [Hr][Wr][res_in_ch][B]
+    int res_in_ch;          // channels of the source
+    int res_limit;          // inject only into n < res_limit
+    int res_pool;           // 2x2 max over a source twice the output size
+    int32_t* res_out;       // [PH][PW][N][B]
+    // split-K (FC-shaped problems only): partial popcounts are atomically added into
+    // workspace[n*B + b] and a finishing kernel applies the epilogue
+    int32_t* workspace;
+    int ksplit;
 };
 
 int launch_bgemm_popc(const BgemmParams& p, hipStream_t stream);
 int launch_bgemm_mfma(const BgemmParams& p, int variant, hipStream_t stream);
 int validate_bgemm(const BgemmParams& p);
+// zero the split-K workspace / apply the epilogue to it (shared by both engines)
+int launch_splitk_clear(const BgemmParams& p, hipStream_t stream);
+int launch_splitk_finish(const BgemmParams& p, hipStream_t stream);
+// profiler-style kernel names for a problem
+void bgemm_popc_kernel_name(const BgemmParams& p, char* buf, size_t len);
+void bgemm_mfma_kernel_name(const BgemmParams& p, int variant, char* buf, size_t len);
+// number of K splits wanted for a problem (1 = none)
+int choose_ksplit(const BgemmParams& p);
 
 }  // namespace tcbnn

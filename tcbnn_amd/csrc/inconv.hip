@@ -7,23 +7,31 @@
 // are no multiplies (the sign is applied by flipping the fp32 sign bit with a
 // precomputed mask), hence no FMA contraction either.
 //
-// Mapping: lane = one pooled output pixel of one image, x fastest, so the 64
-// lanes of a wave read neighbouring input columns of the same image row; the
-// filter sign masks are wave-uniform (scalar loads).  A lane owns 32 output
-// channels per pass and builds the packed word in registers.
+// Two kernels:
+//   inconv_tiled_kernel (pool 1x1): workgroup = one output row y, 4 consecutive output
+//     columns (one per wave), 64 images (lane = image).  For each filter row the needed
+//     input row segment of the 64 images is read with lanes running along the image row
+//     (contiguous runs) and transposed through LDS to image-innermost order, so the
+//     compute phase reads LDS without bank conflicts, the filter sign masks are
+//     wave-uniform scalar loads, and the packed words / int32 residuals are written as
+//     contiguous 256-byte runs of the batch-innermost output layouts.
+//   inconv_generic_kernel (any pooling): one lane per pooled output pixel.
 #include "common.h"
 
 namespace tcbnn {
 namespace {
 
 constexpr int kThreads = 256;
+constexpr int kXT = 4;        // output columns per workgroup (one per wave)
+constexpr int kLB = 65;       // LDS row pitch in floats for 64 images (+1 against conflicts)
+constexpr int kMaxCols = 32;  // (kXT-1)*stride + S must fit
 
 struct InConvParams {
     const float* in;       // [B][3][H][W]
     const uint4* masks;    // [taps][opad32] {m0, m1, m2, 0}
     const float* bn;
-    uint32_t* out;         // [OH][OW][B][ow]
-    int32_t* res;          // [PH][PW][B][O] or null
+    uint32_t* out;         // [OH][OW][ow][B]
+    int32_t* res;          // [PH][PW][O][B] or null
     int H, W, B, O, opad, ow;
     int R, S, stride_h, stride_w, pad_h, pad_w;
     int PH, PW, pool_h, pool_w, OH, OW;
@@ -33,13 +41,105 @@ __device__ __forceinline__ float flip(float f, uint32_t m) {
     return __uint_as_float(__float_as_uint(f) ^ m);
 }
 
-__global__ __launch_bounds__(kThreads) void inconv_kernel(const InConvParams p) {
+// The read-only operands are separate __restrict__ kernel arguments so that the
+// wave-uniform mask / threshold loads become scalar loads (s_load) feeding v_xor directly.
+__global__ __launch_bounds__(kThreads) void inconv_tiled_kernel(
+    const InConvParams p, const float* __restrict__ in, const uint4* __restrict__ masks,
+    const float* __restrict__ bn, uint32_t* __restrict__ out, int32_t* __restrict__ res, int b_tiles,
+    int x_groups) {
+    __shared__ float tile[3 * kMaxCols * kLB];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int bt = blockIdx.x % b_tiles;
+    const int xg = (blockIdx.x / b_tiles) % x_groups;
+    const int y = blockIdx.x / (b_tiles * x_groups);
+    const int x0 = xg * kXT;
+    const int x = x0 + wave;
+    const bool x_ok = x < p.PW;  // wave-uniform
+    const int b0 = bt * 64;
+    const int b = b0 + lane;
+    const int ncols = (kXT - 1) * p.stride_w + p.S;
+    const int ax_base = x0 * p.stride_w - p.pad_w;
+    const size_t plane = (size_t)p.H * p.W;
+    const int n_groups = (p.O + 63) / 64;
+
+    for (int g = 0; g < n_groups; ++g) {
+        float acc[64];
+#pragma unroll
+        for (int n = 0; n < 64; ++n) acc[n] = 0.0f;
+        const bool second_half = g * 64 + 32 < p.opad;  // uniform
+
+        for (int r = 0; r < p.R; ++r) {
+            const int ay = y * p.stride_h - p.pad_h + r;
+            if (ay < 0 || ay >= p.H) continue;  // uniform for the whole workgroup
+            __syncthreads();
+            // stage: lanes run along the image row (contiguous), LDS is image-innermost
+            for (int e = tid; e < 3 * 64 * ncols; e += kThreads) {
+                const int col = e % ncols;
+                const int bc = e / ncols;
+                const int bl = bc & 63;
+                const int c = bc >> 6;
+                const int ax = ax_base + col;
+                const int bb = min(b0 + bl, p.B - 1);
+                float v = 0.0f;
+                if (ax >= 0 && ax < p.W) v = in[((size_t)bb * 3 + c) * plane + (size_t)ay * p.W + ax];
+                tile[(c * ncols + col) * kLB + bl] = v;
+            }
+            __syncthreads();
+            if (!x_ok) continue;
+            for (int s = 0; s < p.S; ++s) {
+                const int col = wave * p.stride_w + s;
+                const int ax = ax_base + col;
+                if (ax < 0 || ax >= p.W) continue;  // wave-uniform
+                const float f0 = tile[(0 * ncols + col) * kLB + lane];
+                const float f1 = tile[(1 * ncols + col) * kLB + lane];
+                const float f2 = tile[(2 * ncols + col) * kLB + lane];
+                const uint4* mk = masks + (size_t)(r * p.S + s) * p.opad + g * 64;
+#pragma unroll
+                for (int n = 0; n < 32; ++n) {
+                    const uint4 mm = mk[n];
+                    acc[n] += (flip(f0, mm.x) + flip(f1, mm.y)) + flip(f2, mm.z);
+                }
+                if (second_half) {
+#pragma unroll
+                    for (int n = 32; n < 64; ++n) {
+                        const uint4 mm = mk[n];
+                        acc[n] += (flip(f0, mm.x) + flip(f1, mm.y)) + flip(f2, mm.z);
+                    }
+                }
+            }
+        }
+
+        if (x_ok && b < p.B) {
+            const size_t pix = (size_t)y * p.PW + x;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int wi = g * 2 + h;
+                if (wi >= p.ow) continue;
+                uint32_t word = 0;
+#pragma unroll
+                for (int n = 0; n < 32; ++n) {
+                    const int ch = wi * 32 + n;
+                    if (ch < p.O) {
+                        word |= (acc[h * 32 + n] < bn[ch] ? 0u : 1u) << (31 - n);
+                        if (res != nullptr) res[(pix * p.O + ch) * p.B + b] = (int)acc[h * 32 + n];
+                    }
+                }
+                out[(pix * p.ow + wi) * p.B + b] = word;
+            }
+        }
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void inconv_generic_kernel(const InConvParams p) {
     const long long m = (long long)blockIdx.x * kThreads + threadIdx.x;
     const long long total = (long long)p.B * p.OH * p.OW;
     if (m >= total) return;
-    const int ox = (int)(m % p.OW);
-    const int oy = (int)((m / p.OW) % p.OH);
-    const int b = (int)(m / ((long long)p.OW * p.OH));
+    const int b = (int)(m % p.B);
+    const int ox = (int)((m / p.B) % p.OW);
+    const int oy = (int)(m / ((long long)p.B * p.OW));
     const size_t plane = (size_t)p.H * p.W;
     const float* img = p.in + (size_t)b * 3 * plane;
 
@@ -77,14 +177,14 @@ __global__ __launch_bounds__(kThreads) void inconv_kernel(const InConvParams p) 
                     if (ch < p.O) word |= (acc[n] < p.bn[ch] ? 0u : 1u) << (31 - n);
                 }
                 if (p.res != nullptr) {
-                    int32_t* dst = p.res + (((size_t)y * p.PW + x) * p.B + b) * p.O;
+                    int32_t* dst = p.res + ((size_t)y * p.PW + x) * p.O * p.B + b;
 #pragma unroll
                     for (int n = 0; n < 32; ++n)
-                        if (g * 32 + n < p.O) dst[g * 32 + n] = (int)acc[n];
+                        if (g * 32 + n < p.O) dst[(size_t)(g * 32 + n) * p.B] = (int)acc[n];
                 }
             }
         }
-        p.out[(((size_t)oy * p.OW + ox) * p.B + b) * p.ow + g] = word;
+        p.out[(((size_t)oy * p.OW + ox) * p.ow + g) * p.B + b] = word;
     }
 }
 
@@ -136,11 +236,23 @@ extern "C" int tcbnn_inconv128_forward(const tcbnn_inconv128_desc* d, void* stre
     TCBNN_REQUIRE(p.PH > 0 && p.PW > 0, "inconv128: empty output");
     p.OH = (p.PH + p.pool_h - 1) / p.pool_h;
     p.OW = (p.PW + p.pool_w - 1) / p.pool_w;
+
+    const bool tiled = p.pool_h == 1 && p.pool_w == 1 && (kXT - 1) * p.stride_w + p.S <= kMaxCols;
+    if (tiled) {
+        const int b_tiles = (p.B + 63) / 64;
+        const int x_groups = (p.PW + kXT - 1) / kXT;
+        const long long blocks = (long long)b_tiles * x_groups * p.PH;
+        TCBNN_REQUIRE(blocks <= 0x7fffffffLL, "inconv128: grid too large");
+        hipLaunchKernelGGL(inconv_tiled_kernel, dim3((unsigned)blocks), dim3(kThreads), 0,
+                           (hipStream_t)stream, p, p.in, p.masks, p.bn, p.out, p.res, b_tiles, x_groups);
+        TCBNN_LAUNCH_CHECK("inconv_tiled_kernel");
+        return TCBNN_OK;
+    }
     const long long total = (long long)p.B * p.OH * p.OW;
     const long long blocks = (total + kThreads - 1) / kThreads;
     TCBNN_REQUIRE(blocks <= 0x7fffffffLL, "inconv128: grid too large");
-    hipLaunchKernelGGL(inconv_kernel, dim3((unsigned)blocks), dim3(kThreads), 0,
+    hipLaunchKernelGGL(inconv_generic_kernel, dim3((unsigned)blocks), dim3(kThreads), 0,
                        (hipStream_t)stream, p);
-    TCBNN_LAUNCH_CHECK("inconv_kernel");
+    TCBNN_LAUNCH_CHECK("inconv_generic_kernel");
     return TCBNN_OK;
 }

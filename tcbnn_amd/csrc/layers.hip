@@ -73,6 +73,7 @@ static BgemmParams fc_problem(const uint32_t* input, const uint32_t* weight, int
     p.pool_h = p.pool_w = 1;
     p.N = n;
     p.k_tap = k;
+    p.ksplit = 1;
     return p;
 }
 
@@ -133,8 +134,10 @@ int tcbnn_fc128_forward(const tcbnn_fc128_desc* d, void* stream) {
     p.bn = d->bn;
     p.out_bits = d->output;
     p.bits_pix_stride = 0;
-    p.bits_b_stride = kw128(d->weight_width);
     p.bits_row_words = kw128(d->weight_width);
+    if (d->workspace != nullptr &&
+        d->workspace_words >= (size_t)pad32(d->weight_width) * d->input_height)
+        p.workspace = d->workspace;
     return run_bgemm(p, d->variant, (hipStream_t)stream);
 }
 
@@ -195,16 +198,11 @@ int tcbnn_conv128_forward(const tcbnn_conv128_desc* d, void* stream) {
     p.bn = d->bn;
     p.out_bits = d->output;
     const int ow = step32(p.N);
-    if (d->ahead_fc) {
-        const int ow128 = kw128(p.N);
-        p.bits_pix_stride = ow128;
-        p.bits_b_stride = (long long)p.OH * p.OW * ow128;
-        p.bits_row_words = ow128;
-    } else {
-        p.bits_pix_stride = (long long)p.B * ow;
-        p.bits_b_stride = ow;
-        p.bits_row_words = ow;
-    }
+    // FC-ready output pads every pixel's channels to 128 (kernel.cuh:798-808); with the
+    // batch-innermost layout that is the only difference from the normal conv output
+    p.bits_row_words = d->ahead_fc ? kw128(p.N) : ow;
+    p.bits_pix_stride = (long long)p.bits_row_words * p.B;
+    p.ksplit = 1;
     if (d->inject_residual) {
         TCBNN_NOTNULL(d->input_residual);
         TCBNN_REQUIRE(d->input_residual_channels > 0, "conv128: input_residual_channels unset");
@@ -219,6 +217,48 @@ int tcbnn_conv128_forward(const tcbnn_conv128_desc* d, void* stream) {
         p.res_out = d->output_residual;
     }
     return run_bgemm(p, d->variant, (hipStream_t)stream);
+}
+
+static int kernel_name(const BgemmParams& p, int variant, char* buf, size_t len) {
+    TCBNN_NOTNULL(buf);
+    TCBNN_REQUIRE(len > 0, "kernel_name: empty buffer");
+    const int v = resolve_variant(variant);
+    if (v == TCBNN_VARIANT_POPC)
+        bgemm_popc_kernel_name(p, buf, len);
+    else
+        bgemm_mfma_kernel_name(p, v, buf, len);
+    return TCBNN_OK;
+}
+
+int tcbnn_conv128_kernel_name(const tcbnn_conv128_desc* d, char* buf, size_t len) {
+    TCBNN_NOTNULL(d);
+    BgemmParams p;
+    memset(&p, 0, sizeof(p));
+    p.B = d->batch;
+    p.cw = step32(d->input_channels);
+    p.R = d->filter_height;
+    p.S = d->filter_width;
+    p.pool_h = d->pool_height;
+    p.pool_w = d->pool_width;
+    p.PH = tcbnn_conv_out(d->input_height, p.R, d->stride_height, d->padding, 1);
+    p.PW = tcbnn_conv_out(d->input_width, p.S, d->stride_width, d->padding, 1);
+    p.OH = (p.PH + p.pool_h - 1) / p.pool_h;
+    p.OW = (p.PW + p.pool_w - 1) / p.pool_w;
+    p.N = d->output_channels;
+    p.ksplit = 1;
+    p.mode = EPI_THRESH;
+    // only nullness matters for the name
+    p.res_in = d->inject_residual ? reinterpret_cast<const int32_t*>(d) : nullptr;
+    p.res_out = d->save_residual ? reinterpret_cast<int32_t*>(const_cast<tcbnn_conv128_desc*>(d)) : nullptr;
+    return kernel_name(p, d->variant, buf, len);
+}
+int tcbnn_fc128_kernel_name(const tcbnn_fc128_desc* d, char* buf, size_t len) {
+    TCBNN_NOTNULL(d);
+    BgemmParams p = fc_problem(nullptr, nullptr, d->input_height, d->input_width, d->weight_width);
+    if (d->workspace != nullptr &&
+        d->workspace_words >= (size_t)pad32(d->weight_width) * d->input_height)
+        p.workspace = d->workspace;
+    return kernel_name(p, d->variant, buf, len);
 }
 
 int tcbnn_bmm(const uint32_t* a, const uint32_t* b, int32_t* c, int m, int n, int k, int variant,
@@ -243,6 +283,7 @@ int tcbnn_bmm(const uint32_t* a, const uint32_t* b, int32_t* c, int m, int n, in
     p.N = n;
     p.k_tap = k;
     p.mode = EPI_RAW;
+    p.ksplit = 1;
     p.out_i32 = c;
     p.raw_pix_stride = 0;
     p.raw_b_stride = n;
@@ -280,6 +321,7 @@ int tcbnn_bconv(const uint32_t* input, const uint32_t* filter, int32_t* output, 
     p.N = out_ch;
     p.k_tap = in_ch;
     p.mode = EPI_RAW;
+    p.ksplit = 1;
     p.out_i32 = output;
     p.raw_pix_stride = out_ch;
     p.raw_b_stride = (long long)out_h * out_w * out_ch;

@@ -16,12 +16,15 @@ inline unsigned blocks_for(long long n, int per_block = kThreads) {
 
 // One wave binarises 64 consecutive elements of one row with a ballot:
 // a fully coalesced 256-byte read yields two MSB-first words.
-// src element (row, k) at src[row*row_stride + k*k_stride].
+// src element (row, k) at src[row*row_stride + k*k_stride]; word (row, w) goes to
+// dst[row*dst_row_stride + w*dst_word_stride].
 __global__ __launch_bounds__(kThreads) void pack_rows_kernel(const float* __restrict__ src,
                                                              uint32_t* __restrict__ dst,
                                                              long long rows, int k,
                                                              long long row_stride,
-                                                             long long k_stride, int k_words) {
+                                                             long long k_stride, int k_words,
+                                                             long long dst_row_stride,
+                                                             long long dst_word_stride) {
     const int lane = threadIdx.x & 63;
     const long long wave = ((long long)blockIdx.x * kThreads + threadIdx.x) >> 6;
     const int segs = (k_words + 1) >> 1;  // 64-element segments per row
@@ -32,8 +35,9 @@ __global__ __launch_bounds__(kThreads) void pack_rows_kernel(const float* __rest
     const float f = kk < k ? src[row * row_stride + kk * k_stride] : -1.0f;
     const unsigned long long m = __ballot(f >= 0.0f);
     if (lane == 0) {
-        dst[row * k_words + 2 * seg] = __brev((unsigned)(m & 0xffffffffull));
-        if (2 * seg + 1 < k_words) dst[row * k_words + 2 * seg + 1] = __brev((unsigned)(m >> 32));
+        uint32_t* d = dst + row * dst_row_stride;
+        d[(2 * seg) * dst_word_stride] = __brev((unsigned)(m & 0xffffffffull));
+        if (2 * seg + 1 < k_words) d[(2 * seg + 1) * dst_word_stride] = __brev((unsigned)(m >> 32));
     }
 }
 
@@ -72,15 +76,15 @@ __global__ void pack_inconv_filter_kernel(const float* __restrict__ f, uint32_t*
     dst[idx] = m;
 }
 
-// NHWC fp32 -> [H][W][B][cw]; one thread per output word.
+// NHWC fp32 -> [H][W][cw][B]; one thread per output word.
 __global__ void pack_conv_input_nhwc_kernel(const float* __restrict__ src,
                                             uint32_t* __restrict__ dst, int batch, int height,
                                             int width, int ch, int cw) {
     const long long idx = (long long)blockIdx.x * kThreads + threadIdx.x;
     const long long total = (long long)height * width * batch * cw;
     if (idx >= total) return;
-    const int w = (int)(idx % cw);
-    const int b = (int)((idx / cw) % batch);
+    const int b = (int)(idx % batch);
+    const int w = (int)((idx / batch) % cw);
     const long long pix = idx / ((long long)cw * batch);
     const float* s = src + ((size_t)b * height * width + pix) * ch + w * 32;
     uint32_t word = 0;
@@ -95,7 +99,7 @@ __global__ void unpack_fc_kernel(const uint32_t* __restrict__ packed, float* __r
     if (idx >= (long long)batch * features) return;
     const int k = (int)(idx % features);
     const long long b = idx / features;
-    const uint32_t w = packed[b * kw + (k >> 5)];
+    const uint32_t w = packed[(long long)(k >> 5) * batch + b];
     out[idx] = 2.0f * (float)((w >> (31 - (k & 31))) & 1u) - 1.0f;
 }
 
@@ -107,11 +111,11 @@ __global__ void unpack_conv_kernel(const uint32_t* __restrict__ packed, float* _
     const int c = (int)(idx % ch);
     const long long pix = (idx / ch) % ((long long)height * width);
     const long long b = idx / ((long long)ch * height * width);
-    const uint32_t w = packed[(pix * batch + b) * cw + (c >> 5)];
+    const uint32_t w = packed[(pix * cw + (c >> 5)) * batch + b];
     out[idx] = 2.0f * (float)((w >> (31 - (c & 31))) & 1u) - 1.0f;
 }
 
-// engine rows [rows][row_words] <-> reference tiles [groups][ceil(rows/8)][row128][8][4]
+// engine [groups][row_words][rows] <-> reference tiles [groups][ceil(rows/8)][row128][8][4]
 // where `groups` is the number of leading (pixel) blocks, each holding `rows` rows.
 // to_fmt != 0: fmt is written (zero where the engine has no word); else packed is written.
 __global__ void fmt_convert_kernel(uint32_t* __restrict__ packed, uint32_t* __restrict__ fmt,
@@ -131,7 +135,7 @@ __global__ void fmt_convert_kernel(uint32_t* __restrict__ packed, uint32_t* __re
     const int row = rt * 8 + r;
     const int word = kc * 4 + w;
     const bool has = row < rows && word < row_words;
-    const long long pidx = (g * rows + row) * row_words + word;
+    const long long pidx = (g * row_words + word) * rows + row;
     if (to_fmt)
         fmt[idx] = has ? packed[pidx] : 0u;
     else if (has)
@@ -146,7 +150,7 @@ __global__ void residual_to_reference_kernel(const int32_t* __restrict__ res,
     const int c = (int)(idx % c128);
     const int b = (int)((idx / c128) % b8);
     const long long pix = idx / ((long long)c128 * b8);
-    ref[idx] = (b < batch && c < ch) ? res[(pix * batch + b) * ch + c] : 0;
+    ref[idx] = (b < batch && c < ch) ? res[(pix * ch + c) * batch + b] : 0;
 }
 
 }  // namespace
@@ -164,7 +168,7 @@ int tcbnn_pack_rows(const float* src, uint32_t* packed, int rows, int k, int ld,
     const long long waves = (long long)rows * ((k_words + 1) / 2);
     hipLaunchKernelGGL(pack_rows_kernel, dim3(blocks_for(waves * 64)), dim3(kThreads), 0,
                        (hipStream_t)stream, src, packed, (long long)rows, k, (long long)ld, 1LL,
-                       k_words);
+                       k_words, 1LL, (long long)rows);
     TCBNN_LAUNCH_CHECK("pack_rows_kernel");
     return TCBNN_OK;
 }
@@ -176,7 +180,7 @@ int tcbnn_pack_cols(const float* src, uint32_t* packed, int k, int n, int k_word
     const long long waves = (long long)n * ((k_words + 1) / 2);
     hipLaunchKernelGGL(pack_rows_kernel, dim3(blocks_for(waves * 64)), dim3(kThreads), 0,
                        (hipStream_t)stream, src, packed, (long long)n, k, 1LL, (long long)n,
-                       k_words);
+                       k_words, (long long)k_words, 1LL);
     TCBNN_LAUNCH_CHECK("pack_cols_kernel");
     return TCBNN_OK;
 }

@@ -9,7 +9,9 @@ Conv128LayerParam.  Differences forced by the redesign:
     the device function called inside the reference's cooperative network kernel;
   * `download_output()` returns the packed activations in the reference's
     tile-contiguous layout (what the reference's download_output() yields);
-    `download_packed()` returns the engine layout.
+    `download_packed()` returns them as plain row-major words ([B][KW] for FC layers,
+    [H][W][B][CW] for conv layers), transposed on the host from the engine's
+    batch-innermost device layout.
 All compute goes through the C ABI of libtcbnn_hip.so.
 """
 import ctypes as C
@@ -118,7 +120,8 @@ class In128LayerParam:
         check(lib.tcbnn_in128_forward(C.byref(d), _stream_handle(stream)))
 
     def download_packed(self):
-        return self.output_gpu.to_numpy(np.uint32, (self.output_height, 4 * STEP128(self.output_width)))
+        eng = self.output_gpu.to_numpy(np.uint32, (4 * STEP128(self.output_width), self.output_height))
+        return np.ascontiguousarray(eng.T)
 
     def download_output(self):
         return _fc_download_fmt(self.output_gpu, self.output_height, self.output_width)
@@ -183,6 +186,9 @@ class Fc128LayerParam:
         self.bn = np.array(config_file.launch_array(self.bn_size()), dtype=np.float32)
         self.bn_gpu = DeviceBuffer.from_numpy(self.bn)
         self.output_gpu = DeviceBuffer(4 * lib.tcbnn_fc_act_words(self.output_height, self.output_width))
+        # scratch for split-K: int32 [PAD32(N)][B]
+        self.workspace_words = PAD32(self.weight_width) * self.input_height
+        self.workspace_gpu = DeviceBuffer(4 * self.workspace_words)
         self.set_input_gpu(prev_layer_gpu)
         if self.input_gpu is None:
             raise _lib.TcbnnError("Error: NULL pointer (input_gpu)")
@@ -191,13 +197,24 @@ class Fc128LayerParam:
     def get_output_gpu(self):
         return self.output_gpu
 
+    def _desc(self):
+        return _lib.Fc128Desc(self.input_gpu.ptr, self.weight_gpu.ptr, self.bn_gpu.ptr, self.output_gpu.ptr,
+                              self.input_height, self.input_width, self.weight_width, self.variant,
+                              self.workspace_gpu.ptr, self.workspace_words)
+
     def forward(self, stream=None):
-        d = _lib.Fc128Desc(self.input_gpu.ptr, self.weight_gpu.ptr, self.bn_gpu.ptr, self.output_gpu.ptr,
-                           self.input_height, self.input_width, self.weight_width, self.variant, None, 0)
+        d = self._desc()
         check(lib.tcbnn_fc128_forward(C.byref(d), _stream_handle(stream)))
 
+    def kernel_name(self):
+        buf = C.create_string_buffer(128)
+        d = self._desc()
+        check(lib.tcbnn_fc128_kernel_name(C.byref(d), buf, 128))
+        return buf.value.decode()
+
     def download_packed(self):
-        return self.output_gpu.to_numpy(np.uint32, (self.output_height, 4 * STEP128(self.output_width)))
+        eng = self.output_gpu.to_numpy(np.uint32, (4 * STEP128(self.output_width), self.output_height))
+        return np.ascontiguousarray(eng.T)
 
     def download_output(self):
         return _fc_download_fmt(self.output_gpu, self.output_height, self.output_width)
@@ -206,10 +223,10 @@ class Fc128LayerParam:
         return _fc_download_full(self.output_gpu, self.output_height, self.output_width)
 
     def release(self):
-        for b in (self.weight_gpu, self.bn_gpu, self.output_gpu):
+        for b in (self.weight_gpu, self.bn_gpu, self.output_gpu, getattr(self, "workspace_gpu", None)):
             if b is not None:
                 b.free()
-        self.weight_gpu = self.bn_gpu = self.output_gpu = None
+        self.weight_gpu = self.bn_gpu = self.output_gpu = self.workspace_gpu = None
 
 
 class Out128LayerParam:
@@ -301,9 +318,10 @@ class _ConvGeometry:
         return self.output_residual_gpu
 
     def download_residual(self):
-        """Saved residual in the engine layout int32 [P][Q][B][O]."""
-        return self.output_residual_gpu.to_numpy(
-            np.int32, (self.buf_height, self.buf_width, self.batch, self.output_channels))
+        """Saved residual as int32 [P][Q][B][O] (host transpose of the engine's [P][Q][O][B])."""
+        eng = self.output_residual_gpu.to_numpy(
+            np.int32, (self.buf_height, self.buf_width, self.output_channels, self.batch))
+        return np.ascontiguousarray(eng.transpose(0, 1, 3, 2))
 
     def download_residual_reference(self):
         """Saved residual in the reference layout int32 [P][Q][PAD8(B)][PAD128(O)]."""
@@ -319,10 +337,12 @@ class _ConvGeometry:
 
     def download_packed(self):
         if self._is_fc_ready():
-            return self.output_gpu.to_numpy(
-                np.uint32, (self.batch, self.output_height * self.output_width * 4 * STEP128(self.output_channels)))
-        return self.output_gpu.to_numpy(
-            np.uint32, (self.output_height, self.output_width, self.batch, STEP32(self.output_channels)))
+            eng = self.output_gpu.to_numpy(
+                np.uint32, (self.output_height * self.output_width * 4 * STEP128(self.output_channels), self.batch))
+            return np.ascontiguousarray(eng.T)
+        eng = self.output_gpu.to_numpy(
+            np.uint32, (self.output_height, self.output_width, STEP32(self.output_channels), self.batch))
+        return np.ascontiguousarray(eng.transpose(0, 1, 3, 2))
 
     def download_output(self):
         if self._is_fc_ready():
@@ -471,9 +491,9 @@ class Conv128LayerParam(_ConvGeometry):
             raise _lib.TcbnnError("Error: NULL pointer (input_gpu)")
         return self
 
-    def forward(self, stream=None):
+    def _desc(self):
         rin = self.input_residual_gpu if self.inject_residual else None
-        d = _lib.Conv128Desc(
+        return _lib.Conv128Desc(
             self.input_gpu.ptr, self.filter_gpu.ptr, self.bn_gpu.ptr, self.output_gpu.ptr,
             rin.ptr if rin is not None else None,
             self.output_residual_gpu.ptr if self.output_residual_gpu is not None else None,
@@ -482,7 +502,16 @@ class Conv128LayerParam(_ConvGeometry):
             self.pool_height, self.pool_width, int(self.ahead_fc), int(self.save_residual),
             int(self.inject_residual), self.residual_channels, int(self.residual_pool),
             rin.channels if rin is not None else 0, self.variant)
+
+    def forward(self, stream=None):
+        d = self._desc()
         check(lib.tcbnn_conv128_forward(C.byref(d), _stream_handle(stream)))
+
+    def kernel_name(self):
+        buf = C.create_string_buffer(128)
+        d = self._desc()
+        check(lib.tcbnn_conv128_kernel_name(C.byref(d), buf, 128))
+        return buf.value.decode()
 
     def release(self):
         for b in (self.filter_gpu, self.bn_gpu, self.output_gpu, self.output_residual_gpu):

@@ -53,14 +53,21 @@ def in128(x):
     return out
 
 
-def fc128(inp_buf, w_buf, bn, b, k, n, variant=0):
+def fc128(inp_buf, w_buf, bn, b, k, n, variant=0, workspace=True):
+    """Returns the packed output as [B][KW128(n)] rows."""
     out = DeviceBuffer(4 * lib.tcbnn_fc_act_words(b, n))
     out.fill(0xAB)  # the call must overwrite every word, padding included
     bnb = dev(bn.astype(np.float32))
-    d = _lib.Fc128Desc(inp_buf.ptr, w_buf.ptr, bnb.ptr, out.ptr, b, k, n, variant, None, 0)
+    ws_words = ((n + 31) // 32) * 32 * b
+    ws = DeviceBuffer(4 * ws_words) if workspace else None
+    if ws is not None:
+        ws.fill(0x5A)  # the call must clear what it accumulates into
+    d = _lib.Fc128Desc(inp_buf.ptr, w_buf.ptr, bnb.ptr, out.ptr, b, k, n, variant,
+                       ws.ptr if ws else None, ws_words if ws else 0)
     check(lib.tcbnn_fc128_forward(C.byref(d), None))
     sync()
-    return out
+    kw = lib.tcbnn_fc_act_words(1, n)
+    return np.ascontiguousarray(out.to_numpy(np.uint32, (kw, b)).T)
 
 
 def out128(inp_buf, w_buf, scale, bias, b, k, n, variant=0):
@@ -73,7 +80,8 @@ def out128(inp_buf, w_buf, scale, bias, b, k, n, variant=0):
 
 
 def bmm(a_packed, b_packed, m, n, k, variant=0):
-    a, b = dev(a_packed), dev(b_packed)
+    """a_packed: [M][K/32] rows (uploaded in the engine's [K/32][M] layout); b_packed: [N][K/32]."""
+    a, b = dev(np.ascontiguousarray(a_packed.T)), dev(b_packed)
     c = DeviceBuffer(4 * m * n)
     check(lib.tcbnn_bmm(a.ptr, b.ptr, c.ptr, m, n, k, variant, None))
     sync()

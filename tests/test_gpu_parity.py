@@ -61,8 +61,9 @@ def test_fc128(gpu, variant, b, k, n):
     want = orc.fc128(orc.in128(x), wl, bn, k, n)
     inp = gpuops.in128(x)
     wbuf = gpuops.pack_fc_weight(w)
-    out = gpuops.fc128(inp, wbuf, bn, b, k, n, _variant(gpu, variant))
-    got = out.to_numpy(np.uint32, (b, orc.kw128(n)))
+    got = gpuops.fc128(inp, wbuf, bn, b, k, n, _variant(gpu, variant))
+    np.testing.assert_array_equal(got, want)
+    got = gpuops.fc128(inp, wbuf, bn, b, k, n, _variant(gpu, variant), workspace=False)  # no split-K
     np.testing.assert_array_equal(got, want)
     # packed weights agree with the oracle's packing (rows >= N are zero)
     wg = wbuf.to_numpy(np.uint32, (((n + 31) // 32) * 32, orc.kw128(k)))
@@ -77,7 +78,7 @@ def test_fc128_nan_threshold(gpu, variant):
     w = rm.pm1(r, (128, 32))
     bn = np.full(32, np.nan, np.float32)
     out = gpuops.fc128(gpuops.in128(x), gpuops.pack_fc_weight(w), bn, 8, 128, 32, _variant(gpu, variant))
-    assert not out.to_numpy(np.uint32, (8, 4)).any()
+    assert out.shape == (8, 4) and not out.any()
 
 
 @pytest.mark.parametrize("variant", VARIANTS)
@@ -109,7 +110,8 @@ def test_bconv_sweep_shapes(gpu, variant, h, c):
     pad, buf, _ = orc.conv_geometry(h, 3, 1)
     want = orc.bconv(orc.pack_conv_input_nhwc(x), orc.pack_conv_filter(f), c, c, 3, 3, 1, pad, buf, buf)
     inp, filt = gpuops.pack_conv_input(x), gpuops.pack_conv_filter(f)
-    np.testing.assert_array_equal(inp.to_numpy(np.uint32, (h, h, b, c // 32)), orc.pack_conv_input_nhwc(x))
+    np.testing.assert_array_equal(inp.to_numpy(np.uint32, (h, h, c // 32, b)).transpose(0, 1, 3, 2),
+                                  orc.pack_conv_input_nhwc(x))
     got = gpuops.bconv(inp, filt, b, h, h, c, c, 3, 3, 1, pad, buf, buf, _variant(gpu, variant))
     np.testing.assert_array_equal(got, want)
 
@@ -147,7 +149,7 @@ def _run_conv_layer(gpu, variant, x, f, bn, stride=1, pool=1, ahead_fc=False, sa
     src = gpuops.pack_conv_input(x)
     rbuf = None
     if inject_residual:
-        rbuf = gpuops.dev(res_in.astype(np.int32))
+        rbuf = gpuops.dev(np.ascontiguousarray(res_in.astype(np.int32).transpose(0, 1, 3, 2)))  # [Hr][Wr][C][B]
         rbuf.channels = res_in.shape[-1]
     layer.initialize(gpu.ArrayWeights([f, bn]), src, rbuf)
     layer.output_gpu.fill(0xCD)  # every output word must be written by the call
