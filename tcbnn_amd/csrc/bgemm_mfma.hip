@@ -1,14 +1,453 @@
-// Matrix-core variants of the implicit GEMM (placeholder until the MFMA kernels land).
+// Matrix-core variants of the bit implicit GEMM for gfx950.
+//
+// CDNA4 has no 1-bit MFMA, so the packed +-1 operands are expanded on the fly to the
+// narrowest type the matrix cores multiply exactly:
+//   FMT_F4: FP4 E2M1 nibbles (+1.0 = 0x2, -1.0 = 0xA, 0 = 0x0), v_mfma_f32_32x32x64_f8f6f4.
+//           Products are exactly +-1 or 0 and every partial sum is an integer below 2^24,
+//           so the fp32 accumulator is exact whatever the internal summation order.
+//   FMT_I8: int8 bytes (+1 = 0x01, -1 = 0xFF, 0), v_mfma_i32_32x32x32_i8, int32 accumulate.
+// A 32-bit word of packed bits becomes 4 dwords of FP4 with 7 VALU ops (shift, and-or),
+// which is amortised over the 32*NT output channels the wave multiplies it with.
+//
+// Operand roles are transposed with respect to the usual GEMM: the MFMA "A" operand holds
+// 32 output channels (weights), the "B" operand 32 images, so in the accumulator a lane owns
+// ONE image and 16 channels.  With the batch-innermost layouts this gives
+//   - activation loads: lane (image j, k-half h) reads word 2t+h of its image: two contiguous
+//     128-byte runs per wave load;
+//   - epilogue: threshold -> bit -> shift/or builds a 16-channel half-word in the lane, one
+//     cross-lane swap (lane ^ 32) completes the 32-channel word, 128-byte contiguous stores;
+//     residual loads/stores are contiguous runs as well; no atomics, pool windows are a
+//     sequential loop (OR), every output word is written exactly once.
+// The weight rows of a channel tile are permuted when they are staged so that accumulator
+// register v of lane half h is channel 16h+v.  Weights are expanded once per workgroup into
+// LDS in MFMA-fragment order ([k-step][channel tile][lane] x 16 bytes, conflict-free
+// ds_read_b128); pad bits and out-of-range channels are staged as zeros, so the true K / Cin
+// enters the result without any correction term, and zero padding of the convolution is
+// simply a skipped tap (kernel.cuh:752-768 "exclude").
+//
+// Semantics: Fc128LayerFMT / Out128LayerFMT / Conv128LayerFMT (kernel.cuh:174-280, 676-827),
+// BMMAS / BTC_Conv2d_balance (tensorcore_kernel.cu:305-356, bmma_kernel.cu:101-165).
 #include "common.h"
 
 namespace tcbnn {
-int launch_bgemm_mfma(const BgemmParams& p, int variant, hipStream_t stream) {
-    (void)p;
-    (void)stream;
-    return fail(TCBNN_EUNSUPPORTED, "MFMA variant %d is not built", variant);
+namespace {
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+constexpr int FMT_F4 = 0;
+constexpr int FMT_I8 = 1;
+constexpr int kWaves = 4;
+constexpr int kThreads = 64 * kWaves;
+constexpr int kNT = 2;    // 32-channel tiles per wave
+constexpr int kQB = 24;   // k-steps of weights staged in LDS at a time (24 * kNT KiB)
+
+enum MfmaMode : int { MM_THRESH = 0, MM_THRESH_RES = 1, MM_OTHER = 2 };
+
+// ---- bit expansion ----------------------------------------------------------------
+// FP4: bit value 1 -> nibble 0xA (-1.0), 0 -> 0x2 (+1.0): the sign is flipped for BOTH
+// operands, so products are unchanged.  dword j takes bits {4p + (3-j)}.
+__device__ __forceinline__ v4i expand_f4(uint32_t x) {
+    v4i r;
+    r[0] = ((x << 3) & 0x88888888u) | 0x22222222u;
+    r[1] = ((x << 2) & 0x88888888u) | 0x22222222u;
+    r[2] = ((x << 1) & 0x88888888u) | 0x22222222u;
+    r[3] = (x & 0x88888888u) | 0x22222222u;
+    return r;
 }
+// nibbles whose bit is not `valid` become FP4 zero
+__device__ __forceinline__ v4i expand_f4_masked(uint32_t x, uint32_t valid) {
+    v4i r = expand_f4(x);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t t = ((valid << (3 - j)) & 0x88888888u) >> 3;  // 0x1 per valid nibble
+        r[j] &= (int)(t * 15u);
+    }
+    return r;
+}
+// int8: lane half h of a 32-bit word takes bits {q + 4h + 8p}; bit 1 -> 0x01, bit 0 -> 0xFF
+__device__ __forceinline__ v4i expand_i8(uint32_t x, int h) {
+    v4i r;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const uint32_t d = (x >> (q + 4 * h)) & 0x01010101u;
+        const uint32_t m = (d << 8) - d;  // 0xFF in every byte whose bit is set
+        r[q] = (int)(~m | 0x01010101u);
+    }
+    return r;
+}
+__device__ __forceinline__ v4i expand_i8_masked(uint32_t x, uint32_t valid, int h) {
+    v4i r = expand_i8(x, h);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const uint32_t d = (valid >> (q + 4 * h)) & 0x01010101u;
+        r[q] &= (int)((d << 8) - d);
+    }
+    return r;
+}
+
+template <int FMT>
+struct Acc;
+template <>
+struct Acc<FMT_F4> {
+    using type = v16f;
+    static __device__ __forceinline__ type mma(v4i a, v4i b, type c) {
+        const v8i a8 = {a[0], a[1], a[2], a[3], 0, 0, 0, 0};
+        const v8i b8 = {b[0], b[1], b[2], b[3], 0, 0, 0, 0};
+        // cbsz = blgp = 4: both operands FP4; scale operands 0 select the unscaled instruction
+        return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8, b8, c, 4, 4, 0, 0, 0, 0);
+    }
+    static __device__ __forceinline__ int to_int(float v) { return (int)v; }
+};
+template <>
+struct Acc<FMT_I8> {
+    using type = v16i;
+    static __device__ __forceinline__ type mma(v4i a, v4i b, type c) {
+        return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ int to_int(int v) { return v; }
+};
+
+__device__ __forceinline__ uint32_t thresh_bit(int res, float thr, int nan_bit) {
+    const float rf = (float)res;
+    return nan_bit ? (rf < thr ? 0u : 1u) : (rf >= thr ? 1u : 0u);
+}
+
+// MFMA row i of a channel tile holds channel perm(i), so that accumulator register v of
+// lane half h (row 8*(v/4) + 4h + v%4) is channel 16h + v.
+__device__ __forceinline__ int row_to_channel(int i) {
+    return 16 * ((i >> 2) & 1) + 4 * (i >> 3) + (i & 3);
+}
+
+template <int FMT, int MT, int MM>
+__global__ __launch_bounds__(kThreads) void bgemm_mfma_kernel(
+    const BgemmParams p, const uint32_t* __restrict__ act, const uint32_t* __restrict__ wgt,
+    const float* __restrict__ bnp, const int32_t* __restrict__ rin, int n_groups, int row_waves,
+    int b_groups, int row_blocks) {
+    using A = Acc<FMT>;
+    using acc_t = typename A::type;
+    __shared__ v4i lds_w[kQB * kNT * 64];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int j = lane & 31;   // image within a 32-image tile
+    const int h = lane >> 5;   // k half (operands) / channel half (accumulator)
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int ng = blockIdx.x % n_groups;
+    const int rb = (blockIdx.x / n_groups) % row_blocks;
+    const int ks = blockIdx.x / (n_groups * row_blocks);
+    const int rw = rb * kWaves + wave;
+    const bool active = rw < row_waves;
+    const int n0 = ng * (32 * kNT);
+
+    const int taps = p.R * p.S;
+    const int kw_tot = taps * p.cw;
+    const int steps = FMT == FMT_F4 ? (p.cw + 1) / 2 : p.cw;  // k-steps per tap
+    const int nq_all = taps * steps;
+    const int q_per = (nq_all + p.ksplit - 1) / p.ksplit;
+    const int q_begin = ks * q_per;
+    const int q_end = min(nq_all, q_begin + q_per);
+    const bool single_block = q_end - q_begin <= kQB;
+
+    const int opix = active ? rw / b_groups : 0;
+    const int bg = active ? rw % b_groups : 0;
+    const int oy = opix / p.OW, ox = opix % p.OW;
+
+    int bimg[MT], bload[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        bimg[mt] = (bg * MT + mt) * 32 + j;
+        bload[mt] = min(bimg[mt], p.B - 1);
+    }
+
+    // stage k-steps [q0, q0+cnt) of this channel group, expanded, in fragment order
+    auto stage_weights = [&](int q0) {
+        const int cnt = min(kQB, q_end - q0);
+        for (int f = wave; f < cnt * kNT; f += kWaves) {
+            const int ql = f / kNT, nt = f % kNT;
+            const int q = q0 + ql;
+            const int tap = q / steps, t = q % steps;
+            const int c = n0 + nt * 32 + row_to_channel(j);
+            const int word = FMT == FMT_F4 ? 2 * t + h : t;  // word of the tap this lane expands
+            uint32_t x = 0, valid = 0;
+            if (word < p.cw && c < p.N) {
+                x = wgt[(size_t)c * kw_tot + tap * p.cw + word];
+                const int nbits = p.k_tap - 32 * word;  // true bits in this word
+                valid = nbits >= 32 ? 0xffffffffu : (nbits <= 0 ? 0u : 0xffffffffu << (32 - nbits));
+            }
+            lds_w[(ql * kNT + nt) * 64 + lane] =
+                FMT == FMT_F4 ? expand_f4_masked(x, valid) : expand_i8_masked(x, valid, h);
+        }
+    };
+
+    if (single_block && q_end > q_begin) {
+        stage_weights(q_begin);
+        __syncthreads();
+    }
+
+    uint32_t outword[MT][kNT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < kNT; ++nt) outword[mt][nt] = 0;
+
+    const int pool_n = p.pool_h * p.pool_w;
+    for (int pp = 0; pp < pool_n; ++pp) {
+        const int y = oy * p.pool_h + pp / p.pool_w;
+        const int x = ox * p.pool_w + pp % p.pool_w;
+        const bool valid = active && y < p.PH && x < p.PW;  // wave-uniform
+        const int ay0 = y * p.stride_h - p.pad_h;
+        const int ax0 = x * p.stride_w - p.pad_w;
+
+        acc_t acc[MT][kNT];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+            for (int nt = 0; nt < kNT; ++nt)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[mt][nt][v] = 0;
+
+        // activation word this lane needs for k-step (tap row tr, tap col ts, step t)
+        auto load_step = [&](int tr, int ts, int t, uint32_t* dst) {
+            const int ay = ay0 + tr, ax = ax0 + ts;
+            const bool in_frame = valid && ay >= 0 && ay < p.H && ax >= 0 && ax < p.W;
+            if (in_frame) {
+                const int word = FMT == FMT_F4 ? min(2 * t + h, p.cw - 1) : t;
+                const uint32_t* src = act + ((size_t)(ay * p.W + ax) * p.cw + word) * p.B;
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) dst[mt] = src[bload[mt]];
+            }
+            return in_frame;
+        };
+
+        int tr = (q_begin / steps) / p.S, ts = (q_begin / steps) % p.S, t = q_begin % steps;
+        uint32_t cur[MT], nxt[MT];
+        bool cur_ok = q_begin < q_end ? load_step(tr, ts, t, cur) : false;
+        for (int q0 = q_begin; q0 < q_end; q0 += kQB) {
+            if (!single_block) {
+                __syncthreads();
+                stage_weights(q0);
+                __syncthreads();
+            }
+            const int cnt = min(kQB, q_end - q0);
+            for (int ql = 0; ql < cnt; ++ql) {
+                // advance the (tap, step) counters and prefetch the next step's words
+                int ntr = tr, nts = ts, nt_ = t + 1;
+                if (nt_ == steps) {
+                    nt_ = 0;
+                    if (++nts == p.S) {
+                        nts = 0;
+                        ++ntr;
+                    }
+                }
+                const bool nxt_ok = (q0 + ql + 1 < q_end) ? load_step(ntr, nts, nt_, nxt) : false;
+                if (cur_ok) {
+                    v4i bfrag[MT];
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt)
+                        bfrag[mt] = FMT == FMT_F4 ? expand_f4(cur[mt]) : expand_i8(cur[mt], h);
+#pragma unroll
+                    for (int nt = 0; nt < kNT; ++nt) {
+                        const v4i afrag = lds_w[(ql * kNT + nt) * 64 + lane];
+#pragma unroll
+                        for (int mt = 0; mt < MT; ++mt)
+                            acc[mt][nt] = A::mma(afrag, bfrag[mt], acc[mt][nt]);
+                    }
+                }
+                tr = ntr;
+                ts = nts;
+                t = nt_;
+                cur_ok = nxt_ok;
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) cur[mt] = nxt[mt];
+            }
+        }
+
+        if (!valid) continue;
+
+        // ---------------- epilogue for pre-pool pixel (y, x) ----------------
+        const size_t pix = (size_t)y * p.PW + x;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int b = bimg[mt];
+            const bool b_ok = b < p.B;
+            const int bb = bload[mt];
+#pragma unroll
+            for (int nt = 0; nt < kNT; ++nt) {
+                const int cbase = n0 + nt * 32 + 16 * h;  // this lane's channels: cbase + v
+                if constexpr (MM == MM_THRESH || MM == MM_THRESH_RES) {
+                    int rv[16];
+                    if constexpr (MM == MM_THRESH_RES) {
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) {
+                            const int c = cbase + v;
+                            int val = 0;
+                            if (rin != nullptr && c < p.res_limit && c < p.res_in_ch && c < p.N) {
+                                if (p.res_pool) {
+                                    const size_t rw2 = 2 * (size_t)p.PW;
+                                    const int32_t* s00 =
+                                        rin + (((size_t)(2 * y) * rw2 + 2 * x) * p.res_in_ch + c) * p.B + bb;
+                                    const size_t dx = (size_t)p.res_in_ch * p.B, dy = rw2 * dx;
+                                    val = max(max(s00[0], s00[dx]), max(s00[dy], s00[dy + dx]));
+                                } else {
+                                    val = rin[(pix * p.res_in_ch + c) * p.B + bb];
+                                }
+                            }
+                            rv[v] = val;
+                        }
+                    }
+                    int32_t* __restrict__ rout = p.res_out;
+                    uint32_t hw = 0;
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int c = cbase + v;
+                        int res = A::to_int(acc[mt][nt][v]);
+                        uint32_t bit = 0;
+                        if (c < p.N) {
+                            if constexpr (MM == MM_THRESH_RES) {
+                                res += rv[v];
+                                if (rout != nullptr && b_ok) rout[(pix * p.N + c) * p.B + b] = res;
+                            }
+                            bit = thresh_bit(res, bnp[c], p.nan_bit);
+                        }
+                        hw = (hw << 1) | bit;
+                    }
+                    const uint32_t other = (uint32_t)__shfl_xor((int)hw, 32);
+                    outword[mt][nt] |= h == 0 ? (hw << 16) | other : (other << 16) | hw;
+                } else {
+                    if (!b_ok) continue;
+                    if (p.ksplit > 1) {  // partial dot products; the finishing kernel does the rest
+#pragma unroll
+                        for (int v = 0; v < 16; ++v)
+                            if (cbase + v < p.N)
+                                atomicAdd(p.workspace + (size_t)(cbase + v) * p.B + b,
+                                          A::to_int(acc[mt][nt][v]));
+                    } else if (p.mode == EPI_AFFINE) {
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) {
+                            const int c = cbase + v;
+                            // the +-1 dot product equals (float)K - (float)popc*2.0f exactly
+                            if (c < p.N)
+                                p.out_f32[(size_t)b * p.N + c] = __fadd_rn(
+                                    __fmul_rn((float)A::to_int(acc[mt][nt][v]), bnp[c]), p.bn_bias[c]);
+                        }
+                    } else {
+                        int32_t* dst = p.out_i32 + pix * p.raw_pix_stride + (size_t)b * p.raw_b_stride;
+#pragma unroll
+                        for (int v = 0; v < 16; ++v)
+                            if (cbase + v < p.N) dst[cbase + v] = A::to_int(acc[mt][nt][v]);
+                    }
+                }
+            }
+        }
+    }
+
+    if ((MM == MM_THRESH || MM == MM_THRESH_RES) && active && h == 0) {
+        const int n_words = (p.N + 31) / 32;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            if (bimg[mt] >= p.B) continue;
+            uint32_t* dst = p.out_bits + (size_t)opix * p.bits_pix_stride + bimg[mt];
+#pragma unroll
+            for (int nt = 0; nt < kNT; ++nt) {
+                const int w = ng * kNT + nt;
+                if (w < p.bits_row_words) dst[(size_t)w * p.B] = outword[mt][nt];
+            }
+            if (ng == n_groups - 1)  // zero the pixel's padding words
+                for (int w = max(n_words, n_groups * kNT); w < p.bits_row_words; ++w)
+                    dst[(size_t)w * p.B] = 0;
+        }
+    }
+}
+
+int images_per_wave_tiles(const BgemmParams& p) {
+    const long long pix = (long long)p.OH * p.OW;
+    const int n_groups = (p.N + 32 * kNT - 1) / (32 * kNT);
+    for (int mt = 4; mt > 1; mt >>= 1) {
+        if (p.B <= 32 * (mt / 2)) continue;
+        const long long waves = pix * ((p.B + 32 * mt - 1) / (32 * mt)) * n_groups * p.ksplit;
+        if (waves >= 2048) return mt;
+    }
+    return 1;
+}
+
+int mfma_mode(const BgemmParams& p) {
+    if (p.ksplit > 1 || p.mode != EPI_THRESH) return MM_OTHER;
+    return (p.res_in != nullptr || p.res_out != nullptr) ? MM_THRESH_RES : MM_THRESH;
+}
+
+template <int FMT, int MT, int MM>
+int launch_t(const BgemmParams& p, hipStream_t stream) {
+    const int n_groups = (p.N + 32 * kNT - 1) / (32 * kNT);
+    const int b_groups = (p.B + 32 * MT - 1) / (32 * MT);
+    const long long row_waves = (long long)p.OH * p.OW * b_groups;
+    const long long row_blocks = (row_waves + kWaves - 1) / kWaves;
+    const long long blocks = row_blocks * n_groups * p.ksplit;
+    if (blocks <= 0 || blocks > 0x7fffffffLL) return fail(TCBNN_EINVAL, "bgemm grid too large");
+    hipLaunchKernelGGL((bgemm_mfma_kernel<FMT, MT, MM>), dim3((unsigned)blocks), dim3(kThreads), 0,
+                       stream, p, p.act, p.wgt, p.mode == EPI_AFFINE ? p.bn_scale : p.bn, p.res_in,
+                       n_groups, (int)row_waves, b_groups, (int)row_blocks);
+    TCBNN_LAUNCH_CHECK("bgemm_mfma_kernel");
+    return TCBNN_OK;
+}
+
+template <int FMT, int MT>
+int launch_m(const BgemmParams& p, hipStream_t stream) {
+    switch (mfma_mode(p)) {
+        case MM_THRESH:
+            return launch_t<FMT, MT, MM_THRESH>(p, stream);
+        case MM_THRESH_RES:
+            return launch_t<FMT, MT, MM_THRESH_RES>(p, stream);
+        default:
+            return launch_t<FMT, MT, MM_OTHER>(p, stream);
+    }
+}
+
+template <int FMT>
+int launch_f(const BgemmParams& p, hipStream_t stream) {
+    switch (images_per_wave_tiles(p)) {
+        case 4:
+            return launch_m<FMT, 4>(p, stream);
+        case 2:
+            return launch_m<FMT, 2>(p, stream);
+        default:
+            return launch_m<FMT, 1>(p, stream);
+    }
+}
+
+int mfma_ksplit(const BgemmParams& p, int variant) {
+    if (p.workspace == nullptr || p.PH * p.PW != 1 || p.R * p.S != 1 || p.res_in || p.res_out)
+        return 1;
+    const int n_groups = (p.N + 32 * kNT - 1) / (32 * kNT);
+    const long long waves = (long long)((p.B + 31) / 32) * n_groups;
+    const int steps = variant == TCBNN_VARIANT_MFMA_F4 ? (p.cw + 1) / 2 : p.cw;
+    int ks = (int)(2048 / waves);
+    ks = min(ks, steps / 8);
+    return ks < 2 ? 1 : min(ks, 64);
+}
+
+}  // namespace
+
 void bgemm_mfma_kernel_name(const BgemmParams& p, int variant, char* buf, size_t len) {
-    (void)p;
-    snprintf(buf, len, "bgemm_mfma_kernel<%d>", variant);
+    BgemmParams q = p;
+    q.ksplit = mfma_ksplit(p, variant);
+    snprintf(buf, len, "bgemm_mfma_kernel<%d, %d, %d>", variant == TCBNN_VARIANT_MFMA_F4 ? FMT_F4 : FMT_I8,
+             images_per_wave_tiles(q), mfma_mode(q));
 }
+
+int launch_bgemm_mfma(const BgemmParams& p_in, int variant, hipStream_t stream) {
+    if (int rc = validate_bgemm(p_in)) return rc;
+    BgemmParams p = p_in;
+    p.ksplit = mfma_ksplit(p, variant);
+    p.ws_is_dot = 1;
+    if (p.ksplit > 1)
+        if (int rc = launch_splitk_clear(p, stream)) return rc;
+    const int rc = variant == TCBNN_VARIANT_MFMA_F4 ? launch_f<FMT_F4>(p, stream) : launch_f<FMT_I8>(p, stream);
+    if (rc) return rc;
+    if (p.ksplit > 1) return launch_splitk_finish(p, stream);
+    return TCBNN_OK;
+}
+
 }  // namespace tcbnn

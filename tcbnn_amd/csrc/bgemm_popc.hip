@@ -84,7 +84,11 @@ enum KernelMode : int {
 template <int RPL, int CH, int KM>
 __global__ __launch_bounds__(kThreads)
     __attribute__((amdgpu_waves_per_eu(RPL == 1 ? 4 : (RPL == 2 ? 3 : 2)))) void bgemm_popc_kernel(
-        const BgemmParams p, int n_tiles, int row_waves, int b_tiles, int row_blocks) {
+        const BgemmParams p, const uint32_t* __restrict__ act, const uint32_t* __restrict__ wgt,
+        const float* __restrict__ bnp, const int32_t* __restrict__ rin, int n_tiles, int row_waves,
+        int b_tiles, int row_blocks) {
+    // act / wgt / bnp / rin repeat p.act / p.wgt / p.bn (or p.bn_scale) / p.res_in as __restrict__
+    // arguments: read-only and unaliased, so wave-uniform loads from them become scalar loads
     using V = typename WordVec<CH>::type;
     __shared__ __attribute__((aligned(16))) uint32_t lds_w[kLdsWords];
 
@@ -124,7 +128,7 @@ __global__ __launch_bounds__(kThreads)
     auto stage_weights = [&](int q0) {
         const int cnt = min(kQB, q_end - q0);
         const int blk_words = cnt * CH;  // words per weight row in this block
-        const uint32_t* wrow = p.wgt + (size_t)nt * kNTile * kw_tot + (size_t)q0 * CH;
+        const uint32_t* wrow = wgt + (size_t)nt * kNTile * kw_tot + (size_t)q0 * CH;
         for (int idx = tid; idx < blk_words * kNTile; idx += kThreads) {
             const int n = idx / blk_words;
             const int kk = idx - n * blk_words;
@@ -174,7 +178,7 @@ __global__ __launch_bounds__(kThreads)
                     if (in_frame) {
                         uint32_t a[RPL][CH];
                         const uint32_t* src =
-                            p.act + ((size_t)(ay * p.W + ax) * p.cw + kc * CH) * p.B;
+                            act + ((size_t)(ay * p.W + ax) * p.cw + kc * CH) * p.B;
 #pragma unroll
                         for (int j = 0; j < CH; ++j)
 #pragma unroll
@@ -227,7 +231,6 @@ __global__ __launch_bounds__(kThreads)
                 if constexpr (KM == KM_THRESH_RES) {
                     // all residual loads first (one contiguous run per channel across the
                     // wave), so they are in flight together before any store is issued
-                    const int32_t* __restrict__ rin = p.res_in;
 #pragma unroll
                     for (int n = 0; n < kNTile; ++n) {
                         const int ch = n0 + n;
@@ -246,7 +249,7 @@ __global__ __launch_bounds__(kThreads)
                         rv[n] = v;
                     }
                 }
-                const float* __restrict__ bn = p.bn;
+                const float* __restrict__ bn = bnp;
                 int32_t* __restrict__ rout = p.res_out;
 #pragma unroll
                 for (int n = 0; n < kNTile; ++n) {
@@ -269,7 +272,7 @@ __global__ __launch_bounds__(kThreads)
                         // (float)K - (float)c*2.0f is exact; multiply and add are kept
                         // separate (no FMA contraction) so the result is reproducible.
                         const float d = (float)p.k_tap - (float)acc[r][n] * 2.0f;
-                        dst[ch] = __fadd_rn(__fmul_rn(d, p.bn_scale[ch]), p.bn_bias[ch]);
+                        dst[ch] = __fadd_rn(__fmul_rn(d, bnp[ch]), p.bn_bias[ch]);
                     }
                 }
             } else if constexpr (KM == KM_RAW) {
@@ -305,25 +308,25 @@ __global__ __launch_bounds__(256) void splitk_finish_kernel(const BgemmParams p,
     const int b = (int)(i % p.B);
     const int nt = (int)(i / p.B);
     const int n0 = nt * kNTile;
+    // the +-1 dot product from what the engine accumulated
+    auto dot = [&](int n) {
+        const int w = p.workspace[(size_t)(n0 + n) * p.B + b];
+        return p.ws_is_dot ? w : p.k_tap - 2 * w;
+    };
     if (p.mode == EPI_THRESH) {
         uint32_t word = 0;
-        for (int n = 0; n < kNTile && n0 + n < p.N; ++n) {
-            const int res = p.k_tap - 2 * p.workspace[(size_t)(n0 + n) * p.B + b];
-            word |= thresh_bit(res, p.bn[n0 + n], p.nan_bit) << (31 - n);
-        }
+        for (int n = 0; n < kNTile && n0 + n < p.N; ++n)
+            word |= thresh_bit(dot(n), p.bn[n0 + n], p.nan_bit) << (31 - n);
         p.out_bits[(size_t)nt * p.B + b] = word;
         if (nt == n_tiles - 1)
             for (int w = n_tiles; w < p.bits_row_words; ++w) p.out_bits[(size_t)w * p.B + b] = 0;
     } else if (p.mode == EPI_AFFINE) {
-        for (int n = 0; n < kNTile && n0 + n < p.N; ++n) {
-            const float d = (float)p.k_tap - (float)p.workspace[(size_t)(n0 + n) * p.B + b] * 2.0f;
+        for (int n = 0; n < kNTile && n0 + n < p.N; ++n)
             p.out_f32[(size_t)b * p.N + n0 + n] =
-                __fadd_rn(__fmul_rn(d, p.bn_scale[n0 + n]), p.bn_bias[n0 + n]);
-        }
+                __fadd_rn(__fmul_rn((float)dot(n), p.bn_scale[n0 + n]), p.bn_bias[n0 + n]);
     } else {
         for (int n = 0; n < kNTile && n0 + n < p.N; ++n)
-            p.out_i32[(size_t)b * p.raw_b_stride + n0 + n] =
-                p.k_tap - 2 * p.workspace[(size_t)(n0 + n) * p.B + b];
+            p.out_i32[(size_t)b * p.raw_b_stride + n0 + n] = dot(n);
     }
 }
 
@@ -349,7 +352,8 @@ int launch_t(const BgemmParams& p, hipStream_t stream) {
     const long long blocks = row_blocks * n_tiles * p.ksplit;
     if (blocks <= 0 || blocks > 0x7fffffffLL) return fail(TCBNN_EINVAL, "bgemm grid too large");
     hipLaunchKernelGGL((bgemm_popc_kernel<RPL, CH, KM>), dim3((unsigned)blocks), dim3(kThreads), 0,
-                       stream, p, n_tiles, (int)row_waves, b_tiles, (int)row_blocks);
+                       stream, p, p.act, p.wgt, p.mode == EPI_AFFINE ? p.bn_scale : p.bn, p.res_in, n_tiles,
+                       (int)row_waves, b_tiles, (int)row_blocks);
     TCBNN_LAUNCH_CHECK("bgemm_popc_kernel");
     return TCBNN_OK;
 }

@@ -88,6 +88,7 @@ struct BgemmParams {
     // workspace[n*B + b] and a finishing kernel applies the epilogue
     int32_t* workspace;
     int ksplit;
+    int ws_is_dot;  // workspace holds +-1 dot products (matrix-core engines) instead of popcounts
 };
 
 int launch_bgemm_popc(const BgemmParams& p, hipStream_t stream);

@@ -10,7 +10,7 @@ from tests import gpuops, refmath as rm
 
 pytestmark = pytest.mark.gpu
 
-VARIANTS = ["popc"]
+VARIANTS = ["popc", "mfma_f4", "mfma_i8"]
 
 
 def rng(seed):
