@@ -1,0 +1,717 @@
+// C++ host mirror of the reference's layer objects (param.h:115-1065) over the C ABI of
+// libtcbnn_hip.so.  Same class names, constructor signatures, public fields and method
+// names, so a driver written against the reference's param.h keeps compiling:
+//
+//     Conv128LayerParam* c = new Conv128LayerParam("L1B1C2", h, w, 3, 3, 64, 64, batch,
+//                                                  1, 1, true, 1, 1, false, true, true, 64);
+//     c->initialize(config_file, prev->get_output_gpu(), stem->get_output_residual_gpu());
+//
+// What differs, by design:
+//   * initialize() returns `this` (the reference returns the device shadow that its
+//     cooperative network kernel dereferences); each layer is run with forward(stream),
+//     one stream-ordered launch, in place of the call inside the network kernel
+//     (imagenet_resnet.cu:34-125).  forward() is idempotent: outputs are plainly stored,
+//     not OR-accumulated into a once-zeroed buffer (param.h:973-974).
+//   * device buffers use the engine's batch-innermost layouts; download_output() converts
+//     to the reference's tile-contiguous layout, so it returns what the reference returns.
+//   * errors follow the reference convention: message on stderr and exit(-1)
+//     (utility.h:57-92); the C ABI underneath returns codes instead.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <map>
+#include <vector>
+
+#include "../../include/tcbnn_hip.h"
+
+// ---- utility.h:25-52 ---------------------------------------------------------------
+typedef unsigned char uin8;
+typedef unsigned short uin16;
+typedef unsigned int uin32;
+typedef unsigned long long uin64;
+
+#define STEP8(X) (((X) + 7) >> 3)
+#define STEP32(X) (((X) + 31) >> 5)
+#define STEP128(X) (((X) + 127) >> 7)
+#define PAD8(X) (STEP8(X) << 3)
+#define PAD32(X) (STEP32(X) << 5)
+#define PAD128(X) (STEP128(X) << 7)
+
+// ---- error convention, utility.h:57-92 ------------------------------------------------
+#define HIP_SAFE_CALL(err) tcbnn_host::hip_safe_call((err), __FILE__, __LINE__)
+#define TCBNN_SAFE_CALL(rc) tcbnn_host::tcbnn_safe_call((rc), __FILE__, __LINE__)
+#define CHECK_NULL_POINTER(X) tcbnn_host::check_null((const void*)(X), __FILE__, __LINE__)
+#define SAFE_ALOC_GPU(X, Y) HIP_SAFE_CALL(hipMalloc((void**)&(X), (Y) > 0 ? (size_t)(Y) : 4))
+#define SAFE_ALOC_HOST(X, Y) HIP_SAFE_CALL(hipHostMalloc((void**)&(X), (Y) > 0 ? (size_t)(Y) : 4))
+#define SAFE_FREE_GPU(X)               \
+    if ((X) != NULL) {                 \
+        HIP_SAFE_CALL(hipFree((X)));   \
+        (X) = NULL;                    \
+    }
+#define SAFE_FREE_HOST(X)                \
+    if ((X) != NULL) {                   \
+        HIP_SAFE_CALL(hipHostFree((X))); \
+        (X) = NULL;                      \
+    }
+
+namespace tcbnn_host {
+
+inline void hip_safe_call(hipError_t err, const char* file, int line) {
+    if (err != hipSuccess) {
+        fprintf(stderr, "hipSafeCall() failed at %s:%i : %s\n", file, line, hipGetErrorString(err));
+        exit(-1);
+    }
+}
+inline void tcbnn_safe_call(int rc, const char* file, int line) {
+    if (rc != TCBNN_OK) {
+        fprintf(stderr, "tcbnn call failed at %s:%i : %s\n", file, line, tcbnn_last_error());
+        exit(-1);
+    }
+}
+inline void check_null(const void* p, const char* file, int line) {
+    if (p == NULL) {
+        fprintf(stderr, "Error: NULL pointer at %s:%i.\n", file, line);
+        exit(-1);
+    }
+}
+
+// load weights from file, utility.h:188-196
+inline void launch_array(FILE* cf, float* array, unsigned array_size) {
+    if (cf == NULL) {
+        fprintf(stderr, "NULL pointer to the network configuration file.\n");
+        exit(1);
+    }
+    for (unsigned i = 0; i < array_size; i++) {
+        int c;
+        while ((c = fgetc(cf)) == ',') {  // the reference's files are white-space separated; tolerate commas
+        }
+        if (c != EOF) ungetc(c, cf);
+        if (fscanf(cf, "%f", &array[i]) != 1) {
+            fprintf(stderr, "network configuration file ended after %u of %u values.\n", i, array_size);
+            exit(1);
+        }
+    }
+}
+
+// Where a layer's parameters come from: the reference's text weight file, or an in-memory
+// float array consumed in the same order.  Converts implicitly from FILE*, so
+// initialize(config_file, ...) reads exactly like the reference.
+class ConfigSource {
+   public:
+    ConfigSource(FILE* f) : file_(f), cursor_(NULL), end_(NULL) {}
+    ConfigSource(const float** cursor, const float* end) : file_(NULL), cursor_(cursor), end_(end) {}
+    void read(float* dst, unsigned n) {
+        if (cursor_ != NULL) {
+            if (*cursor_ + n > end_) {
+                fprintf(stderr, "in-memory network configuration ended early.\n");
+                exit(1);
+            }
+            memcpy(dst, *cursor_, (size_t)n * sizeof(float));
+            *cursor_ += n;
+        } else {
+            launch_array(file_, dst, n);
+        }
+    }
+
+   private:
+    FILE* file_;
+    const float** cursor_;
+    const float* end_;
+};
+
+// The reference infers the channel stride of an injected residual from PAD128 of the
+// consumer's residual_channels (kernel.cuh:778-791).  The engine stores residuals with their
+// true channel count, so the producer records it here, keyed by device pointer.
+inline std::map<const void*, int>& residual_channels_registry() {
+    static std::map<const void*, int> reg;
+    return reg;
+}
+
+}  // namespace tcbnn_host
+
+using tcbnn_host::launch_array;
+
+// ======================================================================================
+class In128LayerParam {  // param.h:115-222
+   public:
+    In128LayerParam(const char* _name, int _input_height, int _input_width)
+        : input(NULL), input_gpu(NULL), output(NULL), output_gpu(NULL), input_width(_input_width),
+          input_height(_input_height), output_width(_input_width), output_height(_input_height), gpu(this) {
+        strncpy(name, _name, 8);
+    }
+    int input_size() { return input_height * input_width; }
+    int input_bytes() { return input_size() * sizeof(float); }
+    int output_size() { return output_height * output_width; }
+    int output_bytes() { return output_size() * sizeof(float); }
+    int output_bit_size() { return PAD8(output_height) * STEP128(output_width); }
+    int output_bit_bytes() { return output_bit_size() * 16; }
+
+    In128LayerParam* initialize(float* input) {
+        CHECK_NULL_POINTER(input);
+        this->input = input;
+        SAFE_ALOC_GPU(input_gpu, input_bytes());
+        HIP_SAFE_CALL(hipMemcpy(input_gpu, input, input_bytes(), hipMemcpyHostToDevice));
+        SAFE_ALOC_GPU(output_gpu, 4 * tcbnn_fc_act_words(output_height, output_width));
+        return this;
+    }
+    void set_output_gpu(uin32* _output_gpu) { this->output_gpu = _output_gpu; }
+    uin32* get_output_gpu() { return this->output_gpu; }
+    void forward(hipStream_t stream = 0) {
+        tcbnn_in128_desc d = {input_gpu, output_gpu, input_height, input_width};
+        TCBNN_SAFE_CALL(tcbnn_in128_forward(&d, stream));
+    }
+    uin32* download_output() {  // reference tile layout, PAD8(B)*STEP128(K) 128-bit units
+        if (output == NULL) SAFE_ALOC_HOST(output, output_bit_bytes());
+        uin32* tmp = NULL;
+        SAFE_ALOC_GPU(tmp, output_bit_bytes());
+        TCBNN_SAFE_CALL(tcbnn_fc_to_reference_fmt(output_gpu, tmp, output_height, output_width, 0));
+        HIP_SAFE_CALL(hipMemcpy(output, tmp, output_bit_bytes(), hipMemcpyDeviceToHost));
+        SAFE_FREE_GPU(tmp);
+        return this->output;
+    }
+    float* download_full_output() {  // +-1.0f [B][K] (UnPackFcOutput128FMT, param.h:87-104)
+        float* full_output = NULL;
+        SAFE_ALOC_HOST(full_output, output_bytes());
+        float* full_output_gpu = NULL;
+        SAFE_ALOC_GPU(full_output_gpu, output_bytes());
+        TCBNN_SAFE_CALL(tcbnn_unpack_fc_output(output_gpu, full_output_gpu, output_height, output_width, 0));
+        HIP_SAFE_CALL(hipMemcpy(full_output, full_output_gpu, output_bytes(), hipMemcpyDeviceToHost));
+        SAFE_FREE_GPU(full_output_gpu);
+        return full_output;
+    }
+    void release() {
+        SAFE_FREE_GPU(input_gpu);
+        SAFE_FREE_GPU(output_gpu);
+        SAFE_FREE_HOST(output);
+    }
+    ~In128LayerParam() { release(); }
+
+   public:
+    float* input;
+    float* input_gpu;
+    uin32* output;
+    uin32* output_gpu;
+    int input_width;
+    int input_height;
+    int output_width;
+    int output_height;
+    In128LayerParam* gpu;
+    char name[8];
+};
+
+// ======================================================================================
+class Fc128LayerParam {  // param.h:224-385
+   public:
+    Fc128LayerParam(const char* name, int _input_height, int _input_width, int _weight_width)
+        : input(NULL), input_gpu(NULL), input_width(_input_width), input_height(_input_height), weight(NULL),
+          weight_gpu(NULL), weight_width(_weight_width), weight_height(_input_width), output(NULL),
+          output_gpu(NULL), output_width(_weight_width), output_height(_input_height), bn(NULL), bn_gpu(NULL),
+          bn_width(_weight_width), gpu(this), variant(TCBNN_VARIANT_AUTO), workspace_gpu(NULL) {
+        strncpy(this->name, name, 8);
+    }
+    int weight_size() { return weight_height * weight_width; }
+    int weight_bytes() { return weight_size() * sizeof(float); }
+    int output_size() { return output_height * output_width; }
+    int output_bytes() { return output_size() * sizeof(float); }
+    int output_bit_size() { return PAD8(output_height) * STEP128(output_width); }
+    int output_bit_bytes() { return output_bit_size() * 16; }
+    int bn_size() { return bn_width; }
+    int bn_bytes() { return bn_size() * sizeof(float); }
+    size_t workspace_words() { return (size_t)PAD32(weight_width) * input_height; }
+
+    void set_input_gpu(uin32* _input_gpu) { this->input_gpu = _input_gpu; }
+    Fc128LayerParam* initialize(tcbnn_host::ConfigSource config_file, uin32* prev_layer_gpu) {
+        SAFE_ALOC_HOST(weight, weight_bytes());
+        config_file.read(this->weight, weight_size());
+        SAFE_ALOC_GPU(weight_gpu, 4 * tcbnn_fc_weight_words(weight_height, weight_width));
+        float* weight_float = NULL;
+        SAFE_ALOC_GPU(weight_float, weight_bytes());
+        HIP_SAFE_CALL(hipMemcpy(weight_float, weight, weight_bytes(), hipMemcpyHostToDevice));
+        TCBNN_SAFE_CALL(tcbnn_pack_fc_weight(weight_float, weight_gpu, weight_height, weight_width, 0));
+        HIP_SAFE_CALL(hipDeviceSynchronize());
+        SAFE_FREE_GPU(weight_float);
+        SAFE_ALOC_HOST(bn, bn_bytes());
+        config_file.read(this->bn, bn_size());
+        SAFE_ALOC_GPU(bn_gpu, bn_bytes());
+        HIP_SAFE_CALL(hipMemcpy(bn_gpu, bn, bn_bytes(), hipMemcpyHostToDevice));
+        SAFE_ALOC_GPU(output_gpu, 4 * tcbnn_fc_act_words(output_height, output_width));
+        SAFE_ALOC_GPU(workspace_gpu, 4 * workspace_words());
+        set_input_gpu(prev_layer_gpu);
+        CHECK_NULL_POINTER(input_gpu);
+        return this;
+    }
+    uin32* get_output_gpu() { return this->output_gpu; }
+    void forward(hipStream_t stream = 0) {
+        tcbnn_fc128_desc d = {input_gpu, weight_gpu, bn_gpu,  output_gpu,    input_height,
+                              input_width, weight_width, variant, workspace_gpu, workspace_words()};
+        TCBNN_SAFE_CALL(tcbnn_fc128_forward(&d, stream));
+    }
+    uin32* download_output() {
+        if (output == NULL) SAFE_ALOC_HOST(output, output_bit_bytes());
+        uin32* tmp = NULL;
+        SAFE_ALOC_GPU(tmp, output_bit_bytes());
+        TCBNN_SAFE_CALL(tcbnn_fc_to_reference_fmt(output_gpu, tmp, output_height, output_width, 0));
+        HIP_SAFE_CALL(hipMemcpy(output, tmp, output_bit_bytes(), hipMemcpyDeviceToHost));
+        SAFE_FREE_GPU(tmp);
+        return this->output;
+    }
+    float* download_full_output() {
+        float* full_output = NULL;
+        SAFE_ALOC_HOST(full_output, output_bytes());
+        float* full_output_gpu = NULL;
+        SAFE_ALOC_GPU(full_output_gpu, output_bytes());
+        TCBNN_SAFE_CALL(tcbnn_unpack_fc_output(output_gpu, full_output_gpu, output_height, output_width, 0));
+        HIP_SAFE_CALL(hipMemcpy(full_output, full_output_gpu, output_bytes(), hipMemcpyDeviceToHost));
+        SAFE_FREE_GPU(full_output_gpu);
+        return full_output;
+    }
+    void release() {
+        SAFE_FREE_HOST(weight);
+        SAFE_FREE_HOST(bn);
+        SAFE_FREE_HOST(output);
+        SAFE_FREE_GPU(weight_gpu);
+        SAFE_FREE_GPU(bn_gpu);
+        SAFE_FREE_GPU(output_gpu);
+        SAFE_FREE_GPU(workspace_gpu);
+    }
+    ~Fc128LayerParam() { release(); }
+
+   public:
+    uin32* input;
+    uin32* input_gpu;
+    int input_width;
+    int input_height;
+    float* weight;
+    uin32* weight_gpu;
+    int weight_width;
+    int weight_height;
+    uin32* output;
+    uin32* output_gpu;
+    int output_width;
+    int output_height;
+    float* bn;
+    float* bn_gpu;
+    int bn_width;
+    Fc128LayerParam* gpu;
+    char name[8];
+    int variant;             // TCBNN_VARIANT_* (no counterpart in the reference)
+    int32_t* workspace_gpu;  // split-K scratch (no counterpart in the reference)
+};
+
+// ======================================================================================
+class Out128LayerParam {  // param.h:388-531
+   public:
+    Out128LayerParam(const char* name, int _input_height, int _input_width, int _weight_width)
+        : input(NULL), input_gpu(NULL), input_width(_input_width), input_height(_input_height), weight(NULL),
+          weight_gpu(NULL), weight_width(_weight_width), weight_height(_input_width), output(NULL),
+          output_gpu(NULL), output_height(_input_height), output_width(_weight_width), has_bn(true),
+          bn_scale(NULL), bn_scale_gpu(NULL), bn_bias(NULL), bn_bias_gpu(NULL), gpu(this),
+          variant(TCBNN_VARIANT_AUTO) {
+        strncpy(this->name, name, 8);
+    }
+    int weight_size() { return weight_height * weight_width; }
+    int weight_bytes() { return weight_size() * sizeof(float); }
+    int output_size() { return output_height * output_width; }
+    int output_bytes() { return output_size() * sizeof(float); }
+    int bn_size() { return output_width; }
+    int bn_bytes() { return output_width * sizeof(float); }
+
+    void set_input_gpu(uin32* input_gpu) { this->input_gpu = input_gpu; }
+    float* get_output_gpu() { return this->output_gpu; }
+    Out128LayerParam* initialize(tcbnn_host::ConfigSource config_file, uin32* prev_layer_gpu) {
+        SAFE_ALOC_HOST(weight, weight_bytes());
+        config_file.read(this->weight, weight_size());
+        SAFE_ALOC_GPU(weight_gpu, 4 * tcbnn_fc_weight_words(weight_height, weight_width));
+        float* weight_float = NULL;
+        SAFE_ALOC_GPU(weight_float, weight_bytes());
+        HIP_SAFE_CALL(hipMemcpy(weight_float, weight, weight_bytes(), hipMemcpyHostToDevice));
+        TCBNN_SAFE_CALL(tcbnn_pack_fc_weight(weight_float, weight_gpu, weight_height, weight_width, 0));
+        HIP_SAFE_CALL(hipDeviceSynchronize());
+        SAFE_FREE_GPU(weight_float);
+        SAFE_ALOC_HOST(bn_scale, bn_bytes());
+        config_file.read(this->bn_scale, bn_size());
+        SAFE_ALOC_GPU(bn_scale_gpu, bn_bytes());
+        HIP_SAFE_CALL(hipMemcpy(bn_scale_gpu, bn_scale, bn_bytes(), hipMemcpyHostToDevice));
+        SAFE_ALOC_HOST(bn_bias, bn_bytes());
+        config_file.read(this->bn_bias, bn_size());
+        SAFE_ALOC_GPU(bn_bias_gpu, bn_bytes());
+        HIP_SAFE_CALL(hipMemcpy(bn_bias_gpu, bn_bias, bn_bytes(), hipMemcpyHostToDevice));
+        SAFE_ALOC_GPU(output_gpu, output_bytes());
+        HIP_SAFE_CALL(hipMemset(this->output_gpu, 0, output_bytes()));
+        set_input_gpu(prev_layer_gpu);
+        CHECK_NULL_POINTER(input_gpu);
+        return this;
+    }
+    void forward(hipStream_t stream = 0) {
+        tcbnn_out128_desc d = {input_gpu,    weight_gpu,  bn_scale_gpu, bn_bias_gpu, output_gpu,
+                               input_height, input_width, weight_width, variant};
+        TCBNN_SAFE_CALL(tcbnn_out128_forward(&d, stream));
+    }
+    float* download_output() {
+        if (output == NULL) SAFE_ALOC_HOST(output, output_bytes());
+        HIP_SAFE_CALL(hipMemcpy(output, output_gpu, output_bytes(), hipMemcpyDeviceToHost));
+        return this->output;
+    }
+    void release() {
+        SAFE_FREE_HOST(weight);
+        SAFE_FREE_HOST(output);
+        SAFE_FREE_HOST(bn_scale);
+        SAFE_FREE_HOST(bn_bias);
+        SAFE_FREE_GPU(weight_gpu);
+        SAFE_FREE_GPU(output_gpu);
+        SAFE_FREE_GPU(bn_scale_gpu);
+        SAFE_FREE_GPU(bn_bias_gpu);
+    }
+    ~Out128LayerParam() { release(); }
+
+   public:
+    uin32* input;
+    uin32* input_gpu;
+    int input_width;
+    int input_height;
+    float* weight;
+    uin32* weight_gpu;
+    int weight_width;
+    int weight_height;
+    float* output;
+    float* output_gpu;
+    int output_height;
+    int output_width;
+    bool has_bn;
+    float* bn_scale;
+    float* bn_scale_gpu;
+    float* bn_bias;
+    float* bn_bias_gpu;
+    Out128LayerParam* gpu;
+    char name[8];
+    int variant;
+};
+
+// ======================================================================================
+// Geometry shared by both conv constructors (param.h:719-728, 897-906).
+#define TCBNN_CONV_GEOMETRY()                                                                          \
+    this->pad_h = tcbnn_conv_pad(input_height, filter_height, stride_height, padding);                 \
+    this->pad_w = tcbnn_conv_pad(input_width, filter_width, stride_width, padding);                    \
+    buf_height = tcbnn_conv_out(input_height, filter_height, stride_height, padding, 1);               \
+    buf_width = tcbnn_conv_out(input_width, filter_width, stride_width, padding, 1);                   \
+    output_height = tcbnn_conv_out(input_height, filter_height, stride_height, padding, pool_height);  \
+    output_width = tcbnn_conv_out(input_width, filter_width, stride_width, padding, pool_width);
+
+class InConv128LayerParam {  // param.h:701-870
+   public:
+    InConv128LayerParam(const char* name, int _input_height, int _input_width, int _filter_height,
+                        int _filter_width, int _input_channels, int _output_channels, int _batch,
+                        int _stride_height = 1, int _stride_width = 1, bool _padding = true,
+                        int _pool_height = 1, int _pool_width = 1, bool _save_residual = false)
+        : input(NULL), input_gpu(NULL), input_width(_input_width), input_height(_input_height),
+          input_channels(_input_channels), filter(NULL), filter_gpu(NULL), filter_width(_filter_width),
+          filter_height(_filter_height), output(NULL), output_gpu(NULL), output_channels(_output_channels),
+          padding(_padding), bn(NULL), bn_gpu(NULL), batch(_batch), stride_height(_stride_height),
+          stride_width(_stride_width), pool_width(_pool_width), pool_height(_pool_height),
+          save_residual(_save_residual), output_residual_gpu(NULL), gpu(this) {
+        strncpy(this->name, name, 8);
+        TCBNN_CONV_GEOMETRY();
+    }
+    int input_size() { return input_channels * input_height * input_width * batch; }
+    int input_bytes() { return input_size() * sizeof(float); }
+    int filter_size() { return output_channels * input_channels * filter_height * filter_width; }
+    int filter_bytes() { return filter_size() * sizeof(float); }
+    int output_size() { return output_channels * output_height * output_width * batch; }
+    int output_bytes() { return output_size() * sizeof(uin32); }
+    int output_bit_size() { return STEP128(output_channels) * output_height * output_width * PAD8(batch); }
+    int output_bit_bytes() { return output_bit_size() * 16; }
+    int bn_size() { return output_channels; }
+    int bn_bytes() { return bn_size() * sizeof(float); }
+    // engine residual: int32 [P][Q][O][B], true sizes (the reference pads to 8 x 128, param.h:756-758)
+    size_t residual_size() { return (size_t)output_channels * batch * buf_height * buf_width; }
+    size_t residual_bytes() { return residual_size() * sizeof(int); }
+
+    InConv128LayerParam* initialize(float* input, tcbnn_host::ConfigSource config_file) {
+        CHECK_NULL_POINTER(input);
+        this->input = input;
+        SAFE_ALOC_GPU(input_gpu, input_bytes());
+        HIP_SAFE_CALL(hipMemcpy(input_gpu, input, input_bytes(), hipMemcpyHostToDevice));
+        SAFE_ALOC_HOST(filter, filter_bytes());
+        config_file.read(this->filter, filter_size());
+        SAFE_ALOC_GPU(filter_gpu,
+                      4 * tcbnn_inconv_filter_words(filter_height, filter_width, input_channels, output_channels));
+        float* filter_float = NULL;
+        SAFE_ALOC_GPU(filter_float, filter_bytes());
+        HIP_SAFE_CALL(hipMemcpy(filter_float, filter, filter_bytes(), hipMemcpyHostToDevice));
+        TCBNN_SAFE_CALL(tcbnn_pack_inconv_filter(filter_float, filter_gpu, filter_height, filter_width,
+                                                 input_channels, output_channels, 0));
+        HIP_SAFE_CALL(hipDeviceSynchronize());
+        SAFE_FREE_GPU(filter_float);
+        SAFE_ALOC_HOST(bn, bn_bytes());
+        config_file.read(bn, bn_size());
+        SAFE_ALOC_GPU(bn_gpu, bn_bytes());
+        HIP_SAFE_CALL(hipMemcpy(this->bn_gpu, this->bn, bn_bytes(), hipMemcpyHostToDevice));
+        SAFE_ALOC_GPU(output_gpu, 4 * tcbnn_conv_act_words(output_height, output_width, batch, output_channels));
+        if (save_residual) {
+            SAFE_ALOC_GPU(output_residual_gpu, residual_bytes());
+            tcbnn_host::residual_channels_registry()[output_residual_gpu] = output_channels;
+        }
+        return this;
+    }
+    uin32* get_output_gpu() { return this->output_gpu; }
+    int* get_output_residual_gpu() { return this->output_residual_gpu; }
+    void forward(hipStream_t stream = 0) {
+        tcbnn_inconv128_desc d = {input_gpu,      filter_gpu,     bn_gpu,        output_gpu,   output_residual_gpu,
+                                  input_height,   input_width,    input_channels, filter_height, filter_width,
+                                  output_channels, batch,         stride_height, stride_width, padding ? 1 : 0,
+                                  pool_height,    pool_width,     save_residual ? 1 : 0};
+        TCBNN_SAFE_CALL(tcbnn_inconv128_forward(&d, stream));
+    }
+    unsigned* download_output() {
+        if (output == NULL) SAFE_ALOC_HOST(output, output_bit_bytes());
+        uin32* tmp = NULL;
+        SAFE_ALOC_GPU(tmp, output_bit_bytes());
+        TCBNN_SAFE_CALL(
+            tcbnn_conv_to_reference_fmt(output_gpu, tmp, output_height, output_width, batch, output_channels, 0));
+        HIP_SAFE_CALL(hipMemcpy(output, tmp, output_bit_bytes(), hipMemcpyDeviceToHost));
+        SAFE_FREE_GPU(tmp);
+        return this->output;
+    }
+    float* download_full_output() {  // +-1.0f NHWC (UnpackConvOutput32FMT, param.h:661-688)
+        float* full_output = NULL;
+        SAFE_ALOC_HOST(full_output, output_bytes());
+        float* full_output_gpu = NULL;
+        SAFE_ALOC_GPU(full_output_gpu, output_bytes());
+        TCBNN_SAFE_CALL(tcbnn_unpack_conv_output(output_gpu, full_output_gpu, output_height, output_width,
+                                                 output_channels, batch, 0));
+        HIP_SAFE_CALL(hipMemcpy(full_output, full_output_gpu, output_bytes(), hipMemcpyDeviceToHost));
+        SAFE_FREE_GPU(full_output_gpu);
+        return full_output;
+    }
+    void release() {
+        SAFE_FREE_HOST(filter);
+        SAFE_FREE_HOST(bn);
+        SAFE_FREE_HOST(output);
+        SAFE_FREE_GPU(input_gpu);
+        SAFE_FREE_GPU(output_gpu);
+        SAFE_FREE_GPU(filter_gpu);
+        SAFE_FREE_GPU(bn_gpu);
+        if (output_residual_gpu != NULL) tcbnn_host::residual_channels_registry().erase(output_residual_gpu);
+        SAFE_FREE_GPU(output_residual_gpu);
+    }
+    ~InConv128LayerParam() { release(); }
+
+   public:
+    float* input;
+    float* input_gpu;
+    int input_width;
+    int input_height;
+    int input_channels;
+    float* filter;
+    uin32* filter_gpu;
+    int filter_width;
+    int filter_height;
+    uin32* output;
+    uin32* output_gpu;
+    int output_width;
+    int output_height;
+    int output_channels;
+    bool padding;
+    float* bn;
+    float* bn_gpu;
+    int batch;
+    int stride_height;
+    int stride_width;
+    int pad_h;
+    int pad_w;
+    int pool_width;
+    int pool_height;
+    bool save_residual;
+    int* output_residual_gpu;
+    InConv128LayerParam* gpu;
+    char name[8];
+    int buf_height, buf_width;  // conv output size before pooling
+};
+
+// ======================================================================================
+class Conv128LayerParam {  // param.h:872-1065
+   public:
+    Conv128LayerParam(const char* name, int _input_height, int _input_width, int _filter_height,
+                      int _filter_width, int _input_channels, int _output_channels, int _batch,
+                      int _stride_height = 1, int _stride_width = 1, bool _padding = true, int _pool_height = 1,
+                      int _pool_width = 1, bool _ahead_fc = false, bool _save_residual = false,
+                      bool _inject_residual = false, int _residual_channels = 0, bool _residual_pool = false)
+        : input(NULL), input_gpu(NULL), input_width(_input_width), input_height(_input_height),
+          input_channels(_input_channels), filter(NULL), filter_gpu(NULL), filter_width(_filter_width),
+          filter_height(_filter_height), output(NULL), output_gpu(NULL), output_channels(_output_channels),
+          bn(NULL), bn_gpu(NULL), batch(_batch), stride_height(_stride_height), stride_width(_stride_width),
+          padding(_padding), pool_width(_pool_width), pool_height(_pool_height), ahead_fc(_ahead_fc),
+          save_residual(_save_residual), output_residual_gpu(NULL), inject_residual(_inject_residual),
+          input_residual_gpu(NULL), residual_channels(_residual_channels), residual_pool(_residual_pool),
+          gpu(this), variant(TCBNN_VARIANT_AUTO), input_residual_channels(0) {
+        strncpy(this->name, name, 8);
+        TCBNN_CONV_GEOMETRY();
+    }
+    int filter_size() { return output_channels * input_channels * filter_height * filter_width; }
+    int filter_bytes() { return filter_size() * sizeof(float); }
+    int output_size() { return output_channels * output_height * output_width * batch; }
+    int output_bytes() { return output_size() * sizeof(uin32); }
+    int output_bit_size() { return STEP128(output_channels) * output_height * output_width * PAD8(batch); }
+    int output_bit_bytes() { return output_bit_size() * 16; }
+    int bn_size() { return output_channels; }
+    int bn_bytes() { return bn_size() * sizeof(float); }
+    size_t residual_size() { return (size_t)output_channels * batch * buf_height * buf_width; }
+    size_t residual_bytes() { return residual_size() * sizeof(int); }
+
+    void set_input_gpu(uin32* input_gpu) { this->input_gpu = input_gpu; }
+    void set_input_residual_gpu(int* input_residual_gpu) {
+        this->input_residual_gpu = input_residual_gpu;
+        std::map<const void*, int>& reg = tcbnn_host::residual_channels_registry();
+        std::map<const void*, int>::iterator it = reg.find(input_residual_gpu);
+        // a residual that no layer of this library produced: assume the consumer's limit
+        input_residual_channels = it != reg.end() ? it->second : residual_channels;
+    }
+    Conv128LayerParam* initialize(tcbnn_host::ConfigSource config_file, uin32* prev_layer_gpu,
+                                  int* input_residual_gpu = NULL) {
+        SAFE_ALOC_HOST(filter, filter_bytes());
+        config_file.read(filter, filter_size());
+        SAFE_ALOC_GPU(filter_gpu,
+                      4 * tcbnn_conv_filter_words(filter_height, filter_width, input_channels, output_channels));
+        float* filter_float = NULL;
+        SAFE_ALOC_GPU(filter_float, filter_bytes());
+        HIP_SAFE_CALL(hipMemcpy(filter_float, filter, filter_bytes(), hipMemcpyHostToDevice));
+        TCBNN_SAFE_CALL(tcbnn_pack_conv_filter(filter_float, filter_gpu, filter_height, filter_width, input_channels,
+                                               output_channels, 0));
+        HIP_SAFE_CALL(hipDeviceSynchronize());
+        SAFE_FREE_GPU(filter_float);
+        SAFE_ALOC_HOST(bn, bn_bytes());
+        config_file.read(bn, bn_size());
+        SAFE_ALOC_GPU(bn_gpu, bn_bytes());
+        HIP_SAFE_CALL(hipMemcpy(bn_gpu, bn, bn_bytes(), hipMemcpyHostToDevice));
+        const size_t words =
+            ahead_fc ? tcbnn_fc_act_words(batch, output_height * output_width * PAD128(output_channels))
+                     : tcbnn_conv_act_words(output_height, output_width, batch, output_channels);
+        SAFE_ALOC_GPU(output_gpu, 4 * words);
+        set_input_gpu(prev_layer_gpu);
+        if (save_residual) {
+            SAFE_ALOC_GPU(output_residual_gpu, residual_bytes());
+            tcbnn_host::residual_channels_registry()[output_residual_gpu] = output_channels;
+        }
+        if (inject_residual) {
+            set_input_residual_gpu(input_residual_gpu);
+            CHECK_NULL_POINTER(this->input_residual_gpu);
+        }
+        CHECK_NULL_POINTER(input_gpu);
+        return this;
+    }
+    uin32* get_output_gpu() { return this->output_gpu; }
+    int* get_output_residual_gpu() { return this->output_residual_gpu; }
+    void forward(hipStream_t stream = 0) {
+        tcbnn_conv128_desc d;
+        memset(&d, 0, sizeof(d));
+        d.input = input_gpu;
+        d.filter = filter_gpu;
+        d.bn = bn_gpu;
+        d.output = output_gpu;
+        d.input_residual = inject_residual ? input_residual_gpu : NULL;
+        d.output_residual = output_residual_gpu;
+        d.input_height = input_height;
+        d.input_width = input_width;
+        d.input_channels = input_channels;
+        d.filter_height = filter_height;
+        d.filter_width = filter_width;
+        d.output_channels = output_channels;
+        d.batch = batch;
+        d.stride_height = stride_height;
+        d.stride_width = stride_width;
+        d.padding = padding ? 1 : 0;
+        d.pool_height = pool_height;
+        d.pool_width = pool_width;
+        d.ahead_fc = ahead_fc ? 1 : 0;
+        d.save_residual = save_residual ? 1 : 0;
+        d.inject_residual = inject_residual ? 1 : 0;
+        d.residual_channels = residual_channels;
+        d.residual_pool = residual_pool ? 1 : 0;
+        d.input_residual_channels = input_residual_channels;
+        d.variant = variant;
+        TCBNN_SAFE_CALL(tcbnn_conv128_forward(&d, stream));
+    }
+    unsigned* download_output() {
+        if (output == NULL) SAFE_ALOC_HOST(output, output_bit_bytes());
+        uin32* tmp = NULL;
+        SAFE_ALOC_GPU(tmp, output_bit_bytes());
+        if (ahead_fc)  // FC-ready: an FC activation of OH*OW*PAD128(O) features (kernel.cuh:798-808)
+            TCBNN_SAFE_CALL(tcbnn_fc_to_reference_fmt(output_gpu, tmp, batch,
+                                                      output_height * output_width * PAD128(output_channels), 0));
+        else
+            TCBNN_SAFE_CALL(tcbnn_conv_to_reference_fmt(output_gpu, tmp, output_height, output_width, batch,
+                                                        output_channels, 0));
+        HIP_SAFE_CALL(hipMemcpy(output, tmp, output_bit_bytes(), hipMemcpyDeviceToHost));
+        SAFE_FREE_GPU(tmp);
+        return this->output;
+    }
+    float* download_full_output() {
+        float* full_output = NULL;
+        SAFE_ALOC_HOST(full_output, output_bytes());
+        float* full_output_gpu = NULL;
+        SAFE_ALOC_GPU(full_output_gpu, output_bytes());
+        if (ahead_fc) {
+            fprintf(stderr, "download_full_output(): not available for an FC-ready (ahead_fc) layer.\n");
+            exit(-1);
+        }
+        TCBNN_SAFE_CALL(tcbnn_unpack_conv_output(output_gpu, full_output_gpu, output_height, output_width,
+                                                 output_channels, batch, 0));
+        HIP_SAFE_CALL(hipMemcpy(full_output, full_output_gpu, output_bytes(), hipMemcpyDeviceToHost));
+        SAFE_FREE_GPU(full_output_gpu);
+        return full_output;
+    }
+    void release() {
+        SAFE_FREE_HOST(filter);
+        SAFE_FREE_HOST(bn);
+        SAFE_FREE_HOST(output);
+        SAFE_FREE_GPU(output_gpu);
+        SAFE_FREE_GPU(filter_gpu);
+        SAFE_FREE_GPU(bn_gpu);
+        if (output_residual_gpu != NULL) tcbnn_host::residual_channels_registry().erase(output_residual_gpu);
+        SAFE_FREE_GPU(output_residual_gpu);
+    }
+    ~Conv128LayerParam() { release(); }
+
+   public:
+    uin32* input;
+    uin32* input_gpu;
+    int input_width;
+    int input_height;
+    int input_channels;
+    float* filter;
+    uin32* filter_gpu;
+    int filter_width;
+    int filter_height;
+    uin32* output;
+    uin32* output_gpu;
+    int output_width;
+    int output_height;
+    int output_channels;
+    float* bn;
+    float* bn_gpu;
+    int batch;
+    int stride_height;
+    int stride_width;
+    bool padding;
+    int pad_h;
+    int pad_w;
+    int pool_width;
+    int pool_height;
+    bool ahead_fc;
+    bool save_residual;
+    int* output_residual_gpu;
+    bool inject_residual;
+    int* input_residual_gpu;
+    int residual_channels;
+    bool residual_pool;
+    Conv128LayerParam* gpu;
+    char name[8];
+    int variant;
+    int input_residual_channels;
+    int buf_height, buf_width;
+};

@@ -1,0 +1,81 @@
+"""The C++ host layer (tcbnn_layers.hpp classes + drivers) against the CPU oracle: the driver
+binaries read a weight file in the reference's text format and a raw input file, and their
+logits must match the oracle's on the same data."""
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+from oracle import nets as orc_nets
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BIN = os.path.join(ROOT, "tcbnn_amd", "bin")
+
+
+def _write_weight_file(path, arrays):
+    with open(path, "w") as f:
+        for a in arrays:
+            a = np.asarray(a, np.float32).ravel()
+            if np.all(np.abs(a) == 1.0):
+                f.write(" ".join("1" if v > 0 else "-1" for v in a))
+            else:
+                f.write(" ".join(repr(float(v)) for v in a))  # repr(float(float32)) round-trips
+            f.write("\n")
+
+
+def _run_driver(tmp_path, name, spec, extra, seed, variant):
+    import tcbnn_amd
+    exe = os.path.join(BIN, name)
+    assert os.path.exists(exe), "%s is not built (run __graft_entry__.build())" % exe
+    weights = tcbnn_amd.synthetic_weights(spec, seed)
+    x = tcbnn_amd.synthetic_input(spec, seed)
+    wf, xf, of = (str(tmp_path / n) for n in ("w.csv", "x.f32", "logits.f32"))
+    _write_weight_file(wf, weights)
+    x.astype(np.float32).tofile(xf)
+    batch = spec[0]["batch"]
+    cmd = [exe, "--batch", str(batch), "--weights", wf, "--input", xf, "--out", of, "--reps", "2", "--warmup", "1",
+           "--variant", variant] + extra
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=280)
+    assert proc.returncode == 0, proc.stdout
+    classes = spec[-1]["out"]
+    got = np.fromfile(of, np.float32).reshape(batch, classes)
+    want = orc_nets.run(spec, weights, x)[spec[-1]["name"]]["out"]
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=0)
+    np.testing.assert_array_equal(got, want)
+    return proc.stdout
+
+
+@pytest.mark.parametrize("variant", ["popc", "mfma_f4"])
+def test_mnist_mlp_driver(gpu, tmp_path, variant):
+    from tcbnn_amd import nets
+    out = _run_driver(tmp_path, "mnist_mlp", nets.mnist_mlp_spec(batch=200), [], 5, variant)
+    assert '"net": "mnist_mlp"' in out
+
+
+def test_cifar10_vgg_driver(gpu, tmp_path):
+    from tcbnn_amd import nets
+    _run_driver(tmp_path, "cifar10_vgg", nets.cifar10_vgg_spec(batch=8, image=16), ["--image", "16"], 6, "popc")
+
+
+def test_imagenet_resnet_driver(gpu, tmp_path):
+    from tcbnn_amd import nets
+    spec = nets.imagenet_resnet_spec(batch=8, image=64, output_size=100)
+    _run_driver(tmp_path, "imagenet_resnet", spec, ["--image", "64", "--classes", "100"], 7, "mfma_f4")
+
+
+def test_driver_synthetic_mode_runs(gpu):
+    exe = os.path.join(BIN, "imagenet_resnet")
+    proc = subprocess.run([exe, "--batch", "8", "--image", "64", "--classes", "10", "--reps", "2"],
+                          stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
+    assert proc.returncode == 0 and '"images_per_s"' in proc.stdout, proc.stdout
+
+
+def test_driver_error_convention_is_print_and_exit(gpu):
+    """Reference convention (utility.h:57-92): message on stderr and exit(-1), no exception."""
+    exe = os.path.join(BIN, "mnist_mlp")
+    proc = subprocess.run([exe, "--weights", "/nonexistent.csv"], stdout=subprocess.PIPE, stderr=subprocess.PIPE,
+                          text=True, timeout=60)
+    assert proc.returncode != 0 and "NULL pointer" in proc.stderr
