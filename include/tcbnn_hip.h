@@ -80,7 +80,7 @@ size_t tcbnn_fc_act_words(int batch, int features);                    /* B*KW12
 size_t tcbnn_conv_act_words(int height, int width, int batch, int ch); /* H*W*B*CW         */
 size_t tcbnn_fc_weight_words(int in_features, int out_features);       /* NPAD32*KW128     */
 size_t tcbnn_conv_filter_words(int r, int s, int in_ch, int out_ch);   /* NPAD32*R*S*CW    */
-size_t tcbnn_inconv_filter_words(int r, int s, int in_ch, int out_ch); /* R*S*OPAD32*4     */
+size_t tcbnn_inconv_filter_words(int r, int s, int in_ch, int out_ch); /* R*S*OPAD32*(4+1/8) */
 
 /* ------------------------------------------------- one-time weight packing */
 /* fp32 [K][N] (param.h:58-59) -> packed [NPAD32][KW128].  Replaces
@@ -91,10 +91,11 @@ int tcbnn_pack_fc_weight(const float* weight_kn, uint32_t* packed, int in_featur
  * PackFiltersByInChannels128FMT (param.h:560-581). */
 int tcbnn_pack_conv_filter(const float* filter_hwio, uint32_t* packed, int r, int s, int in_ch,
                            int out_ch, void* stream);
-/* fp32 HWIO [R][S][3][O] -> sign-mask table uint32 [R*S][OPAD32][4]: entry c<3 is
- * 0 if the weight is >= 0 and 0x80000000 otherwise (the bit the first layer
- * flips on the fp32 input, kernel.cuh:636-638).  Replaces
- * PackFiltersByOutChannels32 (param.h:613-632). */
+/* fp32 HWIO [R][S][3][O] -> sign table uint32 [R*S][OPAD32][4]: entry c<3 is 0 if the
+ * weight of input channel c is >= 0 and 0x80000000 otherwise (the bit the first layer
+ * flips on the fp32 input, kernel.cuh:636-638); entry 3 is the sign pattern index
+ * 4*neg0 + 2*neg1 + neg2.  A second table [R*S][OPAD32/8] follows with the same patterns
+ * packed 8 per word.  Replaces PackFiltersByOutChannels32 (param.h:613-632). */
 int tcbnn_pack_inconv_filter(const float* filter_hwio, uint32_t* packed, int r, int s, int in_ch,
                              int out_ch, void* stream);
 /* fp32 +-1 matrix rows -> packed activation matrix, MSB first, batch (row) innermost:

@@ -16,6 +16,8 @@
 //     wave-uniform scalar loads, and the packed words / int32 residuals are written as
 //     contiguous 256-byte runs of the batch-innermost output layouts.
 //   inconv_generic_kernel (any pooling): one lane per pooled output pixel.
+#include <stdlib.h>
+
 #include "common.h"
 
 namespace tcbnn {
@@ -41,20 +43,93 @@ __device__ __forceinline__ float flip(float f, uint32_t m) {
     return __uint_as_float(__float_as_uint(f) ^ m);
 }
 
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+// The eight possible values of ((+-f0) + (+-f1)) + (+-f2), indexed by the sign pattern
+// 4*neg0 + 2*neg1 + neg2.  With t = f0 + f1 and u = f0 - f1 (round-to-nearest is symmetric
+// under negation, so (-f0) + f1 == -(f0 - f1) bit for bit, up to the sign of a zero):
+//   0: t + f2   1: t - f2   2: u + f2   3: u - f2   4: -(u - f2)   5: -(u + f2)   6: -(t - f2)   7: -(t + f2)
+// A filter tap then costs 6 adds + 4 negations per lane once, and each output channel one
+// register-indexed move (the pattern is wave-uniform) plus one add, instead of 3 sign flips
+// and 3 adds.  16 elements (8 unused) make the compiler select VGPR index mode for c[idx].
+__device__ __forceinline__ v16f sign_combos(float f0, float f1, float f2) {
+    const float t = f0 + f1, u = f0 - f1;
+    v16f c;
+    c[0] = t + f2;
+    c[1] = t - f2;
+    c[2] = u + f2;
+    c[3] = u - f2;
+    c[4] = -c[3];
+    c[5] = -c[2];
+    c[6] = -c[1];
+    c[7] = -c[0];
+#pragma unroll
+    for (int i = 8; i < 16; ++i) c[i] = 0.0f;
+    return c;
+}
+
+typedef float v8f __attribute__((ext_vector_type(8)));
+
+// acc[k] += c[idx_k] for 8 output channels with ONE switch into VGPR-index mode: the combo
+// vector is pinned to v[120:127], source 0 of each v_add_f32 is v120 displaced by the index in
+// M0 (s_set_gpr_idx_idx only rewrites that index, it does not touch the MODE register).
+// Wait states between a write of the index (M0) and the VALU instruction that uses it.  The
+// hardware does not interlock this pair: without them an add occasionally used the previous
+// index (seen as rare wrong sums when few waves share a SIMD).
+#define IDX_WAIT "s_nop 1\n\t"
+__device__ __forceinline__ void add_indexed8(float* acc, v8f c, int i0, int i1, int i2, int i3, int i4,
+                                             int i5, int i6, int i7) {
+    asm volatile(
+        "s_set_gpr_idx_on %8, gpr_idx(SRC0)\n\t" IDX_WAIT
+        "v_add_f32_e32 %0, v120, %0\n\t"
+        "s_set_gpr_idx_idx %9\n\t" IDX_WAIT
+        "v_add_f32_e32 %1, v120, %1\n\t"
+        "s_set_gpr_idx_idx %10\n\t" IDX_WAIT
+        "v_add_f32_e32 %2, v120, %2\n\t"
+        "s_set_gpr_idx_idx %11\n\t" IDX_WAIT
+        "v_add_f32_e32 %3, v120, %3\n\t"
+        "s_set_gpr_idx_idx %12\n\t" IDX_WAIT
+        "v_add_f32_e32 %4, v120, %4\n\t"
+        "s_set_gpr_idx_idx %13\n\t" IDX_WAIT
+        "v_add_f32_e32 %5, v120, %5\n\t"
+        "s_set_gpr_idx_idx %14\n\t" IDX_WAIT
+        "v_add_f32_e32 %6, v120, %6\n\t"
+        "s_set_gpr_idx_idx %15\n\t" IDX_WAIT
+        "v_add_f32_e32 %7, v120, %7\n\t"
+        "s_set_gpr_idx_off"
+        : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]), "+v"(acc[4]), "+v"(acc[5]), "+v"(acc[6]),
+          "+v"(acc[7])
+        : "s"(i0), "s"(i1), "s"(i2), "s"(i3), "s"(i4), "s"(i5), "s"(i6), "s"(i7), "{v[120:127]}"(c)
+        : "m0");
+}
+
 // The read-only operands are separate __restrict__ kernel arguments so that the
 // wave-uniform mask / threshold loads become scalar loads (s_load) feeding v_xor directly.
 __global__ __launch_bounds__(kThreads) void inconv_tiled_kernel(
     const InConvParams p, const float* __restrict__ in, const uint4* __restrict__ masks,
     const float* __restrict__ bn, uint32_t* __restrict__ out, int32_t* __restrict__ res, int b_tiles,
-    int x_groups) {
+    int x_groups, int y_phases, int div_magic) {
     __shared__ float tile[3 * kMaxCols * kLB];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int bt = blockIdx.x % b_tiles;
-    const int xg = (blockIdx.x / b_tiles) % x_groups;
-    const int y = blockIdx.x / (b_tiles * x_groups);
+    // Workgroups are dealt round-robin to the 8 XCDs (each with its own L2).  When the number
+    // of image tiles divides 8, XCD slot = (image tile, row phase) and consecutive workgroups of
+    // a slot walk along x, so the input cache lines shared by neighbouring column groups are
+    // re-used in one L2 instead of being fetched into several.
+    int bt, xg, y;
+    if (y_phases > 0) {
+        const int slot = blockIdx.x & 7, j = blockIdx.x >> 3;
+        bt = slot % b_tiles;
+        xg = j % x_groups;
+        y = (j / x_groups) * y_phases + slot / b_tiles;
+        if (y >= p.PH) return;  // whole workgroup: grid padding
+    } else {
+        bt = blockIdx.x % b_tiles;
+        xg = (blockIdx.x / b_tiles) % x_groups;
+        y = blockIdx.x / (b_tiles * x_groups);
+    }
     const int x0 = xg * kXT;
     const int x = x0 + wave;
     const bool x_ok = x < p.PW;  // wave-uniform
@@ -64,6 +139,8 @@ __global__ __launch_bounds__(kThreads) void inconv_tiled_kernel(
     const int ax_base = x0 * p.stride_w - p.pad_w;
     const size_t plane = (size_t)p.H * p.W;
     const int n_groups = (p.O + 63) / 64;
+    const uint32_t* __restrict__ pats =
+        reinterpret_cast<const uint32_t*>(masks) + (size_t)p.R * p.S * p.opad * 4;  // packed pattern table
 
     for (int g = 0; g < n_groups; ++g) {
         float acc[64];
@@ -75,10 +152,12 @@ __global__ __launch_bounds__(kThreads) void inconv_tiled_kernel(
             const int ay = y * p.stride_h - p.pad_h + r;
             if (ay < 0 || ay >= p.H) continue;  // uniform for the whole workgroup
             __syncthreads();
-            // stage: lanes run along the image row (contiguous), LDS is image-innermost
+            // stage: lanes run along the image row (contiguous runs of ncols floats per
+            // (channel, image)), LDS is image-innermost.  e / ncols by multiply-shift (the host
+            // checked the magic constant over the whole range).
             for (int e = tid; e < 3 * 64 * ncols; e += kThreads) {
-                const int col = e % ncols;
-                const int bc = e / ncols;
+                const int bc = (int)(((unsigned)e * (unsigned)div_magic) >> 16);
+                const int col = e - bc * ncols;
                 const int bl = bc & 63;
                 const int c = bc >> 6;
                 const int ax = ax_base + col;
@@ -96,17 +175,22 @@ __global__ __launch_bounds__(kThreads) void inconv_tiled_kernel(
                 const float f0 = tile[(0 * ncols + col) * kLB + lane];
                 const float f1 = tile[(1 * ncols + col) * kLB + lane];
                 const float f2 = tile[(2 * ncols + col) * kLB + lane];
-                const uint4* mk = masks + (size_t)(r * p.S + s) * p.opad + g * 64;
+                // sign patterns of this tap's channels, 8 per word (scalar loads)
+                const uint32_t* pw = pats + ((size_t)(r * p.S + s) * p.opad + g * 64) / 8;
+                const v16f c16 = sign_combos(f0, f1, f2);
+                const v8f c = {c16[0], c16[1], c16[2], c16[3], c16[4], c16[5], c16[6], c16[7]};
 #pragma unroll
-                for (int n = 0; n < 32; ++n) {
-                    const uint4 mm = mk[n];
-                    acc[n] += (flip(f0, mm.x) + flip(f1, mm.y)) + flip(f2, mm.z);
+                for (int n = 0; n < 32; n += 8) {
+                    const uint32_t w = pw[n / 8];
+                    add_indexed8(&acc[n], c, w & 7, (w >> 4) & 7, (w >> 8) & 7, (w >> 12) & 7, (w >> 16) & 7,
+                                 (w >> 20) & 7, (w >> 24) & 7, (w >> 28) & 7);
                 }
                 if (second_half) {
 #pragma unroll
-                    for (int n = 32; n < 64; ++n) {
-                        const uint4 mm = mk[n];
-                        acc[n] += (flip(f0, mm.x) + flip(f1, mm.y)) + flip(f2, mm.z);
+                    for (int n = 32; n < 64; n += 8) {
+                        const uint32_t w = pw[n / 8];
+                        add_indexed8(&acc[n], c, w & 7, (w >> 4) & 7, (w >> 8) & 7, (w >> 12) & 7,
+                                     (w >> 16) & 7, (w >> 20) & 7, (w >> 24) & 7, (w >> 28) & 7);
                     }
                 }
             }
@@ -241,10 +325,22 @@ extern "C" int tcbnn_inconv128_forward(const tcbnn_inconv128_desc* d, void* stre
     if (tiled) {
         const int b_tiles = (p.B + 63) / 64;
         const int x_groups = (p.PW + kXT - 1) / kXT;
-        const long long blocks = (long long)b_tiles * x_groups * p.PH;
+        // e / ncols == (e * magic) >> 16 for every e the staging loop uses
+        const int ncols = (kXT - 1) * p.stride_w + p.S;
+        const int div_magic = 65536 / ncols + 1;
+        for (int e = 0; e < 3 * 64 * ncols; ++e)
+            TCBNN_REQUIRE((int)(((unsigned)e * (unsigned)div_magic) >> 16) == e / ncols,
+                          "inconv128: internal error (division constant)");
+        // XCD-aware order when the image tiles divide the 8 XCD slots (see the kernel)
+        static const bool plain_order = getenv("TCBNN_INCONV_ORDER") != nullptr;  // tuning switch
+        const int y_phases = (!plain_order && 8 % b_tiles == 0) ? 8 / b_tiles : 0;
+        const long long blocks = y_phases > 0
+                                     ? 8LL * x_groups * ((p.PH + y_phases - 1) / y_phases)
+                                     : (long long)b_tiles * x_groups * p.PH;
         TCBNN_REQUIRE(blocks <= 0x7fffffffLL, "inconv128: grid too large");
         hipLaunchKernelGGL(inconv_tiled_kernel, dim3((unsigned)blocks), dim3(kThreads), 0,
-                           (hipStream_t)stream, p, p.in, p.masks, p.bn, p.out, p.res, b_tiles, x_groups);
+                           (hipStream_t)stream, p, p.in, p.masks, p.bn, p.out, p.res, b_tiles, x_groups,
+                           y_phases, div_magic);
         TCBNN_LAUNCH_CHECK("inconv_tiled_kernel");
         return TCBNN_OK;
     }

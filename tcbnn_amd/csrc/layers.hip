@@ -116,7 +116,7 @@ size_t tcbnn_conv_filter_words(int r, int s, int in_ch, int out_ch) {
 }
 size_t tcbnn_inconv_filter_words(int r, int s, int in_ch, int out_ch) {
     (void)in_ch;
-    return (size_t)r * s * pad32(out_ch) * 4;
+    return (size_t)r * s * pad32(out_ch) * 4 + (size_t)r * s * pad32(out_ch) / 8;
 }
 
 int tcbnn_fc128_forward(const tcbnn_fc128_desc* d, void* stream) {

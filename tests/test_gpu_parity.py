@@ -259,6 +259,26 @@ def test_inconv128_layer(gpu, b, h, R, stride, cout, pool, save):
     layer.release()
 
 
+def test_inconv128_small_batch_is_repeatable(gpu):
+    """Few waves per SIMD is the worst case for the register-indexed accumulation of the
+    first layer (index write -> use needs wait states): every repeat must match the oracle."""
+    r = rng(226)
+    b, h, cout = 2, 224, 64
+    x = r.standard_normal((b, 3, h, h)).astype(np.float32)
+    f = rm.pm1(r, (7, 7, 3, cout))
+    bn = r.normal(0, 12, cout).astype(np.float32)
+    want, wres = orc.inconv128(x, f, bn, 4, True, 1, True)
+    layer = gpu.InConv128LayerParam("Conv1", h, h, 7, 7, 3, cout, b, 4, 4, True, 1, 1, True)
+    layer.initialize(x, gpu.ArrayWeights([f, bn]))
+    for _ in range(12):
+        layer.output_gpu.fill(0)
+        layer.forward()
+        gpuops.sync()
+        np.testing.assert_array_equal(layer.download_packed(), want)
+        np.testing.assert_array_equal(layer.download_residual(), wres)
+    layer.release()
+
+
 def test_inconv128_presigned_input_is_exact_integer_conv(gpu):
     """The config's 'input binarized by sign' variant: +-1.0f input, sums are exact integers."""
     r = rng(5)
