@@ -55,13 +55,23 @@ struct WordVec<1> {
     using type = uint32_t;
 };
 
-__device__ __forceinline__ int xpopc(const uint32_t* a, uint4 w) {
-    return __popc(a[0] ^ w.x) + __popc(a[1] ^ w.y) + __popc(a[2] ^ w.z) + __popc(a[3] ^ w.w);
+// acc += popcount(x) in ONE instruction: v_bcnt_u32_b32 adds its second operand.  (Written
+// as inline asm because the compiler otherwise popcounts into temporaries and sums them with
+// v_add3_u32: 5 instead of 4 VALU operations per two words.)
+__device__ __forceinline__ void popc_acc(int& acc, uint32_t x) {
+    asm("v_bcnt_u32_b32 %0, %1, %0" : "+v"(acc) : "v"(x));
 }
-__device__ __forceinline__ int xpopc(const uint32_t* a, uint2 w) {
-    return __popc(a[0] ^ w.x) + __popc(a[1] ^ w.y);
+__device__ __forceinline__ void xpopc(int& acc, const uint32_t* a, uint4 w) {
+    popc_acc(acc, a[0] ^ w.x);
+    popc_acc(acc, a[1] ^ w.y);
+    popc_acc(acc, a[2] ^ w.z);
+    popc_acc(acc, a[3] ^ w.w);
 }
-__device__ __forceinline__ int xpopc(const uint32_t* a, uint32_t w) { return __popc(a[0] ^ w); }
+__device__ __forceinline__ void xpopc(int& acc, const uint32_t* a, uint2 w) {
+    popc_acc(acc, a[0] ^ w.x);
+    popc_acc(acc, a[1] ^ w.y);
+}
+__device__ __forceinline__ void xpopc(int& acc, const uint32_t* a, uint32_t w) { popc_acc(acc, a[0] ^ w); }
 
 // Threshold compare of the reference: conv layers emit (res < bn) ? 0 : 1
 // (kernel.cuh:795-796), FC layers emit (res >= bn) (kernel.cuh:210-213); the two differ
@@ -78,6 +88,7 @@ enum KernelMode : int {
     KM_AFFINE = 2,      // fp32 affine output
     KM_RAW = 3,         // int32 dot products
     KM_PARTIAL = 4,     // split-K partial popcounts -> workspace
+    KM_THRESH_FC = 5,   // threshold + pack with the FC compare (res >= bn: 0 when bn is NaN)
 };
 
 // register budget: 32*RPL accumulators + operands; keep as many waves per SIMD as that allows
@@ -161,9 +172,27 @@ __global__ __launch_bounds__(kThreads)
             for (int n = 0; n < kNTile; ++n) acc[r][n] = 0;
         int exclude = 0;
 
+        // Activation words of one k-chunk for this lane's rows; returns the (wave-uniform)
+        // in-frame predicate.  Loads are issued one chunk ahead of their use so that their
+        // latency overlaps the 32*RPL*CH xor+popcount pairs of the current chunk.
+        auto load_chunk = [&](int tr, int ts, int kc, uint32_t (*dst)[CH]) {
+            const int ay = ay0 + tr, ax = ax0 + ts;
+            const bool in_frame = valid && ay >= 0 && ay < p.H && ax >= 0 && ax < p.W;
+            if (in_frame) {
+                const uint32_t* src = act + ((size_t)(ay * p.W + ax) * p.cw + kc * CH) * p.B;
+#pragma unroll
+                for (int j = 0; j < CH; ++j)
+#pragma unroll
+                    for (int r = 0; r < RPL; ++r) dst[r][j] = src[(size_t)j * p.B + bload[r]];
+            }
+            return in_frame;
+        };
+
         // running (tap row, tap col, chunk) counters: no integer division in the loop
         int tr = (q_begin / cw_chunks) / p.S, ts = (q_begin / cw_chunks) % p.S,
             kc = q_begin % cw_chunks;
+        uint32_t a[RPL][CH], a_next[RPL][CH];
+        bool in_frame = q_begin < q_end ? load_chunk(tr, ts, kc, a) : false;
         for (int q0 = q_begin; q0 < q_end; q0 += kQB) {
             if (!single_block) {
                 __syncthreads();
@@ -172,36 +201,35 @@ __global__ __launch_bounds__(kThreads)
             }
             const int cnt = min(kQB, q_end - q0);
             for (int ql = 0; ql < cnt; ++ql) {
-                const int ay = ay0 + tr, ax = ax0 + ts;
-                const bool in_frame = ay >= 0 && ay < p.H && ax >= 0 && ax < p.W;
-                if (valid) {
-                    if (in_frame) {
-                        uint32_t a[RPL][CH];
-                        const uint32_t* src =
-                            act + ((size_t)(ay * p.W + ax) * p.cw + kc * CH) * p.B;
-#pragma unroll
-                        for (int j = 0; j < CH; ++j)
-#pragma unroll
-                            for (int r = 0; r < RPL; ++r)
-                                a[r][j] = src[(size_t)j * p.B + bload[r]];
-                        const V* wl = reinterpret_cast<const V*>(lds_w) + ql * kNTile;
-#pragma unroll
-                        for (int n = 0; n < kNTile; ++n) {
-                            const V w = wl[n];
-#pragma unroll
-                            for (int r = 0; r < RPL; ++r) acc[r][n] += xpopc(a[r], w);
-                        }
-                    } else if (kc == 0) {
-                        ++exclude;
+                int ntr = tr, nts = ts, nkc = kc + 1;
+                if (nkc == cw_chunks) {
+                    nkc = 0;
+                    if (++nts == p.S) {
+                        nts = 0;
+                        ++ntr;
                     }
                 }
-                if (++kc == cw_chunks) {
-                    kc = 0;
-                    if (++ts == p.S) {
-                        ts = 0;
-                        ++tr;
+                const bool next_in_frame =
+                    (q0 + ql + 1 < q_end) ? load_chunk(ntr, nts, nkc, a_next) : false;
+                if (in_frame) {
+                    const V* wl = reinterpret_cast<const V*>(lds_w) + ql * kNTile;
+#pragma unroll
+                    for (int n = 0; n < kNTile; ++n) {
+                        const V w = wl[n];
+#pragma unroll
+                        for (int r = 0; r < RPL; ++r) xpopc(acc[r][n], a[r], w);
                     }
+                } else if (valid && kc == 0) {
+                    ++exclude;
                 }
+                tr = ntr;
+                ts = nts;
+                kc = nkc;
+                in_frame = next_in_frame;
+#pragma unroll
+                for (int r = 0; r < RPL; ++r)
+#pragma unroll
+                    for (int j = 0; j < CH; ++j) a[r][j] = a_next[r][j];
             }
         }
 
@@ -225,7 +253,7 @@ __global__ __launch_bounds__(kThreads)
         for (int r = 0; r < RPL; ++r) {
             if (brow[r] >= p.B) continue;
             const int b = brow[r];
-            if constexpr (KM == KM_THRESH || KM == KM_THRESH_RES) {
+            if constexpr (KM == KM_THRESH || KM == KM_THRESH_RES || KM == KM_THRESH_FC) {
                 uint32_t word = 0;
                 int rv[kNTile];
                 if constexpr (KM == KM_THRESH_RES) {
@@ -254,13 +282,19 @@ __global__ __launch_bounds__(kThreads)
 #pragma unroll
                 for (int n = 0; n < kNTile; ++n) {
                     const int ch = n0 + n;
-                    if (ch >= p.N) continue;  // (no break: the loop must stay fully unrolled)
-                    int res = base - 2 * acc[r][n];
-                    if constexpr (KM == KM_THRESH_RES) {
-                        res += rv[n];
-                        if (rout != nullptr) rout[(pix * p.N + ch) * p.B + b] = res;
+                    uint32_t bit = 0;
+                    if (ch < p.N) {  // wave-uniform
+                        int res = base - 2 * acc[r][n];
+                        if constexpr (KM == KM_THRESH_RES) {
+                            res += rv[n];
+                            if (rout != nullptr) rout[(pix * p.N + ch) * p.B + b] = res;
+                        }
+                        if constexpr (KM == KM_THRESH_FC)
+                            bit = (float)res >= bn[ch] ? 1u : 0u;
+                        else
+                            bit = (float)res < bn[ch] ? 0u : 1u;
                     }
-                    word |= thresh_bit(res, bn[ch], p.nan_bit) << (31 - n);
+                    word = word + word + bit;  // shift the next channel in (MSB first)
                 }
                 outword[r] |= word;
             } else if constexpr (KM == KM_AFFINE) {
@@ -284,7 +318,7 @@ __global__ __launch_bounds__(kThreads)
         }
     }
 
-    if ((KM == KM_THRESH || KM == KM_THRESH_RES) && active) {
+    if ((KM == KM_THRESH || KM == KM_THRESH_RES || KM == KM_THRESH_FC) && active) {
 #pragma unroll
         for (int r = 0; r < RPL; ++r)
             if (brow[r] < p.B) {
@@ -362,7 +396,10 @@ int kernel_mode(const BgemmParams& p) {
     if (p.ksplit > 1) return KM_PARTIAL;
     if (p.mode == EPI_AFFINE) return KM_AFFINE;
     if (p.mode == EPI_RAW) return KM_RAW;
-    return (p.res_in != nullptr || p.res_out != nullptr) ? KM_THRESH_RES : KM_THRESH;
+    if (p.res_in != nullptr || p.res_out != nullptr) return KM_THRESH_RES;
+    // the FC compare differs from the conv compare only for NaN thresholds; it is only
+    // instantiated for FC-shaped problems (whole 128-bit words per row)
+    return (p.nan_bit == 0 && p.cw % 4 == 0) ? KM_THRESH_FC : KM_THRESH;
 }
 
 template <int RPL, int CH>
@@ -376,6 +413,9 @@ int launch_m(const BgemmParams& p, hipStream_t stream) {
             return launch_t<RPL, CH, KM_AFFINE>(p, stream);
         case KM_RAW:
             return launch_t<RPL, CH, KM_RAW>(p, stream);
+        case KM_THRESH_FC:
+            if constexpr (CH == 4) return launch_t<RPL, CH, KM_THRESH_FC>(p, stream);
+            return fail(TCBNN_EINVAL, "bgemm: FC compare needs 128-bit aligned rows");
         default:
             return launch_t<RPL, CH, KM_PARTIAL>(p, stream);
     }
