@@ -28,98 +28,17 @@
 // Semantics: Fc128LayerFMT / Out128LayerFMT / Conv128LayerFMT (kernel.cuh:174-280, 676-827),
 // BMMAS / BTC_Conv2d_balance (tensorcore_kernel.cu:305-356, bmma_kernel.cu:101-165).
 #include "common.h"
+#include "mfma_util.h"
 
 namespace tcbnn {
 namespace {
 
-typedef int v8i __attribute__((ext_vector_type(8)));
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef float v16f __attribute__((ext_vector_type(16)));
-typedef int v16i __attribute__((ext_vector_type(16)));
+using namespace mfma;
 
-constexpr int FMT_F4 = 0;
-constexpr int FMT_I8 = 1;
 constexpr int kWaves = 4;
 constexpr int kThreads = 64 * kWaves;
 constexpr int kNT = 2;    // 32-channel tiles per wave
 constexpr int kQB = 24;   // k-steps of weights staged in LDS at a time (24 * kNT KiB)
-
-enum MfmaMode : int { MM_THRESH = 0, MM_THRESH_RES = 1, MM_OTHER = 2 };
-
-// ---- bit expansion ----------------------------------------------------------------
-// FP4: bit value 1 -> nibble 0xA (-1.0), 0 -> 0x2 (+1.0): the sign is flipped for BOTH
-// operands, so products are unchanged.  dword j takes bits {4p + (3-j)}.
-__device__ __forceinline__ v4i expand_f4(uint32_t x) {
-    v4i r;
-    r[0] = ((x << 3) & 0x88888888u) | 0x22222222u;
-    r[1] = ((x << 2) & 0x88888888u) | 0x22222222u;
-    r[2] = ((x << 1) & 0x88888888u) | 0x22222222u;
-    r[3] = (x & 0x88888888u) | 0x22222222u;
-    return r;
-}
-// nibbles whose bit is not `valid` become FP4 zero
-__device__ __forceinline__ v4i expand_f4_masked(uint32_t x, uint32_t valid) {
-    v4i r = expand_f4(x);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const uint32_t t = ((valid << (3 - j)) & 0x88888888u) >> 3;  // 0x1 per valid nibble
-        r[j] &= (int)(t * 15u);
-    }
-    return r;
-}
-// int8: lane half h of a 32-bit word takes bits {q + 4h + 8p}; bit 1 -> 0x01, bit 0 -> 0xFF
-__device__ __forceinline__ v4i expand_i8(uint32_t x, int h) {
-    v4i r;
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-        const uint32_t d = (x >> (q + 4 * h)) & 0x01010101u;
-        const uint32_t m = (d << 8) - d;  // 0xFF in every byte whose bit is set
-        r[q] = (int)(~m | 0x01010101u);
-    }
-    return r;
-}
-__device__ __forceinline__ v4i expand_i8_masked(uint32_t x, uint32_t valid, int h) {
-    v4i r = expand_i8(x, h);
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-        const uint32_t d = (valid >> (q + 4 * h)) & 0x01010101u;
-        r[q] &= (int)((d << 8) - d);
-    }
-    return r;
-}
-
-template <int FMT>
-struct Acc;
-template <>
-struct Acc<FMT_F4> {
-    using type = v16f;
-    static __device__ __forceinline__ type mma(v4i a, v4i b, type c) {
-        const v8i a8 = {a[0], a[1], a[2], a[3], 0, 0, 0, 0};
-        const v8i b8 = {b[0], b[1], b[2], b[3], 0, 0, 0, 0};
-        // cbsz = blgp = 4: both operands FP4; scale operands 0 select the unscaled instruction
-        return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8, b8, c, 4, 4, 0, 0, 0, 0);
-    }
-    static __device__ __forceinline__ int to_int(float v) { return (int)v; }
-};
-template <>
-struct Acc<FMT_I8> {
-    using type = v16i;
-    static __device__ __forceinline__ type mma(v4i a, v4i b, type c) {
-        return __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c, 0, 0, 0);
-    }
-    static __device__ __forceinline__ int to_int(int v) { return v; }
-};
-
-__device__ __forceinline__ uint32_t thresh_bit(int res, float thr, int nan_bit) {
-    const float rf = (float)res;
-    return nan_bit ? (rf < thr ? 0u : 1u) : (rf >= thr ? 1u : 0u);
-}
-
-// MFMA row i of a channel tile holds channel perm(i), so that accumulator register v of
-// lane half h (row 8*(v/4) + 4h + v%4) is channel 16h + v.
-__device__ __forceinline__ int row_to_channel(int i) {
-    return 16 * ((i >> 2) & 1) + 4 * (i >> 3) + (i & 3);
-}
 
 template <int FMT, int MT, int MM>
 __global__ __launch_bounds__(kThreads) void bgemm_mfma_kernel(
@@ -431,6 +350,10 @@ int mfma_ksplit(const BgemmParams& p, int variant) {
 }  // namespace
 
 void bgemm_mfma_kernel_name(const BgemmParams& p, int variant, char* buf, size_t len) {
+    if (variant == TCBNN_VARIANT_MFMA_F4 && conv3x3_mfma_applicable(p)) {
+        conv3x3_mfma_kernel_name(p, buf, len);
+        return;
+    }
     BgemmParams q = p;
     q.ksplit = mfma_ksplit(p, variant);
     snprintf(buf, len, "bgemm_mfma_kernel<%d, %d, %d>", variant == TCBNN_VARIANT_MFMA_F4 ? FMT_F4 : FMT_I8,
@@ -439,6 +362,8 @@ void bgemm_mfma_kernel_name(const BgemmParams& p, int variant, char* buf, size_t
 
 int launch_bgemm_mfma(const BgemmParams& p_in, int variant, hipStream_t stream) {
     if (int rc = validate_bgemm(p_in)) return rc;
+    if (variant == TCBNN_VARIANT_MFMA_F4 && conv3x3_mfma_applicable(p_in))
+        return launch_conv3x3_mfma(p_in, stream);
     BgemmParams p = p_in;
     p.ksplit = mfma_ksplit(p, variant);
     p.ws_is_dot = 1;

@@ -100,6 +100,10 @@ int launch_splitk_finish(const BgemmParams& p, hipStream_t stream);
 // profiler-style kernel names for a problem
 void bgemm_popc_kernel_name(const BgemmParams& p, char* buf, size_t len);
 void bgemm_mfma_kernel_name(const BgemmParams& p, int variant, char* buf, size_t len);
+// persistent FP4 matrix-core kernel for 3x3 convolutions with Cin = 64 / 128 / 256
+bool conv3x3_mfma_applicable(const BgemmParams& p);
+int launch_conv3x3_mfma(const BgemmParams& p, hipStream_t stream);
+void conv3x3_mfma_kernel_name(const BgemmParams& p, char* buf, size_t len);
 // number of K splits wanted for a problem (1 = none)
 int choose_ksplit(const BgemmParams& p);
 
