@@ -1,5 +1,5 @@
 // Persistent FP4 matrix-core kernel for the 3x3 bit convolutions that carry almost all of a
-// binarized ResNet / VGG (Conv128LayerFMT, kernel.cuh:676-827, pool 1x1, Cin = 64 / 128 / 256).
+// binarized ResNet / VGG (Conv128LayerFMT, kernel.cuh:676-827, pool 1x1, Cin = 64 .. 512).
 //
 // Same operand mapping as bgemm_mfma.hip (MFMA "A" = 32 output channels, "B" = 32 images, a lane
 // of the accumulator owns one image and 16 channels), plus what a short-K convolution needs to
@@ -9,7 +9,8 @@
 //     KiB) and its thresholds are staged in LDS ONCE, then every wave walks a strided list of
 //     (pixel, 64-image) tiles; no barrier after the staging;
 //   - whole-chunk register prefetch: all activation words a wave needs for the next chunk of
-//     taps (the whole tile for Cin <= 128, one filter row for Cin = 256) are requested while
+//     taps (the whole tile for Cin <= 128, one filter row for Cin = 256, one tap for Cin = 512)
+//     are requested while
 //     the current chunk is multiplied, double-buffered across tile boundaries, so the loads of
 //     tile i+1 fly under the MFMAs and the epilogue of tile i;
 //   - wave-uniform border handling: a tap outside the frame is a cleared bit in a scalar mask
@@ -31,16 +32,17 @@ using namespace mfma;
 
 constexpr int kWaves = 4;
 constexpr int kThreads = 64 * kWaves;
-constexpr int MT = 2;  // 32-image tiles per wave
 constexpr int NT = 2;  // 32-channel tiles per wave
 
-// SPT = k-steps (64 bits) per filter tap = Cin / 64
-template <int SPT, int MM>
-__global__ __launch_bounds__(kThreads) void conv3x3_mfma_f4_kernel(
+// SPT = k-steps (64 bits) per filter tap = Cin / 64; MT = 32-image tiles per wave (2 for plain
+// layers; 1 for residual layers, whose int32 traffic wants more waves per SIMD in flight)
+template <int SPT, int MM, int MT>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) void
+conv3x3_mfma_f4_kernel(
     const BgemmParams p, const uint32_t* __restrict__ act, const uint32_t* __restrict__ wgt,
     const float* __restrict__ bnp, const int32_t* __restrict__ rin, int n_groups, int b_groups,
     int pix_streams) {
-    constexpr int TPC = SPT == 4 ? 3 : 9;  // taps per prefetch chunk
+    constexpr int TPC = SPT == 8 ? 1 : (SPT == 4 ? 3 : 9);  // taps per prefetch chunk
     constexpr int NCH = 9 / TPC;           // chunks per tile
     constexpr int NQ = 9 * SPT;            // k-steps per tile
     extern __shared__ v4i lds_dyn[];
@@ -92,8 +94,8 @@ __global__ __launch_bounds__(kThreads) void conv3x3_mfma_f4_kernel(
         uint32_t mask = 0;
 #pragma unroll
         for (int tl = 0; tl < TPC; ++tl) {
-            const int r = TPC == 9 ? tl / 3 : chunk;
-            const int s = tl % 3;
+            const int r = TPC == 9 ? tl / 3 : (TPC == 3 ? chunk : chunk / 3);
+            const int s = TPC == 1 ? chunk % 3 : tl % 3;
             const int ay = yy * p.stride_h - p.pad_h + r, ax = xx * p.stride_w - p.pad_w + s;
             if (ay >= 0 && ay < p.H && ax >= 0 && ax < p.W) {
                 mask |= 1u << tl;
@@ -139,6 +141,37 @@ __global__ __launch_bounds__(kThreads) void conv3x3_mfma_f4_kernel(
         }
     };
 
+    // Residual operand of the tile at pixel (yy, xx), requested before the tile's last chunk is
+    // multiplied so that the loads fly under the MFMAs (kernel.cuh:770-794).
+    int rv[MM == MM_THRESH_RES ? MT : 1][NT][16];
+    auto load_residual = [&](int yy, int xx) {
+        if constexpr (MM == MM_THRESH_RES) {
+            const size_t pix = (size_t)yy * p.PW + xx;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int c = n0 + nt * 32 + 16 * h + v;
+                        const int bb = bload[mt];
+                        int val = 0;
+                        if (rin != nullptr && c < p.res_limit && c < p.res_in_ch && c < p.N) {
+                            if (p.res_pool) {
+                                const size_t rw2 = 2 * (size_t)p.PW;
+                                const int32_t* s00 =
+                                    rin + (((size_t)(2 * yy) * rw2 + 2 * xx) * p.res_in_ch + c) * p.B + bb;
+                                const size_t ddx = (size_t)p.res_in_ch * p.B, ddy = rw2 * ddx;
+                                val = max(max(s00[0], s00[ddx]), max(s00[ddy], s00[ddy + ddx]));
+                            } else {
+                                val = rin[(pix * p.res_in_ch + c) * p.B + bb];
+                            }
+                        }
+                        rv[mt][nt][v] = val;
+                    }
+        }
+    };
+
     auto epilogue = [&](int yy, int xx) {
         const size_t pix = (size_t)yy * p.PW + xx;
         uint32_t* dst_bits = p.out_bits + pix * p.bits_pix_stride;
@@ -163,30 +196,11 @@ __global__ __launch_bounds__(kThreads) void conv3x3_mfma_f4_kernel(
                 const bool b_ok = b < p.B;
                 uint32_t hw = 0;
                 if constexpr (MM == MM_THRESH_RES) {
-                    const int bb = bload[mt];
-                    int rv[16];
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        const int c = cbase + v;
-                        int val = 0;
-                        if (rin != nullptr && c < p.res_limit && c < p.res_in_ch && c < p.N) {
-                            if (p.res_pool) {
-                                const size_t rw2 = 2 * (size_t)p.PW;
-                                const int32_t* s00 =
-                                    rin + (((size_t)(2 * yy) * rw2 + 2 * xx) * p.res_in_ch + c) * p.B + bb;
-                                const size_t ddx = (size_t)p.res_in_ch * p.B, ddy = rw2 * ddx;
-                                val = max(max(s00[0], s00[ddx]), max(s00[ddy], s00[ddy + ddx]));
-                            } else {
-                                val = rin[(pix * p.res_in_ch + c) * p.B + bb];
-                            }
-                        }
-                        rv[v] = val;
-                    }
                     int32_t* __restrict__ rout = p.res_out;
 #pragma unroll
                     for (int v = 0; v < 16; ++v) {
                         const int c = cbase + v;
-                        const int res = (int)acc[mt][nt][v] + rv[v];
+                        const int res = (int)acc[mt][nt][v] + rv[mt][nt][v];
                         if (rout != nullptr && b_ok && c < p.N) rout[(pix * p.N + c) * p.B + b] = res;
                         const uint32_t bit = (c < p.N && !((float)res < thr[v])) ? 1u : 0u;
                         hw = hw + hw + bit;
@@ -235,6 +249,7 @@ __global__ __launch_bounds__(kThreads) void conv3x3_mfma_f4_kernel(
         }
         const bool nhave = npi < npix;
         if (nhave) mnxt = load_chunk(ny, nx, nchunk, nxt);
+        if (chunk == NCH - 1) load_residual(y, x);
         compute_chunk(chunk, cur, mcur);
         if (chunk == NCH - 1) {
             epilogue(y, x);
@@ -254,13 +269,13 @@ __global__ __launch_bounds__(kThreads) void conv3x3_mfma_f4_kernel(
     }
 }
 
-template <int SPT, int MM>
+template <int SPT, int MM, int MT>
 int launch_t(const BgemmParams& p, hipStream_t stream) {
     constexpr int NQ = 9 * SPT;
     const size_t lds_bytes = (size_t)NQ * NT * 64 * 16 + NT * 32 * sizeof(float);
     static bool attr_set = false;  // per instantiation
     if (!attr_set) {
-        if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&conv3x3_mfma_f4_kernel<SPT, MM>),
+        if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&conv3x3_mfma_f4_kernel<SPT, MM, MT>),
                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes),
                                "hipFuncSetAttribute(MaxDynamicSharedMemorySize)"))
             return rc;
@@ -269,8 +284,9 @@ int launch_t(const BgemmParams& p, hipStream_t stream) {
     const int n_groups = (p.N + 32 * NT - 1) / (32 * NT);
     const int b_groups = (p.B + 32 * MT - 1) / (32 * MT);
     const int quads = (p.PH * p.PW + kWaves - 1) / kWaves;  // pixel quads (one pixel per wave)
-    // about two workgroups per CU, with the pixel quads spread as evenly as possible
-    const int target = std::max(1, 512 / (n_groups * b_groups));
+    // about two (plain) or three (residual) workgroups per CU, with the pixel quads spread as
+    // evenly as possible
+    const int target = std::max(1, (MT == 1 ? 768 : 512) / (n_groups * b_groups));
     int best = std::min(target, quads);
     double best_waste = 1e30;
     for (int ps = std::max(1, target / 2); ps <= std::min(quads, target * 2); ++ps) {
@@ -282,7 +298,7 @@ int launch_t(const BgemmParams& p, hipStream_t stream) {
         }
     }
     const long long blocks = (long long)best * n_groups * b_groups;
-    hipLaunchKernelGGL((conv3x3_mfma_f4_kernel<SPT, MM>), dim3((unsigned)blocks), dim3(kThreads), lds_bytes,
+    hipLaunchKernelGGL((conv3x3_mfma_f4_kernel<SPT, MM, MT>), dim3((unsigned)blocks), dim3(kThreads), lds_bytes,
                        stream, p, p.act, p.wgt, p.bn, p.res_in, n_groups, b_groups, best);
     TCBNN_LAUNCH_CHECK("conv3x3_mfma_f4_kernel");
     return TCBNN_OK;
@@ -290,21 +306,22 @@ int launch_t(const BgemmParams& p, hipStream_t stream) {
 
 template <int SPT>
 int launch_m(const BgemmParams& p, hipStream_t stream) {
-    if (p.res_in != nullptr || p.res_out != nullptr) return launch_t<SPT, MM_THRESH_RES>(p, stream);
-    return launch_t<SPT, MM_THRESH>(p, stream);
+    if (p.res_in != nullptr || p.res_out != nullptr) return launch_t<SPT, MM_THRESH_RES, 1>(p, stream);
+    return launch_t<SPT, MM_THRESH, 2>(p, stream);
 }
 
 }  // namespace
 
 bool conv3x3_mfma_applicable(const BgemmParams& p) {
     return p.R == 3 && p.S == 3 && p.pool_h == 1 && p.pool_w == 1 && p.mode == EPI_THRESH && p.nan_bit == 1 &&
-           p.ksplit <= 1 && (p.cw == 2 || p.cw == 4 || p.cw == 8) && p.k_tap == 32 * p.cw &&
+           p.ksplit <= 1 && (p.cw == 2 || p.cw == 4 || p.cw == 8 || p.cw == 16) && p.k_tap == 32 * p.cw &&
            (long long)p.PH * p.PW < (1 << 24);
 }
 
 void conv3x3_mfma_kernel_name(const BgemmParams& p, char* buf, size_t len) {
-    snprintf(buf, len, "conv3x3_mfma_f4_kernel<%d, %d>", p.cw / 2,
-             (p.res_in != nullptr || p.res_out != nullptr) ? MM_THRESH_RES : MM_THRESH);
+    const bool res = p.res_in != nullptr || p.res_out != nullptr;
+    snprintf(buf, len, "conv3x3_mfma_f4_kernel<%d, %d, %d>", p.cw / 2, res ? MM_THRESH_RES : MM_THRESH,
+             res ? 1 : 2);
 }
 
 int launch_conv3x3_mfma(const BgemmParams& p, hipStream_t stream) {
@@ -313,8 +330,10 @@ int launch_conv3x3_mfma(const BgemmParams& p, hipStream_t stream) {
             return launch_m<1>(p, stream);
         case 4:
             return launch_m<2>(p, stream);
-        default:
+        case 8:
             return launch_m<4>(p, stream);
+        default:
+            return launch_m<8>(p, stream);
     }
 }
 
