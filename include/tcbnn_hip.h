@@ -52,7 +52,8 @@ extern "C" {
 #define TCBNN_EHIP (-3)     /* HIP runtime error (utility.h:57-81)           */
 #define TCBNN_EUNSUPPORTED (-4)
 
-/* Inner-product engines.  AUTO picks per shape. */
+/* Inner-product engines.  AUTO is the process-wide default (FP4 matrix cores unless
+ * changed by tcbnn_set_default_variant or the environment). */
 #define TCBNN_VARIANT_AUTO 0
 #define TCBNN_VARIANT_POPC 1      /* v_xor_b32 + v_bcnt_u32_b32 on the VALU   */
 #define TCBNN_VARIANT_MFMA_I8 2   /* +-1 unpacked to int8, v_mfma_i32_32x32x32_i8 */
@@ -80,7 +81,7 @@ size_t tcbnn_fc_act_words(int batch, int features);                    /* B*KW12
 size_t tcbnn_conv_act_words(int height, int width, int batch, int ch); /* H*W*B*CW         */
 size_t tcbnn_fc_weight_words(int in_features, int out_features);       /* NPAD32*KW128     */
 size_t tcbnn_conv_filter_words(int r, int s, int in_ch, int out_ch);   /* NPAD32*R*S*CW    */
-size_t tcbnn_inconv_filter_words(int r, int s, int in_ch, int out_ch); /* R*S*OPAD32*(4+1/8) */
+size_t tcbnn_inconv_filter_words(int r, int s, int in_ch, int out_ch); /* R*S*OPAD32*5     */
 
 /* ------------------------------------------------- one-time weight packing */
 /* fp32 [K][N] (param.h:58-59) -> packed [NPAD32][KW128].  Replaces
@@ -94,8 +95,8 @@ int tcbnn_pack_conv_filter(const float* filter_hwio, uint32_t* packed, int r, in
 /* fp32 HWIO [R][S][3][O] -> sign table uint32 [R*S][OPAD32][4]: entry c<3 is 0 if the
  * weight of input channel c is >= 0 and 0x80000000 otherwise (the bit the first layer
  * flips on the fp32 input, kernel.cuh:636-638); entry 3 is the sign pattern index
- * 4*neg0 + 2*neg1 + neg2.  A second table [R*S][OPAD32/8] follows with the same patterns
- * packed 8 per word.  Replaces PackFiltersByOutChannels32 (param.h:613-632). */
+ * 4*neg0 + 2*neg1 + neg2.  A second table [R*S][OPAD32] follows with the patterns alone,
+ * one per word.  Replaces PackFiltersByOutChannels32 (param.h:613-632). */
 int tcbnn_pack_inconv_filter(const float* filter_hwio, uint32_t* packed, int r, int s, int in_ch,
                              int out_ch, void* stream);
 /* fp32 +-1 matrix rows -> packed activation matrix, MSB first, batch (row) innermost:

@@ -105,7 +105,11 @@ __device__ __forceinline__ void add_indexed8(float* acc, v8f c, int i0, int i1, 
 
 // The read-only operands are separate __restrict__ kernel arguments so that the
 // wave-uniform mask / threshold loads become scalar loads (s_load) feeding v_xor directly.
-__global__ __launch_bounds__(kThreads) void inconv_tiled_kernel(
+typedef uint32_t u16v __attribute__((ext_vector_type(16)));
+
+// NST = floats each thread stages per filter row = ceil(3 * 64 * ncols / 256)
+template <int NST>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3))) void inconv_tiled_kernel(
     const InConvParams p, const float* __restrict__ in, const uint4* __restrict__ masks,
     const float* __restrict__ bn, uint32_t* __restrict__ out, int32_t* __restrict__ res, int b_tiles,
     int x_groups, int y_phases, int div_magic) {
@@ -148,50 +152,69 @@ __global__ __launch_bounds__(kThreads) void inconv_tiled_kernel(
         for (int n = 0; n < 64; ++n) acc[n] = 0.0f;
         const bool second_half = g * 64 + 32 < p.opad;  // uniform
 
-        for (int r = 0; r < p.R; ++r) {
-            const int ay = y * p.stride_h - p.pad_h + r;
-            if (ay < 0 || ay >= p.H) continue;  // uniform for the whole workgroup
-            __syncthreads();
-            // stage: lanes run along the image row (contiguous runs of ncols floats per
-            // (channel, image)), LDS is image-innermost.  e / ncols by multiply-shift (the host
-            // checked the magic constant over the whole range).
-            for (int e = tid; e < 3 * 64 * ncols; e += kThreads) {
+        // Filter rows inside the frame: r_lo <= r < r_hi (uniform for the whole workgroup).
+        const int ay0 = y * p.stride_h - p.pad_h;
+        const int r_lo = max(0, -ay0), r_hi = min(p.R, p.H - ay0);
+        const int n_stage = 3 * 64 * ncols;
+
+        // Software-pipelined staging: the input row segment of filter row r+1 is requested
+        // from HBM into registers before row r is multiplied, and written to LDS afterwards.
+        // Lanes run along the image row (contiguous runs of ncols floats per (channel, image)),
+        // LDS is image-innermost; e / ncols by multiply-shift (the host checked the constant).
+        float stg[NST];
+        auto fetch_row = [&](int r) {
+            const size_t row_off = (size_t)(ay0 + r) * p.W;
+#pragma unroll
+            for (int k = 0; k < NST; ++k) {
+                const int e = tid + k * kThreads;
                 const int bc = (int)(((unsigned)e * (unsigned)div_magic) >> 16);
                 const int col = e - bc * ncols;
-                const int bl = bc & 63;
-                const int c = bc >> 6;
                 const int ax = ax_base + col;
-                const int bb = min(b0 + bl, p.B - 1);
+                const int bb = min(b0 + (bc & 63), p.B - 1);
                 float v = 0.0f;
-                if (ax >= 0 && ax < p.W) v = in[((size_t)bb * 3 + c) * plane + (size_t)ay * p.W + ax];
-                tile[(c * ncols + col) * kLB + bl] = v;
+                if (e < n_stage && ax >= 0 && ax < p.W) v = in[((size_t)bb * 3 + (bc >> 6)) * plane + row_off + ax];
+                stg[k] = v;
             }
+        };
+        auto store_row = [&]() {
+#pragma unroll
+            for (int k = 0; k < NST; ++k) {
+                const int e = tid + k * kThreads;
+                const int bc = (int)(((unsigned)e * (unsigned)div_magic) >> 16);
+                const int col = e - bc * ncols;
+                if (e < n_stage) tile[((bc >> 6) * ncols + col) * kLB + (bc & 63)] = stg[k];
+            }
+        };
+
+        if (r_lo < r_hi) fetch_row(r_lo);
+        for (int r = r_lo; r < r_hi; ++r) {
             __syncthreads();
+            store_row();
+            __syncthreads();
+            if (r + 1 < r_hi) fetch_row(r + 1);
             if (!x_ok) continue;
             for (int s = 0; s < p.S; ++s) {
                 const int col = wave * p.stride_w + s;
                 const int ax = ax_base + col;
                 if (ax < 0 || ax >= p.W) continue;  // wave-uniform
+                // sign patterns of this tap's channels, one per word (wide scalar loads)
+                const u16v* pw = reinterpret_cast<const u16v*>(pats + (size_t)(r * p.S + s) * p.opad + g * 64);
+                const u16v i0 = pw[0], i1 = pw[1];
                 const float f0 = tile[(0 * ncols + col) * kLB + lane];
                 const float f1 = tile[(1 * ncols + col) * kLB + lane];
                 const float f2 = tile[(2 * ncols + col) * kLB + lane];
-                // sign patterns of this tap's channels, 8 per word (scalar loads)
-                const uint32_t* pw = pats + ((size_t)(r * p.S + s) * p.opad + g * 64) / 8;
                 const v16f c16 = sign_combos(f0, f1, f2);
                 const v8f c = {c16[0], c16[1], c16[2], c16[3], c16[4], c16[5], c16[6], c16[7]};
-#pragma unroll
-                for (int n = 0; n < 32; n += 8) {
-                    const uint32_t w = pw[n / 8];
-                    add_indexed8(&acc[n], c, w & 7, (w >> 4) & 7, (w >> 8) & 7, (w >> 12) & 7, (w >> 16) & 7,
-                                 (w >> 20) & 7, (w >> 24) & 7, (w >> 28) & 7);
-                }
+                add_indexed8(&acc[0], c, i0[0], i0[1], i0[2], i0[3], i0[4], i0[5], i0[6], i0[7]);
+                add_indexed8(&acc[8], c, i0[8], i0[9], i0[10], i0[11], i0[12], i0[13], i0[14], i0[15]);
+                add_indexed8(&acc[16], c, i1[0], i1[1], i1[2], i1[3], i1[4], i1[5], i1[6], i1[7]);
+                add_indexed8(&acc[24], c, i1[8], i1[9], i1[10], i1[11], i1[12], i1[13], i1[14], i1[15]);
                 if (second_half) {
-#pragma unroll
-                    for (int n = 32; n < 64; n += 8) {
-                        const uint32_t w = pw[n / 8];
-                        add_indexed8(&acc[n], c, w & 7, (w >> 4) & 7, (w >> 8) & 7, (w >> 12) & 7,
-                                     (w >> 16) & 7, (w >> 20) & 7, (w >> 24) & 7, (w >> 28) & 7);
-                    }
+                    const u16v i2 = pw[2], i3 = pw[3];
+                    add_indexed8(&acc[32], c, i2[0], i2[1], i2[2], i2[3], i2[4], i2[5], i2[6], i2[7]);
+                    add_indexed8(&acc[40], c, i2[8], i2[9], i2[10], i2[11], i2[12], i2[13], i2[14], i2[15]);
+                    add_indexed8(&acc[48], c, i3[0], i3[1], i3[2], i3[3], i3[4], i3[5], i3[6], i3[7]);
+                    add_indexed8(&acc[56], c, i3[8], i3[9], i3[10], i3[11], i3[12], i3[13], i3[14], i3[15]);
                 }
             }
         }
@@ -338,9 +361,17 @@ extern "C" int tcbnn_inconv128_forward(const tcbnn_inconv128_desc* d, void* stre
                                      ? 8LL * x_groups * ((p.PH + y_phases - 1) / y_phases)
                                      : (long long)b_tiles * x_groups * p.PH;
         TCBNN_REQUIRE(blocks <= 0x7fffffffLL, "inconv128: grid too large");
-        hipLaunchKernelGGL(inconv_tiled_kernel, dim3((unsigned)blocks), dim3(kThreads), 0,
-                           (hipStream_t)stream, p, p.in, p.masks, p.bn, p.out, p.res, b_tiles, x_groups,
-                           y_phases, div_magic);
+        const int nst = (3 * 64 * ncols + kThreads - 1) / kThreads;
+        auto launch = [&](auto kernel) {
+            hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(kThreads), 0, (hipStream_t)stream, p, p.in,
+                               p.masks, p.bn, p.out, p.res, b_tiles, x_groups, y_phases, div_magic);
+        };
+        if (nst <= 5)
+            launch(inconv_tiled_kernel<5>);
+        else if (nst <= 15)
+            launch(inconv_tiled_kernel<15>);
+        else
+            launch(inconv_tiled_kernel<24>);
         TCBNN_LAUNCH_CHECK("inconv_tiled_kernel");
         return TCBNN_OK;
     }

@@ -62,27 +62,22 @@ __global__ void pack_conv_filter_kernel(const float* __restrict__ f, uint32_t* _
 // HWIO fp32 [R*S][3][O] -> two tables:
 //   [R*S][opad32][4]  sign masks of the three input channels (0x80000000 where the weight is
 //                     negative) and, in the 4th word, the sign pattern 4*neg0 + 2*neg1 + neg2;
-//   [R*S][opad32/8]   the same patterns packed 8 per word (nibble k of word j = channel 8j+k),
-//                     so one scalar load fetches the patterns of 64 channels.
+//   [R*S][opad32]     the same patterns, one per word, contiguous (read with wide scalar loads).
 __global__ void pack_inconv_filter_kernel(const float* __restrict__ f, uint32_t* __restrict__ dst,
                                           int taps, int in_ch, int out_ch, int opad) {
     const long long idx = (long long)blockIdx.x * kThreads + threadIdx.x;
     const long long n_mask = (long long)taps * opad * 4;
-    if (idx >= n_mask + (long long)taps * opad / 8) return;
-    if (idx >= n_mask) {  // packed pattern table
+    if (idx >= n_mask + (long long)taps * opad) return;
+    if (idx >= n_mask) {  // pattern table
         const long long j = idx - n_mask;
-        const int t = (int)(j / (opad / 8));
-        const int o0 = (int)(j % (opad / 8)) * 8;
-        uint32_t w = 0;
-        for (int k = 0; k < 8; ++k) {
-            uint32_t pat = 0;
-            for (int cc = 0; cc < 3; ++cc) {
-                const float v = o0 + k < out_ch ? f[((size_t)t * in_ch + cc) * out_ch + o0 + k] : -1.0f;
-                pat = pat * 2 + (v >= 0.0f ? 0u : 1u);
-            }
-            w |= pat << (4 * k);
+        const int t = (int)(j / opad);
+        const int oo = (int)(j % opad);
+        uint32_t pat = 0;
+        for (int cc = 0; cc < 3; ++cc) {
+            const float v = oo < out_ch ? f[((size_t)t * in_ch + cc) * out_ch + oo] : -1.0f;
+            pat = pat * 2 + (v >= 0.0f ? 0u : 1u);
         }
-        dst[idx] = w;
+        dst[idx] = pat;
         return;
     }
     const int c = (int)(idx & 3);
@@ -243,7 +238,7 @@ int tcbnn_pack_inconv_filter(const float* filter_hwio, uint32_t* packed, int r, 
     TCBNN_REQUIRE(r > 0 && s > 0 && out_ch > 0, "pack_inconv_filter: bad shape");
     TCBNN_REQUIRE(in_ch == 3, "first-layer convolution has 3 input channels (kernel.cuh:620-625)");
     const int opad = pad32(out_ch);
-    const long long total = (long long)r * s * opad * 4 + (long long)r * s * opad / 8;
+    const long long total = (long long)r * s * opad * 5;
     hipLaunchKernelGGL(pack_inconv_filter_kernel, dim3(blocks_for(total)), dim3(kThreads), 0,
                        (hipStream_t)stream, filter_hwio, packed, r * s, in_ch, out_ch, opad);
     TCBNN_LAUNCH_CHECK("pack_inconv_filter_kernel");

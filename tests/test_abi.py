@@ -45,7 +45,7 @@ def test_size_helpers():
     assert L.tcbnn_conv_act_words(56, 56, 256, 64) == 56 * 56 * 256 * 2
     assert L.tcbnn_fc_weight_words(784, 10) == 32 * 28
     assert L.tcbnn_conv_filter_words(3, 3, 64, 64) == 64 * 9 * 2
-    assert L.tcbnn_inconv_filter_words(7, 7, 3, 64) == 49 * 64 * 4 + 49 * 64 // 8
+    assert L.tcbnn_inconv_filter_words(7, 7, 3, 64) == 49 * 64 * 5
 
 
 def test_errors_are_codes_not_exits():
