@@ -22,13 +22,78 @@ if ROOT not in sys.path:
 
 PAPER_IMAGES_PER_S = 5600.0  # README.md:16 of the reference (ResNet-18, ImageNet, Turing)
 
-# Rooflines.  VALU: 256 CU x 64 lane-ops/clk x 2.4 GHz = 39.3 T lane-op/s; one v_xor_b32 +
+# Published MI355X peaks.  The XOR+popcount engine runs on the VALU, for which there is no
+# published figure: 256 CU x 64 lane-ops/clk x 2.4 GHz = 39.3 T lane-op/s, and one v_xor_b32 +
 # one v_bcnt_u32_b32 (2 lane-ops) do 32 multiply-accumulates = 64 binary ops.
-PEAKS = {
+HBM_PEAK_GBS = 8000.0
+COMPUTE_PEAKS_TOPS = {
     "popc": ("valu", 256 * 64 * 2.4e9 / 2 * 64 / 1e12),  # 1258.3 T binary op/s
-    "mfma_i8": ("mfma", 5000.0),                          # published dense int8, TOP/s
-    "mfma_f4": ("mfma", 10100.0),                         # published dense fp4, TFLOP/s
+    "mfma_i8": ("mfma", 5000.0),                          # dense int8
+    "mfma_f4": ("mfma", 10100.0),                         # dense fp4
 }
+
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch,
+# scaled by what the same counters read for a plain device-to-device copy of known size); the
+# runs and the scale factor are recorded in profiles/.  Keyed by kernel name; None = not measured.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def layer_work(L, spec=()):
+    """Algorithmic work of one layer launch: binary ops (2 per +-1 multiply-accumulate, border taps
+    included), fp32 adds of the first layer, and the HBM bytes the launch has to move once
+    (inputs + outputs + weights, packed activations at 1 bit per value, residuals int32)."""
+    from tcbnn_amd import nets
+    bops, flops = nets.binary_ops([L])
+    B = L["batch"]
+    if L["kind"] == "in":
+        byts = B * L["features"] * 4 + B * L["features"] / 8
+    elif L["kind"] in ("fc", "out"):
+        byts = B * L["inp"] / 8 + L["inp"] * L["out"] / 8 + (B * L["out"] * 4 if L["kind"] == "out" else B * L["out"] / 8)
+    else:
+        oh = -(-L["h"] // L["stride"]); ow = -(-L["w"] // L["stride"])
+        poh, pow_ = -(-oh // L["pool"]), -(-ow // L["pool"])
+        out_bits = B * poh * pow_ * L["cout"] / 8
+        if L["kind"] == "inconv":
+            byts = B * 3 * L["h"] * L["w"] * 4 + out_bits + L["r"] * L["s"] * 3 * L["cout"] * 4
+            if L["save_residual"]:
+                byts += B * oh * ow * L["cout"] * 4
+        else:
+            byts = B * L["h"] * L["w"] * L["cin"] / 8 + out_bits + L["r"] * L["s"] * L["cin"] * L["cout"] / 8
+            if L["save_residual"]:
+                byts += B * oh * ow * L["cout"] * 4
+            if L["inject_residual"]:
+                # channels actually injected: those the source layer saved, capped by residual_channels
+                src_ch = [S["cout"] for S in spec if S["name"] == L.get("res_src")]
+                ch = min([L["residual_channels"], L["cout"]] + src_ch)
+                byts += B * oh * ow * (4 if L["residual_pool"] else 1) * ch * 4
+    return dict(bops=bops, flops=flops, bytes=float(byts))
+
+
+def roofline_of(name, g, variant):
+    """Roofline record of one kernel (all its launches in a step): the binding roof is HBM when the
+    kernel's arithmetic intensity is below the ridge of the compute peak, else the compute peak."""
+    bound_c, peak_c = COMPUTE_PEAKS_TOPS[variant]
+    secs = g["ms"] * 1e-3
+    tops = g["bops"] / secs / 1e12
+    gbs = g["bytes"] / secs / 1e9
+    ridge = peak_c * 1e12 / (HBM_PEAK_GBS * 1e9)  # binary ops per byte
+    intensity = g["bops"] / g["bytes"] if g["bytes"] else float("inf")
+    hbm_bound = g["bops"] == 0 or intensity < ridge
+    rec = {
+        "bound": "hbm" if hbm_bound else bound_c,
+        "achieved": round(gbs if hbm_bound else tops, 2),
+        "peak": HBM_PEAK_GBS if hbm_bound else round(peak_c, 1),
+        "unit": "GB/s" if hbm_bound else ("TFLOP/s" if variant == "mfma_f4" else "TOP/s"),
+        "frac": round((gbs / HBM_PEAK_GBS) if hbm_bound else (tops / peak_c), 4),
+        "traffic": MEASURED_TRAFFIC_BYTES.get(name),
+        "kernel": name, "launches_per_step": g["launches"],
+        "avg_launch_ms": round(g["ms"] / g["launches"], 4),
+        "algorithmic_bytes_per_launch": round(g["bytes"] / g["launches"]),
+        "algorithmic_ops_per_launch": round(g["bops"] / g["launches"]),
+        "ops_per_byte": round(intensity, 1) if g["bytes"] else None,
+        "binary_tops": round(tops, 2), "hbm_gbs": round(gbs, 1),
+    }
+    return rec
 
 
 def main():
@@ -100,32 +165,29 @@ def main():
     # group launches by device kernel, as a profiler does
     groups = {}
     for L, layer in zip(spec, net.order):
-        if L["kind"] in ("conv", "fc"):
-            name = layer.kernel_name()
-            ops = nets.binary_ops([L])[0]
-            g = groups.setdefault(name, dict(ops=0.0, ms=0.0, launches=0))
-            g["ops"] += ops
-            g["ms"] += layer_ms[L["name"]]
-            g["launches"] += 1
-    dom_name, dom = max(groups.items(), key=lambda kv: kv[1]["ms"])
-    bound, peak = PEAKS[variant]
-    achieved = dom["ops"] / (dom["ms"] * 1e-3) / 1e12
-    roofline = {
-        "bound": bound, "achieved": round(achieved, 2), "peak": round(peak, 1), "unit": "TOP/s",
-        "frac": round(achieved / peak, 4), "traffic": None, "kernel": dom_name,
-        "launches_per_step": dom["launches"], "avg_launch_ms": round(dom["ms"] / dom["launches"], 4),
-        "algorithmic_ops_per_launch": dom["ops"] / dom["launches"],
-        "bit_layers_tops": round(sum(g["ops"] for g in groups.values()) /
-                                 (sum(g["ms"] for g in groups.values()) * 1e-3) / 1e12, 2),
-    }
+        name = layer.kernel_name() if hasattr(layer, "kernel_name") else \
+            {"inconv": "inconv_tiled_kernel", "in": "pack_rows_kernel", "out": "bgemm (output layer)"}[L["kind"]]
+        w = layer_work(L, spec)
+        g = groups.setdefault(name, dict(bops=0.0, bytes=0.0, ms=0.0, launches=0))
+        g["bops"] += w["bops"]
+        g["bytes"] += w["bytes"]
+        g["ms"] += layer_ms[L["name"]]
+        g["launches"] += 1
+    by_time = sorted(groups.items(), key=lambda kv: -kv[1]["ms"])
+    roofline = roofline_of(by_time[0][0], by_time[0][1], variant)
+    roofline_all = [roofline_of(n, g, variant) for n, g in by_time]
+    bit = [g for n, g in groups.items() if g["bops"] > 0]
+    bit_layers_tops = round(sum(g["bops"] for g in bit) / (sum(g["ms"] for g in bit) * 1e-3) / 1e12, 2)
 
     if args.layers:
-        sys.stderr.write("%-8s %-34s %10s %10s\n" % ("layer", "kernel", "ms", "TOP/s"))
+        sys.stderr.write("%-8s %-34s %10s %10s %9s\n" % ("layer", "kernel", "ms", "TOP/s", "GB/s"))
         for L, layer in zip(spec, net.order):
             ops = nets.binary_ops([L])[0]
             kn = layer.kernel_name() if hasattr(layer, "kernel_name") else L["kind"]
+            byts = layer_work(L, spec)["bytes"]
             ms = layer_ms[L["name"]]
-            sys.stderr.write("%-8s %-34s %10.4f %10.1f\n" % (L["name"], kn, ms, ops / (ms * 1e-3) / 1e12))
+            sys.stderr.write("%-8s %-34s %10.4f %10.1f %9.0f\n" % (L["name"], kn, ms, ops / (ms * 1e-3) / 1e12,
+                                                                   byts / (ms * 1e-3) / 1e9))
         sys.stderr.write("sum of layers: %.4f ms; step: %.4f ms\n" % (sum(layer_ms.values()), ms_per_step))
 
     # ------------------------------------------------------------------ CPU baseline (bounded sample)
@@ -173,6 +235,8 @@ def main():
         "binary_ops_per_step": bops, "fp32_first_layer_flops_per_step": flops,
         "roofline": roofline,
         "cpu_baseline": cpu,
+        "bit_layers_binary_tops": bit_layers_tops,
+        "roofline_all_kernels": roofline_all,
     }
     net.release()
     print(json.dumps(out))
