@@ -32,19 +32,31 @@ using namespace mfma;
 
 constexpr int kWaves = 4;
 constexpr int kThreads = 64 * kWaves;
-constexpr int NT = 2;  // 32-channel tiles per wave
+
+// Residual mode of an instantiation.
+constexpr int RM_NONE = 0;    // threshold only
+constexpr int RM_PLAIN = 1;   // residual injected from a source of the same size and / or saved
+constexpr int RM_POOLED = 2;  // residual injected as the 2x2 max of a source twice the size
+
+// Waves per SIMD the register allocator is asked to make room for: the residual layers are
+// bound by HBM and want more memory requests in flight, the plain layers want registers.
+constexpr int waves_hint(int spt, int rm, int nt) { return rm == RM_PLAIN && spt * nt <= 2 ? 3 : 2; }
 
 // SPT = k-steps (64 bits) per filter tap = Cin / 64; MT = 32-image tiles per wave (2 for plain
-// layers; 1 for residual layers, whose int32 traffic wants more waves per SIMD in flight)
-template <int SPT, int MM, int MT>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) void
+// layers, 1 for residual layers); NT = 32-channel tiles per wave.
+template <int SPT, int RM, int MT, int NT>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(waves_hint(SPT, RM, NT)))) void
 conv3x3_mfma_f4_kernel(
     const BgemmParams p, const uint32_t* __restrict__ act, const uint32_t* __restrict__ wgt,
-    const float* __restrict__ bnp, const int32_t* __restrict__ rin, int n_groups, int b_groups,
-    int pix_streams) {
-    constexpr int TPC = SPT == 8 ? 1 : (SPT == 4 ? 3 : 9);  // taps per prefetch chunk
+    const float* __restrict__ bnp, const int32_t* __restrict__ rin, int32_t* __restrict__ rout, int res_lim,
+    int n_groups, int b_groups, int pix_streams) {
+    static_assert(RM == RM_NONE || MT == 1, "residual instantiations own one image tile per wave");
+    constexpr int TPC = SPT >= 4 ? 3 : 9;  // taps per prefetch chunk (a filter row, or all of it)
     constexpr int NCH = 9 / TPC;           // chunks per tile
     constexpr int NQ = 9 * SPT;            // k-steps per tile
+    // A tile of one chunk is shorter than the memory latency: its residual operand is then
+    // requested a whole tile ahead (double-buffered); otherwise with the tile's first chunk.
+    constexpr bool kAhead = RM != RM_NONE && NCH == 1;
     extern __shared__ v4i lds_dyn[];
     v4i* lds_w = lds_dyn;  // [NQ][NT][64] fragments
     float* lds_thr = reinterpret_cast<float*>(lds_dyn + NQ * NT * 64);  // [NT*32]
@@ -141,43 +153,66 @@ conv3x3_mfma_f4_kernel(
         }
     };
 
-    // Residual operand of the tile at pixel (yy, xx), requested before the tile's last chunk is
-    // multiplied so that the loads fly under the MFMAs (kernel.cuh:770-794).
-    int rv[MM == MM_THRESH_RES ? MT : 1][NT][16];
-    auto load_residual = [&](int yy, int xx) {
-        if constexpr (MM == MM_THRESH_RES) {
-            const size_t pix = (size_t)yy * p.PW + xx;
+    // ---- residual operand (kernel.cuh:770-794).  A lane owns channels n0 + 32 nt + 16 h + v of
+    // image bload[0]; every load is a wave-uniform base plus this per-lane element offset.
+    constexpr int NRV = RM != RM_NONE ? NT : 1;
+    constexpr int NTMP = RM == RM_POOLED ? 3 : 1;
+    int tmp[NTMP][NRV][16];  // pooled: the other three pixels of the 2x2 window
+    const unsigned lane_off = (unsigned)(16 * h) * (unsigned)p.B + (unsigned)bload[0];
+
+    auto request_residual = [&](int yy, int xx, int (*rv)[16]) {
+        if constexpr (RM != RM_NONE) {
+            const size_t ch_b = (size_t)p.res_in_ch * p.B;
+            const size_t pix = RM == RM_POOLED ? ((size_t)(2 * yy) * (2 * p.PW) + 2 * xx) : ((size_t)yy * p.PW + xx);
+            const size_t ddy = (size_t)(2 * p.PW) * ch_b;
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt)
+            for (int nt = 0; nt < NT; ++nt) {
+                const int cb = n0 + nt * 32;
+                const int32_t* __restrict__ base = rin + pix * ch_b + (size_t)cb * p.B;  // wave-uniform
+                if (cb + 32 <= res_lim) {
 #pragma unroll
                     for (int v = 0; v < 16; ++v) {
-                        const int c = n0 + nt * 32 + 16 * h + v;
-                        const int bb = bload[mt];
-                        int val = 0;
-                        if (rin != nullptr && c < p.res_limit && c < p.res_in_ch && c < p.N) {
-                            if (p.res_pool) {
-                                const size_t rw2 = 2 * (size_t)p.PW;
-                                const int32_t* s00 =
-                                    rin + (((size_t)(2 * yy) * rw2 + 2 * xx) * p.res_in_ch + c) * p.B + bb;
-                                const size_t ddx = (size_t)p.res_in_ch * p.B, ddy = rw2 * ddx;
-                                val = max(max(s00[0], s00[ddx]), max(s00[ddy], s00[ddy + ddx]));
-                            } else {
-                                val = rin[(pix * p.res_in_ch + c) * p.B + bb];
-                            }
+                        const int32_t* s = base + (size_t)v * p.B;
+                        rv[nt][v] = s[lane_off];
+                        if constexpr (RM == RM_POOLED) {
+                            tmp[0][nt][v] = s[ch_b + lane_off];
+                            tmp[1][nt][v] = s[ddy + lane_off];
+                            tmp[2][nt][v] = s[ddy + ch_b + lane_off];
                         }
-                        rv[mt][nt][v] = val;
                     }
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const bool ok = cb + 16 * h + v < res_lim;
+                        const int32_t* s = base + (size_t)v * p.B;
+                        rv[nt][v] = ok ? s[lane_off] : 0;
+                        if constexpr (RM == RM_POOLED) {
+                            tmp[0][nt][v] = ok ? s[ch_b + lane_off] : 0;
+                            tmp[1][nt][v] = ok ? s[ddy + lane_off] : 0;
+                            tmp[2][nt][v] = ok ? s[ddy + ch_b + lane_off] : 0;
+                        }
+                    }
+                }
+            }
+        }
+    };
+    auto reduce_residual = [&](int (*rv)[16]) {
+        if constexpr (RM == RM_POOLED) {
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    rv[nt][v] = max(max(rv[nt][v], tmp[0][nt][v]), max(tmp[1][nt][v], tmp[2][nt][v]));
         }
     };
 
-    auto epilogue = [&](int yy, int xx) {
+    auto epilogue = [&](int yy, int xx, int (*rv)[16]) {
         const size_t pix = (size_t)yy * p.PW + xx;
         uint32_t* dst_bits = p.out_bits + pix * p.bits_pix_stride;
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
             const int cbase = n0 + nt * 32 + 16 * h;  // this lane's channels: cbase + v
+            const bool n_full = n0 + nt * 32 + 32 <= p.N;  // wave-uniform
             float thr[16];
             {
                 const float4* t4 = reinterpret_cast<const float4*>(lds_thr + nt * 32 + 16 * h);
@@ -195,21 +230,33 @@ conv3x3_mfma_f4_kernel(
                 const int b = bimg[mt];
                 const bool b_ok = b < p.B;
                 uint32_t hw = 0;
-                if constexpr (MM == MM_THRESH_RES) {
-                    int32_t* __restrict__ rout = p.res_out;
+                if constexpr (RM != RM_NONE) {
+                    int res[16];
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) res[v] = (int)acc[mt][nt][v] + rv[nt][v];
+                    if (rout != nullptr && b_ok) {
+                        int32_t* __restrict__ dst = rout + (pix * p.N + n0 + nt * 32) * p.B;  // wave-uniform
+                        const unsigned off = (unsigned)(16 * h) * (unsigned)p.B + (unsigned)b;
+                        if (n_full) {
+#pragma unroll
+                            for (int v = 0; v < 16; ++v) (dst + (size_t)v * p.B)[off] = res[v];
+                        } else {
+#pragma unroll
+                            for (int v = 0; v < 16; ++v)
+                                if (cbase + v < p.N) (dst + (size_t)v * p.B)[off] = res[v];
+                        }
+                    }
 #pragma unroll
                     for (int v = 0; v < 16; ++v) {
-                        const int c = cbase + v;
-                        const int res = (int)acc[mt][nt][v] + rv[mt][nt][v];
-                        if (rout != nullptr && b_ok && c < p.N) rout[(pix * p.N + c) * p.B + b] = res;
-                        const uint32_t bit = (c < p.N && !((float)res < thr[v])) ? 1u : 0u;
+                        const uint32_t bit = ((n_full || cbase + v < p.N) && !((float)res[v] < thr[v])) ? 1u : 0u;
                         hw = hw + hw + bit;
                     }
                 } else {
 #pragma unroll
                     for (int v = 0; v < 16; ++v) {
                         // the accumulator is the exact integer sum: compare it directly
-                        const uint32_t bit = (cbase + v < p.N && !(acc[mt][nt][v] < thr[v])) ? 1u : 0u;
+                        const uint32_t bit =
+                            ((n_full || cbase + v < p.N) && !(acc[mt][nt][v] < thr[v])) ? 1u : 0u;
                         hw = hw + hw + bit;
                     }
                 }
@@ -229,13 +276,21 @@ conv3x3_mfma_f4_kernel(
 
     // ---- persistent loop over this wave's tiles, chunks double-buffered in registers
     uint32_t buf0[TPC * SPT][MT], buf1[TPC * SPT][MT];
+    int rv0[NRV][16], rv1[kAhead ? NRV : 1][kAhead ? 16 : 1];
     uint32_t m0 = 0, m1 = 0;
     int chunk = 0;
     bool have = pi < npix;
-    if (have) m0 = load_chunk(y, x, 0, buf0);
+    if (have) {
+        m0 = load_chunk(y, x, 0, buf0);
+        if constexpr (kAhead) {
+            request_residual(y, x, rv0);
+            reduce_residual(rv0);
+        }
+    }
     zero_acc();
 
-    auto step = [&](uint32_t (*cur)[MT], uint32_t mcur, uint32_t (*nxt)[MT], uint32_t& mnxt) {
+    auto step = [&](uint32_t (*cur)[MT], uint32_t mcur, uint32_t (*nxt)[MT], uint32_t& mnxt, int (*rcur)[16],
+                    int (*rnxt)[16]) {
         int nchunk = chunk + 1, ny = y, nx = x, npi = pi;
         if (nchunk == NCH) {
             nchunk = 0;
@@ -249,10 +304,18 @@ conv3x3_mfma_f4_kernel(
         }
         const bool nhave = npi < npix;
         if (nhave) mnxt = load_chunk(ny, nx, nchunk, nxt);
-        if (chunk == NCH - 1) load_residual(y, x);
+        if constexpr (kAhead) {
+            if (nhave) request_residual(ny, nx, rnxt);
+        } else if constexpr (RM != RM_NONE) {
+            if (chunk == 0) request_residual(y, x, rcur);
+        }
         compute_chunk(chunk, cur, mcur);
+        if constexpr (kAhead) {
+            if (nhave) reduce_residual(rnxt);
+        }
         if (chunk == NCH - 1) {
-            epilogue(y, x);
+            if constexpr (!kAhead) reduce_residual(rcur);
+            epilogue(y, x, rcur);
             zero_acc();
         }
         chunk = nchunk;
@@ -263,30 +326,39 @@ conv3x3_mfma_f4_kernel(
     };
 
     while (have) {
-        step(buf0, m0, buf1, m1);
-        if (!have) break;
-        step(buf1, m1, buf0, m0);
+        if constexpr (kAhead) {
+            step(buf0, m0, buf1, m1, rv0, rv1);
+            if (!have) break;
+            step(buf1, m1, buf0, m0, rv1, rv0);
+        } else {
+            step(buf0, m0, buf1, m1, rv0, rv0);
+            if (!have) break;
+            step(buf1, m1, buf0, m0, rv0, rv0);
+        }
     }
 }
 
-template <int SPT, int MM, int MT>
+template <int SPT, int RM, int MT, int NT>
 int launch_t(const BgemmParams& p, hipStream_t stream) {
     constexpr int NQ = 9 * SPT;
     const size_t lds_bytes = (size_t)NQ * NT * 64 * 16 + NT * 32 * sizeof(float);
     static bool attr_set = false;  // per instantiation
     if (!attr_set) {
-        if (int rc = check_hip(hipFuncSetAttribute(reinterpret_cast<const void*>(&conv3x3_mfma_f4_kernel<SPT, MM, MT>),
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes),
-                               "hipFuncSetAttribute(MaxDynamicSharedMemorySize)"))
+        if (int rc = check_hip(
+                hipFuncSetAttribute(reinterpret_cast<const void*>(&conv3x3_mfma_f4_kernel<SPT, RM, MT, NT>),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes),
+                "hipFuncSetAttribute(MaxDynamicSharedMemorySize)"))
             return rc;
         attr_set = true;
     }
     const int n_groups = (p.N + 32 * NT - 1) / (32 * NT);
     const int b_groups = (p.B + 32 * MT - 1) / (32 * MT);
     const int quads = (p.PH * p.PW + kWaves - 1) / kWaves;  // pixel quads (one pixel per wave)
-    // about two (plain) or three (residual) workgroups per CU, with the pixel quads spread as
-    // evenly as possible
-    const int target = std::max(1, (MT == 1 ? 768 : 512) / (n_groups * b_groups));
+    // as many workgroups as are resident at once (two per CU for plain layers, three for residual
+    // layers, fewer when their LDS does not fit), so that the weights are staged once per CU
+    // slot, with the pixel quads spread as evenly as possible
+    const int wg_per_cu = std::max(1, std::min(MT == 1 ? 3 : 2, (int)(160 * 1024 / lds_bytes)));
+    const int target = std::max(1, 256 * wg_per_cu / (n_groups * b_groups));
     int best = std::min(target, quads);
     double best_waste = 1e30;
     for (int ps = std::max(1, target / 2); ps <= std::min(quads, target * 2); ++ps) {
@@ -297,17 +369,43 @@ int launch_t(const BgemmParams& p, hipStream_t stream) {
             best = ps;
         }
     }
+    // channels that receive an injected residual: o < residual_channels, and only those the
+    // source tensor holds (kernel.cuh:770)
+    const int res_lim = p.res_in != nullptr ? std::min(std::min(p.res_limit, p.res_in_ch), p.N) : 0;
     const long long blocks = (long long)best * n_groups * b_groups;
-    hipLaunchKernelGGL((conv3x3_mfma_f4_kernel<SPT, MM, MT>), dim3((unsigned)blocks), dim3(kThreads), lds_bytes,
-                       stream, p, p.act, p.wgt, p.bn, p.res_in, n_groups, b_groups, best);
+    hipLaunchKernelGGL((conv3x3_mfma_f4_kernel<SPT, RM, MT, NT>), dim3((unsigned)blocks), dim3(kThreads), lds_bytes,
+                       stream, p, p.act, p.wgt, p.bn, p.res_in, p.res_out, res_lim, n_groups, b_groups, best);
     TCBNN_LAUNCH_CHECK("conv3x3_mfma_f4_kernel");
     return TCBNN_OK;
 }
 
+// Which instantiation serves a layer.  Measured on ResNet-18 at batch 256: the HBM-bound residual
+// layers run best with one image tile per wave and, from Cin = 256 on, one channel tile (more
+// workgroups fit a CU's LDS, so more residual requests are in flight); plain layers want the 2 x 2
+// tile (each operand fragment feeds two MFMAs) until the weights of 64 channels no longer leave
+// room for a second workgroup (Cin = 512).
+struct Pick {
+    int rm, mt, nt;
+};
+constexpr int pick_nt(int spt, int rm) {
+    return rm == RM_POOLED ? 1 : (rm == RM_PLAIN ? (spt >= 4 ? 1 : 2) : (spt >= 8 ? 1 : 2));
+}
+Pick pick(const BgemmParams& p) {
+    const int rm = p.res_in == nullptr && p.res_out == nullptr ? RM_NONE
+                                                                : (p.res_in != nullptr && p.res_pool ? RM_POOLED : RM_PLAIN);
+    return {rm, rm == RM_NONE ? 2 : 1, pick_nt(p.cw / 2, rm)};
+}
+
 template <int SPT>
 int launch_m(const BgemmParams& p, hipStream_t stream) {
-    if (p.res_in != nullptr || p.res_out != nullptr) return launch_t<SPT, MM_THRESH_RES, 1>(p, stream);
-    return launch_t<SPT, MM_THRESH, 2>(p, stream);
+    switch (pick(p).rm) {
+        case RM_NONE:
+            return launch_t<SPT, RM_NONE, 2, pick_nt(SPT, RM_NONE)>(p, stream);
+        case RM_PLAIN:
+            return launch_t<SPT, RM_PLAIN, 1, pick_nt(SPT, RM_PLAIN)>(p, stream);
+        default:
+            return launch_t<SPT, RM_POOLED, 1, pick_nt(SPT, RM_POOLED)>(p, stream);
+    }
 }
 
 }  // namespace
@@ -319,9 +417,8 @@ bool conv3x3_mfma_applicable(const BgemmParams& p) {
 }
 
 void conv3x3_mfma_kernel_name(const BgemmParams& p, char* buf, size_t len) {
-    const bool res = p.res_in != nullptr || p.res_out != nullptr;
-    snprintf(buf, len, "conv3x3_mfma_f4_kernel<%d, %d, %d>", p.cw / 2, res ? MM_THRESH_RES : MM_THRESH,
-             res ? 1 : 2);
+    const Pick k = pick(p);
+    snprintf(buf, len, "conv3x3_mfma_f4_kernel<%d, %d, %d, %d>", p.cw / 2, k.rm, k.mt, k.nt);
 }
 
 int launch_conv3x3_mfma(const BgemmParams& p, hipStream_t stream) {

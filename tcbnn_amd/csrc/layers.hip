@@ -253,6 +253,7 @@ int tcbnn_conv128_kernel_name(const tcbnn_conv128_desc* d, char* buf, size_t len
     p.k_tap = d->input_channels;
     p.stride_h = d->stride_height;
     p.stride_w = d->stride_width;
+    p.res_pool = d->residual_pool;
     // only nullness matters for the name
     p.res_in = d->inject_residual ? reinterpret_cast<const int32_t*>(d) : nullptr;
     p.res_out = d->save_residual ? reinterpret_cast<int32_t*>(const_cast<tcbnn_conv128_desc*>(d)) : nullptr;
