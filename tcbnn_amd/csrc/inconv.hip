@@ -9,7 +9,8 @@
 //
 // Two kernels:
 //   inconv_tiled_kernel (pool 1x1): workgroup = one output row y, 4 consecutive output
-//     columns (one per wave), 64 images (lane = image).  For each filter row the needed
+//     columns, 64 images (lane = image); a wave owns two of the columns and 32 of the 64 output
+//     channels of a pass.  For each filter row the needed
 //     input row segment of the 64 images is read with lanes running along the image row
 //     (contiguous runs) and transposed through LDS to image-innermost order, so the
 //     compute phase reads LDS without bank conflicts, the filter sign masks are
@@ -43,18 +44,19 @@ __device__ __forceinline__ float flip(float f, uint32_t m) {
     return __uint_as_float(__float_as_uint(f) ^ m);
 }
 
-typedef float v16f __attribute__((ext_vector_type(16)));
+typedef float v8f __attribute__((ext_vector_type(8)));
 
 // The eight possible values of ((+-f0) + (+-f1)) + (+-f2), indexed by the sign pattern
 // 4*neg0 + 2*neg1 + neg2.  With t = f0 + f1 and u = f0 - f1 (round-to-nearest is symmetric
 // under negation, so (-f0) + f1 == -(f0 - f1) bit for bit, up to the sign of a zero):
 //   0: t + f2   1: t - f2   2: u + f2   3: u - f2   4: -(u - f2)   5: -(u + f2)   6: -(t - f2)   7: -(t + f2)
 // A filter tap then costs 6 adds + 4 negations per lane once, and each output channel one
-// register-indexed move (the pattern is wave-uniform) plus one add, instead of 3 sign flips
-// and 3 adds.  16 elements (8 unused) make the compiler select VGPR index mode for c[idx].
-__device__ __forceinline__ v16f sign_combos(float f0, float f1, float f2) {
+// register-indexed add (the pattern is wave-uniform), instead of 3 sign flips and 3 adds.
+// A tap outside the frame reads zeros from the staged tile: all eight values are then +-0, and
+// adding them leaves every accumulator as it was, which is the reference's "skip the tap".
+__device__ __forceinline__ v8f sign_combos(float f0, float f1, float f2) {
     const float t = f0 + f1, u = f0 - f1;
-    v16f c;
+    v8f c;
     c[0] = t + f2;
     c[1] = t - f2;
     c[2] = u + f2;
@@ -63,43 +65,51 @@ __device__ __forceinline__ v16f sign_combos(float f0, float f1, float f2) {
     c[5] = -c[2];
     c[6] = -c[1];
     c[7] = -c[0];
-#pragma unroll
-    for (int i = 8; i < 16; ++i) c[i] = 0.0f;
     return c;
 }
 
-typedef float v8f __attribute__((ext_vector_type(8)));
-
-// acc[k] += c[idx_k] for 8 output channels with ONE switch into VGPR-index mode: the combo
-// vector is pinned to v[120:127], source 0 of each v_add_f32 is v120 displaced by the index in
-// M0 (s_set_gpr_idx_idx only rewrites that index, it does not touch the MODE register).
-// Wait states between a write of the index (M0) and the VALU instruction that uses it.  The
-// hardware does not interlock this pair: without them an add occasionally used the previous
-// index (seen as rare wrong sums when few waves share a SIMD).
+// a[k] += ca[idx_k] and b[k] += cb[idx_k] for 8 output channels of two pixels with ONE switch
+// into VGPR-index mode and one index write per channel: the combination vectors are pinned to
+// v[120:127] and v[112:119], source 0 of each v_add_f32 is that base displaced by the index in
+// M0 (s_set_gpr_idx_idx only rewrites the index, it does not touch the MODE register).  The
+// scalar unit issues one instruction per cycle for the whole CU, so an index write per add
+// would hold the four SIMDs back; shared by the two pixels it does not.
+// Wait states between a write of the index (M0) and the VALU instruction that uses it: the
+// hardware does not interlock this pair.  Without them an add can use a stale M0, i.e. a
+// register far outside v[112:127].  Never remove them.
 #define IDX_WAIT "s_nop 1\n\t"
-__device__ __forceinline__ void add_indexed8(float* acc, v8f c, int i0, int i1, int i2, int i3, int i4,
-                                             int i5, int i6, int i7) {
+__device__ __forceinline__ void add_indexed8x2(float* a, float* b, v8f ca, v8f cb, int i0, int i1, int i2, int i3,
+                                               int i4, int i5, int i6, int i7) {
     asm volatile(
-        "s_set_gpr_idx_on %8, gpr_idx(SRC0)\n\t" IDX_WAIT
+        "s_set_gpr_idx_on %16, gpr_idx(SRC0)\n\t" IDX_WAIT
         "v_add_f32_e32 %0, v120, %0\n\t"
-        "s_set_gpr_idx_idx %9\n\t" IDX_WAIT
+        "v_add_f32_e32 %8, v112, %8\n\t"
+        "s_set_gpr_idx_idx %17\n\t" IDX_WAIT
         "v_add_f32_e32 %1, v120, %1\n\t"
-        "s_set_gpr_idx_idx %10\n\t" IDX_WAIT
+        "v_add_f32_e32 %9, v112, %9\n\t"
+        "s_set_gpr_idx_idx %18\n\t" IDX_WAIT
         "v_add_f32_e32 %2, v120, %2\n\t"
-        "s_set_gpr_idx_idx %11\n\t" IDX_WAIT
+        "v_add_f32_e32 %10, v112, %10\n\t"
+        "s_set_gpr_idx_idx %19\n\t" IDX_WAIT
         "v_add_f32_e32 %3, v120, %3\n\t"
-        "s_set_gpr_idx_idx %12\n\t" IDX_WAIT
+        "v_add_f32_e32 %11, v112, %11\n\t"
+        "s_set_gpr_idx_idx %20\n\t" IDX_WAIT
         "v_add_f32_e32 %4, v120, %4\n\t"
-        "s_set_gpr_idx_idx %13\n\t" IDX_WAIT
+        "v_add_f32_e32 %12, v112, %12\n\t"
+        "s_set_gpr_idx_idx %21\n\t" IDX_WAIT
         "v_add_f32_e32 %5, v120, %5\n\t"
-        "s_set_gpr_idx_idx %14\n\t" IDX_WAIT
+        "v_add_f32_e32 %13, v112, %13\n\t"
+        "s_set_gpr_idx_idx %22\n\t" IDX_WAIT
         "v_add_f32_e32 %6, v120, %6\n\t"
-        "s_set_gpr_idx_idx %15\n\t" IDX_WAIT
+        "v_add_f32_e32 %14, v112, %14\n\t"
+        "s_set_gpr_idx_idx %23\n\t" IDX_WAIT
         "v_add_f32_e32 %7, v120, %7\n\t"
+        "v_add_f32_e32 %15, v112, %15\n\t"
         "s_set_gpr_idx_off"
-        : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]), "+v"(acc[4]), "+v"(acc[5]), "+v"(acc[6]),
-          "+v"(acc[7])
-        : "s"(i0), "s"(i1), "s"(i2), "s"(i3), "s"(i4), "s"(i5), "s"(i6), "s"(i7), "{v[120:127]}"(c)
+        : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(a[4]), "+v"(a[5]), "+v"(a[6]), "+v"(a[7]),
+          "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]), "+v"(b[4]), "+v"(b[5]), "+v"(b[6]), "+v"(b[7])
+        : "s"(i0), "s"(i1), "s"(i2), "s"(i3), "s"(i4), "s"(i5), "s"(i6), "s"(i7), "{v[120:127]}"(ca),
+          "{v[112:119]}"(cb)
         : "m0");
 }
 
@@ -107,12 +117,18 @@ __device__ __forceinline__ void add_indexed8(float* acc, v8f c, int i0, int i1, 
 // wave-uniform mask / threshold loads become scalar loads (s_load) feeding v_xor directly.
 typedef uint32_t u16v __attribute__((ext_vector_type(16)));
 
-// NST = floats each thread stages per filter row = ceil(3 * 64 * ncols / 256)
-template <int NST>
+// Staging of one filter row: the 3 x 64 (channel, image) row segments of ncols floats each.
+//   ROWS = true (ncols <= 21): a wave takes rpw (a multiple of 3) segments at a time, lanes
+//     running along the segment; segments are numbered in memory order (image * 3 + channel),
+//     so that the address of pass k is a wave-uniform base plus a per-lane constant and the
+//     LDS slot a constant plus an immediate: no per-element address arithmetic.  NST = passes =
+//     ceil(192 / (4 rpw)).
+//   ROWS = false: the elements are dealt to the threads linearly, NST = ceil(3 * 64 * ncols / 256).
+template <int NST, bool ROWS>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3))) void inconv_tiled_kernel(
     const InConvParams p, const float* __restrict__ in, const uint4* __restrict__ masks,
     const float* __restrict__ bn, uint32_t* __restrict__ out, int32_t* __restrict__ res, int b_tiles,
-    int x_groups, int y_phases, int div_magic) {
+    int x_groups, int y_phases, int div_magic, int rpw) {
     __shared__ float tile[3 * kMaxCols * kLB];
 
     const int tid = threadIdx.x;
@@ -135,8 +151,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3))) v
         y = blockIdx.x / (b_tiles * x_groups);
     }
     const int x0 = xg * kXT;
-    const int x = x0 + wave;
-    const bool x_ok = x < p.PW;  // wave-uniform
+    const int pp = wave & 1;    // which pair of the workgroup's four columns
+    const int chh = wave >> 1;  // which 32 of the pass's 64 channels
+    const int xa = x0 + 2 * pp, xb = xa + 1;
+    const bool xa_ok = xa < p.PW, xb_ok = xb < p.PW;  // wave-uniform
     const int b0 = bt * 64;
     const int b = b0 + lane;
     const int ncols = (kXT - 1) * p.stride_w + p.S;
@@ -147,10 +165,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3))) v
         reinterpret_cast<const uint32_t*>(masks) + (size_t)p.R * p.S * p.opad * 4;  // packed pattern table
 
     for (int g = 0; g < n_groups; ++g) {
-        float acc[64];
+        float acca[32], accb[32];  // this wave's 32 channels of pixels xa and xb
 #pragma unroll
-        for (int n = 0; n < 64; ++n) acc[n] = 0.0f;
-        const bool second_half = g * 64 + 32 < p.opad;  // uniform
+        for (int n = 0; n < 32; ++n) acca[n] = accb[n] = 0.0f;
+        const int wi = g * 2 + chh;                       // output word = channel tile of this wave
+        const bool work = xa_ok && wi * 32 < p.opad;      // uniform
 
         // Filter rows inside the frame: r_lo <= r < r_hi (uniform for the whole workgroup).
         const int ay0 = y * p.stride_h - p.pad_h;
@@ -162,27 +181,75 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3))) v
         // Lanes run along the image row (contiguous runs of ncols floats per (channel, image)),
         // LDS is image-innermost; e / ncols by multiply-shift (the host checked the constant).
         float stg[NST];
+        // ROWS scheme: per-lane constants
+        const int rp = 4 * rpw;                      // segments per pass of the workgroup
+        const int sub = lane / ncols;                // segment of the wave's rpw this lane reads
+        const int scol = lane - sub * ncols;         // column in the segment
+        const int seg0 = wave * rpw + sub;           // segment (image * 3 + channel) in pass 0
+        const int sax = ax_base + scol;
+        const bool lane_ok = sub < rpw && sax >= 0 && sax < p.W;  // constant over passes and rows
+        // Buffer addressing: descriptor = this workgroup's 64 images, per-lane byte offset (one
+        // constant), wave-uniform scalar offset per (row, pass).  A lane outside the frame carries an
+        // offset beyond the descriptor's range: the hardware returns 0 for it without touching memory.
+        constexpr unsigned kOutOfRange = 0x80000000u;
+        const unsigned imgs_here = (unsigned)min(64, p.B - b0);
+        const unsigned tile_bytes = imgs_here * 3u * (unsigned)plane * 4u;  // host checked: below 2 GiB
+        const unsigned voff = lane_ok ? ((unsigned)seg0 * (unsigned)plane + (unsigned)sax) * 4u : kOutOfRange;
+        const int lds0 = ((seg0 % 3) * ncols + scol) * kLB + seg0 / 3;
+        // every pass of every lane inside the 192 segments and the batch (wave-uniform)?
+        const bool all_in = NST * rp == 3 * 64 && b0 + 64 <= p.B;
+        __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<float*>(in + (size_t)b0 * 3 * plane), 0, (int)tile_bytes, 0x00020000);
         auto fetch_row = [&](int r) {
-            const size_t row_off = (size_t)(ay0 + r) * p.W;
+            if constexpr (ROWS) {
+                const unsigned row_bytes = (unsigned)(ay0 + r) * (unsigned)p.W * 4u;       // uniform
+                const unsigned pass_bytes = (unsigned)rp * (unsigned)plane * 4u;           // uniform
+                if (all_in) {
 #pragma unroll
-            for (int k = 0; k < NST; ++k) {
-                const int e = tid + k * kThreads;
-                const int bc = (int)(((unsigned)e * (unsigned)div_magic) >> 16);
-                const int col = e - bc * ncols;
-                const int ax = ax_base + col;
-                const int bb = min(b0 + (bc & 63), p.B - 1);
-                float v = 0.0f;
-                if (e < n_stage && ax >= 0 && ax < p.W) v = in[((size_t)bb * 3 + (bc >> 6)) * plane + row_off + ax];
-                stg[k] = v;
+                    for (int k = 0; k < NST; ++k)
+                        stg[k] = __builtin_bit_cast(
+                            float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)voff, (int)(row_bytes + k * pass_bytes), 0));
+                } else {
+#pragma unroll
+                    for (int k = 0; k < NST; ++k) {
+                        const int seg = seg0 + k * rp;
+                        const bool ok = seg < 3 * 64 && b0 + seg / 3 < p.B;
+                        stg[k] = __builtin_bit_cast(
+                            float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)(ok ? voff : kOutOfRange),
+                                                                        (int)(row_bytes + k * pass_bytes), 0));
+                    }
+                }
+            } else {
+                const size_t row_off = (size_t)(ay0 + r) * p.W;
+#pragma unroll
+                for (int k = 0; k < NST; ++k) {
+                    const int e = tid + k * kThreads;
+                    const int bc = (int)(((unsigned)e * (unsigned)div_magic) >> 16);
+                    const int col = e - bc * ncols;
+                    const int ax = ax_base + col;
+                    const int bb = min(b0 + (bc & 63), p.B - 1);
+                    float v = 0.0f;
+                    if (e < n_stage && ax >= 0 && ax < p.W)
+                        v = in[((size_t)bb * 3 + (bc >> 6)) * plane + row_off + ax];
+                    stg[k] = v;
+                }
             }
         };
         auto store_row = [&]() {
+            if constexpr (ROWS) {
+                if (sub < rpw) {
 #pragma unroll
-            for (int k = 0; k < NST; ++k) {
-                const int e = tid + k * kThreads;
-                const int bc = (int)(((unsigned)e * (unsigned)div_magic) >> 16);
-                const int col = e - bc * ncols;
-                if (e < n_stage) tile[((bc >> 6) * ncols + col) * kLB + (bc & 63)] = stg[k];
+                    for (int k = 0; k < NST; ++k)
+                        if (all_in || seg0 + k * rp < 3 * 64) tile[lds0 + k * (rp / 3)] = stg[k];
+                }
+            } else {
+#pragma unroll
+                for (int k = 0; k < NST; ++k) {
+                    const int e = tid + k * kThreads;
+                    const int bc = (int)(((unsigned)e * (unsigned)div_magic) >> 16);
+                    const int col = e - bc * ncols;
+                    if (e < n_stage) tile[((bc >> 6) * ncols + col) * kLB + (bc & 63)] = stg[k];
+                }
             }
         };
 
@@ -192,46 +259,38 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3))) v
             store_row();
             __syncthreads();
             if (r + 1 < r_hi) fetch_row(r + 1);
-            if (!x_ok) continue;
+            if (!work) continue;
             for (int s = 0; s < p.S; ++s) {
-                const int col = wave * p.stride_w + s;
-                const int ax = ax_base + col;
-                if (ax < 0 || ax >= p.W) continue;  // wave-uniform
-                // sign patterns of this tap's channels, one per word (wide scalar loads)
-                const u16v* pw = reinterpret_cast<const u16v*>(pats + (size_t)(r * p.S + s) * p.opad + g * 64);
+                const int cola = 2 * pp * p.stride_w + s, colb = cola + p.stride_w;
+                // sign patterns of this tap's 32 channels, one per word (wide scalar loads)
+                const u16v* pw = reinterpret_cast<const u16v*>(pats + (size_t)(r * p.S + s) * p.opad + wi * 32);
                 const u16v i0 = pw[0], i1 = pw[1];
-                const float f0 = tile[(0 * ncols + col) * kLB + lane];
-                const float f1 = tile[(1 * ncols + col) * kLB + lane];
-                const float f2 = tile[(2 * ncols + col) * kLB + lane];
-                const v16f c16 = sign_combos(f0, f1, f2);
-                const v8f c = {c16[0], c16[1], c16[2], c16[3], c16[4], c16[5], c16[6], c16[7]};
-                add_indexed8(&acc[0], c, i0[0], i0[1], i0[2], i0[3], i0[4], i0[5], i0[6], i0[7]);
-                add_indexed8(&acc[8], c, i0[8], i0[9], i0[10], i0[11], i0[12], i0[13], i0[14], i0[15]);
-                add_indexed8(&acc[16], c, i1[0], i1[1], i1[2], i1[3], i1[4], i1[5], i1[6], i1[7]);
-                add_indexed8(&acc[24], c, i1[8], i1[9], i1[10], i1[11], i1[12], i1[13], i1[14], i1[15]);
-                if (second_half) {
-                    const u16v i2 = pw[2], i3 = pw[3];
-                    add_indexed8(&acc[32], c, i2[0], i2[1], i2[2], i2[3], i2[4], i2[5], i2[6], i2[7]);
-                    add_indexed8(&acc[40], c, i2[8], i2[9], i2[10], i2[11], i2[12], i2[13], i2[14], i2[15]);
-                    add_indexed8(&acc[48], c, i3[0], i3[1], i3[2], i3[3], i3[4], i3[5], i3[6], i3[7]);
-                    add_indexed8(&acc[56], c, i3[8], i3[9], i3[10], i3[11], i3[12], i3[13], i3[14], i3[15]);
-                }
+                const v8f ca = sign_combos(tile[(0 * ncols + cola) * kLB + lane], tile[(1 * ncols + cola) * kLB + lane],
+                                           tile[(2 * ncols + cola) * kLB + lane]);
+                const v8f cb = sign_combos(tile[(0 * ncols + colb) * kLB + lane], tile[(1 * ncols + colb) * kLB + lane],
+                                           tile[(2 * ncols + colb) * kLB + lane]);
+                add_indexed8x2(&acca[0], &accb[0], ca, cb, i0[0], i0[1], i0[2], i0[3], i0[4], i0[5], i0[6], i0[7]);
+                add_indexed8x2(&acca[8], &accb[8], ca, cb, i0[8], i0[9], i0[10], i0[11], i0[12], i0[13], i0[14],
+                               i0[15]);
+                add_indexed8x2(&acca[16], &accb[16], ca, cb, i1[0], i1[1], i1[2], i1[3], i1[4], i1[5], i1[6], i1[7]);
+                add_indexed8x2(&acca[24], &accb[24], ca, cb, i1[8], i1[9], i1[10], i1[11], i1[12], i1[13], i1[14],
+                               i1[15]);
             }
         }
 
-        if (x_ok && b < p.B) {
-            const size_t pix = (size_t)y * p.PW + x;
+        if (work && b < p.B && wi < p.ow) {
 #pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                const int wi = g * 2 + h;
-                if (wi >= p.ow) continue;
+            for (int px = 0; px < 2; ++px) {
+                if (px == 1 && !xb_ok) continue;
+                const float* acc = px == 0 ? acca : accb;
+                const size_t pix = (size_t)y * p.PW + xa + px;
                 uint32_t word = 0;
 #pragma unroll
                 for (int n = 0; n < 32; ++n) {
                     const int ch = wi * 32 + n;
                     if (ch < p.O) {
-                        word |= (acc[h * 32 + n] < bn[ch] ? 0u : 1u) << (31 - n);
-                        if (res != nullptr) res[(pix * p.O + ch) * p.B + b] = (int)acc[h * 32 + n];
+                        word |= (acc[n] < bn[ch] ? 0u : 1u) << (31 - n);
+                        if (res != nullptr) res[(pix * p.O + ch) * p.B + b] = (int)acc[n];
                     }
                 }
                 out[(pix * p.ow + wi) * p.B + b] = word;
@@ -361,17 +420,27 @@ extern "C" int tcbnn_inconv128_forward(const tcbnn_inconv128_desc* d, void* stre
                                      ? 8LL * x_groups * ((p.PH + y_phases - 1) / y_phases)
                                      : (long long)b_tiles * x_groups * p.PH;
         TCBNN_REQUIRE(blocks <= 0x7fffffffLL, "inconv128: grid too large");
-        const int nst = (3 * 64 * ncols + kThreads - 1) / kThreads;
+        // staging scheme (see the kernel): whole segments per wave when at least 3 fit its 64 lanes
+        const int rpw = (64 / ncols) / 3 * 3;
         auto launch = [&](auto kernel) {
             hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(kThreads), 0, (hipStream_t)stream, p, p.in,
-                               p.masks, p.bn, p.out, p.res, b_tiles, x_groups, y_phases, div_magic);
+                               p.masks, p.bn, p.out, p.res, b_tiles, x_groups, y_phases, div_magic, rpw);
         };
-        if (nst <= 5)
-            launch(inconv_tiled_kernel<5>);
-        else if (nst <= 15)
-            launch(inconv_tiled_kernel<15>);
-        else
-            launch(inconv_tiled_kernel<24>);
+        if (rpw >= 3 && 64LL * 3 * p.H * p.W * 4 < (1LL << 31)) {
+            const int passes = (3 * 64 + 4 * rpw - 1) / (4 * rpw);
+            if (passes <= 4)
+                launch(inconv_tiled_kernel<4, true>);
+            else if (passes <= 8)
+                launch(inconv_tiled_kernel<8, true>);
+            else
+                launch(inconv_tiled_kernel<16, true>);
+        } else {
+            const int nst = (3 * 64 * ncols + kThreads - 1) / kThreads;
+            if (nst <= 15)
+                launch(inconv_tiled_kernel<15, false>);
+            else
+                launch(inconv_tiled_kernel<24, false>);
+        }
         TCBNN_LAUNCH_CHECK("inconv_tiled_kernel");
         return TCBNN_OK;
     }

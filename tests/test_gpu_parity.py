@@ -241,7 +241,12 @@ def test_conv128_rejects_residual_with_pooling(gpu):
 # --------------------------------------------------------------------------- first layer
 @pytest.mark.parametrize("b,h,R,stride,cout,pool,save", [(8, 32, 3, 1, 128, 1, False), (5, 20, 7, 4, 64, 1, True),
                                                          (70, 12, 3, 1, 32, 2, False), (3, 13, 5, 2, 96, 1, True),
-                                                         (2, 224, 7, 4, 64, 1, True)])
+                                                         (2, 224, 7, 4, 64, 1, True),
+                                                         # staging schemes of the tiled kernel: wide filter (linear
+                                                         # scheme), partial image tiles, whole tiles, odd channel counts
+                                                         (70, 24, 11, 4, 64, 1, True), (66, 20, 7, 4, 40, 1, True),
+                                                         (9, 17, 3, 2, 33, 1, True), (64, 16, 7, 4, 64, 1, True),
+                                                         (128, 10, 3, 1, 64, 1, True)])
 def test_inconv128_layer(gpu, b, h, R, stride, cout, pool, save):
     r = rng(b + h + R + cout)
     x = r.standard_normal((b, 3, h, h)).astype(np.float32)
