@@ -38,10 +38,13 @@ COMPUTE_PEAKS_TOPS = {
 MEASURED_TRAFFIC_BYTES = {}
 
 
-def layer_work(L, spec=()):
+def layer_work(L, spec=(), res_bytes=None):
     """Algorithmic work of one layer launch: binary ops (2 per +-1 multiply-accumulate, border taps
     included), fp32 adds of the first layer, and the HBM bytes the launch has to move once
-    (inputs + outputs + weights, packed activations at 1 bit per value, residuals int32)."""
+    (inputs + outputs + weights, packed activations at 1 bit per value, residuals at the width
+    they are stored in: res_bytes[layer name] = 2 or 4 bytes per value of that layer's saved
+    residual, 4 = the reference's int32 when not given)."""
+    res_bytes = res_bytes or {}
     from tcbnn_amd import nets
     bops, flops = nets.binary_ops([L])
     B = L["batch"]
@@ -56,16 +59,16 @@ def layer_work(L, spec=()):
         if L["kind"] == "inconv":
             byts = B * 3 * L["h"] * L["w"] * 4 + out_bits + L["r"] * L["s"] * 3 * L["cout"] * 4
             if L["save_residual"]:
-                byts += B * oh * ow * L["cout"] * 4
+                byts += B * oh * ow * L["cout"] * res_bytes.get(L["name"], 4)
         else:
             byts = B * L["h"] * L["w"] * L["cin"] / 8 + out_bits + L["r"] * L["s"] * L["cin"] * L["cout"] / 8
             if L["save_residual"]:
-                byts += B * oh * ow * L["cout"] * 4
+                byts += B * oh * ow * L["cout"] * res_bytes.get(L["name"], 4)
             if L["inject_residual"]:
                 # channels actually injected: those the source layer saved, capped by residual_channels
                 src_ch = [S["cout"] for S in spec if S["name"] == L.get("res_src")]
                 ch = min([L["residual_channels"], L["cout"]] + src_ch)
-                byts += B * oh * ow * (4 if L["residual_pool"] else 1) * ch * 4
+                byts += B * oh * ow * (4 if L["residual_pool"] else 1) * ch * res_bytes.get(L.get("res_src"), 4)
     return dict(bops=bops, flops=flops, bytes=float(byts))
 
 
@@ -162,12 +165,15 @@ def main():
             per_layer[L["name"]].append(evs[i].elapsed_ms(evs[i + 1]))
     layer_ms = {k: float(np.median(v)) for k, v in per_layer.items()}
 
+    # width each saved residual is stored in (16 bits where its bound proves that exact)
+    res_bytes = {L["name"]: (2 if net.layers[L["name"]].output_residual_gpu.format == _lib.RES_I16 else 4)
+                 for L in spec if L.get("save_residual")}
     # group launches by device kernel, as a profiler does
     groups = {}
     for L, layer in zip(spec, net.order):
         name = layer.kernel_name() if hasattr(layer, "kernel_name") else \
             {"inconv": "inconv_tiled_kernel", "in": "pack_rows_kernel", "out": "bgemm (output layer)"}[L["kind"]]
-        w = layer_work(L, spec)
+        w = layer_work(L, spec, res_bytes)
         g = groups.setdefault(name, dict(bops=0.0, bytes=0.0, ms=0.0, launches=0))
         g["bops"] += w["bops"]
         g["bytes"] += w["bytes"]
@@ -184,7 +190,7 @@ def main():
         for L, layer in zip(spec, net.order):
             ops = nets.binary_ops([L])[0]
             kn = layer.kernel_name() if hasattr(layer, "kernel_name") else L["kind"]
-            byts = layer_work(L, spec)["bytes"]
+            byts = layer_work(L, spec, res_bytes)["bytes"]
             ms = layer_ms[L["name"]]
             sys.stderr.write("%-8s %-34s %10.4f %10.1f %9.0f\n" % (L["name"], kn, ms, ops / (ms * 1e-3) / 1e12,
                                                                    byts / (ms * 1e-3) / 1e9))
@@ -230,7 +236,10 @@ def main():
                                % (args.net, {"imagenet_resnet": "imagenet_resnet.cu:223-325",
                                              "cifar10_vgg": "cifar10_vgg.cu:162-199",
                                              "mnist_mlp": "mnist_mlp.cu:111-124"}[args.net], batch),
-                   "variant": variant, "layers": len(spec)},
+                   "variant": variant, "layers": len(spec),
+                   "residual_storage": ("int16 where the bound of |residual| proves it exact (%d of %d tensors), "
+                                        "else int32" % (sum(1 for v in res_bytes.values() if v == 2), len(res_bytes)))
+                   if res_bytes else "none"},
         "binary_tops": round(bops * args.steps / wall / 1e12, 2),
         "binary_ops_per_step": bops, "fp32_first_layer_flops_per_step": flops,
         "roofline": roofline,

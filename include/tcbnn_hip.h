@@ -30,7 +30,10 @@
  *   packed weights   : uint32 [NPAD32][KWTOT]     one row per output neuron/channel,
  *                                                 FC: KWTOT = KW128; conv: KWTOT = R*S*CW,
  *                                                 K index = (r*S+s)*32*CW + c; rows >= N are 0
- *   residual tensors : int32  [P][Q][O][B]        true channel count, no 128-padding
+ *   residual tensors : TCBNN_RES_I32: int32 [P][Q][O][B], true channel count, no 128-padding;
+ *                      TCBNN_RES_I16: int16 [P][Q][ceil(O/2)][B][2] (channels 2k and 2k+1 of
+ *                      an image share one 32-bit word, 2k in the low half) for tensors whose
+ *                      values provably fit 16 bits (see "residual formats" below)
  *   fp32 stem input  : float  [B][3][H][W]        (kernel.cuh:620-625)
  * The reference's own tile-contiguous "FMT" layouts ([.../8][.../128][8][4],
  * kernel.cuh:170,222,650-660,798-815) are produced / consumed by the
@@ -59,6 +62,16 @@ extern "C" {
 #define TCBNN_VARIANT_MFMA_I8 2   /* +-1 unpacked to int8, v_mfma_i32_32x32x32_i8 */
 #define TCBNN_VARIANT_MFMA_F4 3   /* +-1 unpacked to FP4 E2M1, v_mfma_f32_32x32x64_f8f6f4 (exact: |sum| < 2^24) */
 
+/* Residual storage formats.  The reference keeps residuals (pre-threshold sums, kernel.cuh:
+ * 662-669, 818-824) as int32.  They are this path's dominant HBM traffic, and their magnitude
+ * is bounded by construction: |first-layer sum| <= R*S*3*max|input|, and every bit
+ * convolution adds at most Cin*R*S.  A tensor whose bound is <= 32767 may be stored as
+ * int16 without changing a single value; the caller states the format per tensor and is
+ * responsible for the bound (tcbnn_*_residual_bound compute it, the layer classes above
+ * this ABI track it from the actual input data).  Producer and consumer must agree. */
+#define TCBNN_RES_I32 0
+#define TCBNN_RES_I16 1
+
 /* ------------------------------------------------------------------ misc */
 int tcbnn_abi_version(void);
 /* Message of the last failing call on this thread ("" if none). */
@@ -82,6 +95,16 @@ size_t tcbnn_conv_act_words(int height, int width, int batch, int ch); /* H*W*B*
 size_t tcbnn_fc_weight_words(int in_features, int out_features);       /* NPAD32*KW128     */
 size_t tcbnn_conv_filter_words(int r, int s, int in_ch, int out_ch);   /* NPAD32*R*S*CW    */
 size_t tcbnn_inconv_filter_words(int r, int s, int in_ch, int out_ch); /* R*S*OPAD32*5     */
+/* bytes of a residual tensor of `channels` channels in the given TCBNN_RES_* format */
+size_t tcbnn_residual_bytes(int height, int width, int channels, int batch, int format);
+/* Upper bound of |residual| of a first layer whose input satisfies |x| <= input_abs_max
+ * (R*S*3 terms plus rounding slack), and of a bit convolution that adds its own
+ * Cin*R*S to an injected residual bounded by injected_bound (0 if none).  INT32_MAX
+ * when unknown (non-finite input_abs_max, overflow).  tcbnn_residual_format_for_bound:
+ * TCBNN_RES_I16 when 0 <= bound <= 32767, else TCBNN_RES_I32. */
+int tcbnn_inconv_residual_bound(int filter_height, int filter_width, float input_abs_max);
+int tcbnn_conv_residual_bound(int input_channels, int filter_height, int filter_width, int injected_bound);
+int tcbnn_residual_format_for_bound(int bound);
 
 /* ------------------------------------------------- one-time weight packing */
 /* fp32 [K][N] (param.h:58-59) -> packed [NPAD32][KW128].  Replaces
@@ -165,7 +188,7 @@ typedef struct tcbnn_inconv128_desc {
     const uint32_t* filter;    /* tcbnn_pack_inconv_filter output */
     const float* bn;           /* [output_channels] */
     uint32_t* output;          /* [OH][OW][CW(output_channels)][B] */
-    int32_t* output_residual;  /* [P][Q][O][B] or NULL */
+    int32_t* output_residual;  /* residual tensor in `residual_format`, or NULL */
     int input_height, input_width, input_channels;
     int filter_height, filter_width;
     int output_channels, batch;
@@ -173,6 +196,7 @@ typedef struct tcbnn_inconv128_desc {
     int padding;               /* bool */
     int pool_height, pool_width;
     int save_residual;         /* bool */
+    int residual_format;       /* TCBNN_RES_* of output_residual */
 } tcbnn_inconv128_desc;
 int tcbnn_inconv128_forward(const tcbnn_inconv128_desc* d, void* stream);
 
@@ -192,8 +216,8 @@ typedef struct tcbnn_conv128_desc {
     const uint32_t* filter;        /* tcbnn_pack_conv_filter output */
     const float* bn;               /* [output_channels] */
     uint32_t* output;              /* [OH][OW][CW(O)][B]; ahead_fc: [OH][OW][CW128(O)][B] */
-    const int32_t* input_residual; /* [Hr][Wr][input_residual_channels][B] or NULL */
-    int32_t* output_residual;      /* [P][Q][O][B] or NULL */
+    const int32_t* input_residual; /* source tensor (Hr x Wr x input_residual_channels) or NULL */
+    int32_t* output_residual;      /* P x Q x O tensor or NULL */
     int input_height, input_width, input_channels;
     int filter_height, filter_width;
     int output_channels, batch;
@@ -205,6 +229,8 @@ typedef struct tcbnn_conv128_desc {
     int residual_pool;
     int input_residual_channels;   /* channel count of the source tensor */
     int variant;
+    int input_residual_format;     /* TCBNN_RES_* of input_residual */
+    int output_residual_format;    /* TCBNN_RES_* of output_residual */
 } tcbnn_conv128_desc;
 int tcbnn_conv128_forward(const tcbnn_conv128_desc* d, void* stream);
 
@@ -251,10 +277,10 @@ int tcbnn_conv_to_reference_fmt(const uint32_t* packed, uint32_t* fmt, int heigh
                                 int batch, int ch, void* stream);
 int tcbnn_conv_from_reference_fmt(const uint32_t* fmt, uint32_t* packed, int height, int width,
                                   int batch, int ch, void* stream);
-/* Engine residual [P][Q][O][B] -> reference [P][Q][PAD8(B)][PAD128(O)] with zero
- * fill (kernel.cuh:666-668, 820-823). */
+/* Engine residual (either format) -> reference int32 [P][Q][PAD8(B)][PAD128(O)] with
+ * zero fill (kernel.cuh:666-668, 820-823). */
 int tcbnn_residual_to_reference(const int32_t* res, int32_t* ref, int height, int width,
-                                int batch, int ch, void* stream);
+                                int batch, int ch, int format, void* stream);
 
 #ifdef __cplusplus
 }

@@ -51,7 +51,7 @@ class InConv128Desc(C.Structure):
                 ("input_channels", c_int), ("filter_height", c_int), ("filter_width", c_int),
                 ("output_channels", c_int), ("batch", c_int), ("stride_height", c_int),
                 ("stride_width", c_int), ("padding", c_int), ("pool_height", c_int),
-                ("pool_width", c_int), ("save_residual", c_int)]
+                ("pool_width", c_int), ("save_residual", c_int), ("residual_format", c_int)]
 
 
 class Conv128Desc(C.Structure):
@@ -63,7 +63,8 @@ class Conv128Desc(C.Structure):
                 ("padding", c_int), ("pool_height", c_int), ("pool_width", c_int),
                 ("ahead_fc", c_int), ("save_residual", c_int), ("inject_residual", c_int),
                 ("residual_channels", c_int), ("residual_pool", c_int),
-                ("input_residual_channels", c_int), ("variant", c_int)]
+                ("input_residual_channels", c_int), ("variant", c_int),
+                ("input_residual_format", c_int), ("output_residual_format", c_int)]
 
 
 # name -> (restype, argtypes); the complete list of symbols include/tcbnn_hip.h declares.
@@ -79,6 +80,10 @@ ABI = {
     "tcbnn_fc_weight_words": (c_size_t, [c_int] * 2),
     "tcbnn_conv_filter_words": (c_size_t, [c_int] * 4),
     "tcbnn_inconv_filter_words": (c_size_t, [c_int] * 4),
+    "tcbnn_residual_bytes": (c_size_t, [c_int] * 5),
+    "tcbnn_inconv_residual_bound": (c_int, [c_int, c_int, C.c_float]),
+    "tcbnn_conv_residual_bound": (c_int, [c_int] * 4),
+    "tcbnn_residual_format_for_bound": (c_int, [c_int]),
     "tcbnn_pack_fc_weight": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "tcbnn_pack_conv_filter": (c_int, [c_void_p, c_void_p] + [c_int] * 4 + [c_void_p]),
     "tcbnn_pack_inconv_filter": (c_int, [c_void_p, c_void_p] + [c_int] * 4 + [c_void_p]),
@@ -100,7 +105,7 @@ ABI = {
     "tcbnn_fc_from_reference_fmt": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "tcbnn_conv_to_reference_fmt": (c_int, [c_void_p, c_void_p] + [c_int] * 4 + [c_void_p]),
     "tcbnn_conv_from_reference_fmt": (c_int, [c_void_p, c_void_p] + [c_int] * 4 + [c_void_p]),
-    "tcbnn_residual_to_reference": (c_int, [c_void_p, c_void_p] + [c_int] * 4 + [c_void_p]),
+    "tcbnn_residual_to_reference": (c_int, [c_void_p, c_void_p] + [c_int] * 5 + [c_void_p]),
 }
 
 for _name, (_res, _args) in ABI.items():
@@ -110,6 +115,8 @@ for _name, (_res, _args) in ABI.items():
 
 VARIANT_AUTO, VARIANT_POPC, VARIANT_MFMA_I8, VARIANT_MFMA_F4 = 0, 1, 2, 3
 VARIANTS = {"auto": 0, "popc": 1, "mfma_i8": 2, "mfma_f4": 3}
+RES_I32, RES_I16 = 0, 1
+INT32_MAX = 2 ** 31 - 1
 
 
 def check(rc):

@@ -205,13 +205,13 @@ __global__ __launch_bounds__(kThreads) void bgemm_mfma_kernel(
                             int val = 0;
                             if (rin != nullptr && c < p.res_limit && c < p.res_in_ch && c < p.N) {
                                 if (p.res_pool) {
-                                    const size_t rw2 = 2 * (size_t)p.PW;
-                                    const int32_t* s00 =
-                                        rin + (((size_t)(2 * y) * rw2 + 2 * x) * p.res_in_ch + c) * p.B + bb;
-                                    const size_t dx = (size_t)p.res_in_ch * p.B, dy = rw2 * dx;
-                                    val = max(max(s00[0], s00[dx]), max(s00[dy], s00[dy + dx]));
+                                    const size_t rw2 = 2 * (size_t)p.PW, p00 = (size_t)(2 * y) * rw2 + 2 * x;
+                                    auto at = [&](size_t sp) {
+                                        return residual_load(rin, p.res_in_fmt, sp, p.res_in_ch, c, p.B, bb);
+                                    };
+                                    val = max(max(at(p00), at(p00 + 1)), max(at(p00 + rw2), at(p00 + rw2 + 1)));
                                 } else {
-                                    val = rin[(pix * p.res_in_ch + c) * p.B + bb];
+                                    val = residual_load(rin, p.res_in_fmt, pix, p.res_in_ch, c, p.B, bb);
                                 }
                             }
                             rv[v] = val;
@@ -227,7 +227,7 @@ __global__ __launch_bounds__(kThreads) void bgemm_mfma_kernel(
                         if (c < p.N) {
                             if constexpr (MM == MM_THRESH_RES) {
                                 res += rv[v];
-                                if (rout != nullptr && b_ok) rout[(pix * p.N + c) * p.B + b] = res;
+                                if (rout != nullptr && b_ok) residual_store(rout, p.res_out_fmt, pix, p.N, c, p.B, b, res);
                             }
                             bit = thresh_bit(res, bnp[c], p.nan_bit);
                         }

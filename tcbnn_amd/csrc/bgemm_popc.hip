@@ -265,13 +265,13 @@ __global__ __launch_bounds__(kThreads)
                         int v = 0;
                         if (rin != nullptr && ch < p.res_limit && ch < p.res_in_ch && ch < p.N) {
                             if (p.res_pool) {
-                                const size_t rw2 = 2 * (size_t)p.PW;
-                                const int32_t* s00 =
-                                    rin + (((size_t)(2 * y) * rw2 + 2 * x) * p.res_in_ch + ch) * p.B + b;
-                                const size_t dx = (size_t)p.res_in_ch * p.B, dy = rw2 * dx;
-                                v = max(max(s00[0], s00[dx]), max(s00[dy], s00[dy + dx]));
+                                const size_t rw2 = 2 * (size_t)p.PW, p00 = (size_t)(2 * y) * rw2 + 2 * x;
+                                auto at = [&](size_t sp) {
+                                    return residual_load(rin, p.res_in_fmt, sp, p.res_in_ch, ch, p.B, b);
+                                };
+                                v = max(max(at(p00), at(p00 + 1)), max(at(p00 + rw2), at(p00 + rw2 + 1)));
                             } else {
-                                v = rin[(pix * p.res_in_ch + ch) * p.B + b];
+                                v = residual_load(rin, p.res_in_fmt, pix, p.res_in_ch, ch, p.B, b);
                             }
                         }
                         rv[n] = v;
@@ -287,7 +287,7 @@ __global__ __launch_bounds__(kThreads)
                         int res = base - 2 * acc[r][n];
                         if constexpr (KM == KM_THRESH_RES) {
                             res += rv[n];
-                            if (rout != nullptr) rout[(pix * p.N + ch) * p.B + b] = res;
+                            if (rout != nullptr) residual_store(rout, p.res_out_fmt, pix, p.N, ch, p.B, b, res);
                         }
                         if constexpr (KM == KM_THRESH_FC)
                             bit = (float)res >= bn[ch] ? 1u : 0u;

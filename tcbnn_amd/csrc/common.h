@@ -84,12 +84,33 @@ struct BgemmParams {
     int res_limit;          // inject only into n < res_limit
     int res_pool;           // 2x2 max over a source twice the output size
     int32_t* res_out;       // [PH][PW][N][B]
+    int res_in_fmt, res_out_fmt;  // TCBNN_RES_* of res_in / res_out
     // split-K (FC-shaped problems only): partial popcounts are atomically added into
     // workspace[n*B + b] and a finishing kernel applies the epilogue
     int32_t* workspace;
     int ksplit;
     int ws_is_dot;  // workspace holds +-1 dot products (matrix-core engines) instead of popcounts
 };
+
+// One residual value in either storage format (TCBNN_RES_I32: int32 [pix][ch][B];
+// TCBNN_RES_I16: int16 [pix][ceil(ch/2)][B][2], channel 2k in the low half of a word).
+__device__ __forceinline__ int residual_load(const int32_t* __restrict__ base, int fmt, size_t pix, int channels,
+                                             int c, int batch, int b) {
+    if (fmt == TCBNN_RES_I16) {
+        const int16_t* s = reinterpret_cast<const int16_t*>(base);
+        return s[((pix * (size_t)((channels + 1) / 2) + (c >> 1)) * batch + b) * 2 + (c & 1)];
+    }
+    return base[(pix * channels + c) * batch + b];
+}
+__device__ __forceinline__ void residual_store(int32_t* __restrict__ base, int fmt, size_t pix, int channels, int c,
+                                               int batch, int b, int v) {
+    if (fmt == TCBNN_RES_I16) {
+        int16_t* s = reinterpret_cast<int16_t*>(base);
+        s[((pix * (size_t)((channels + 1) / 2) + (c >> 1)) * batch + b) * 2 + (c & 1)] = (int16_t)v;
+    } else {
+        base[(pix * channels + c) * batch + b] = v;
+    }
+}
 
 int launch_bgemm_popc(const BgemmParams& p, hipStream_t stream);
 int launch_bgemm_mfma(const BgemmParams& p, int variant, hipStream_t stream);

@@ -49,7 +49,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(waves_
 conv3x3_mfma_f4_kernel(
     const BgemmParams p, const uint32_t* __restrict__ act, const uint32_t* __restrict__ wgt,
     const float* __restrict__ bnp, const int32_t* __restrict__ rin, int32_t* __restrict__ rout, int res_lim,
-    int n_groups, int b_groups, int pix_streams) {
+    int rin_fmt, int rout_fmt, int n_groups, int b_groups, int pix_streams) {
     static_assert(RM == RM_NONE || MT == 1, "residual instantiations own one image tile per wave");
     constexpr int TPC = SPT >= 4 ? 3 : 9;  // taps per prefetch chunk (a filter row, or all of it)
     constexpr int NCH = 9 / TPC;           // chunks per tile
@@ -155,54 +155,91 @@ conv3x3_mfma_f4_kernel(
 
     // ---- residual operand (kernel.cuh:770-794).  A lane owns channels n0 + 32 nt + 16 h + v of
     // image bload[0]; every load is a wave-uniform base plus this per-lane element offset.
+    // TCBNN_RES_I16 tensors hold two channels per word: 8 loads per channel tile instead of 16,
+    // unpacked (and, for a pooled source, reduced) by finish_residual.
     constexpr int NRV = RM != RM_NONE ? NT : 1;
     constexpr int NTMP = RM == RM_POOLED ? 3 : 1;
     int tmp[NTMP][NRV][16];  // pooled: the other three pixels of the 2x2 window
     const unsigned lane_off = (unsigned)(16 * h) * (unsigned)p.B + (unsigned)bload[0];
+    const unsigned lane_off16 = (unsigned)(8 * h) * (unsigned)p.B + (unsigned)bload[0];
 
     auto request_residual = [&](int yy, int xx, int (*rv)[16]) {
         if constexpr (RM != RM_NONE) {
-            const size_t ch_b = (size_t)p.res_in_ch * p.B;
+            const bool i16 = rin_fmt == TCBNN_RES_I16;  // wave-uniform
+            // words per source pixel, words between channel rows of a lane, lane offset
+            const size_t ch_b = (size_t)(i16 ? (p.res_in_ch + 1) / 2 : p.res_in_ch) * p.B;
+            const unsigned loff = i16 ? lane_off16 : lane_off;
+            const int nld = i16 ? 8 : 16;
             const size_t pix = RM == RM_POOLED ? ((size_t)(2 * yy) * (2 * p.PW) + 2 * xx) : ((size_t)yy * p.PW + xx);
             const size_t ddy = (size_t)(2 * p.PW) * ch_b;
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
                 const int cb = n0 + nt * 32;
-                const int32_t* __restrict__ base = rin + pix * ch_b + (size_t)cb * p.B;  // wave-uniform
+                const int32_t* __restrict__ base = rin + pix * ch_b + (size_t)(i16 ? cb / 2 : cb) * p.B;  // uniform
                 if (cb + 32 <= res_lim) {
 #pragma unroll
                     for (int v = 0; v < 16; ++v) {
+                        if (v >= nld) continue;  // uniform
                         const int32_t* s = base + (size_t)v * p.B;
-                        rv[nt][v] = s[lane_off];
+                        rv[nt][v] = s[loff];
                         if constexpr (RM == RM_POOLED) {
-                            tmp[0][nt][v] = s[ch_b + lane_off];
-                            tmp[1][nt][v] = s[ddy + lane_off];
-                            tmp[2][nt][v] = s[ddy + ch_b + lane_off];
+                            tmp[0][nt][v] = s[ch_b + loff];
+                            tmp[1][nt][v] = s[ddy + loff];
+                            tmp[2][nt][v] = s[ddy + ch_b + loff];
                         }
                     }
                 } else {
 #pragma unroll
                     for (int v = 0; v < 16; ++v) {
-                        const bool ok = cb + 16 * h + v < res_lim;
+                        if (v >= nld) continue;  // uniform
+                        const bool ok = cb + 16 * h + (i16 ? 2 * v : v) < res_lim;
                         const int32_t* s = base + (size_t)v * p.B;
-                        rv[nt][v] = ok ? s[lane_off] : 0;
+                        rv[nt][v] = ok ? s[loff] : 0;
                         if constexpr (RM == RM_POOLED) {
-                            tmp[0][nt][v] = ok ? s[ch_b + lane_off] : 0;
-                            tmp[1][nt][v] = ok ? s[ddy + lane_off] : 0;
-                            tmp[2][nt][v] = ok ? s[ddy + ch_b + lane_off] : 0;
+                            tmp[0][nt][v] = ok ? s[ch_b + loff] : 0;
+                            tmp[1][nt][v] = ok ? s[ddy + loff] : 0;
+                            tmp[2][nt][v] = ok ? s[ddy + ch_b + loff] : 0;
                         }
                     }
                 }
             }
         }
     };
-    auto reduce_residual = [&](int (*rv)[16]) {
-        if constexpr (RM == RM_POOLED) {
+    // Turns what request_residual loaded into one int per channel: unpack 16-bit pairs, take the
+    // 2x2 maximum of a pooled source, clear channels that receive no residual.
+    auto finish_residual = [&](int (*rv)[16]) {
+        if constexpr (RM != RM_NONE) {
+            if (rin_fmt == TCBNN_RES_I16) {
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
+                for (int nt = 0; nt < NT; ++nt) {
+                    const int cb = n0 + nt * 32;
 #pragma unroll
-                for (int v = 0; v < 16; ++v)
-                    rv[nt][v] = max(max(rv[nt][v], tmp[0][nt][v]), max(tmp[1][nt][v], tmp[2][nt][v]));
+                    for (int k = 7; k >= 0; --k) {  // downwards: slot k is read before 2k, 2k+1 are written
+                        const int w = rv[nt][k];
+                        int lo = (int)(short)(w & 0xffff), hi = w >> 16;
+                        if constexpr (RM == RM_POOLED) {
+#pragma unroll
+                            for (int t = 0; t < 3; ++t) {
+                                const int wt = tmp[t][nt][k];
+                                lo = max(lo, (int)(short)(wt & 0xffff));
+                                hi = max(hi, wt >> 16);
+                            }
+                        }
+                        if (cb + 32 > res_lim) {  // uniform: partial channel tile
+                            if (cb + 16 * h + 2 * k >= res_lim) lo = 0;
+                            if (cb + 16 * h + 2 * k + 1 >= res_lim) hi = 0;
+                        }
+                        rv[nt][2 * k] = lo;
+                        rv[nt][2 * k + 1] = hi;
+                    }
+                }
+            } else if constexpr (RM == RM_POOLED) {
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v)
+                        rv[nt][v] = max(max(rv[nt][v], tmp[0][nt][v]), max(tmp[1][nt][v], tmp[2][nt][v]));
+            }
         }
     };
 
@@ -235,15 +272,27 @@ conv3x3_mfma_f4_kernel(
 #pragma unroll
                     for (int v = 0; v < 16; ++v) res[v] = (int)acc[mt][nt][v] + rv[nt][v];
                     if (rout != nullptr && b_ok) {
-                        int32_t* __restrict__ dst = rout + (pix * p.N + n0 + nt * 32) * p.B;  // wave-uniform
-                        const unsigned off = (unsigned)(16 * h) * (unsigned)p.B + (unsigned)b;
-                        if (n_full) {
+                        if (rout_fmt == TCBNN_RES_I16) {  // two channels per word
+                            int32_t* __restrict__ dst =
+                                rout + (pix * ((p.N + 1) / 2) + (n0 + nt * 32) / 2) * p.B;  // wave-uniform
+                            const unsigned off = (unsigned)(8 * h) * (unsigned)p.B + (unsigned)b;
 #pragma unroll
-                            for (int v = 0; v < 16; ++v) (dst + (size_t)v * p.B)[off] = res[v];
+                            for (int k = 0; k < 8; ++k) {
+                                const int c0 = cbase + 2 * k;
+                                const int hi = (n_full || c0 + 1 < p.N) ? res[2 * k + 1] : 0;
+                                if (n_full || c0 < p.N) (dst + (size_t)k * p.B)[off] = (res[2 * k] & 0xffff) | (hi << 16);
+                            }
                         } else {
+                            int32_t* __restrict__ dst = rout + (pix * p.N + n0 + nt * 32) * p.B;  // wave-uniform
+                            const unsigned off = (unsigned)(16 * h) * (unsigned)p.B + (unsigned)b;
+                            if (n_full) {
 #pragma unroll
-                            for (int v = 0; v < 16; ++v)
-                                if (cbase + v < p.N) (dst + (size_t)v * p.B)[off] = res[v];
+                                for (int v = 0; v < 16; ++v) (dst + (size_t)v * p.B)[off] = res[v];
+                            } else {
+#pragma unroll
+                                for (int v = 0; v < 16; ++v)
+                                    if (cbase + v < p.N) (dst + (size_t)v * p.B)[off] = res[v];
+                            }
                         }
                     }
 #pragma unroll
@@ -284,7 +333,7 @@ conv3x3_mfma_f4_kernel(
         m0 = load_chunk(y, x, 0, buf0);
         if constexpr (kAhead) {
             request_residual(y, x, rv0);
-            reduce_residual(rv0);
+            if constexpr (RM == RM_POOLED) finish_residual(rv0);
         }
     }
     zero_acc();
@@ -310,11 +359,13 @@ conv3x3_mfma_f4_kernel(
             if (chunk == 0) request_residual(y, x, rcur);
         }
         compute_chunk(chunk, cur, mcur);
-        if constexpr (kAhead) {
-            if (nhave) reduce_residual(rnxt);
+        // a pooled source is reduced as soon as its tile has been multiplied (frees the registers of the
+        // window); otherwise the operand is left in flight until its own epilogue
+        if constexpr (kAhead && RM == RM_POOLED) {
+            if (nhave) finish_residual(rnxt);
         }
         if (chunk == NCH - 1) {
-            if constexpr (!kAhead) reduce_residual(rcur);
+            if constexpr (!(kAhead && RM == RM_POOLED)) finish_residual(rcur);
             epilogue(y, x, rcur);
             zero_acc();
         }
@@ -374,7 +425,8 @@ int launch_t(const BgemmParams& p, hipStream_t stream) {
     const int res_lim = p.res_in != nullptr ? std::min(std::min(p.res_limit, p.res_in_ch), p.N) : 0;
     const long long blocks = (long long)best * n_groups * b_groups;
     hipLaunchKernelGGL((conv3x3_mfma_f4_kernel<SPT, RM, MT, NT>), dim3((unsigned)blocks), dim3(kThreads), lds_bytes,
-                       stream, p, p.act, p.wgt, p.bn, p.res_in, p.res_out, res_lim, n_groups, b_groups, best);
+                       stream, p, p.act, p.wgt, p.bn, p.res_in, p.res_out, res_lim, p.res_in_fmt, p.res_out_fmt, n_groups,
+                       b_groups, best);
     TCBNN_LAUNCH_CHECK("conv3x3_mfma_f4_kernel");
     return TCBNN_OK;
 }

@@ -34,7 +34,8 @@ struct InConvParams {
     const uint4* masks;    // [taps][opad32] {m0, m1, m2, 0}
     const float* bn;
     uint32_t* out;         // [OH][OW][ow][B]
-    int32_t* res;          // [PH][PW][O][B] or null
+    int32_t* res;          // residual tensor in format res_fmt, or null
+    int res_fmt;           // TCBNN_RES_*
     int H, W, B, O, opad, ow;
     int R, S, stride_h, stride_w, pad_h, pad_w;
     int PH, PW, pool_h, pool_w, OH, OW;
@@ -288,12 +289,25 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3))) v
 #pragma unroll
                 for (int n = 0; n < 32; ++n) {
                     const int ch = wi * 32 + n;
-                    if (ch < p.O) {
-                        word |= (acc[n] < bn[ch] ? 0u : 1u) << (31 - n);
-                        if (res != nullptr) res[(pix * p.O + ch) * p.B + b] = (int)acc[n];
-                    }
+                    if (ch < p.O) word |= (acc[n] < bn[ch] ? 0u : 1u) << (31 - n);
                 }
                 out[(pix * p.ow + wi) * p.B + b] = word;
+                if (res != nullptr) {
+                    if (p.res_fmt == TCBNN_RES_I16) {  // two channels per word, even one in the low half
+                        int32_t* __restrict__ dst = res + (pix * ((p.O + 1) / 2) + wi * 16) * p.B + b;
+#pragma unroll
+                        for (int k = 0; k < 16; ++k) {
+                            const int ch = wi * 32 + 2 * k;
+                            const int hi = ch + 1 < p.O ? (int)acc[2 * k + 1] : 0;
+                            if (ch < p.O) dst[(size_t)k * p.B] = ((int)acc[2 * k] & 0xffff) | (hi << 16);
+                        }
+                    } else {
+                        int32_t* __restrict__ dst = res + (pix * p.O + wi * 32) * p.B + b;
+#pragma unroll
+                        for (int n = 0; n < 32; ++n)
+                            if (wi * 32 + n < p.O) dst[(size_t)n * p.B] = (int)acc[n];
+                    }
+                }
             }
         }
     }
@@ -343,10 +357,10 @@ __global__ __launch_bounds__(kThreads) void inconv_generic_kernel(const InConvPa
                     if (ch < p.O) word |= (acc[n] < p.bn[ch] ? 0u : 1u) << (31 - n);
                 }
                 if (p.res != nullptr) {
-                    int32_t* dst = p.res + ((size_t)y * p.PW + x) * p.O * p.B + b;
 #pragma unroll
                     for (int n = 0; n < 32; ++n)
-                        if (g * 32 + n < p.O) dst[(size_t)(g * 32 + n) * p.B] = (int)acc[n];
+                        if (g * 32 + n < p.O)
+                            residual_store(p.res, p.res_fmt, (size_t)y * p.PW + x, p.O, g * 32 + n, p.B, b, (int)acc[n]);
                 }
             }
         }
@@ -383,6 +397,9 @@ extern "C" int tcbnn_inconv128_forward(const tcbnn_inconv128_desc* d, void* stre
     p.bn = d->bn;
     p.out = d->output;
     p.res = d->save_residual ? d->output_residual : nullptr;
+    p.res_fmt = d->residual_format;
+    TCBNN_REQUIRE(!d->save_residual || p.res_fmt == TCBNN_RES_I32 || p.res_fmt == TCBNN_RES_I16,
+                  "inconv128: unknown residual_format");
     p.H = d->input_height;
     p.W = d->input_width;
     p.B = d->batch;

@@ -6,6 +6,9 @@
 
 #include <atomic>
 
+#include <cmath>
+#include <cstdint>
+
 #include "common.h"
 
 namespace tcbnn {
@@ -85,7 +88,7 @@ using namespace tcbnn;
 
 extern "C" {
 
-int tcbnn_abi_version(void) { return 1; }
+int tcbnn_abi_version(void) { return 2; }
 const char* tcbnn_last_error(void) { return g_err; }
 
 int tcbnn_set_default_variant(int variant) {
@@ -119,6 +122,31 @@ size_t tcbnn_conv_filter_words(int r, int s, int in_ch, int out_ch) {
 size_t tcbnn_inconv_filter_words(int r, int s, int in_ch, int out_ch) {
     (void)in_ch;
     return (size_t)r * s * pad32(out_ch) * 5;
+}
+
+size_t tcbnn_residual_bytes(int height, int width, int channels, int batch, int format) {
+    if (height <= 0 || width <= 0 || channels <= 0 || batch <= 0) return 0;
+    const size_t pix_b = (size_t)height * width * batch;
+    return format == TCBNN_RES_I16 ? pix_b * ((channels + 1) / 2) * 4 : pix_b * channels * 4;
+}
+
+int tcbnn_inconv_residual_bound(int filter_height, int filter_width, float input_abs_max) {
+    if (filter_height <= 0 || filter_width <= 0 || !(input_abs_max >= 0.0f) || std::isinf(input_abs_max))
+        return INT32_MAX;
+    // R*S*3 terms of magnitude <= input_abs_max; fp32 rounding of the running sum adds far less
+    // than the 0.1 % + 1 of slack taken here
+    const double bound = (double)filter_height * filter_width * 3.0 * (double)input_abs_max * 1.001 + 1.0;
+    return bound < (double)(INT32_MAX / 2) ? (int)std::ceil(bound) : INT32_MAX;
+}
+
+int tcbnn_conv_residual_bound(int input_channels, int filter_height, int filter_width, int injected_bound) {
+    if (input_channels <= 0 || filter_height <= 0 || filter_width <= 0 || injected_bound < 0) return INT32_MAX;
+    const long long bound = (long long)input_channels * filter_height * filter_width + injected_bound;
+    return bound < INT32_MAX / 2 ? (int)bound : INT32_MAX;
+}
+
+int tcbnn_residual_format_for_bound(int bound) {
+    return bound >= 0 && bound <= 32767 ? TCBNN_RES_I16 : TCBNN_RES_I32;
 }
 
 int tcbnn_fc128_forward(const tcbnn_fc128_desc* d, void* stream) {
@@ -213,10 +241,16 @@ int tcbnn_conv128_forward(const tcbnn_conv128_desc* d, void* stream) {
         p.res_in_ch = d->input_residual_channels;
         p.res_limit = d->residual_channels;
         p.res_pool = d->residual_pool ? 1 : 0;
+        TCBNN_REQUIRE(d->input_residual_format == TCBNN_RES_I32 || d->input_residual_format == TCBNN_RES_I16,
+                      "conv128: unknown input_residual_format");
+        p.res_in_fmt = d->input_residual_format;
     }
     if (d->save_residual) {
         TCBNN_NOTNULL(d->output_residual);
+        TCBNN_REQUIRE(d->output_residual_format == TCBNN_RES_I32 || d->output_residual_format == TCBNN_RES_I16,
+                      "conv128: unknown output_residual_format");
         p.res_out = d->output_residual;
+        p.res_out_fmt = d->output_residual_format;
     }
     return run_bgemm(p, d->variant, (hipStream_t)stream);
 }
@@ -254,6 +288,8 @@ int tcbnn_conv128_kernel_name(const tcbnn_conv128_desc* d, char* buf, size_t len
     p.stride_h = d->stride_height;
     p.stride_w = d->stride_width;
     p.res_pool = d->residual_pool;
+    p.res_in_fmt = d->input_residual_format;
+    p.res_out_fmt = d->output_residual_format;
     // only nullness matters for the name
     p.res_in = d->inject_residual ? reinterpret_cast<const int32_t*>(d) : nullptr;
     p.res_out = d->save_residual ? reinterpret_cast<int32_t*>(const_cast<tcbnn_conv128_desc*>(d)) : nullptr;

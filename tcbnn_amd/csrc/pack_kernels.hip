@@ -164,13 +164,13 @@ __global__ void fmt_convert_kernel(uint32_t* __restrict__ packed, uint32_t* __re
 
 __global__ void residual_to_reference_kernel(const int32_t* __restrict__ res,
                                              int32_t* __restrict__ ref, long long pixels,
-                                             int batch, int ch, int b8, int c128) {
+                                             int batch, int ch, int b8, int c128, int fmt) {
     const long long idx = (long long)blockIdx.x * kThreads + threadIdx.x;
     if (idx >= pixels * b8 * c128) return;
     const int c = (int)(idx % c128);
     const int b = (int)((idx / c128) % b8);
     const long long pix = idx / ((long long)c128 * b8);
-    ref[idx] = (b < batch && c < ch) ? res[(pix * ch + c) * batch + b] : 0;
+    ref[idx] = (b < batch && c < ch) ? residual_load(res, fmt, (size_t)pix, ch, c, batch, b) : 0;
 }
 
 }  // namespace
@@ -335,14 +335,15 @@ int tcbnn_conv_from_reference_fmt(const uint32_t* fmt, uint32_t* packed, int hei
 }
 
 int tcbnn_residual_to_reference(const int32_t* res, int32_t* ref, int height, int width, int batch,
-                                int ch, void* stream) {
+                                int ch, int format, void* stream) {
     TCBNN_NOTNULL(res);
     TCBNN_NOTNULL(ref);
     TCBNN_REQUIRE(batch > 0 && height > 0 && width > 0 && ch > 0, "residual_to_reference: bad shape");
+    TCBNN_REQUIRE(format == TCBNN_RES_I32 || format == TCBNN_RES_I16, "residual_to_reference: unknown format");
     const long long pixels = (long long)height * width;
     const long long total = pixels * pad8(batch) * pad128(ch);
     hipLaunchKernelGGL(residual_to_reference_kernel, dim3(blocks_for(total)), dim3(kThreads), 0,
-                       (hipStream_t)stream, res, ref, pixels, batch, ch, pad8(batch), pad128(ch));
+                       (hipStream_t)stream, res, ref, pixels, batch, ch, pad8(batch), pad128(ch), format);
     TCBNN_LAUNCH_CHECK("residual_to_reference_kernel");
     return TCBNN_OK;
 }

@@ -124,12 +124,23 @@ class ConfigSource {
     const float* end_;
 };
 
-// The reference infers the channel stride of an injected residual from PAD128 of the
-// consumer's residual_channels (kernel.cuh:778-791).  The engine stores residuals with their
-// true channel count, so the producer records it here, keyed by device pointer.
-inline std::map<const void*, int>& residual_channels_registry() {
-    static std::map<const void*, int> reg;
+// What a consumer has to know about a saved residual, recorded by its producer and keyed by the
+// device pointer that get_output_residual_gpu() hands out:
+//   channels: the reference infers the channel stride of an injected residual from PAD128 of the
+//             consumer's residual_channels (kernel.cuh:778-791); the engine stores the true count;
+//   bound:    upper bound of |value| (first layer: from the actual input; each bit convolution
+//             adds Cin*R*S), INT32_MAX when unknown;
+//   format:   TCBNN_RES_I16 when the bound proves that 16 bits hold every value, else int32.
+struct ResidualInfo {
+    int channels, bound, format;
+};
+inline std::map<const void*, ResidualInfo>& residual_registry() {
+    static std::map<const void*, ResidualInfo> reg;
     return reg;
+}
+inline ResidualInfo make_residual_info(int channels, int bound) {
+    ResidualInfo info = {channels, bound, tcbnn_residual_format_for_bound(bound)};
+    return info;
 }
 
 }  // namespace tcbnn_host
@@ -414,6 +425,7 @@ class InConv128LayerParam {  // param.h:701-870
           padding(_padding), bn(NULL), bn_gpu(NULL), batch(_batch), stride_height(_stride_height),
           stride_width(_stride_width), pool_width(_pool_width), pool_height(_pool_height),
           save_residual(_save_residual), output_residual_gpu(NULL), gpu(this) {
+        residual_info = tcbnn_host::make_residual_info(_output_channels, INT32_MAX);
         strncpy(this->name, name, 8);
         TCBNN_CONV_GEOMETRY();
     }
@@ -427,13 +439,23 @@ class InConv128LayerParam {  // param.h:701-870
     int output_bit_bytes() { return output_bit_size() * 16; }
     int bn_size() { return output_channels; }
     int bn_bytes() { return bn_size() * sizeof(float); }
-    // engine residual: int32 [P][Q][O][B], true sizes (the reference pads to 8 x 128, param.h:756-758)
+    // engine residual: true sizes (the reference pads to 8 x 128, param.h:756-758), 16 or 32 bits
     size_t residual_size() { return (size_t)output_channels * batch * buf_height * buf_width; }
-    size_t residual_bytes() { return residual_size() * sizeof(int); }
+    size_t residual_bytes() {
+        return tcbnn_residual_bytes(buf_height, buf_width, output_channels, batch, residual_info.format);
+    }
 
     InConv128LayerParam* initialize(float* input, tcbnn_host::ConfigSource config_file) {
         CHECK_NULL_POINTER(input);
         this->input = input;
+        // |first-layer sum| <= R*S*3*max|x|: decides whether the saved residual fits 16 bits
+        float input_abs_max = 0.0f;
+        for (int i = 0; i < input_size(); ++i) {
+            const float a = input[i] < 0 ? -input[i] : input[i];
+            if (!(a <= input_abs_max)) input_abs_max = a;  // also catches NaN
+        }
+        residual_info = tcbnn_host::make_residual_info(
+            output_channels, tcbnn_inconv_residual_bound(filter_height, filter_width, input_abs_max));
         SAFE_ALOC_GPU(input_gpu, input_bytes());
         HIP_SAFE_CALL(hipMemcpy(input_gpu, input, input_bytes(), hipMemcpyHostToDevice));
         SAFE_ALOC_HOST(filter, filter_bytes());
@@ -454,7 +476,7 @@ class InConv128LayerParam {  // param.h:701-870
         SAFE_ALOC_GPU(output_gpu, 4 * tcbnn_conv_act_words(output_height, output_width, batch, output_channels));
         if (save_residual) {
             SAFE_ALOC_GPU(output_residual_gpu, residual_bytes());
-            tcbnn_host::residual_channels_registry()[output_residual_gpu] = output_channels;
+            tcbnn_host::residual_registry()[output_residual_gpu] = residual_info;
         }
         return this;
     }
@@ -464,7 +486,7 @@ class InConv128LayerParam {  // param.h:701-870
         tcbnn_inconv128_desc d = {input_gpu,      filter_gpu,     bn_gpu,        output_gpu,   output_residual_gpu,
                                   input_height,   input_width,    input_channels, filter_height, filter_width,
                                   output_channels, batch,         stride_height, stride_width, padding ? 1 : 0,
-                                  pool_height,    pool_width,     save_residual ? 1 : 0};
+                                  pool_height,    pool_width,     save_residual ? 1 : 0, residual_info.format};
         TCBNN_SAFE_CALL(tcbnn_inconv128_forward(&d, stream));
     }
     unsigned* download_output() {
@@ -496,7 +518,7 @@ class InConv128LayerParam {  // param.h:701-870
         SAFE_FREE_GPU(output_gpu);
         SAFE_FREE_GPU(filter_gpu);
         SAFE_FREE_GPU(bn_gpu);
-        if (output_residual_gpu != NULL) tcbnn_host::residual_channels_registry().erase(output_residual_gpu);
+        if (output_residual_gpu != NULL) tcbnn_host::residual_registry().erase(output_residual_gpu);
         SAFE_FREE_GPU(output_residual_gpu);
     }
     ~InConv128LayerParam() { release(); }
@@ -528,6 +550,7 @@ class InConv128LayerParam {  // param.h:701-870
     int pool_height;
     bool save_residual;
     int* output_residual_gpu;
+    tcbnn_host::ResidualInfo residual_info;  // channels / bound / format of output_residual_gpu
     InConv128LayerParam* gpu;
     char name[8];
     int buf_height, buf_width;  // conv output size before pooling
@@ -549,6 +572,7 @@ class Conv128LayerParam {  // param.h:872-1065
           save_residual(_save_residual), output_residual_gpu(NULL), inject_residual(_inject_residual),
           input_residual_gpu(NULL), residual_channels(_residual_channels), residual_pool(_residual_pool),
           gpu(this), variant(TCBNN_VARIANT_AUTO), input_residual_channels(0) {
+        residual_info = input_residual_info = tcbnn_host::make_residual_info(_output_channels, INT32_MAX);
         strncpy(this->name, name, 8);
         TCBNN_CONV_GEOMETRY();
     }
@@ -561,15 +585,27 @@ class Conv128LayerParam {  // param.h:872-1065
     int bn_size() { return output_channels; }
     int bn_bytes() { return bn_size() * sizeof(float); }
     size_t residual_size() { return (size_t)output_channels * batch * buf_height * buf_width; }
-    size_t residual_bytes() { return residual_size() * sizeof(int); }
+    size_t residual_bytes() {
+        return tcbnn_residual_bytes(buf_height, buf_width, output_channels, batch, residual_info.format);
+    }
 
     void set_input_gpu(uin32* input_gpu) { this->input_gpu = input_gpu; }
     void set_input_residual_gpu(int* input_residual_gpu) {
         this->input_residual_gpu = input_residual_gpu;
-        std::map<const void*, int>& reg = tcbnn_host::residual_channels_registry();
-        std::map<const void*, int>::iterator it = reg.find(input_residual_gpu);
-        // a residual that no layer of this library produced: assume the consumer's limit
-        input_residual_channels = it != reg.end() ? it->second : residual_channels;
+        std::map<const void*, tcbnn_host::ResidualInfo>& reg = tcbnn_host::residual_registry();
+        std::map<const void*, tcbnn_host::ResidualInfo>::iterator it = reg.find(input_residual_gpu);
+        // a residual that no layer of this library produced: int32 with the consumer's channel
+        // limit and no known bound
+        const tcbnn_host::ResidualInfo foreign = {residual_channels, INT32_MAX, TCBNN_RES_I32};
+        input_residual_info = it != reg.end() ? it->second : foreign;
+        input_residual_channels = input_residual_info.channels;
+        if (output_residual_gpu != NULL &&
+            tcbnn_conv_residual_bound(input_channels, filter_height, filter_width,
+                                      input_residual_info.bound < INT32_MAX / 4 ? input_residual_info.bound
+                                                                                : INT32_MAX / 4) > residual_info.bound) {
+            fprintf(stderr, "Error: the injected residual exceeds the bound the saved residual was sized for.\n");
+            exit(-1);
+        }
     }
     Conv128LayerParam* initialize(tcbnn_host::ConfigSource config_file, uin32* prev_layer_gpu,
                                   int* input_residual_gpu = NULL) {
@@ -593,13 +629,18 @@ class Conv128LayerParam {  // param.h:872-1065
                      : tcbnn_conv_act_words(output_height, output_width, batch, output_channels);
         SAFE_ALOC_GPU(output_gpu, 4 * words);
         set_input_gpu(prev_layer_gpu);
-        if (save_residual) {
-            SAFE_ALOC_GPU(output_residual_gpu, residual_bytes());
-            tcbnn_host::residual_channels_registry()[output_residual_gpu] = output_channels;
-        }
         if (inject_residual) {
             set_input_residual_gpu(input_residual_gpu);
             CHECK_NULL_POINTER(this->input_residual_gpu);
+        }
+        if (save_residual) {
+            const int injected = inject_residual ? input_residual_info.bound : 0;
+            residual_info = tcbnn_host::make_residual_info(
+                output_channels, injected < INT32_MAX / 4 ? tcbnn_conv_residual_bound(input_channels, filter_height,
+                                                                                      filter_width, injected)
+                                                          : INT32_MAX);
+            SAFE_ALOC_GPU(output_residual_gpu, residual_bytes());
+            tcbnn_host::residual_registry()[output_residual_gpu] = residual_info;
         }
         CHECK_NULL_POINTER(input_gpu);
         return this;
@@ -634,6 +675,8 @@ class Conv128LayerParam {  // param.h:872-1065
         d.residual_pool = residual_pool ? 1 : 0;
         d.input_residual_channels = input_residual_channels;
         d.variant = variant;
+        d.input_residual_format = input_residual_info.format;
+        d.output_residual_format = residual_info.format;
         TCBNN_SAFE_CALL(tcbnn_conv128_forward(&d, stream));
     }
     unsigned* download_output() {
@@ -672,7 +715,7 @@ class Conv128LayerParam {  // param.h:872-1065
         SAFE_FREE_GPU(output_gpu);
         SAFE_FREE_GPU(filter_gpu);
         SAFE_FREE_GPU(bn_gpu);
-        if (output_residual_gpu != NULL) tcbnn_host::residual_channels_registry().erase(output_residual_gpu);
+        if (output_residual_gpu != NULL) tcbnn_host::residual_registry().erase(output_residual_gpu);
         SAFE_FREE_GPU(output_residual_gpu);
     }
     ~Conv128LayerParam() { release(); }
@@ -705,6 +748,7 @@ class Conv128LayerParam {  // param.h:872-1065
     bool ahead_fc;
     bool save_residual;
     int* output_residual_gpu;
+    tcbnn_host::ResidualInfo residual_info;        // of output_residual_gpu
     bool inject_residual;
     int* input_residual_gpu;
     int residual_channels;
@@ -713,5 +757,6 @@ class Conv128LayerParam {  // param.h:872-1065
     char name[8];
     int variant;
     int input_residual_channels;
+    tcbnn_host::ResidualInfo input_residual_info;  // of input_residual_gpu
     int buf_height, buf_width;
 };

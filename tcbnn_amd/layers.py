@@ -80,9 +80,13 @@ def _stream_handle(stream):
     return stream.handle if stream is not None else None
 
 
-def _residual_buffer(nbytes, channels, height, width):
-    buf = DeviceBuffer(nbytes)
-    buf.channels, buf.height, buf.width = channels, height, width
+def _residual_buffer(channels, height, width, batch, bound, force_format=None):
+    """Device buffer of a saved residual.  `bound` is an upper bound of |value| (INT32_MAX when
+    unknown); the 16-bit format is chosen when the bound allows it (or as `force_format` says)."""
+    fmt = lib.tcbnn_residual_format_for_bound(bound) if force_format is None else force_format
+    buf = DeviceBuffer(lib.tcbnn_residual_bytes(height, width, channels, batch, fmt))
+    buf.channels, buf.height, buf.width, buf.batch = channels, height, width, batch
+    buf.bound, buf.format = bound, fmt
     return buf
 
 
@@ -318,9 +322,13 @@ class _ConvGeometry:
         return self.output_residual_gpu
 
     def download_residual(self):
-        """Saved residual as int32 [P][Q][B][O] (host transpose of the engine's [P][Q][O][B])."""
-        eng = self.output_residual_gpu.to_numpy(
-            np.int32, (self.buf_height, self.buf_width, self.output_channels, self.batch))
+        """Saved residual as int32 [P][Q][B][O] (host transpose of the engine's layouts)."""
+        P, Q, O, B = self.buf_height, self.buf_width, self.output_channels, self.batch
+        if self.output_residual_gpu.format == _lib.RES_I16:
+            eng = self.output_residual_gpu.to_numpy(np.int16, (P, Q, (O + 1) // 2, B, 2))
+            return np.ascontiguousarray(
+                eng.transpose(0, 1, 3, 2, 4).reshape(P, Q, B, 2 * ((O + 1) // 2))[..., :O].astype(np.int32))
+        eng = self.output_residual_gpu.to_numpy(np.int32, (P, Q, O, B))
         return np.ascontiguousarray(eng.transpose(0, 1, 3, 2))
 
     def download_residual_reference(self):
@@ -328,7 +336,8 @@ class _ConvGeometry:
         shape = (self.buf_height, self.buf_width, PAD8(self.batch), PAD128(self.output_channels))
         tmp = DeviceBuffer(4 * int(np.prod(shape)))
         check(lib.tcbnn_residual_to_reference(self.output_residual_gpu.ptr, tmp.ptr, self.buf_height,
-                                              self.buf_width, self.batch, self.output_channels, None))
+                                              self.buf_width, self.batch, self.output_channels,
+                                              self.output_residual_gpu.format, None))
         _lib.device_synchronize()
         return tmp.to_numpy(np.int32, shape)
 
@@ -375,8 +384,9 @@ class InConv128LayerParam(_ConvGeometry):
 
     def __init__(self, name, input_height, input_width, filter_height, filter_width, input_channels,
                  output_channels, batch, stride_height=1, stride_width=1, padding=True, pool_height=1,
-                 pool_width=1, save_residual=False):
+                 pool_width=1, save_residual=False, residual_format=None):
         self.name = name
+        self.residual_format = residual_format  # None: narrowest exact format; or _lib.RES_I32 / RES_I16
         self.input_height, self.input_width = input_height, input_width
         self.filter_height, self.filter_width = filter_height, filter_width
         self.input_channels, self.output_channels, self.batch = input_channels, output_channels, batch
@@ -396,6 +406,7 @@ class InConv128LayerParam(_ConvGeometry):
         x = np.ascontiguousarray(input, dtype=np.float32)
         assert x.size == self.input_size(), (x.size, self.input_size())
         self.input_gpu = DeviceBuffer.from_numpy(x)
+        self.input_abs_max = float(np.max(np.abs(x))) if x.size else 0.0
         self.filter = np.array(config_file.launch_array(self.filter_size()), dtype=np.float32)
         self.filter_gpu = DeviceBuffer(4 * lib.tcbnn_inconv_filter_words(
             self.filter_height, self.filter_width, self.input_channels, self.output_channels))
@@ -409,13 +420,18 @@ class InConv128LayerParam(_ConvGeometry):
         self.output_gpu = DeviceBuffer(4 * lib.tcbnn_conv_act_words(
             self.output_height, self.output_width, self.batch, self.output_channels))
         if self.save_residual:
-            self.output_residual_gpu = _residual_buffer(
-                4 * self.buf_height * self.buf_width * self.batch * self.output_channels,
-                self.output_channels, self.buf_height, self.buf_width)
+            bound = lib.tcbnn_inconv_residual_bound(self.filter_height, self.filter_width, self.input_abs_max)
+            self.output_residual_gpu = _residual_buffer(self.output_channels, self.buf_height, self.buf_width,
+                                                        self.batch, bound, self.residual_format)
         return self
 
     def set_input(self, input):
-        self.input_gpu.upload(np.ascontiguousarray(input, dtype=np.float32))
+        x = np.ascontiguousarray(input, dtype=np.float32)
+        amax = float(np.max(np.abs(x))) if x.size else 0.0
+        if self.save_residual and lib.tcbnn_inconv_residual_bound(
+                self.filter_height, self.filter_width, amax) > self.output_residual_gpu.bound:
+            raise _lib.TcbnnError("input magnitude exceeds the bound the residual format was chosen for")
+        self.input_gpu.upload(x)
 
     def forward(self, stream=None):
         d = _lib.InConv128Desc(
@@ -423,7 +439,8 @@ class InConv128LayerParam(_ConvGeometry):
             self.output_residual_gpu.ptr if self.output_residual_gpu is not None else None,
             self.input_height, self.input_width, self.input_channels, self.filter_height, self.filter_width,
             self.output_channels, self.batch, self.stride_height, self.stride_width, int(self.padding),
-            self.pool_height, self.pool_width, int(self.save_residual))
+            self.pool_height, self.pool_width, int(self.save_residual),
+            self.output_residual_gpu.format if self.output_residual_gpu is not None else 0)
         check(lib.tcbnn_inconv128_forward(C.byref(d), _stream_handle(stream)))
 
     def release(self):
@@ -439,8 +456,9 @@ class Conv128LayerParam(_ConvGeometry):
     def __init__(self, name, input_height, input_width, filter_height, filter_width, input_channels,
                  output_channels, batch, stride_height=1, stride_width=1, padding=True, pool_height=1,
                  pool_width=1, ahead_fc=False, save_residual=False, inject_residual=False,
-                 residual_channels=0, residual_pool=False, variant=_lib.VARIANT_AUTO):
+                 residual_channels=0, residual_pool=False, variant=_lib.VARIANT_AUTO, residual_format=None):
         self.name = name
+        self.residual_format = residual_format  # None: narrowest exact format; or _lib.RES_I32 / RES_I16
         self.input_height, self.input_width = input_height, input_width
         self.filter_height, self.filter_width = filter_height, filter_width
         self.input_channels, self.output_channels, self.batch = input_channels, output_channels, batch
@@ -458,6 +476,11 @@ class Conv128LayerParam(_ConvGeometry):
         self.input_gpu = input_gpu
 
     def set_input_residual_gpu(self, input_residual_gpu):
+        out = self.output_residual_gpu
+        if out is not None and input_residual_gpu is not None and self.inject_residual and \
+                lib.tcbnn_conv_residual_bound(self.input_channels, self.filter_height, self.filter_width,
+                                              min(input_residual_gpu.bound, _lib.INT32_MAX // 4)) > out.bound:
+            raise _lib.TcbnnError("injected residual exceeds the bound the saved residual's format was chosen for")
         self.input_residual_gpu = input_residual_gpu
 
     def initialize(self, config_file, prev_layer_gpu, input_residual_gpu=None):
@@ -479,14 +502,16 @@ class Conv128LayerParam(_ConvGeometry):
                                              self.output_channels)
         self.output_gpu = DeviceBuffer(4 * words)
         self.set_input_gpu(prev_layer_gpu)
-        if self.save_residual:
-            self.output_residual_gpu = _residual_buffer(
-                4 * self.buf_height * self.buf_width * self.batch * self.output_channels,
-                self.output_channels, self.buf_height, self.buf_width)
         if self.inject_residual:
             self.set_input_residual_gpu(input_residual_gpu)
             if self.input_residual_gpu is None:
                 raise _lib.TcbnnError("Error: NULL pointer (input_residual_gpu)")
+        if self.save_residual:
+            injected = self.input_residual_gpu.bound if self.inject_residual else 0
+            bound = lib.tcbnn_conv_residual_bound(self.input_channels, self.filter_height, self.filter_width,
+                                                  injected) if injected < _lib.INT32_MAX else _lib.INT32_MAX
+            self.output_residual_gpu = _residual_buffer(self.output_channels, self.buf_height, self.buf_width,
+                                                        self.batch, bound, self.residual_format)
         if self.input_gpu is None:
             raise _lib.TcbnnError("Error: NULL pointer (input_gpu)")
         return self
@@ -501,7 +526,9 @@ class Conv128LayerParam(_ConvGeometry):
             self.output_channels, self.batch, self.stride_height, self.stride_width, int(self.padding),
             self.pool_height, self.pool_width, int(self.ahead_fc), int(self.save_residual),
             int(self.inject_residual), self.residual_channels, int(self.residual_pool),
-            rin.channels if rin is not None else 0, self.variant)
+            rin.channels if rin is not None else 0, self.variant,
+            rin.format if rin is not None else 0,
+            self.output_residual_gpu.format if self.output_residual_gpu is not None else 0)
 
     def forward(self, stream=None):
         d = self._desc()

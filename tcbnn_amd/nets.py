@@ -152,7 +152,9 @@ def synthetic_input(spec, seed=0):
 class Network:
     """Layer objects of one network, wired as in the reference drivers."""
 
-    def __init__(self, spec, weights, input, variant=_lib.VARIANT_AUTO):
+    def __init__(self, spec, weights, input, variant=_lib.VARIANT_AUTO, residual_format=None):
+        """residual_format: None = every saved residual in the narrowest format that is exact for its
+        bound; _lib.RES_I32 keeps them all as int32 (the reference's type)."""
         self.spec = spec
         self.layers = {}
         self.order = []
@@ -164,12 +166,13 @@ class Network:
             elif k == "inconv":
                 layer = InConv128LayerParam(L["name"], L["h"], L["w"], L["r"], L["s"], L["cin"], L["cout"],
                                             L["batch"], L["stride"], L["stride"], L["padding"], L["pool"],
-                                            L["pool"], L["save_residual"]).initialize(input, src)
+                                            L["pool"], L["save_residual"], residual_format).initialize(input, src)
             elif k == "conv":
                 layer = Conv128LayerParam(L["name"], L["h"], L["w"], L["r"], L["s"], L["cin"], L["cout"],
                                           L["batch"], L["stride"], L["stride"], L["padding"], L["pool"],
                                           L["pool"], L["ahead_fc"], L["save_residual"], L["inject_residual"],
-                                          L["residual_channels"], L["residual_pool"], variant=variant)
+                                          L["residual_channels"], L["residual_pool"], variant=variant,
+                                          residual_format=residual_format)
                 res = self.layers[L["res_src"]].get_output_residual_gpu() if L["res_src"] else None
                 layer.initialize(src, self.layers[L["src"]].get_output_gpu(), res)
             elif k == "fc":

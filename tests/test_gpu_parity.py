@@ -139,20 +139,36 @@ class _PackedSource:
         self.buf = gpuops.dev(packed)
 
 
+def _residual_source(res_in, fmt):
+    """Device copy of a residual [Hr][Wr][B][C] in the engine layout of format `fmt`, tagged the way the
+    layer classes tag the tensors they produce (channel count, format, bound of |value|)."""
+    hr, wr, b, c = res_in.shape
+    if fmt == 1:  # int16 [Hr][Wr][ceil(C/2)][B][2], channel 2k in the low half
+        c2 = (c + 1) // 2
+        pad = np.zeros((hr, wr, b, 2 * c2), np.int16)
+        pad[..., :c] = res_in
+        host = np.ascontiguousarray(pad.reshape(hr, wr, b, c2, 2).transpose(0, 1, 3, 2, 4))
+    else:         # int32 [Hr][Wr][C][B]
+        host = np.ascontiguousarray(res_in.astype(np.int32).transpose(0, 1, 3, 2))
+    rbuf = gpuops.dev(host)
+    rbuf.channels, rbuf.format, rbuf.bound = c, fmt, int(np.abs(res_in).max())
+    return rbuf
+
+
 def _run_conv_layer(gpu, variant, x, f, bn, stride=1, pool=1, ahead_fc=False, save_residual=False,
-                    inject_residual=False, residual_channels=0, residual_pool=False, res_in=None):
+                    inject_residual=False, residual_channels=0, residual_pool=False, res_in=None, in_fmt=0,
+                    out_fmt=None):
     b, h, w, cin = x.shape
     R, S, _, cout = f.shape
     layer = gpu.Conv128LayerParam("C", h, w, R, S, cin, cout, b, stride, stride, True, pool, pool, ahead_fc,
                                   save_residual, inject_residual, residual_channels, residual_pool,
-                                  variant=_variant(gpu, variant))
+                                  variant=_variant(gpu, variant), residual_format=out_fmt)
     src = gpuops.pack_conv_input(x)
-    rbuf = None
-    if inject_residual:
-        rbuf = gpuops.dev(np.ascontiguousarray(res_in.astype(np.int32).transpose(0, 1, 3, 2)))  # [Hr][Wr][C][B]
-        rbuf.channels = res_in.shape[-1]
+    rbuf = _residual_source(res_in, in_fmt) if inject_residual else None
     layer.initialize(gpu.ArrayWeights([f, bn]), src, rbuf)
     layer.output_gpu.fill(0xCD)  # every output word must be written by the call
+    if layer.output_residual_gpu is not None:
+        layer.output_residual_gpu.fill(0xCD)
     layer.forward()
     layer.forward()  # idempotent: a second run on the same objects gives the same result
     gpuops.sync()
@@ -194,39 +210,94 @@ def test_conv128_layer(gpu, variant, b, h, cin, cout, stride, pool, ahead_fc):
     layer.release()
 
 
+# (cin, cout): the persistent 3x3 kernel's instantiations (Cin 64 .. 512), a channel count that is not a
+# multiple of 32 and an odd one (half-filled last 16-bit pair); formats of the injected and saved tensors
+RES_SHAPES = [(64, 96), (128, 64), (256, 35), (512, 64)]
+RES_FORMATS = [(0, 0), (1, 1), (0, 1), (1, 0)]
+
+
 @pytest.mark.parametrize("variant", VARIANTS)
-def test_conv128_residual_modes(gpu, variant):
-    r = rng(41)
-    b, h, cin, cout = 72, 6, 64, 96
+@pytest.mark.parametrize("in_fmt,out_fmt", RES_FORMATS)
+@pytest.mark.parametrize("cin,cout", RES_SHAPES)
+def test_conv128_residual_modes(gpu, variant, cin, cout, in_fmt, out_fmt):
+    if variant != "mfma_f4" and cin > 128:
+        pytest.skip("the other engines share one residual epilogue for every Cin")
+    r = rng(41 + cin + cout)
+    b, h = 72, 6
     x = rm.pm1(r, (b, h, h, cin))
     f = rm.pm1(r, (3, 3, cin, cout))
     bn = r.normal(0, 20, cout).astype(np.float32)
     inp, filt = orc.pack_conv_input_nhwc(x), orc.pack_conv_filter(f)
 
-    layer = _run_conv_layer(gpu, variant, x, f, bn, save_residual=True)
+    layer = _run_conv_layer(gpu, variant, x, f, bn, save_residual=True, out_fmt=out_fmt)
+    assert layer.output_residual_gpu.format == out_fmt
     want, wres = orc.conv128(inp, filt, bn, cin, cout, 3, 3, save_residual=True)
     np.testing.assert_array_equal(layer.download_packed(), want)
     np.testing.assert_array_equal(layer.download_residual(), wres)
     np.testing.assert_array_equal(layer.download_residual_reference(), orc.residual_to_reference(wres))
     layer.release()
 
-    src = r.integers(-300, 300, size=(h, h, b, 64)).astype(np.int32)
+    # source narrower than the consumer and a limit that cuts through a channel tile
+    src_ch, lim = (cout * 2) // 3, (cout * 5) // 6
+    src = r.integers(-3000, 3000, size=(h, h, b, src_ch)).astype(np.int32)
     layer = _run_conv_layer(gpu, variant, x, f, bn, save_residual=True, inject_residual=True,
-                            residual_channels=80, res_in=src)
+                            residual_channels=lim, res_in=src, in_fmt=in_fmt, out_fmt=out_fmt)
     want, wres = orc.conv128(inp, filt, bn, cin, cout, 3, 3, save_residual=True, inject_residual=True,
-                             residual_channels=80, res_in=src)
+                             residual_channels=lim, res_in=src)
     np.testing.assert_array_equal(layer.download_packed(), want)
     np.testing.assert_array_equal(layer.download_residual(), wres)
     layer.release()
 
-    src2 = r.integers(-300, 300, size=(2 * h, 2 * h, b, 96)).astype(np.int32)
+    # 2x2 max of a source twice the size; source wider than the limit
+    src2 = r.integers(-3000, 3000, size=(2 * h, 2 * h, b, cout)).astype(np.int32)
     layer = _run_conv_layer(gpu, variant, x, f, bn, save_residual=True, inject_residual=True,
-                            residual_channels=48, residual_pool=True, res_in=src2)
+                            residual_channels=cout // 2, residual_pool=True, res_in=src2, in_fmt=in_fmt,
+                            out_fmt=out_fmt)
     want, wres = orc.conv128(inp, filt, bn, cin, cout, 3, 3, save_residual=True, inject_residual=True,
-                             residual_channels=48, residual_pool=True, res_in=src2)
+                             residual_channels=cout // 2, residual_pool=True, res_in=src2)
     np.testing.assert_array_equal(layer.download_packed(), want)
     np.testing.assert_array_equal(layer.download_residual(), wres)
     layer.release()
+
+    # inject only (the last block of the ResNet saves nothing)
+    layer = _run_conv_layer(gpu, variant, x, f, bn, inject_residual=True, residual_channels=cout,
+                            res_in=src2[:h, :h], in_fmt=in_fmt)
+    want, _ = orc.conv128(inp, filt, bn, cin, cout, 3, 3, inject_residual=True, residual_channels=cout,
+                          res_in=src2[:h, :h])
+    np.testing.assert_array_equal(layer.download_packed(), want)
+    layer.release()
+
+
+def test_residual_format_follows_the_bound(gpu):
+    """The layer classes store a residual in 16 bits only when |value| <= 32767 is certain: the first
+    layer's bound comes from the actual input, every bit convolution adds Cin*R*S."""
+    lib = gpu.lib
+    assert lib.tcbnn_residual_format_for_bound(32767) == 1 and lib.tcbnn_residual_format_for_bound(32768) == 0
+    assert lib.tcbnn_inconv_residual_bound(7, 7, float("inf")) == 2 ** 31 - 1
+    assert lib.tcbnn_inconv_residual_bound(7, 7, float("nan")) == 2 ** 31 - 1
+    assert 147 * 5 <= lib.tcbnn_inconv_residual_bound(7, 7, 5.0) <= 147 * 5 + 3
+    assert lib.tcbnn_conv_residual_bound(512, 3, 3, 1000) == 5608
+    assert lib.tcbnn_residual_bytes(3, 5, 7, 11, 0) == 3 * 5 * 7 * 11 * 4
+    assert lib.tcbnn_residual_bytes(3, 5, 7, 11, 1) == 3 * 5 * 4 * 11 * 4
+    r = rng(77)
+    b, h, cout = 4, 16, 64
+    f = rm.pm1(r, (7, 7, 3, cout))
+    bn = r.normal(0, 12, cout).astype(np.float32)
+    for scale, fmt in ((1.0, 1), (400.0, 0)):  # 147 * 400 * |x| overflows 16 bits: int32 is kept
+        x = (r.standard_normal((b, 3, h, h)) * scale).astype(np.float32)
+        want, wres = orc.inconv128(x, f, bn, 4, True, 1, True)
+        layer = gpu.InConv128LayerParam("Conv1", h, h, 7, 7, 3, cout, b, 4, 4, True, 1, 1, True)
+        layer.initialize(x, gpu.ArrayWeights([f, bn]))
+        assert layer.output_residual_gpu.format == fmt
+        assert np.abs(wres).max() <= layer.output_residual_gpu.bound
+        layer.forward()
+        gpuops.sync()
+        np.testing.assert_array_equal(layer.download_packed(), want)
+        np.testing.assert_array_equal(layer.download_residual(), wres)
+        if fmt == 1:
+            with pytest.raises(gpu.TcbnnError):
+                layer.set_input(x * 1000)
+        layer.release()
 
 
 def test_conv128_rejects_residual_with_pooling(gpu):
@@ -300,11 +371,11 @@ def test_inconv128_presigned_input_is_exact_integer_conv(gpu):
 
 
 # --------------------------------------------------------------------------- whole networks
-def _compare_network(gpu, spec, seed, variant):
+def _compare_network(gpu, spec, seed, variant, residual_format=None):
     weights = gpu.synthetic_weights(spec, seed)
     x = gpu.synthetic_input(spec, seed)
     want = orc_nets.run(spec, weights, x)
-    net = gpu.Network(spec, weights, x, variant=_variant(gpu, variant))
+    net = gpu.Network(spec, weights, x, variant=_variant(gpu, variant), residual_format=residual_format)
     net.forward()
     logits = net.logits()
     for L in spec:
@@ -337,10 +408,19 @@ def test_cifar10_vgg(gpu, variant):
     _compare_network(gpu, nets.cifar10_vgg_spec(batch=16), 2, variant)
 
 
+@pytest.mark.parametrize("residual_format", [None, 0], ids=["narrowest", "int32"])
 @pytest.mark.parametrize("variant", VARIANTS)
-def test_imagenet_resnet18(gpu, variant):
+def test_imagenet_resnet18(gpu, variant, residual_format):
+    """Residuals in the narrowest exact format (16 bits all the way for N(0,1) input: the test checks that
+    this is what was chosen) and, as the reference stores them, in int32: same bits either way."""
     from tcbnn_amd import nets
-    _compare_network(gpu, nets.imagenet_resnet_spec(batch=8), 3, variant)
+    spec = nets.imagenet_resnet_spec(batch=8)
+    if residual_format is None:
+        net = gpu.Network(spec, gpu.synthetic_weights(spec, 3), gpu.synthetic_input(spec, 3))
+        fmts = {L["name"]: net.layers[L["name"]].output_residual_gpu.format for L in spec if L.get("save_residual")}
+        net.release()
+        assert fmts and all(f == 1 for f in fmts.values()), fmts
+    _compare_network(gpu, spec, 3, variant, residual_format)
 
 
 @pytest.mark.parametrize("variant", VARIANTS)
