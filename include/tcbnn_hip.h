@@ -30,10 +30,11 @@
  *   packed weights   : uint32 [NPAD32][KWTOT]     one row per output neuron/channel,
  *                                                 FC: KWTOT = KW128; conv: KWTOT = R*S*CW,
  *                                                 K index = (r*S+s)*32*CW + c; rows >= N are 0
- *   residual tensors : TCBNN_RES_I32: int32 [P][Q][O][B], true channel count, no 128-padding;
- *                      TCBNN_RES_I16: int16 [P][Q][ceil(O/2)][B][2] (channels 2k and 2k+1 of
- *                      an image share one 32-bit word, 2k in the low half) for tensors whose
- *                      values provably fit 16 bits (see "residual formats" below)
+ *   residual tensors : TCBNN_RES_I32: int32 [P][Q][ceil(O/4)][B][4]; TCBNN_RES_I16: int16
+ *                      [P][Q][ceil(O/8)][B][8] for tensors whose values provably fit 16 bits
+ *                      (see "residual formats" below).  Either way an image's group of 4 / 8
+ *                      consecutive channels is 16 contiguous bytes and consecutive images follow
+ *                      each other; channels are padded to the group, not to 128
  *   fp32 stem input  : float  [B][3][H][W]        (kernel.cuh:620-625)
  * The reference's own tile-contiguous "FMT" layouts ([.../8][.../128][8][4],
  * kernel.cuh:170,222,650-660,798-815) are produced / consumed by the

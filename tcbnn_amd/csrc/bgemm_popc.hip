@@ -17,9 +17,9 @@
 //                     32 +-1 multiply-accumulates.
 //   epilogue        = in-lane: the lane owns all 32 channel sums of its row, so
 //                     threshold -> bit -> shift/or builds the packed output word with
-//                     no ballot, no LDS round trip and no atomics; residual tensors are
-//                     [P][Q][O][B], so each channel's residual load/store is again one
-//                     contiguous run across the wave.  Pool windows are a sequential
+//                     no ballot, no LDS round trip and no atomics; residual tensors keep
+//                     the batch below small channel groups, so consecutive lanes touch
+//                     consecutive 16-byte slots.  Pool windows are a sequential
 //                     loop in the same lane (OR of the words), so every output word is
 //                     written exactly once and re-runs are idempotent.
 //   split-K         = FC-shaped problems with few rows split K over blockIdx; partial

@@ -46,7 +46,7 @@ int resolve_variant(int requested);
 // residual and output access one contiguous run):
 //   activations  uint32 [H][W][cw][B]
 //   weights      uint32 [npad32][taps*cw]
-//   residuals    int32  [P][Q][O][B]
+//   residuals    int32 [P][Q][ceil(O/4)][B][4] or int16 [P][Q][ceil(O/8)][B][8]
 // ---------------------------------------------------------------------------
 enum EpilogueMode : int {
     EPI_THRESH = 0,  // threshold -> bit, OR over the pool window, packed store
@@ -92,24 +92,25 @@ struct BgemmParams {
     int ws_is_dot;  // workspace holds +-1 dot products (matrix-core engines) instead of popcounts
 };
 
-// One residual value in either storage format (TCBNN_RES_I32: int32 [pix][ch][B];
-// TCBNN_RES_I16: int16 [pix][ceil(ch/2)][B][2], channel 2k in the low half of a word).
+// One residual value in either storage format.  Both interleave small groups of channels below
+// the batch index, so that a lane (= image) reads or writes 16 contiguous bytes per access:
+//   TCBNN_RES_I32: int32 [pix][ceil(ch/4)][B][4]     TCBNN_RES_I16: int16 [pix][ceil(ch/8)][B][8]
+__device__ __forceinline__ size_t residual_index(int fmt, size_t pix, int channels, int c, int batch, int b) {
+    if (fmt == TCBNN_RES_I16) return ((pix * (size_t)((channels + 7) / 8) + (c >> 3)) * batch + b) * 8 + (c & 7);
+    return ((pix * (size_t)((channels + 3) / 4) + (c >> 2)) * batch + b) * 4 + (c & 3);
+}
 __device__ __forceinline__ int residual_load(const int32_t* __restrict__ base, int fmt, size_t pix, int channels,
                                              int c, int batch, int b) {
-    if (fmt == TCBNN_RES_I16) {
-        const int16_t* s = reinterpret_cast<const int16_t*>(base);
-        return s[((pix * (size_t)((channels + 1) / 2) + (c >> 1)) * batch + b) * 2 + (c & 1)];
-    }
-    return base[(pix * channels + c) * batch + b];
+    const size_t i = residual_index(fmt, pix, channels, c, batch, b);
+    return fmt == TCBNN_RES_I16 ? (int)reinterpret_cast<const int16_t*>(base)[i] : base[i];
 }
 __device__ __forceinline__ void residual_store(int32_t* __restrict__ base, int fmt, size_t pix, int channels, int c,
                                                int batch, int b, int v) {
-    if (fmt == TCBNN_RES_I16) {
-        int16_t* s = reinterpret_cast<int16_t*>(base);
-        s[((pix * (size_t)((channels + 1) / 2) + (c >> 1)) * batch + b) * 2 + (c & 1)] = (int16_t)v;
-    } else {
-        base[(pix * channels + c) * batch + b] = v;
-    }
+    const size_t i = residual_index(fmt, pix, channels, c, batch, b);
+    if (fmt == TCBNN_RES_I16)
+        reinterpret_cast<int16_t*>(base)[i] = (int16_t)v;
+    else
+        base[i] = v;
 }
 
 int launch_bgemm_popc(const BgemmParams& p, hipStream_t stream);

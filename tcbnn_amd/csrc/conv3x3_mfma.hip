@@ -43,13 +43,15 @@ constexpr int RM_POOLED = 2;  // residual injected as the 2x2 max of a source tw
 constexpr int waves_hint(int spt, int rm, int nt) { return rm == RM_PLAIN && spt * nt <= 2 ? 3 : 2; }
 
 // SPT = k-steps (64 bits) per filter tap = Cin / 64; MT = 32-image tiles per wave (2 for plain
-// layers, 1 for residual layers); NT = 32-channel tiles per wave.
-template <int SPT, int RM, int MT, int NT>
+// layers, 1 for residual layers); NT = 32-channel tiles per wave; R16 = the injected residual is
+// stored as int16 (half the registers hold it while it is in flight).
+template <int SPT, int RM, int MT, int NT, bool R16>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(waves_hint(SPT, RM, NT)))) void
 conv3x3_mfma_f4_kernel(
     const BgemmParams p, const uint32_t* __restrict__ act, const uint32_t* __restrict__ wgt,
     const float* __restrict__ bnp, const int32_t* __restrict__ rin, int32_t* __restrict__ rout, int res_lim,
-    int rin_fmt, int rout_fmt, int n_groups, int b_groups, int pix_streams) {
+    int rin_fmt, int rout_fmt, unsigned act_bytes, unsigned rin_bytes, unsigned rout_bytes, unsigned bits_bytes,
+    int n_groups, int b_groups, int pix_streams) {
     static_assert(RM == RM_NONE || MT == 1, "residual instantiations own one image tile per wave");
     constexpr int TPC = SPT >= 4 ? 3 : 9;  // taps per prefetch chunk (a filter row, or all of it)
     constexpr int NCH = 9 / TPC;           // chunks per tile
@@ -100,6 +102,22 @@ conv3x3_mfma_f4_kernel(
         bload[mt] = min(bimg[mt], p.B - 1);
     }
 
+    // Buffer addressing for every global access of the tile loop: a descriptor per tensor, one
+    // per-lane byte offset (a constant of the lane) and a wave-uniform scalar offset per access, so
+    // that addresses cost scalar adds only.  A lane that must not take part carries an offset beyond
+    // every descriptor (the host checked the tensors are below 2 GiB): its load returns 0, its
+    // store is dropped.
+    constexpr unsigned kOutOfRange = 0x80000000u;
+    auto make_rsrc = [](const void* ptr, unsigned bytes) {
+        return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(ptr), 0, (int)bytes, 0x00020000);
+    };
+    const __amdgpu_buffer_rsrc_t r_act = make_rsrc(act, act_bytes), r_rin = make_rsrc(rin, rin_bytes),
+                                 r_rout = make_rsrc(rout, rout_bytes), r_bits = make_rsrc(p.out_bits, bits_bytes);
+    const unsigned row_b = (unsigned)p.B * 4u;  // bytes between consecutive words / channels of an image
+    unsigned voff_act[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) voff_act[mt] = ((unsigned)h * (unsigned)p.B + (unsigned)bload[mt]) * 4u;
+
     // Requests the activation words of chunk `chunk` of the tile at pixel (yy, xx); returns the
     // wave-uniform mask of its in-frame taps.
     auto load_chunk = [&](int yy, int xx, int chunk, uint32_t (*buf)[MT]) {
@@ -111,12 +129,13 @@ conv3x3_mfma_f4_kernel(
             const int ay = yy * p.stride_h - p.pad_h + r, ax = xx * p.stride_w - p.pad_w + s;
             if (ay >= 0 && ay < p.H && ax >= 0 && ax < p.W) {
                 mask |= 1u << tl;
-                const uint32_t* src = act + ((size_t)(ay * p.W + ax) * p.cw + h) * p.B;
+                const unsigned soff = (unsigned)(ay * p.W + ax) * (unsigned)p.cw * row_b;  // uniform
 #pragma unroll
                 for (int t = 0; t < SPT; ++t)
 #pragma unroll
                     for (int mt = 0; mt < MT; ++mt)
-                        buf[tl * SPT + t][mt] = src[(size_t)(2 * t) * p.B + bload[mt]];
+                        buf[tl * SPT + t][mt] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(
+                            r_act, (int)voff_act[mt], (int)(soff + (unsigned)(2 * t) * row_b), 0);
             }
         }
         return mask;
@@ -155,97 +174,95 @@ conv3x3_mfma_f4_kernel(
 
     // ---- residual operand (kernel.cuh:770-794).  A lane owns channels n0 + 32 nt + 16 h + v of
     // image bload[0]; every load is a wave-uniform base plus this per-lane element offset.
-    // TCBNN_RES_I16 tensors hold two channels per word: 8 loads per channel tile instead of 16,
-    // unpacked (and, for a pooled source, reduced) by finish_residual.
+    // A lane's 16 values arrive as 16 (int32) or 8 (int16 pairs) words; a plain operand stays in
+    // that raw form until its epilogue, a pooled one is reduced to 16 ints by finish_residual.
     constexpr int NRV = RM != RM_NONE ? NT : 1;
     constexpr int NTMP = RM == RM_POOLED ? 3 : 1;
-    int tmp[NTMP][NRV][16];  // pooled: the other three pixels of the 2x2 window
-    const unsigned lane_off = (unsigned)(16 * h) * (unsigned)p.B + (unsigned)bload[0];
-    const unsigned lane_off16 = (unsigned)(8 * h) * (unsigned)p.B + (unsigned)bload[0];
+    constexpr int NRAW = R16 ? 8 : 16;                    // words loaded per channel tile
+    constexpr int NW = RM == RM_POOLED ? 16 : NRAW;       // words kept per channel tile
+    int tmp[NTMP][NRV][NRAW];  // pooled: the other three pixels of the 2x2 window
+    // A lane's 16 channels are 4 groups of 4 (int32) or 2 groups of 8 (int16): 16 bytes each.
+    const unsigned lane_off = ((unsigned)(4 * h) * (unsigned)p.B + (unsigned)bload[0]) * 16u;
+    const unsigned lane_off16 = ((unsigned)(2 * h) * (unsigned)p.B + (unsigned)bload[0]) * 16u;
+    const unsigned grp_b = (unsigned)p.B * 16u;  // bytes between consecutive channel groups
 
-    auto request_residual = [&](int yy, int xx, int (*rv)[16]) {
+    auto request_residual = [&](int yy, int xx, int (*rv)[NW]) {
         if constexpr (RM != RM_NONE) {
-            const bool i16 = rin_fmt == TCBNN_RES_I16;  // wave-uniform
-            // words per source pixel, words between channel rows of a lane, lane offset
-            const size_t ch_b = (size_t)(i16 ? (p.res_in_ch + 1) / 2 : p.res_in_ch) * p.B;
+            constexpr bool i16 = R16;
+            // bytes per source pixel; per-lane offset; 128-bit loads per channel tile.  Groups past the
+            // source's channels read the neighbouring pixel or (at the end of the tensor) zeros; their
+            // values are cleared by finish_residual.
+            const unsigned ch_b = (unsigned)(i16 ? (p.res_in_ch + 7) / 8 : (p.res_in_ch + 3) / 4) * grp_b;
             const unsigned loff = i16 ? lane_off16 : lane_off;
-            const int nld = i16 ? 8 : 16;
-            const size_t pix = RM == RM_POOLED ? ((size_t)(2 * yy) * (2 * p.PW) + 2 * xx) : ((size_t)yy * p.PW + xx);
-            const size_t ddy = (size_t)(2 * p.PW) * ch_b;
+            constexpr int nld = i16 ? 2 : 4;
+            const unsigned pix = RM == RM_POOLED ? (unsigned)(2 * yy) * (unsigned)(2 * p.PW) + (unsigned)(2 * xx)
+                                                 : (unsigned)yy * (unsigned)p.PW + (unsigned)xx;
+            const unsigned ddy = (unsigned)(2 * p.PW) * ch_b;
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
                 const int cb = n0 + nt * 32;
-                const int32_t* __restrict__ base = rin + pix * ch_b + (size_t)(i16 ? cb / 2 : cb) * p.B;  // uniform
-                if (cb + 32 <= res_lim) {
+                if (cb >= res_lim) {  // uniform: this channel tile receives no residual
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        if (v >= nld) continue;  // uniform
-                        const int32_t* s = base + (size_t)v * p.B;
-                        rv[nt][v] = s[loff];
-                        if constexpr (RM == RM_POOLED) {
-                            tmp[0][nt][v] = s[ch_b + loff];
-                            tmp[1][nt][v] = s[ddy + loff];
-                            tmp[2][nt][v] = s[ddy + ch_b + loff];
-                        }
+                    for (int v = 0; v < NW; ++v) rv[nt][v] = 0;
+                    if constexpr (RM == RM_POOLED) {
+#pragma unroll
+                        for (int v = 0; v < NRAW; ++v) tmp[0][nt][v] = tmp[1][nt][v] = tmp[2][nt][v] = 0;
                     }
-                } else {
+                    continue;
+                }
+                const unsigned base = pix * ch_b + (unsigned)(i16 ? cb / 8 : cb / 4) * grp_b;  // uniform
+                auto load4 = [&](int* dst, unsigned so) {
+                    const v4i q = __builtin_amdgcn_raw_buffer_load_b128(r_rin, (int)loff, (int)so, 0);
+                    dst[0] = q[0];
+                    dst[1] = q[1];
+                    dst[2] = q[2];
+                    dst[3] = q[3];
+                };
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        if (v >= nld) continue;  // uniform
-                        const bool ok = cb + 16 * h + (i16 ? 2 * v : v) < res_lim;
-                        const int32_t* s = base + (size_t)v * p.B;
-                        rv[nt][v] = ok ? s[loff] : 0;
-                        if constexpr (RM == RM_POOLED) {
-                            tmp[0][nt][v] = ok ? s[ch_b + loff] : 0;
-                            tmp[1][nt][v] = ok ? s[ddy + loff] : 0;
-                            tmp[2][nt][v] = ok ? s[ddy + ch_b + loff] : 0;
-                        }
+                for (int g = 0; g < 4; ++g) {
+                    if (g >= nld) continue;  // uniform
+                    const unsigned so = base + (unsigned)g * grp_b;
+                    load4(&rv[nt][4 * g], so);
+                    if constexpr (RM == RM_POOLED) {
+                        load4(&tmp[0][nt][4 * g], so + ch_b);
+                        load4(&tmp[1][nt][4 * g], so + ddy);
+                        load4(&tmp[2][nt][4 * g], so + ddy + ch_b);
                     }
                 }
             }
         }
     };
-    // Turns what request_residual loaded into one int per channel: unpack 16-bit pairs, take the
-    // 2x2 maximum of a pooled source, clear channels that receive no residual.
-    auto finish_residual = [&](int (*rv)[16]) {
-        if constexpr (RM != RM_NONE) {
-            if (rin_fmt == TCBNN_RES_I16) {
+    // Pooled source: 2x2 maximum of the four pixels, one int per channel (16-bit pairs unpacked).
+    auto finish_residual = [&](int (*rv)[NW]) {
+        if constexpr (RM == RM_POOLED) {
 #pragma unroll
-                for (int nt = 0; nt < NT; ++nt) {
-                    const int cb = n0 + nt * 32;
+            for (int nt = 0; nt < NT; ++nt) {
+                if constexpr (R16) {
 #pragma unroll
                     for (int k = 7; k >= 0; --k) {  // downwards: slot k is read before 2k, 2k+1 are written
                         const int w = rv[nt][k];
                         int lo = (int)(short)(w & 0xffff), hi = w >> 16;
-                        if constexpr (RM == RM_POOLED) {
 #pragma unroll
-                            for (int t = 0; t < 3; ++t) {
-                                const int wt = tmp[t][nt][k];
-                                lo = max(lo, (int)(short)(wt & 0xffff));
-                                hi = max(hi, wt >> 16);
-                            }
-                        }
-                        if (cb + 32 > res_lim) {  // uniform: partial channel tile
-                            if (cb + 16 * h + 2 * k >= res_lim) lo = 0;
-                            if (cb + 16 * h + 2 * k + 1 >= res_lim) hi = 0;
+                        for (int t = 0; t < 3; ++t) {
+                            const int wt = tmp[t][nt][k];
+                            lo = max(lo, (int)(short)(wt & 0xffff));
+                            hi = max(hi, wt >> 16);
                         }
                         rv[nt][2 * k] = lo;
                         rv[nt][2 * k + 1] = hi;
                     }
-                }
-            } else if constexpr (RM == RM_POOLED) {
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt)
+                } else {
 #pragma unroll
                     for (int v = 0; v < 16; ++v)
                         rv[nt][v] = max(max(rv[nt][v], tmp[0][nt][v]), max(tmp[1][nt][v], tmp[2][nt][v]));
+                }
             }
         }
     };
 
-    auto epilogue = [&](int yy, int xx, int (*rv)[16]) {
-        const size_t pix = (size_t)yy * p.PW + xx;
-        uint32_t* dst_bits = p.out_bits + pix * p.bits_pix_stride;
+    auto epilogue = [&](int yy, int xx, int (*rv)[NW]) {
+        const unsigned pix = (unsigned)yy * (unsigned)p.PW + (unsigned)xx;
+        const unsigned bits_pix = pix * (unsigned)p.bits_pix_stride * 4u;  // uniform
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
             const int cbase = n0 + nt * 32 + 16 * h;  // this lane's channels: cbase + v
@@ -269,29 +286,48 @@ conv3x3_mfma_f4_kernel(
                 uint32_t hw = 0;
                 if constexpr (RM != RM_NONE) {
                     int res[16];
+                    const bool partial = n0 + nt * 32 + 32 > res_lim;  // uniform (also when no residual: zeros)
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) res[v] = (int)acc[mt][nt][v] + rv[nt][v];
-                    if (rout != nullptr && b_ok) {
-                        if (rout_fmt == TCBNN_RES_I16) {  // two channels per word
-                            int32_t* __restrict__ dst =
-                                rout + (pix * ((p.N + 1) / 2) + (n0 + nt * 32) / 2) * p.B;  // wave-uniform
-                            const unsigned off = (unsigned)(8 * h) * (unsigned)p.B + (unsigned)b;
+                    for (int v = 0; v < 16; ++v) {
+                        int val;
+                        if constexpr (RM == RM_PLAIN && R16) {
+                            const int w = rv[nt][v >> 1];
+                            val = (v & 1) ? (w >> 16) : (int)(short)(w & 0xffff);
+                        } else {
+                            val = rv[nt][v];
+                        }
+                        if (partial && cbase + v >= res_lim) val = 0;
+                        res[v] = (int)acc[mt][nt][v] + val;
+                    }
+                    if (rout != nullptr) {
+                        if (!n_full) {  // uniform: channels past N are stored as 0 inside a group
 #pragma unroll
-                            for (int k = 0; k < 8; ++k) {
-                                const int c0 = cbase + 2 * k;
-                                const int hi = (n_full || c0 + 1 < p.N) ? res[2 * k + 1] : 0;
-                                if (n_full || c0 < p.N) (dst + (size_t)k * p.B)[off] = (res[2 * k] & 0xffff) | (hi << 16);
+                            for (int v = 0; v < 16; ++v)
+                                if (cbase + v >= p.N) res[v] = 0;
+                        }
+                        if (rout_fmt == TCBNN_RES_I16) {  // groups of 8 channels, two per word
+                            const unsigned so = (pix * (unsigned)((p.N + 7) / 8) + (unsigned)((n0 + nt * 32) / 8)) * grp_b;
+                            const unsigned vo = b_ok ? ((unsigned)(2 * h) * (unsigned)p.B + (unsigned)b) * 16u : kOutOfRange;
+#pragma unroll
+                            for (int g = 0; g < 2; ++g) {
+                                v4i q;
+#pragma unroll
+                                for (int k = 0; k < 4; ++k)
+                                    q[k] = (res[8 * g + 2 * k] & 0xffff) | (res[8 * g + 2 * k + 1] << 16);
+                                // a group that starts past N belongs to the next pixel: not written
+                                __builtin_amdgcn_raw_buffer_store_b128(
+                                    q, r_rout, (int)(n_full || cbase + 8 * g < p.N ? vo : kOutOfRange),
+                                    (int)(so + (unsigned)g * grp_b), 0);
                             }
                         } else {
-                            int32_t* __restrict__ dst = rout + (pix * p.N + n0 + nt * 32) * p.B;  // wave-uniform
-                            const unsigned off = (unsigned)(16 * h) * (unsigned)p.B + (unsigned)b;
-                            if (n_full) {
+                            const unsigned so = (pix * (unsigned)((p.N + 3) / 4) + (unsigned)((n0 + nt * 32) / 4)) * grp_b;
+                            const unsigned vo = b_ok ? ((unsigned)(4 * h) * (unsigned)p.B + (unsigned)b) * 16u : kOutOfRange;
 #pragma unroll
-                                for (int v = 0; v < 16; ++v) (dst + (size_t)v * p.B)[off] = res[v];
-                            } else {
-#pragma unroll
-                                for (int v = 0; v < 16; ++v)
-                                    if (cbase + v < p.N) (dst + (size_t)v * p.B)[off] = res[v];
+                            for (int g = 0; g < 4; ++g) {
+                                const v4i q = {res[4 * g], res[4 * g + 1], res[4 * g + 2], res[4 * g + 3]};
+                                __builtin_amdgcn_raw_buffer_store_b128(
+                                    q, r_rout, (int)(n_full || cbase + 4 * g < p.N ? vo : kOutOfRange),
+                                    (int)(so + (unsigned)g * grp_b), 0);
                             }
                         }
                     }
@@ -311,21 +347,25 @@ conv3x3_mfma_f4_kernel(
                 }
                 const uint32_t other = (uint32_t)__shfl_xor((int)hw, 32);
                 const int w = ng * NT + nt;
-                if (h == 0 && b_ok && w < p.bits_row_words) dst_bits[(size_t)w * p.B + b] = (hw << 16) | other;
+                if (w < p.bits_row_words)  // uniform
+                    __builtin_amdgcn_raw_buffer_store_b32((int)((hw << 16) | other), r_bits,
+                                                          (int)(h == 0 && b_ok ? (unsigned)b * 4u : kOutOfRange),
+                                                          (int)(bits_pix + (unsigned)w * row_b), 0);
             }
         }
-        if (ng == n_groups - 1 && h == 0) {  // zero the pixel's padding words
+        if (ng == n_groups - 1) {  // zero the pixel's padding words
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
-                if (bimg[mt] < p.B)
-                    for (int w = max((p.N + 31) / 32, n_groups * NT); w < p.bits_row_words; ++w)
-                        dst_bits[(size_t)w * p.B + bimg[mt]] = 0;
+                for (int w = max((p.N + 31) / 32, n_groups * NT); w < p.bits_row_words; ++w)
+                    __builtin_amdgcn_raw_buffer_store_b32(
+                        0, r_bits, (int)(h == 0 && bimg[mt] < p.B ? (unsigned)bimg[mt] * 4u : kOutOfRange),
+                        (int)(bits_pix + (unsigned)w * row_b), 0);
         }
     };
 
     // ---- persistent loop over this wave's tiles, chunks double-buffered in registers
     uint32_t buf0[TPC * SPT][MT], buf1[TPC * SPT][MT];
-    int rv0[NRV][16], rv1[kAhead ? NRV : 1][kAhead ? 16 : 1];
+    int rv0[NRV][NW], rv1[kAhead ? NRV : 1][NW];
     uint32_t m0 = 0, m1 = 0;
     int chunk = 0;
     bool have = pi < npix;
@@ -338,8 +378,8 @@ conv3x3_mfma_f4_kernel(
     }
     zero_acc();
 
-    auto step = [&](uint32_t (*cur)[MT], uint32_t mcur, uint32_t (*nxt)[MT], uint32_t& mnxt, int (*rcur)[16],
-                    int (*rnxt)[16]) {
+    auto step = [&](uint32_t (*cur)[MT], uint32_t mcur, uint32_t (*nxt)[MT], uint32_t& mnxt, int (*rcur)[NW],
+                    int (*rnxt)[NW]) {
         int nchunk = chunk + 1, ny = y, nx = x, npi = pi;
         if (nchunk == NCH) {
             nchunk = 0;
@@ -365,7 +405,7 @@ conv3x3_mfma_f4_kernel(
             if (nhave) finish_residual(rnxt);
         }
         if (chunk == NCH - 1) {
-            if constexpr (!(kAhead && RM == RM_POOLED)) finish_residual(rcur);
+            if constexpr (!kAhead) finish_residual(rcur);
             epilogue(y, x, rcur);
             zero_acc();
         }
@@ -389,14 +429,30 @@ conv3x3_mfma_f4_kernel(
     }
 }
 
-template <int SPT, int RM, int MT, int NT>
+// Sizes in bytes of the tensors the kernel addresses through buffer descriptors.
+struct TensorBytes {
+    long long act, rin, rout, bits;
+};
+TensorBytes tensor_bytes(const BgemmParams& p) {
+    auto res_words = [&](long long pixels, int channels, int fmt) {
+        return pixels * (fmt == TCBNN_RES_I16 ? (channels + 7) / 8 : (channels + 3) / 4) * p.B * 4;
+    };
+    TensorBytes t;
+    t.act = 4LL * p.H * p.W * p.cw * p.B;
+    t.rin = p.res_in != nullptr ? 4 * res_words((long long)p.PH * p.PW * (p.res_pool ? 4 : 1), p.res_in_ch, p.res_in_fmt) : 0;
+    t.rout = p.res_out != nullptr ? 4 * res_words((long long)p.PH * p.PW, p.N, p.res_out_fmt) : 0;
+    t.bits = 4LL * p.PH * p.PW * p.bits_pix_stride;
+    return t;
+}
+
+template <int SPT, int RM, int MT, int NT, bool R16>
 int launch_t(const BgemmParams& p, hipStream_t stream) {
     constexpr int NQ = 9 * SPT;
     const size_t lds_bytes = (size_t)NQ * NT * 64 * 16 + NT * 32 * sizeof(float);
     static bool attr_set = false;  // per instantiation
     if (!attr_set) {
         if (int rc = check_hip(
-                hipFuncSetAttribute(reinterpret_cast<const void*>(&conv3x3_mfma_f4_kernel<SPT, RM, MT, NT>),
+                hipFuncSetAttribute(reinterpret_cast<const void*>(&conv3x3_mfma_f4_kernel<SPT, RM, MT, NT, R16>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes),
                 "hipFuncSetAttribute(MaxDynamicSharedMemorySize)"))
             return rc;
@@ -424,9 +480,10 @@ int launch_t(const BgemmParams& p, hipStream_t stream) {
     // source tensor holds (kernel.cuh:770)
     const int res_lim = p.res_in != nullptr ? std::min(std::min(p.res_limit, p.res_in_ch), p.N) : 0;
     const long long blocks = (long long)best * n_groups * b_groups;
-    hipLaunchKernelGGL((conv3x3_mfma_f4_kernel<SPT, RM, MT, NT>), dim3((unsigned)blocks), dim3(kThreads), lds_bytes,
-                       stream, p, p.act, p.wgt, p.bn, p.res_in, p.res_out, res_lim, p.res_in_fmt, p.res_out_fmt, n_groups,
-                       b_groups, best);
+    const TensorBytes tb = tensor_bytes(p);
+    hipLaunchKernelGGL((conv3x3_mfma_f4_kernel<SPT, RM, MT, NT, R16>), dim3((unsigned)blocks), dim3(kThreads), lds_bytes,
+                       stream, p, p.act, p.wgt, p.bn, p.res_in, p.res_out, res_lim, p.res_in_fmt, p.res_out_fmt,
+                       (unsigned)tb.act, (unsigned)tb.rin, (unsigned)tb.rout, (unsigned)tb.bits, n_groups, b_groups, best);
     TCBNN_LAUNCH_CHECK("conv3x3_mfma_f4_kernel");
     return TCBNN_OK;
 }
@@ -437,7 +494,7 @@ int launch_t(const BgemmParams& p, hipStream_t stream) {
 // tile (each operand fragment feeds two MFMAs) until the weights of 64 channels no longer leave
 // room for a second workgroup (Cin = 512).
 struct Pick {
-    int rm, mt, nt;
+    int rm, mt, nt, r16;
 };
 constexpr int pick_nt(int spt, int rm) {
     return rm == RM_POOLED ? 1 : (rm == RM_PLAIN ? (spt >= 4 ? 1 : 2) : (spt >= 8 ? 1 : 2));
@@ -445,32 +502,43 @@ constexpr int pick_nt(int spt, int rm) {
 Pick pick(const BgemmParams& p) {
     const int rm = p.res_in == nullptr && p.res_out == nullptr ? RM_NONE
                                                                 : (p.res_in != nullptr && p.res_pool ? RM_POOLED : RM_PLAIN);
-    return {rm, rm == RM_NONE ? 2 : 1, pick_nt(p.cw / 2, rm)};
+    return {rm, rm == RM_NONE ? 2 : 1, pick_nt(p.cw / 2, rm), p.res_in != nullptr && p.res_in_fmt == TCBNN_RES_I16};
 }
 
 template <int SPT>
 int launch_m(const BgemmParams& p, hipStream_t stream) {
-    switch (pick(p).rm) {
+    const Pick k = pick(p);
+    switch (k.rm) {
         case RM_NONE:
-            return launch_t<SPT, RM_NONE, 2, pick_nt(SPT, RM_NONE)>(p, stream);
+            return launch_t<SPT, RM_NONE, 2, pick_nt(SPT, RM_NONE), false>(p, stream);
         case RM_PLAIN:
-            return launch_t<SPT, RM_PLAIN, 1, pick_nt(SPT, RM_PLAIN)>(p, stream);
+            return k.r16 ? launch_t<SPT, RM_PLAIN, 1, pick_nt(SPT, RM_PLAIN), true>(p, stream)
+                         : launch_t<SPT, RM_PLAIN, 1, pick_nt(SPT, RM_PLAIN), false>(p, stream);
         default:
-            return launch_t<SPT, RM_POOLED, 1, pick_nt(SPT, RM_POOLED)>(p, stream);
+            return k.r16 ? launch_t<SPT, RM_POOLED, 1, pick_nt(SPT, RM_POOLED), true>(p, stream)
+                         : launch_t<SPT, RM_POOLED, 1, pick_nt(SPT, RM_POOLED), false>(p, stream);
     }
 }
 
 }  // namespace
 
+// the kernel's 32-bit buffer offsets (and its "out of range" lane offset) need every tensor below 2 GiB
+static bool within_2gib(const BgemmParams& p) {
+    const TensorBytes t = tensor_bytes(p);
+    const long long lim = 1LL << 31;
+    return t.act < lim && t.rin < lim && t.rout < lim && t.bits < lim;
+}
+
 bool conv3x3_mfma_applicable(const BgemmParams& p) {
     return p.R == 3 && p.S == 3 && p.pool_h == 1 && p.pool_w == 1 && p.mode == EPI_THRESH && p.nan_bit == 1 &&
            p.ksplit <= 1 && (p.cw == 2 || p.cw == 4 || p.cw == 8 || p.cw == 16) && p.k_tap == 32 * p.cw &&
-           (long long)p.PH * p.PW < (1 << 24);
+           (long long)p.PH * p.PW < (1 << 24) && within_2gib(p);
 }
 
 void conv3x3_mfma_kernel_name(const BgemmParams& p, char* buf, size_t len) {
     const Pick k = pick(p);
-    snprintf(buf, len, "conv3x3_mfma_f4_kernel<%d, %d, %d, %d>", p.cw / 2, k.rm, k.mt, k.nt);
+    snprintf(buf, len, "conv3x3_mfma_f4_kernel<%d, %d, %d, %d, %s>", p.cw / 2, k.rm, k.mt, k.nt,
+             k.r16 ? "true" : "false");
 }
 
 int launch_conv3x3_mfma(const BgemmParams& p, hipStream_t stream) {

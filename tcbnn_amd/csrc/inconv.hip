@@ -293,19 +293,28 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3))) v
                 }
                 out[(pix * p.ow + wi) * p.B + b] = word;
                 if (res != nullptr) {
-                    if (p.res_fmt == TCBNN_RES_I16) {  // two channels per word, even one in the low half
-                        int32_t* __restrict__ dst = res + (pix * ((p.O + 1) / 2) + wi * 16) * p.B + b;
+                    // 16 bytes per (channel group, image): 4 int32 or 8 int16; channels past O are 0
+                    int r32[32];
 #pragma unroll
-                        for (int k = 0; k < 16; ++k) {
-                            const int ch = wi * 32 + 2 * k;
-                            const int hi = ch + 1 < p.O ? (int)acc[2 * k + 1] : 0;
-                            if (ch < p.O) dst[(size_t)k * p.B] = ((int)acc[2 * k] & 0xffff) | (hi << 16);
-                        }
+                    for (int n = 0; n < 32; ++n) r32[n] = wi * 32 + n < p.O ? (int)acc[n] : 0;
+                    int4* __restrict__ dst = reinterpret_cast<int4*>(res);
+                    if (p.res_fmt == TCBNN_RES_I16) {
+                        const size_t g0 = (pix * ((p.O + 7) / 8) + wi * 4) * p.B + b;
+#pragma unroll
+                        for (int g = 0; g < 4; ++g)
+                            if (wi * 32 + 8 * g < p.O)
+                                dst[g0 + (size_t)g * p.B] =
+                                    make_int4((r32[8 * g] & 0xffff) | (r32[8 * g + 1] << 16),
+                                              (r32[8 * g + 2] & 0xffff) | (r32[8 * g + 3] << 16),
+                                              (r32[8 * g + 4] & 0xffff) | (r32[8 * g + 5] << 16),
+                                              (r32[8 * g + 6] & 0xffff) | (r32[8 * g + 7] << 16));
                     } else {
-                        int32_t* __restrict__ dst = res + (pix * p.O + wi * 32) * p.B + b;
+                        const size_t g0 = (pix * ((p.O + 3) / 4) + wi * 8) * p.B + b;
 #pragma unroll
-                        for (int n = 0; n < 32; ++n)
-                            if (wi * 32 + n < p.O) dst[(size_t)n * p.B] = (int)acc[n];
+                        for (int g = 0; g < 8; ++g)
+                            if (wi * 32 + 4 * g < p.O)
+                                dst[g0 + (size_t)g * p.B] =
+                                    make_int4(r32[4 * g], r32[4 * g + 1], r32[4 * g + 2], r32[4 * g + 3]);
                     }
                 }
             }

@@ -127,7 +127,7 @@ size_t tcbnn_inconv_filter_words(int r, int s, int in_ch, int out_ch) {
 size_t tcbnn_residual_bytes(int height, int width, int channels, int batch, int format) {
     if (height <= 0 || width <= 0 || channels <= 0 || batch <= 0) return 0;
     const size_t pix_b = (size_t)height * width * batch;
-    return format == TCBNN_RES_I16 ? pix_b * ((channels + 1) / 2) * 4 : pix_b * channels * 4;
+    return pix_b * 16 * (format == TCBNN_RES_I16 ? (channels + 7) / 8 : (channels + 3) / 4);
 }
 
 int tcbnn_inconv_residual_bound(int filter_height, int filter_width, float input_abs_max) {

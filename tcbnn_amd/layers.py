@@ -324,12 +324,11 @@ class _ConvGeometry:
     def download_residual(self):
         """Saved residual as int32 [P][Q][B][O] (host transpose of the engine's layouts)."""
         P, Q, O, B = self.buf_height, self.buf_width, self.output_channels, self.batch
-        if self.output_residual_gpu.format == _lib.RES_I16:
-            eng = self.output_residual_gpu.to_numpy(np.int16, (P, Q, (O + 1) // 2, B, 2))
-            return np.ascontiguousarray(
-                eng.transpose(0, 1, 3, 2, 4).reshape(P, Q, B, 2 * ((O + 1) // 2))[..., :O].astype(np.int32))
-        eng = self.output_residual_gpu.to_numpy(np.int32, (P, Q, O, B))
-        return np.ascontiguousarray(eng.transpose(0, 1, 3, 2))
+        # engine layouts: int32 [P][Q][ceil(O/4)][B][4] or int16 [P][Q][ceil(O/8)][B][8]
+        grp, dt = (8, np.int16) if self.output_residual_gpu.format == _lib.RES_I16 else (4, np.int32)
+        ng = (O + grp - 1) // grp
+        eng = self.output_residual_gpu.to_numpy(dt, (P, Q, ng, B, grp))
+        return np.ascontiguousarray(eng.transpose(0, 1, 3, 2, 4).reshape(P, Q, B, ng * grp)[..., :O].astype(np.int32))
 
     def download_residual_reference(self):
         """Saved residual in the reference layout int32 [P][Q][PAD8(B)][PAD128(O)]."""

@@ -143,13 +143,11 @@ def _residual_source(res_in, fmt):
     """Device copy of a residual [Hr][Wr][B][C] in the engine layout of format `fmt`, tagged the way the
     layer classes tag the tensors they produce (channel count, format, bound of |value|)."""
     hr, wr, b, c = res_in.shape
-    if fmt == 1:  # int16 [Hr][Wr][ceil(C/2)][B][2], channel 2k in the low half
-        c2 = (c + 1) // 2
-        pad = np.zeros((hr, wr, b, 2 * c2), np.int16)
-        pad[..., :c] = res_in
-        host = np.ascontiguousarray(pad.reshape(hr, wr, b, c2, 2).transpose(0, 1, 3, 2, 4))
-    else:         # int32 [Hr][Wr][C][B]
-        host = np.ascontiguousarray(res_in.astype(np.int32).transpose(0, 1, 3, 2))
+    grp, dt = (8, np.int16) if fmt == 1 else (4, np.int32)  # [Hr][Wr][ceil(C/grp)][B][grp]
+    ng = (c + grp - 1) // grp
+    pad = np.zeros((hr, wr, b, ng * grp), dt)
+    pad[..., :c] = res_in
+    host = np.ascontiguousarray(pad.reshape(hr, wr, b, ng, grp).transpose(0, 1, 3, 2, 4))
     rbuf = gpuops.dev(host)
     rbuf.channels, rbuf.format, rbuf.bound = c, fmt, int(np.abs(res_in).max())
     return rbuf
@@ -277,8 +275,8 @@ def test_residual_format_follows_the_bound(gpu):
     assert lib.tcbnn_inconv_residual_bound(7, 7, float("nan")) == 2 ** 31 - 1
     assert 147 * 5 <= lib.tcbnn_inconv_residual_bound(7, 7, 5.0) <= 147 * 5 + 3
     assert lib.tcbnn_conv_residual_bound(512, 3, 3, 1000) == 5608
-    assert lib.tcbnn_residual_bytes(3, 5, 7, 11, 0) == 3 * 5 * 7 * 11 * 4
-    assert lib.tcbnn_residual_bytes(3, 5, 7, 11, 1) == 3 * 5 * 4 * 11 * 4
+    assert lib.tcbnn_residual_bytes(3, 5, 7, 11, 0) == 3 * 5 * 2 * 11 * 16  # 7 channels: 2 groups of 4
+    assert lib.tcbnn_residual_bytes(3, 5, 9, 11, 1) == 3 * 5 * 2 * 11 * 16  # 9 channels: 2 groups of 8
     r = rng(77)
     b, h, cout = 4, 16, 64
     f = rm.pm1(r, (7, 7, 3, cout))
