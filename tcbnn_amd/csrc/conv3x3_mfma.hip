@@ -21,6 +21,7 @@
 //     contiguous runs.
 #include <algorithm>
 #include <cmath>
+#include <type_traits>
 
 #include "common.h"
 #include "mfma_util.h"
@@ -260,98 +261,111 @@ conv3x3_mfma_f4_kernel(
         }
     };
 
+    // One channel tile of the epilogue.  FAST (wave-uniform choice): all 32 channels exist and, with a
+    // residual, all of them receive it, so no per-channel condition is evaluated at all.
+    auto epilogue_tile = [&](auto fast_tag, int nt, unsigned pix, unsigned bits_pix, int (*rv)[NW]) {
+        constexpr bool FAST = decltype(fast_tag)::value;
+        const int cbase = n0 + nt * 32 + 16 * h;  // this lane's channels: cbase + v
+        float thr[16];
+        {
+            const float4* t4 = reinterpret_cast<const float4*>(lds_thr + nt * 32 + 16 * h);
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const float4 tv = t4[k];
+                thr[4 * k + 0] = tv.x;
+                thr[4 * k + 1] = tv.y;
+                thr[4 * k + 2] = tv.z;
+                thr[4 * k + 3] = tv.w;
+            }
+        }
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int b = bimg[mt];
+            const bool b_ok = b < p.B;
+            uint32_t hw = 0;
+            if constexpr (RM != RM_NONE) {
+                int res[16];
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    int val;
+                    if constexpr (RM == RM_PLAIN && R16) {
+                        const int w = rv[nt][v >> 1];
+                        val = (v & 1) ? (w >> 16) : (int)(short)(w & 0xffff);
+                    } else {
+                        val = rv[nt][v];
+                    }
+                    if constexpr (!FAST) {
+                        if (cbase + v >= res_lim) val = 0;
+                    }
+                    res[v] = (int)acc[mt][nt][v] + val;
+                }
+                if (rout != nullptr) {
+                    if constexpr (!FAST) {  // channels past N are stored as 0 inside a group
+#pragma unroll
+                        for (int v = 0; v < 16; ++v)
+                            if (cbase + v >= p.N) res[v] = 0;
+                    }
+                    if (rout_fmt == TCBNN_RES_I16) {  // groups of 8 channels, two per word
+                        const unsigned so = (pix * (unsigned)((p.N + 7) / 8) + (unsigned)((n0 + nt * 32) / 8)) * grp_b;
+                        const unsigned vo = b_ok ? ((unsigned)(2 * h) * (unsigned)p.B + (unsigned)b) * 16u : kOutOfRange;
+#pragma unroll
+                        for (int g = 0; g < 2; ++g) {
+                            v4i q;
+#pragma unroll
+                            for (int k = 0; k < 4; ++k)
+                                q[k] = (res[8 * g + 2 * k] & 0xffff) | (res[8 * g + 2 * k + 1] << 16);
+                            // a group that starts past N belongs to the next pixel: not written
+                            __builtin_amdgcn_raw_buffer_store_b128(
+                                q, r_rout, (int)(FAST || cbase + 8 * g < p.N ? vo : kOutOfRange),
+                                (int)(so + (unsigned)g * grp_b), 0);
+                        }
+                    } else {
+                        const unsigned so = (pix * (unsigned)((p.N + 3) / 4) + (unsigned)((n0 + nt * 32) / 4)) * grp_b;
+                        const unsigned vo = b_ok ? ((unsigned)(4 * h) * (unsigned)p.B + (unsigned)b) * 16u : kOutOfRange;
+#pragma unroll
+                        for (int g = 0; g < 4; ++g) {
+                            const v4i q = {res[4 * g], res[4 * g + 1], res[4 * g + 2], res[4 * g + 3]};
+                            __builtin_amdgcn_raw_buffer_store_b128(
+                                q, r_rout, (int)(FAST || cbase + 4 * g < p.N ? vo : kOutOfRange),
+                                (int)(so + (unsigned)g * grp_b), 0);
+                        }
+                    }
+                }
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const uint32_t bit = ((FAST || cbase + v < p.N) && !((float)res[v] < thr[v])) ? 1u : 0u;
+                    hw = hw + hw + bit;
+                }
+            } else {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    // the accumulator is the exact integer sum: compare it directly
+                    const uint32_t bit = ((FAST || cbase + v < p.N) && !(acc[mt][nt][v] < thr[v])) ? 1u : 0u;
+                    hw = hw + hw + bit;
+                }
+            }
+            const uint32_t other = (uint32_t)__shfl_xor((int)hw, 32);
+            const int w = ng * NT + nt;
+            if (w < p.bits_row_words)  // uniform
+                __builtin_amdgcn_raw_buffer_store_b32((int)((hw << 16) | other), r_bits,
+                                                      (int)(h == 0 && b_ok ? (unsigned)b * 4u : kOutOfRange),
+                                                      (int)(bits_pix + (unsigned)w * row_b), 0);
+        }
+    };
+
     auto epilogue = [&](int yy, int xx, int (*rv)[NW]) {
         const unsigned pix = (unsigned)yy * (unsigned)p.PW + (unsigned)xx;
         const unsigned bits_pix = pix * (unsigned)p.bits_pix_stride * 4u;  // uniform
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
-            const int cbase = n0 + nt * 32 + 16 * h;  // this lane's channels: cbase + v
-            const bool n_full = n0 + nt * 32 + 32 <= p.N;  // wave-uniform
-            float thr[16];
-            {
-                const float4* t4 = reinterpret_cast<const float4*>(lds_thr + nt * 32 + 16 * h);
-#pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    const float4 tv = t4[k];
-                    thr[4 * k + 0] = tv.x;
-                    thr[4 * k + 1] = tv.y;
-                    thr[4 * k + 2] = tv.z;
-                    thr[4 * k + 3] = tv.w;
-                }
-            }
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                const int b = bimg[mt];
-                const bool b_ok = b < p.B;
-                uint32_t hw = 0;
-                if constexpr (RM != RM_NONE) {
-                    int res[16];
-                    const bool partial = n0 + nt * 32 + 32 > res_lim;  // uniform (also when no residual: zeros)
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        int val;
-                        if constexpr (RM == RM_PLAIN && R16) {
-                            const int w = rv[nt][v >> 1];
-                            val = (v & 1) ? (w >> 16) : (int)(short)(w & 0xffff);
-                        } else {
-                            val = rv[nt][v];
-                        }
-                        if (partial && cbase + v >= res_lim) val = 0;
-                        res[v] = (int)acc[mt][nt][v] + val;
-                    }
-                    if (rout != nullptr) {
-                        if (!n_full) {  // uniform: channels past N are stored as 0 inside a group
-#pragma unroll
-                            for (int v = 0; v < 16; ++v)
-                                if (cbase + v >= p.N) res[v] = 0;
-                        }
-                        if (rout_fmt == TCBNN_RES_I16) {  // groups of 8 channels, two per word
-                            const unsigned so = (pix * (unsigned)((p.N + 7) / 8) + (unsigned)((n0 + nt * 32) / 8)) * grp_b;
-                            const unsigned vo = b_ok ? ((unsigned)(2 * h) * (unsigned)p.B + (unsigned)b) * 16u : kOutOfRange;
-#pragma unroll
-                            for (int g = 0; g < 2; ++g) {
-                                v4i q;
-#pragma unroll
-                                for (int k = 0; k < 4; ++k)
-                                    q[k] = (res[8 * g + 2 * k] & 0xffff) | (res[8 * g + 2 * k + 1] << 16);
-                                // a group that starts past N belongs to the next pixel: not written
-                                __builtin_amdgcn_raw_buffer_store_b128(
-                                    q, r_rout, (int)(n_full || cbase + 8 * g < p.N ? vo : kOutOfRange),
-                                    (int)(so + (unsigned)g * grp_b), 0);
-                            }
-                        } else {
-                            const unsigned so = (pix * (unsigned)((p.N + 3) / 4) + (unsigned)((n0 + nt * 32) / 4)) * grp_b;
-                            const unsigned vo = b_ok ? ((unsigned)(4 * h) * (unsigned)p.B + (unsigned)b) * 16u : kOutOfRange;
-#pragma unroll
-                            for (int g = 0; g < 4; ++g) {
-                                const v4i q = {res[4 * g], res[4 * g + 1], res[4 * g + 2], res[4 * g + 3]};
-                                __builtin_amdgcn_raw_buffer_store_b128(
-                                    q, r_rout, (int)(n_full || cbase + 4 * g < p.N ? vo : kOutOfRange),
-                                    (int)(so + (unsigned)g * grp_b), 0);
-                            }
-                        }
-                    }
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        const uint32_t bit = ((n_full || cbase + v < p.N) && !((float)res[v] < thr[v])) ? 1u : 0u;
-                        hw = hw + hw + bit;
-                    }
-                } else {
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        // the accumulator is the exact integer sum: compare it directly
-                        const uint32_t bit =
-                            ((n_full || cbase + v < p.N) && !(acc[mt][nt][v] < thr[v])) ? 1u : 0u;
-                        hw = hw + hw + bit;
-                    }
-                }
-                const uint32_t other = (uint32_t)__shfl_xor((int)hw, 32);
-                const int w = ng * NT + nt;
-                if (w < p.bits_row_words)  // uniform
-                    __builtin_amdgcn_raw_buffer_store_b32((int)((hw << 16) | other), r_bits,
-                                                          (int)(h == 0 && b_ok ? (unsigned)b * 4u : kOutOfRange),
-                                                          (int)(bits_pix + (unsigned)w * row_b), 0);
-            }
+            const int cb = n0 + nt * 32;
+            // uniform: every channel of the tile exists, and gets a residual if any does (a tile that
+            // gets none at all holds zeros and is fast as well)
+            const bool fast = cb + 32 <= p.N && (RM == RM_NONE || cb + 32 <= res_lim || cb >= res_lim);
+            if (fast)
+                epilogue_tile(std::true_type{}, nt, pix, bits_pix, rv);
+            else
+                epilogue_tile(std::false_type{}, nt, pix, bits_pix, rv);
         }
         if (ng == n_groups - 1) {  // zero the pixel's padding words
 #pragma unroll
