@@ -354,6 +354,10 @@ void bgemm_mfma_kernel_name(const BgemmParams& p, int variant, char* buf, size_t
         conv3x3_mfma_kernel_name(p, buf, len);
         return;
     }
+    if (variant == TCBNN_VARIANT_MFMA_F4 && fc_mfma_applicable(p)) {
+        fc_mfma_kernel_name(p, buf, len);
+        return;
+    }
     BgemmParams q = p;
     q.ksplit = mfma_ksplit(p, variant);
     snprintf(buf, len, "bgemm_mfma_kernel<%d, %d, %d>", variant == TCBNN_VARIANT_MFMA_F4 ? FMT_F4 : FMT_I8,
@@ -364,6 +368,7 @@ int launch_bgemm_mfma(const BgemmParams& p_in, int variant, hipStream_t stream) 
     if (int rc = validate_bgemm(p_in)) return rc;
     if (variant == TCBNN_VARIANT_MFMA_F4 && conv3x3_mfma_applicable(p_in))
         return launch_conv3x3_mfma(p_in, stream);
+    if (variant == TCBNN_VARIANT_MFMA_F4 && fc_mfma_applicable(p_in)) return launch_fc_mfma(p_in, stream);
     BgemmParams p = p_in;
     p.ksplit = mfma_ksplit(p, variant);
     p.ws_is_dot = 1;

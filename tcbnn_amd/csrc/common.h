@@ -126,6 +126,10 @@ void bgemm_mfma_kernel_name(const BgemmParams& p, int variant, char* buf, size_t
 bool conv3x3_mfma_applicable(const BgemmParams& p);
 int launch_conv3x3_mfma(const BgemmParams& p, hipStream_t stream);
 void conv3x3_mfma_kernel_name(const BgemmParams& p, char* buf, size_t len);
+// FP4 matrix-core kernel for small fully connected layers (K split over the waves of a workgroup)
+bool fc_mfma_applicable(const BgemmParams& p);
+int launch_fc_mfma(const BgemmParams& p, hipStream_t stream);
+void fc_mfma_kernel_name(const BgemmParams& p, char* buf, size_t len);
 // number of K splits wanted for a problem (1 = none)
 int choose_ksplit(const BgemmParams& p);
 

@@ -152,23 +152,32 @@ conv3x3_mfma_f4_kernel(
                 for (int v = 0; v < 16; ++v) acc[mt][nt][v] = 0.0f;
     };
 
+    auto compute_tap = [&](int tap, int tl, uint32_t (*buf)[MT]) {
+#pragma unroll
+        for (int t = 0; t < SPT; ++t) {
+            v4i bfrag[MT];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) bfrag[mt] = expand_f4(buf[tl * SPT + t][mt]);
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                const v4i afrag = lds_w[((tap * SPT + t) * NT + nt) * 64 + lane];
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) acc[mt][nt] = Acc<FMT_F4>::mma(afrag, bfrag[mt], acc[mt][nt]);
+            }
+        }
+    };
+    // For Cin <= 128, interior pixels (every tap of the chunk in the frame: the bulk of a layer) run one
+    // straight-line block, so that the weight fragments of the next step are read from LDS while
+    // the current MFMAs execute; border pixels test each tap.
     auto compute_chunk = [&](int chunk, uint32_t (*buf)[MT], uint32_t mask) {
+        if (SPT <= 2 && mask == (1u << TPC) - 1u) {
 #pragma unroll
-        for (int tl = 0; tl < TPC; ++tl) {
-            if (!((mask >> tl) & 1u)) continue;  // wave-uniform
-            const int tap = chunk * TPC + tl;
+            for (int tl = 0; tl < TPC; ++tl) compute_tap(chunk * TPC + tl, tl, buf);
+        } else {
 #pragma unroll
-            for (int t = 0; t < SPT; ++t) {
-                v4i bfrag[MT];
-#pragma unroll
-                for (int mt = 0; mt < MT; ++mt) bfrag[mt] = expand_f4(buf[tl * SPT + t][mt]);
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt) {
-                    const v4i afrag = lds_w[((tap * SPT + t) * NT + nt) * 64 + lane];
-#pragma unroll
-                    for (int mt = 0; mt < MT; ++mt)
-                        acc[mt][nt] = Acc<FMT_F4>::mma(afrag, bfrag[mt], acc[mt][nt]);
-                }
+            for (int tl = 0; tl < TPC; ++tl) {
+                if (!((mask >> tl) & 1u)) continue;  // wave-uniform
+                compute_tap(chunk * TPC + tl, tl, buf);
             }
         }
     };
