@@ -34,8 +34,25 @@ COMPUTE_PEAKS_TOPS = {
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch,
 # scaled by what the same counters read for a plain device-to-device copy of known size); the
-# runs and the scale factor are recorded in profiles/.  Keyed by kernel name; None = not measured.
-MEASURED_TRAFFIC_BYTES = {}
+# runs and the scale factors (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0) are recorded in profiles/.  Average over the
+# launches of a kernel name in one step of the default workload (ResNet-18, batch 256, FP4 engine); a kernel
+# name that is not listed (another network, batch or engine) reports null.
+MEASURED_TRAFFIC_BYTES = {
+    "inconv_tiled_kernel<16, true>": 381400712,
+    "conv3x3_mfma_f4_kernel<1, 0, 2, 2, false>": 16283847,
+    "conv3x3_mfma_f4_kernel<1, 1, 1, 2, true>": 228868160,
+    "conv3x3_mfma_f4_kernel<2, 2, 1, 1, true>": 186302646,
+    "conv3x3_mfma_f4_kernel<2, 0, 2, 2, false>": 12512218,
+    "conv3x3_mfma_f4_kernel<2, 1, 1, 2, true>": 116245214,
+    "conv3x3_mfma_f4_kernel<4, 2, 1, 1, true>": 95096837,
+    "conv3x3_mfma_f4_kernel<4, 0, 2, 2, false>": 11224199,
+    "conv3x3_mfma_f4_kernel<4, 1, 1, 1, true>": 66435010,
+    "conv3x3_mfma_f4_kernel<8, 2, 1, 1, true>": 47223952,
+    "conv3x3_mfma_f4_kernel<8, 0, 2, 1, false>": 7800695,
+    "conv3x3_mfma_f4_kernel<8, 1, 1, 1, true>": 20616829,
+    "fc_mfma_f4_kernel<0>": 8245599,
+    "fc_mfma_f4_kernel<1>": 1385636,
+}
 
 
 def layer_work(L, spec=(), res_bytes=None):
@@ -172,7 +189,7 @@ def main():
     groups = {}
     for L, layer in zip(spec, net.order):
         name = layer.kernel_name() if hasattr(layer, "kernel_name") else \
-            {"inconv": "inconv_tiled_kernel", "in": "pack_rows_kernel", "out": "bgemm (output layer)"}[L["kind"]]
+            {"in": "pack_rows_kernel"}[L["kind"]]
         w = layer_work(L, spec, res_bytes)
         g = groups.setdefault(name, dict(bops=0.0, bytes=0.0, ms=0.0, launches=0))
         g["bops"] += w["bops"]

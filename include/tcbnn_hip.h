@@ -236,12 +236,14 @@ typedef struct tcbnn_conv128_desc {
 int tcbnn_conv128_forward(const tcbnn_conv128_desc* d, void* stream);
 
 /* Name of the device kernel (as a profiler lists it, template arguments included) that
- * tcbnn_conv128_forward / tcbnn_fc128_forward would launch for this descriptor; no
+ * the corresponding *_forward call would launch for this descriptor; no
  * launch happens and no pointer is dereferenced.  No counterpart in the reference
  * (its layers are inlined device functions of one network kernel); used to match
  * per-launch timings with profiler output. */
 int tcbnn_conv128_kernel_name(const tcbnn_conv128_desc* d, char* buf, size_t len);
 int tcbnn_fc128_kernel_name(const tcbnn_fc128_desc* d, char* buf, size_t len);
+int tcbnn_out128_kernel_name(const tcbnn_out128_desc* d, char* buf, size_t len);
+int tcbnn_inconv128_kernel_name(const tcbnn_inconv128_desc* d, char* buf, size_t len);
 
 /* ------------------------------------------------ standalone GEMM / conv */
 /* C[m][n] = K - 2*popc(A[m,:] xor B[n,:]), int32 row major [M][N].  A: [K/32][M]

@@ -97,6 +97,8 @@ ABI = {
     "tcbnn_conv128_forward": (c_int, [C.POINTER(Conv128Desc), c_void_p]),
     "tcbnn_conv128_kernel_name": (c_int, [C.POINTER(Conv128Desc), C.c_char_p, c_size_t]),
     "tcbnn_fc128_kernel_name": (c_int, [C.POINTER(Fc128Desc), C.c_char_p, c_size_t]),
+    "tcbnn_out128_kernel_name": (c_int, [C.POINTER(Out128Desc), C.c_char_p, c_size_t]),
+    "tcbnn_inconv128_kernel_name": (c_int, [C.POINTER(InConv128Desc), C.c_char_p, c_size_t]),
     "tcbnn_bmm": (c_int, [c_void_p] * 3 + [c_int] * 4 + [c_void_p]),
     "tcbnn_bconv": (c_int, [c_void_p] * 3 + [c_int] * 14 + [c_void_p]),
     "tcbnn_unpack_fc_output": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),

@@ -382,12 +382,14 @@ __global__ __launch_bounds__(kThreads) void inconv_generic_kernel(const InConvPa
 
 using namespace tcbnn;
 
-extern "C" int tcbnn_inconv128_forward(const tcbnn_inconv128_desc* d, void* stream) {
+static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name_buf, size_t name_len) {
     TCBNN_NOTNULL(d);
-    TCBNN_NOTNULL(d->input);
-    TCBNN_NOTNULL(d->filter);
-    TCBNN_NOTNULL(d->bn);
-    TCBNN_NOTNULL(d->output);
+    if (name_buf == nullptr) {
+        TCBNN_NOTNULL(d->input);
+        TCBNN_NOTNULL(d->filter);
+        TCBNN_NOTNULL(d->bn);
+        TCBNN_NOTNULL(d->output);
+    }
     TCBNN_REQUIRE(d->input_channels == 3,
                   "inconv128: the first layer takes 3 input channels (kernel.cuh:620-625)");
     TCBNN_REQUIRE(d->input_height > 0 && d->input_width > 0 && d->batch > 0 &&
@@ -396,7 +398,7 @@ extern "C" int tcbnn_inconv128_forward(const tcbnn_inconv128_desc* d, void* stre
                       d->pool_width > 0,
                   "inconv128: bad shape");
     if (d->save_residual) {
-        TCBNN_NOTNULL(d->output_residual);
+        if (name_buf == nullptr) TCBNN_NOTNULL(d->output_residual);
         TCBNN_REQUIRE(d->pool_height == 1 && d->pool_width == 1,
                       "inconv128: save_residual requires pool 1x1");
     }
@@ -430,6 +432,22 @@ extern "C" int tcbnn_inconv128_forward(const tcbnn_inconv128_desc* d, void* stre
     p.OW = (p.PW + p.pool_w - 1) / p.pool_w;
 
     const bool tiled = p.pool_h == 1 && p.pool_w == 1 && (kXT - 1) * p.stride_w + p.S <= kMaxCols;
+    if (name_buf != nullptr) {  // report the kernel instead of launching it
+        if (!tiled) {
+            snprintf(name_buf, name_len, "inconv_generic_kernel");
+            return TCBNN_OK;
+        }
+        const int ncols = (kXT - 1) * p.stride_w + p.S;
+        const int rpw = (64 / ncols) / 3 * 3;
+        if (rpw >= 3 && 64LL * 3 * p.H * p.W * 4 < (1LL << 31)) {
+            const int passes = (3 * 64 + 4 * rpw - 1) / (4 * rpw);
+            snprintf(name_buf, name_len, "inconv_tiled_kernel<%d, true>", passes <= 4 ? 4 : (passes <= 8 ? 8 : 16));
+        } else {
+            snprintf(name_buf, name_len, "inconv_tiled_kernel<%d, false>",
+                     (3 * 64 * ncols + kThreads - 1) / kThreads <= 15 ? 15 : 24);
+        }
+        return TCBNN_OK;
+    }
     if (tiled) {
         const int b_tiles = (p.B + 63) / 64;
         const int x_groups = (p.PW + kXT - 1) / kXT;
@@ -477,4 +495,14 @@ extern "C" int tcbnn_inconv128_forward(const tcbnn_inconv128_desc* d, void* stre
                        (hipStream_t)stream, p);
     TCBNN_LAUNCH_CHECK("inconv_generic_kernel");
     return TCBNN_OK;
+}
+
+extern "C" int tcbnn_inconv128_forward(const tcbnn_inconv128_desc* d, void* stream) {
+    return inconv128_run(d, stream, nullptr, 0);
+}
+
+extern "C" int tcbnn_inconv128_kernel_name(const tcbnn_inconv128_desc* d, char* buf, size_t len) {
+    TCBNN_NOTNULL(buf);
+    TCBNN_REQUIRE(len > 0, "kernel_name: empty buffer");
+    return inconv128_run(d, nullptr, buf, len);
 }

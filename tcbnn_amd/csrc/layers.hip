@@ -304,6 +304,13 @@ int tcbnn_fc128_kernel_name(const tcbnn_fc128_desc* d, char* buf, size_t len) {
     return kernel_name(p, d->variant, buf, len);
 }
 
+int tcbnn_out128_kernel_name(const tcbnn_out128_desc* d, char* buf, size_t len) {
+    TCBNN_NOTNULL(d);
+    BgemmParams p = fc_problem(nullptr, nullptr, d->input_height, d->input_width, d->weight_width);
+    p.mode = EPI_AFFINE;
+    return kernel_name(p, d->variant, buf, len);
+}
+
 int tcbnn_bmm(const uint32_t* a, const uint32_t* b, int32_t* c, int m, int n, int k, int variant,
               void* stream) {
     TCBNN_NOTNULL(a);

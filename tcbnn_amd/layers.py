@@ -274,11 +274,20 @@ class Out128LayerParam:
     def get_output_gpu(self):
         return self.output_gpu
 
+    def _desc(self):
+        return _lib.Out128Desc(self.input_gpu.ptr, self.weight_gpu.ptr, self.bn_scale_gpu.ptr,
+                               self.bn_bias_gpu.ptr, self.output_gpu.ptr, self.input_height,
+                               self.input_width, self.weight_width, self.variant)
+
     def forward(self, stream=None):
-        d = _lib.Out128Desc(self.input_gpu.ptr, self.weight_gpu.ptr, self.bn_scale_gpu.ptr,
-                            self.bn_bias_gpu.ptr, self.output_gpu.ptr, self.input_height,
-                            self.input_width, self.weight_width, self.variant)
+        d = self._desc()
         check(lib.tcbnn_out128_forward(C.byref(d), _stream_handle(stream)))
+
+    def kernel_name(self):
+        buf = C.create_string_buffer(128)
+        d = self._desc()
+        check(lib.tcbnn_out128_kernel_name(C.byref(d), buf, 128))
+        return buf.value.decode()
 
     def download_output(self):
         return self.output_gpu.to_numpy(np.float32, (self.output_height, self.output_width))
@@ -432,15 +441,24 @@ class InConv128LayerParam(_ConvGeometry):
             raise _lib.TcbnnError("input magnitude exceeds the bound the residual format was chosen for")
         self.input_gpu.upload(x)
 
-    def forward(self, stream=None):
-        d = _lib.InConv128Desc(
+    def _desc(self):
+        return _lib.InConv128Desc(
             self.input_gpu.ptr, self.filter_gpu.ptr, self.bn_gpu.ptr, self.output_gpu.ptr,
             self.output_residual_gpu.ptr if self.output_residual_gpu is not None else None,
             self.input_height, self.input_width, self.input_channels, self.filter_height, self.filter_width,
             self.output_channels, self.batch, self.stride_height, self.stride_width, int(self.padding),
             self.pool_height, self.pool_width, int(self.save_residual),
             self.output_residual_gpu.format if self.output_residual_gpu is not None else 0)
+
+    def forward(self, stream=None):
+        d = self._desc()
         check(lib.tcbnn_inconv128_forward(C.byref(d), _stream_handle(stream)))
+
+    def kernel_name(self):
+        buf = C.create_string_buffer(128)
+        d = self._desc()
+        check(lib.tcbnn_inconv128_kernel_name(C.byref(d), buf, 128))
+        return buf.value.decode()
 
     def release(self):
         for b in (self.input_gpu, self.filter_gpu, self.bn_gpu, self.output_gpu, self.output_residual_gpu):
