@@ -421,6 +421,29 @@ def test_imagenet_resnet18(gpu, variant, residual_format):
     _compare_network(gpu, spec, 3, variant, residual_format)
 
 
+def test_imagenet_resnet18_batch256_every_image(gpu):
+    """Full configured size on the default engine, every one of the 256 images and every layer against the
+    oracle (packed activations and residuals bit for bit, logits to 1e-5 relative), three forward passes:
+    kernels whose lanes, tiles or workgroups are only all in use at full batch are only covered here."""
+    from tcbnn_amd import nets
+    spec = nets.imagenet_resnet_spec(batch=256)
+    weights = gpu.synthetic_weights(spec, 0)
+    x = gpu.synthetic_input(spec, 0)
+    want = orc_nets.run(spec, weights, x)
+    net = gpu.Network(spec, weights, x)
+    for _ in range(3):
+        net.forward()
+        logits = net.logits()
+        np.testing.assert_allclose(logits, want["Fout"]["out"], rtol=1e-5, atol=0)
+        for L in spec[:-1]:
+            layer, w = net.layers[L["name"]], want[L["name"]]
+            got = layer.download_packed()
+            np.testing.assert_array_equal(got, w["out"].reshape(got.shape), err_msg=L["name"])
+            if w.get("res") is not None:
+                np.testing.assert_array_equal(layer.download_residual(), w["res"], err_msg=L["name"])
+    net.release()
+
+
 @pytest.mark.parametrize("variant", VARIANTS)
 def test_imagenet_resnet18_batch256_properties(gpu, variant):
     """Full configured size: images are independent, so the first 8 images of a batch-256 run
