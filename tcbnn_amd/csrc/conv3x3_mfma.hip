@@ -314,33 +314,38 @@ conv3x3_mfma_f4_kernel(
                         for (int v = 0; v < 16; ++v)
                             if (cbase + v >= p.N) res[v] = 0;
                     }
-                    // 128-bit stores go through plain global addressing: on this hardware a buffer store of
-                    // more than 64 bits that takes its scalar offset from an SGPR still reads its data
-                    // registers after issue, and the compiler, which assumes that form is safe, lets the
-                    // next VALU instruction overwrite them (seen as rare wrong first words in lanes 12-15 of a row).
-                    char* __restrict__ rbase = reinterpret_cast<char*>(rout);
+                    // 128-bit buffer stores.  On this hardware a buffer store of more than 64 bits still reads
+                    // its data registers after issue even when its scalar offset comes from an SGPR; the
+                    // compiler assumes that form is safe and lets the very next VALU instruction overwrite
+                    // them (seen as rare wrong first words in lanes 12-15 of each 16).  The data vectors are
+                    // therefore kept alive, by the empty-but-for-wait-states asm below, until well after the
+                    // last store has issued.
+                    v4i q[4];
                     if (rout_fmt == TCBNN_RES_I16) {  // groups of 8 channels, two per word
                         const unsigned so = (pix * (unsigned)((p.N + 7) / 8) + (unsigned)((n0 + nt * 32) / 8)) * grp_b;
-                        const unsigned vo = ((unsigned)(2 * h) * (unsigned)p.B + (unsigned)b) * 16u;
+                        const unsigned vo = b_ok ? ((unsigned)(2 * h) * (unsigned)p.B + (unsigned)b) * 16u : kOutOfRange;
 #pragma unroll
                         for (int g = 0; g < 2; ++g) {
-                            v4i q;
 #pragma unroll
                             for (int k = 0; k < 4; ++k)
-                                q[k] = (res[8 * g + 2 * k] & 0xffff) | (res[8 * g + 2 * k + 1] << 16);
+                                q[g][k] = (res[8 * g + 2 * k] & 0xffff) | (res[8 * g + 2 * k + 1] << 16);
                             // a group that starts past N belongs to the next pixel: not written
-                            if (b_ok && (FAST || cbase + 8 * g < p.N))
-                                *reinterpret_cast<v4i*>(rbase + (size_t)(so + (unsigned)g * grp_b) + vo) = q;
+                            __builtin_amdgcn_raw_buffer_store_b128(
+                                q[g], r_rout, (int)(FAST || cbase + 8 * g < p.N ? vo : kOutOfRange),
+                                (int)(so + (unsigned)g * grp_b), 0);
                         }
+                        asm volatile("s_nop 4" ::"v"(q[0]), "v"(q[1]));
                     } else {
                         const unsigned so = (pix * (unsigned)((p.N + 3) / 4) + (unsigned)((n0 + nt * 32) / 4)) * grp_b;
-                        const unsigned vo = ((unsigned)(4 * h) * (unsigned)p.B + (unsigned)b) * 16u;
+                        const unsigned vo = b_ok ? ((unsigned)(4 * h) * (unsigned)p.B + (unsigned)b) * 16u : kOutOfRange;
 #pragma unroll
                         for (int g = 0; g < 4; ++g) {
-                            const v4i q = {res[4 * g], res[4 * g + 1], res[4 * g + 2], res[4 * g + 3]};
-                            if (b_ok && (FAST || cbase + 4 * g < p.N))
-                                *reinterpret_cast<v4i*>(rbase + (size_t)(so + (unsigned)g * grp_b) + vo) = q;
+                            q[g] = v4i{res[4 * g], res[4 * g + 1], res[4 * g + 2], res[4 * g + 3]};
+                            __builtin_amdgcn_raw_buffer_store_b128(
+                                q[g], r_rout, (int)(FAST || cbase + 4 * g < p.N ? vo : kOutOfRange),
+                                (int)(so + (unsigned)g * grp_b), 0);
                         }
+                        asm volatile("s_nop 4" ::"v"(q[0]), "v"(q[1]), "v"(q[2]), "v"(q[3]));
                     }
                 }
 #pragma unroll
