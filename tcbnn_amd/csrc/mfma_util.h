@@ -19,12 +19,21 @@ enum MfmaMode : int { MM_THRESH = 0, MM_THRESH_RES = 1, MM_OTHER = 2 };
 // ---- bit expansion ----------------------------------------------------------------
 // FP4: bit value 1 -> nibble 0xA (-1.0), 0 -> 0x2 (+1.0): the sign is flipped for BOTH
 // operands, so products are unchanged.  dword j takes bits {4p + (3-j)}.
+// One v_bfi_b32 per dword: D = (M & shifted) | (~M & C) with M = 0x88888888 (sign bit of every
+// nibble) and C = 0x22222222 (+1.0 in every nibble), plus the shift: 7 VALU ops per 32 values.
+// Written as asm because two different 32-bit constants do not fit one VOP3 instruction otherwise
+// (the compiler falls back to shift + and + or).
+__device__ __forceinline__ int bfi_sign_nibbles(uint32_t shifted) {
+    int d;
+    asm("v_bfi_b32 %0, %1, %2, %3" : "=v"(d) : "s"(0x88888888u), "v"(shifted), "v"(0x22222222u));
+    return d;
+}
 __device__ __forceinline__ v4i expand_f4(uint32_t x) {
     v4i r;
-    r[0] = ((x << 3) & 0x88888888u) | 0x22222222u;
-    r[1] = ((x << 2) & 0x88888888u) | 0x22222222u;
-    r[2] = ((x << 1) & 0x88888888u) | 0x22222222u;
-    r[3] = (x & 0x88888888u) | 0x22222222u;
+    r[0] = bfi_sign_nibbles(x << 3);
+    r[1] = bfi_sign_nibbles(x << 2);
+    r[2] = bfi_sign_nibbles(x << 1);
+    r[3] = bfi_sign_nibbles(x);
     return r;
 }
 // nibbles whose bit is not `valid` become FP4 zero
