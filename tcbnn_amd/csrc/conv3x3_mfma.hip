@@ -87,7 +87,12 @@ conv3x3_mfma_f4_kernel(
         }
         lds_w[f * 64 + lane] = expand_f4_masked(x, valid);
     }
-    if (tid < NT * 32) lds_thr[tid] = n0 + tid < p.N ? bnp[n0 + tid] : 0.0f;
+    // A NaN threshold always yields bit 1 (!(x < NaN)), exactly like -inf: staged as such, so that
+    // the epilogue can take the bit from the sign of x - threshold.
+    if (tid < NT * 32) {
+        const float t = n0 + tid < p.N ? bnp[n0 + tid] : 0.0f;
+        lds_thr[tid] = t != t ? -__builtin_huge_valf() : t;
+    }
     __syncthreads();
 
     const int npix = p.PH * p.PW;
@@ -348,17 +353,33 @@ conv3x3_mfma_f4_kernel(
                         asm volatile("s_nop 4" ::"v"(q[0]), "v"(q[1]), "v"(q[2]), "v"(q[3]));
                     }
                 }
+                if constexpr (FAST) {
+                    // bit = !(res < thr) = inverted sign of res - thr (never -0: equal operands give +0);
+                    // one subtract and one funnel shift per channel
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const uint32_t bit = ((FAST || cbase + v < p.N) && !((float)res[v] < thr[v])) ? 1u : 0u;
-                    hw = hw + hw + bit;
+                    for (int v = 0; v < 16; ++v)
+                        hw = __builtin_amdgcn_alignbit(hw, __float_as_uint((float)res[v] - thr[v]), 31);
+                    hw = ~hw & 0xffffu;
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const uint32_t bit = (cbase + v < p.N && !((float)res[v] < thr[v])) ? 1u : 0u;
+                        hw = hw + hw + bit;
+                    }
                 }
             } else {
+                // the accumulator is the exact integer sum: compare it directly
+                if constexpr (FAST) {
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    // the accumulator is the exact integer sum: compare it directly
-                    const uint32_t bit = ((FAST || cbase + v < p.N) && !(acc[mt][nt][v] < thr[v])) ? 1u : 0u;
-                    hw = hw + hw + bit;
+                    for (int v = 0; v < 16; ++v)
+                        hw = __builtin_amdgcn_alignbit(hw, __float_as_uint(acc[mt][nt][v] - thr[v]), 31);
+                    hw = ~hw & 0xffffu;
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const uint32_t bit = (cbase + v < p.N && !(acc[mt][nt][v] < thr[v])) ? 1u : 0u;
+                        hw = hw + hw + bit;
+                    }
                 }
             }
             const uint32_t other = (uint32_t)__shfl_xor((int)hw, 32);
