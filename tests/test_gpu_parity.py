@@ -298,6 +298,34 @@ def test_residual_format_follows_the_bound(gpu):
         layer.release()
 
 
+@pytest.mark.parametrize("variant", VARIANTS)
+@pytest.mark.parametrize("with_residual", [False, True])
+def test_conv128_special_thresholds(gpu, variant, with_residual):
+    """NaN, +-inf and exactly met thresholds (kernel.cuh:795-796: bit = (res < bn) ? 0 : 1, so NaN gives 1),
+    on full 32-channel tiles, where the matrix-core kernel derives the bit from the sign of res - bn."""
+    r = rng(99)
+    b, h, cin, cout = 40, 5, 128, 64
+    x = rm.pm1(r, (b, h, h, cin))
+    f = rm.pm1(r, (3, 3, cin, cout))
+    inp, filt = orc.pack_conv_input_nhwc(x), orc.pack_conv_filter(f)
+    src = r.integers(-500, 500, size=(h, h, b, cout)).astype(np.int32) if with_residual else None
+    kw = dict(save_residual=True, inject_residual=True, residual_channels=cout, res_in=src) if with_residual else {}
+    _, res = orc.conv128(inp, filt, np.zeros(cout, np.float32), cin, cout, 3, 3, save_residual=True,
+                         **{k: v for k, v in kw.items() if k != "save_residual"})
+    bn = r.normal(0, 30, cout).astype(np.float32)
+    bn[0:8] = np.nan
+    bn[8:12] = np.inf
+    bn[12:16] = -np.inf
+    bn[16:48] = res[2, 2, 3, 16:48]          # met exactly by one (pixel, image) each
+    bn[48:52] = res[0, 0, 0, 48:52] + 0.5    # half-way values
+    want, _ = orc.conv128(inp, filt, bn, cin, cout, 3, 3, **kw)
+    layer = _run_conv_layer(gpu, variant, x, f, bn, **({"in_fmt": 1, **kw} if with_residual else {}))
+    np.testing.assert_array_equal(layer.download_packed(), want)
+    bits = orc.unpack_bits(want, cout)       # [H][W][B][C] of +-1
+    assert (bits[..., 0:8] == 1).all() and (bits[..., 8:12] == -1).all() and (bits[..., 12:16] == 1).all()
+    layer.release()
+
+
 def test_conv128_rejects_residual_with_pooling(gpu):
     x = rm.pm1(rng(1), (8, 4, 4, 64))
     f = rm.pm1(rng(2), (3, 3, 64, 32))
