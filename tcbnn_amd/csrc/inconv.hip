@@ -126,7 +126,7 @@ typedef uint32_t u16v __attribute__((ext_vector_type(16)));
 //     ceil(192 / (4 rpw)).
 //   ROWS = false: the elements are dealt to the threads linearly, NST = ceil(3 * 64 * ncols / 256).
 template <int NST, bool ROWS>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3))) void inconv_tiled_kernel(
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS ? 4 : 3))) void inconv_tiled_kernel(
     const InConvParams p, const float* __restrict__ in, const uint4* __restrict__ masks,
     const float* __restrict__ bn, uint32_t* __restrict__ out, int32_t* __restrict__ res, int b_tiles,
     int x_groups, int y_phases, int div_magic, int rpw) {
@@ -135,17 +135,19 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(3))) v
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    // Workgroups are dealt round-robin to the 8 XCDs (each with its own L2).  When the number
-    // of image tiles divides 8, XCD slot = (image tile, row phase) and consecutive workgroups of
-    // a slot walk along x, so the input cache lines shared by neighbouring column groups are
-    // re-used in one L2 instead of being fetched into several.
+    // Workgroups are dealt round-robin to the 8 XCDs (each with its own L2).  When the number of
+    // image tiles divides 8, XCD slot = (image tile, range of column groups) and the workgroups of a
+    // slot walk along x and then down the rows, so that the input rows shared by consecutive output
+    // rows (7-row windows at stride 4 overlap by 3) and by neighbouring column groups are found in
+    // that XCD's L2 instead of being fetched from HBM again.
     int bt, xg, y;
-    if (y_phases > 0) {
+    if (y_phases > 0) {  // y_phases = column ranges per image tile
         const int slot = blockIdx.x & 7, j = blockIdx.x >> 3;
+        const int xg_per = (x_groups + y_phases - 1) / y_phases;
         bt = slot % b_tiles;
-        xg = j % x_groups;
-        y = (j / x_groups) * y_phases + slot / b_tiles;
-        if (y >= p.PH) return;  // whole workgroup: grid padding
+        xg = (slot / b_tiles) * xg_per + j % xg_per;
+        y = j / xg_per;
+        if (xg >= x_groups) return;  // whole workgroup: grid padding
     } else {
         bt = blockIdx.x % b_tiles;
         xg = (blockIdx.x / b_tiles) % x_groups;
@@ -461,7 +463,7 @@ static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name
         static const bool plain_order = getenv("TCBNN_INCONV_ORDER") != nullptr;  // tuning switch
         const int y_phases = (!plain_order && 8 % b_tiles == 0) ? 8 / b_tiles : 0;
         const long long blocks = y_phases > 0
-                                     ? 8LL * x_groups * ((p.PH + y_phases - 1) / y_phases)
+                                     ? 8LL * ((x_groups + y_phases - 1) / y_phases) * p.PH
                                      : (long long)b_tiles * x_groups * p.PH;
         TCBNN_REQUIRE(blocks <= 0x7fffffffLL, "inconv128: grid too large");
         // staging scheme (see the kernel): whole segments per wave when at least 3 fit its 64 lanes
