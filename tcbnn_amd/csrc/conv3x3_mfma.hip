@@ -21,6 +21,7 @@
 //     contiguous runs.
 #include <algorithm>
 #include <cmath>
+#include <cstdlib>
 #include <type_traits>
 
 #include "common.h"
@@ -41,7 +42,11 @@ constexpr int RM_POOLED = 2;  // residual injected as the 2x2 max of a source tw
 
 // Waves per SIMD the register allocator is asked to make room for: the residual layers are
 // bound by HBM and want more memory requests in flight, the plain layers want registers.
-constexpr int waves_hint(int spt, int rm, int nt) { return rm == RM_PLAIN && spt * nt <= 2 ? 3 : 2; }
+constexpr int waves_hint(int spt, int rm, int nt) {
+    if (rm == RM_NONE) return 2;
+    if (rm == RM_PLAIN) return spt * nt <= 2 || (nt == 1 && spt <= 4) ? 3 : 2;
+    return 2;
+}
 
 // SPT = k-steps (64 bits) per filter tap = Cin / 64; MT = 32-image tiles per wave (2 for plain
 // layers, 1 for residual layers); NT = 32-channel tiles per wave; R16 = the injected residual is
@@ -513,10 +518,12 @@ int launch_t(const BgemmParams& p, hipStream_t stream) {
     const int n_groups = (p.N + 32 * NT - 1) / (32 * NT);
     const int b_groups = (p.B + 32 * MT - 1) / (32 * MT);
     const int quads = (p.PH * p.PW + kWaves - 1) / kWaves;  // pixel quads (one pixel per wave)
-    // as many workgroups as are resident at once (two per CU for plain layers, three for residual
-    // layers, fewer when their LDS does not fit), so that the weights are staged once per CU
-    // slot, with the pixel quads spread as evenly as possible
-    const int wg_per_cu = std::max(1, std::min(MT == 1 ? 3 : 2, (int)(160 * 1024 / lds_bytes)));
+    // Persistent workgroups: two per CU (four where only a quarter of the LDS is needed per workgroup,
+    // Cin = 256 with one channel tile), fewer when their LDS does not fit.  Measured on every layer
+    // of ResNet-18 at batch 256: more, shorter-lived workgroups stage the weights more often and lose.
+    static const int wg_env = getenv("TCBNN_WG_PER_CU") ? atoi(getenv("TCBNN_WG_PER_CU")) : 0;  // tuning switch
+    const int wg_want = wg_env > 0 ? wg_env : (SPT == 4 && NT == 1 ? 4 : 2);
+    const int wg_per_cu = std::max(1, std::min(wg_want, (int)(160 * 1024 / lds_bytes)));
     const int target = std::max(1, 256 * wg_per_cu / (n_groups * b_groups));
     int best = std::min(target, quads);
     double best_waste = 1e30;
