@@ -42,11 +42,7 @@ constexpr int RM_POOLED = 2;  // residual injected as the 2x2 max of a source tw
 
 // Waves per SIMD the register allocator is asked to make room for: the residual layers are
 // bound by HBM and want more memory requests in flight, the plain layers want registers.
-constexpr int waves_hint(int spt, int rm, int nt) {
-    if (rm == RM_NONE) return 2;
-    if (rm == RM_PLAIN) return spt * nt <= 2 || (nt == 1 && spt <= 4) ? 3 : 2;
-    return 2;
-}
+constexpr int waves_hint(int spt, int rm, int nt) { return rm == RM_PLAIN && spt == 4 && nt == 1 ? 4 : 2; }
 
 // SPT = k-steps (64 bits) per filter tap = Cin / 64; MT = 32-image tiles per wave (2 for plain
 // layers, 1 for residual layers); NT = 32-channel tiles per wave; R16 = the injected residual is
