@@ -94,7 +94,9 @@ int tcbnn_conv_out(int in_size, int filter, int stride, int padding, int pool);
 size_t tcbnn_fc_act_words(int batch, int features);                    /* B*KW128          */
 size_t tcbnn_conv_act_words(int height, int width, int batch, int ch); /* H*W*B*CW         */
 size_t tcbnn_fc_weight_words(int in_features, int out_features);       /* NPAD32*KW128     */
-size_t tcbnn_conv_filter_words(int r, int s, int in_ch, int out_ch);   /* NPAD32*R*S*CW    */
+size_t tcbnn_conv_filter_words(int r, int s, int in_ch, int out_ch);   /* NPAD32*R*S*CW, x5 for 3x3 filters with
+                                                                           Cin = 64/128/256/512: they carry an
+                                                                           FP4-expanded copy after the bit rows */
 size_t tcbnn_inconv_filter_words(int r, int s, int in_ch, int out_ch); /* R*S*OPAD32*5     */
 /* bytes of a residual tensor of `channels` channels in the given TCBNN_RES_* format */
 size_t tcbnn_residual_bytes(int height, int width, int channels, int batch, int format);
@@ -112,8 +114,9 @@ int tcbnn_residual_format_for_bound(int bound);
  * PackFcWeight128FMT (param.h:44-63). */
 int tcbnn_pack_fc_weight(const float* weight_kn, uint32_t* packed, int in_features,
                          int out_features, void* stream);
-/* fp32 HWIO [R][S][C][O] (param.h:573-574) -> packed [OPAD32][R*S][CW].  Replaces
- * PackFiltersByInChannels128FMT (param.h:560-581). */
+/* fp32 HWIO [R][S][C][O] (param.h:573-574) -> packed [OPAD32][R*S][CW] (+ the FP4 fragment copy
+ * for the 3x3 shapes named at tcbnn_conv_filter_words).  `packed` holds
+ * tcbnn_conv_filter_words(...) words.  Replaces PackFiltersByInChannels128FMT (param.h:560-581). */
 int tcbnn_pack_conv_filter(const float* filter_hwio, uint32_t* packed, int r, int s, int in_ch,
                            int out_ch, void* stream);
 /* fp32 HWIO [R][S][3][O] -> sign table uint32 [R*S][OPAD32][4]: entry c<3 is 0 if the

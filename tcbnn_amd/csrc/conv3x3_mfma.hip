@@ -76,17 +76,28 @@ conv3x3_mfma_f4_kernel(
     const int n0 = ng * (32 * NT);
     const int kw_tot = 9 * p.cw;
 
-    // ---- stage this channel group's weights (expanded, fragment order) and thresholds
-    for (int f = wave; f < NQ * NT; f += kWaves) {
-        const int q = f / NT, nt = f % NT;
-        const int tap = q / SPT, t = q % SPT;
-        const int c = n0 + nt * 32 + row_to_channel(j);
-        uint32_t x = 0, valid = 0;
-        if (c < p.N) {
-            x = wgt[(size_t)c * kw_tot + tap * p.cw + 2 * t + h];
-            valid = 0xffffffffu;
+    // ---- stage this channel group's weight fragments (already expanded when the filter was packed)
+    // and thresholds
+    {
+        const v4i* __restrict__ frag = reinterpret_cast<const v4i*>(wgt + (size_t)((p.N + 31) / 32) * 32 * kw_tot);
+        // all requests of a batch are in flight together (a loop of load-then-store would pay the
+        // memory latency once per fragment)
+        constexpr int kPerWave = (NQ * NT + kWaves - 1) / kWaves, kBatch = kPerWave < 9 ? kPerWave : 9;
+#pragma unroll
+        for (int i0 = 0; i0 < kPerWave; i0 += kBatch) {
+            v4i tmp[kBatch];
+#pragma unroll
+            for (int i = 0; i < kBatch; ++i) {
+                const int f = wave + (i0 + i) * kWaves;
+                const int q = f / NT, nt = f % NT;
+                tmp[i] = f < NQ * NT ? frag[((size_t)(ng * NT + nt) * NQ + q) * 64 + lane] : v4i{0, 0, 0, 0};
+            }
+#pragma unroll
+            for (int i = 0; i < kBatch; ++i) {
+                const int f = wave + (i0 + i) * kWaves;
+                if (f < NQ * NT) lds_w[f * 64 + lane] = tmp[i];
+            }
         }
-        lds_w[f * 64 + lane] = expand_f4_masked(x, valid);
     }
     // A NaN threshold always yields bit 1 (!(x < NaN)), exactly like -inf: staged as such, so that
     // the epilogue can take the bit from the sign of x - threshold.
@@ -115,7 +126,7 @@ conv3x3_mfma_f4_kernel(
     // every descriptor (the host checked the tensors are below 2 GiB): its load returns 0, its
     // store is dropped.
     constexpr unsigned kOutOfRange = 0x80000000u;
-    auto make_rsrc = [](const void* ptr, unsigned bytes) {
+    auto make_rsrc = [](const void* ptr, unsigned bytes) __attribute__((always_inline)) {
         return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(ptr), 0, (int)bytes, 0x00020000);
     };
     const __amdgpu_buffer_rsrc_t r_act = make_rsrc(act, act_bytes), r_rin = make_rsrc(rin, rin_bytes),
@@ -127,7 +138,7 @@ conv3x3_mfma_f4_kernel(
 
     // Requests the activation words of chunk `chunk` of the tile at pixel (yy, xx); returns the
     // wave-uniform mask of its in-frame taps.
-    auto load_chunk = [&](int yy, int xx, int chunk, uint32_t (*buf)[MT]) {
+    auto load_chunk = [&](int yy, int xx, int chunk, uint32_t (*buf)[MT]) __attribute__((always_inline)) {
         uint32_t mask = 0;
 #pragma unroll
         for (int tl = 0; tl < TPC; ++tl) {
@@ -149,7 +160,7 @@ conv3x3_mfma_f4_kernel(
     };
 
     v16f acc[MT][NT];
-    auto zero_acc = [&]() {
+    auto zero_acc = [&]() __attribute__((always_inline)) {
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
@@ -158,7 +169,7 @@ conv3x3_mfma_f4_kernel(
                 for (int v = 0; v < 16; ++v) acc[mt][nt][v] = 0.0f;
     };
 
-    auto compute_tap = [&](int tap, int tl, uint32_t (*buf)[MT]) {
+    auto compute_tap = [&](int tap, int tl, uint32_t (*buf)[MT]) __attribute__((always_inline)) {
 #pragma unroll
         for (int t = 0; t < SPT; ++t) {
             v4i bfrag[MT];
@@ -175,7 +186,7 @@ conv3x3_mfma_f4_kernel(
     // For Cin <= 128, interior pixels (every tap of the chunk in the frame: the bulk of a layer) run one
     // straight-line block, so that the weight fragments of the next step are read from LDS while
     // the current MFMAs execute; border pixels test each tap.
-    auto compute_chunk = [&](int chunk, uint32_t (*buf)[MT], uint32_t mask) {
+    auto compute_chunk = [&](int chunk, uint32_t (*buf)[MT], uint32_t mask) __attribute__((always_inline)) {
         if (SPT <= 2 && mask == (1u << TPC) - 1u) {
 #pragma unroll
             for (int tl = 0; tl < TPC; ++tl) compute_tap(chunk * TPC + tl, tl, buf);
@@ -202,7 +213,7 @@ conv3x3_mfma_f4_kernel(
     const unsigned lane_off16 = ((unsigned)(2 * h) * (unsigned)p.B + (unsigned)bload[0]) * 16u;
     const unsigned grp_b = (unsigned)p.B * 16u;  // bytes between consecutive channel groups
 
-    auto request_residual = [&](int yy, int xx, int (*rv)[NW]) {
+    auto request_residual = [&](int yy, int xx, int (*rv)[NW]) __attribute__((always_inline)) {
         if constexpr (RM != RM_NONE) {
             constexpr bool i16 = R16;
             // bytes per source pixel; per-lane offset; 128-bit loads per channel tile.  Groups past the
@@ -227,7 +238,7 @@ conv3x3_mfma_f4_kernel(
                     continue;
                 }
                 const unsigned base = pix * ch_b + (unsigned)(i16 ? cb / 8 : cb / 4) * grp_b;  // uniform
-                auto load4 = [&](int* dst, unsigned so) {
+                auto load4 = [&](int* dst, unsigned so) __attribute__((always_inline)) {
                     const v4i q = __builtin_amdgcn_raw_buffer_load_b128(r_rin, (int)loff, (int)so, 0);
                     dst[0] = q[0];
                     dst[1] = q[1];
@@ -249,7 +260,7 @@ conv3x3_mfma_f4_kernel(
         }
     };
     // Pooled source: 2x2 maximum of the four pixels, one int per channel (16-bit pairs unpacked).
-    auto finish_residual = [&](int (*rv)[NW]) {
+    auto finish_residual = [&](int (*rv)[NW]) __attribute__((always_inline)) {
         if constexpr (RM == RM_POOLED) {
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
@@ -278,7 +289,8 @@ conv3x3_mfma_f4_kernel(
 
     // One channel tile of the epilogue.  FAST (wave-uniform choice): all 32 channels exist and, with a
     // residual, all of them receive it, so no per-channel condition is evaluated at all.
-    auto epilogue_tile = [&](auto fast_tag, int nt, unsigned pix, unsigned bits_pix, int (*rv)[NW]) {
+    auto epilogue_tile = [&](auto fast_tag, int nt, unsigned pix, unsigned bits_pix,
+                             int (*rv)[NW]) __attribute__((always_inline)) {
         constexpr bool FAST = decltype(fast_tag)::value;
         const int cbase = n0 + nt * 32 + 16 * h;  // this lane's channels: cbase + v
         float thr[16];
@@ -392,7 +404,7 @@ conv3x3_mfma_f4_kernel(
         }
     };
 
-    auto epilogue = [&](int yy, int xx, int (*rv)[NW]) {
+    auto epilogue = [&](int yy, int xx, int (*rv)[NW]) __attribute__((always_inline)) {
         const unsigned pix = (unsigned)yy * (unsigned)p.PW + (unsigned)xx;
         const unsigned bits_pix = pix * (unsigned)p.bits_pix_stride * 4u;  // uniform
 #pragma unroll
@@ -416,68 +428,84 @@ conv3x3_mfma_f4_kernel(
         }
     };
 
-    // ---- persistent loop over this wave's tiles, chunks double-buffered in registers
-    uint32_t buf0[TPC * SPT][MT], buf1[TPC * SPT][MT];
-    int rv0[NRV][NW], rv1[kAhead ? NRV : 1][NW];
-    uint32_t m0 = 0, m1 = 0;
-    int chunk = 0;
-    bool have = pi < npix;
-    if (have) {
-        m0 = load_chunk(y, x, 0, buf0);
-        if constexpr (kAhead) {
-            request_residual(y, x, rv0);
-            if constexpr (RM == RM_POOLED) finish_residual(rv0);
+    // ---- persistent loop over this wave's tiles.  The activation chunks rotate through NB register
+    // buffers: the chunk that will be multiplied NB-1 steps from now is requested before the current
+    // one is multiplied (two steps of lookahead for Cin >= 256, where one chunk of MFMAs is shorter
+    // than the memory latency and few waves share a SIMD).
+    constexpr int NB = kAhead ? 2 : (SPT >= 4 ? 3 : 2);
+    constexpr int LOOK = NB - 1;
+    struct Cursor {
+        int pi, y, x, chunk;
+    };
+    auto advance = [&](Cursor& c) __attribute__((always_inline)) {
+        if (++c.chunk == NCH) {
+            c.chunk = 0;
+            c.pi += dpi;
+            c.x += dx;
+            c.y += dy;
+            if (c.x >= p.PW) {
+                c.x -= p.PW;
+                ++c.y;
+            }
+        }
+    };
+    uint32_t buf[NB][TPC * SPT][MT];
+    uint32_t msk[NB];
+    int rv[kAhead ? 2 : 1][NRV][NW];
+    Cursor cc = {pi, y, x, 0};  // chunk being multiplied
+    Cursor lc = cc;             // chunk being requested (LOOK steps ahead)
+#pragma unroll
+    for (int i = 0; i < LOOK; ++i) {
+        msk[i] = 0;
+        if (lc.pi < npix) msk[i] = load_chunk(lc.y, lc.x, lc.chunk, buf[i]);
+        advance(lc);
+    }
+    if constexpr (kAhead) {
+        if (cc.pi < npix) {
+            request_residual(cc.y, cc.x, rv[0]);
+            if constexpr (RM == RM_POOLED) finish_residual(rv[0]);
         }
     }
     zero_acc();
 
-    auto step = [&](uint32_t (*cur)[MT], uint32_t mcur, uint32_t (*nxt)[MT], uint32_t& mnxt, int (*rcur)[NW],
-                    int (*rnxt)[NW]) {
-        int nchunk = chunk + 1, ny = y, nx = x, npi = pi;
-        if (nchunk == NCH) {
-            nchunk = 0;
-            npi = pi + dpi;
-            nx = x + dx;
-            ny = y + dy;
-            if (nx >= p.PW) {
-                nx -= p.PW;
-                ++ny;
+    // one step with compile-time buffer indices: multiply buffer I, request into buffer (I + LOOK) % NB
+    auto step = [&](auto slot) __attribute__((always_inline)) {
+        constexpr int I = decltype(slot)::value;
+        constexpr int J = (I + LOOK) % NB;
+        if (lc.pi < npix) msk[J] = load_chunk(lc.y, lc.x, lc.chunk, buf[J]);
+        advance(lc);
+        int (*rcur)[NW] = rv[kAhead ? I : 0];
+        if constexpr (kAhead) {  // NCH == 1: the next chunk is the next tile
+            Cursor nt = cc;
+            advance(nt);
+            if (nt.pi < npix) request_residual(nt.y, nt.x, rv[1 - I]);
+            compute_chunk(cc.chunk, buf[I], msk[I]);
+            // a pooled source is reduced as soon as its tile has been multiplied (frees the registers of
+            // the window); otherwise the operand is left in flight until its own epilogue
+            if constexpr (RM == RM_POOLED) {
+                if (nt.pi < npix) finish_residual(rv[1 - I]);
             }
+        } else {
+            if constexpr (RM != RM_NONE) {
+                if (cc.chunk == 0) request_residual(cc.y, cc.x, rcur);
+            }
+            compute_chunk(cc.chunk, buf[I], msk[I]);
         }
-        const bool nhave = npi < npix;
-        if (nhave) mnxt = load_chunk(ny, nx, nchunk, nxt);
-        if constexpr (kAhead) {
-            if (nhave) request_residual(ny, nx, rnxt);
-        } else if constexpr (RM != RM_NONE) {
-            if (chunk == 0) request_residual(y, x, rcur);
-        }
-        compute_chunk(chunk, cur, mcur);
-        // a pooled source is reduced as soon as its tile has been multiplied (frees the registers of the
-        // window); otherwise the operand is left in flight until its own epilogue
-        if constexpr (kAhead && RM == RM_POOLED) {
-            if (nhave) finish_residual(rnxt);
-        }
-        if (chunk == NCH - 1) {
+        if (cc.chunk == NCH - 1) {
             if constexpr (!kAhead) finish_residual(rcur);
-            epilogue(y, x, rcur);
+            epilogue(cc.y, cc.x, rcur);
             zero_acc();
         }
-        chunk = nchunk;
-        y = ny;
-        x = nx;
-        pi = npi;
-        have = nhave;
+        advance(cc);
     };
 
-    while (have) {
-        if constexpr (kAhead) {
-            step(buf0, m0, buf1, m1, rv0, rv1);
-            if (!have) break;
-            step(buf1, m1, buf0, m0, rv1, rv0);
-        } else {
-            step(buf0, m0, buf1, m1, rv0, rv0);
-            if (!have) break;
-            step(buf1, m1, buf0, m0, rv0, rv0);
+    while (cc.pi < npix) {
+        step(std::integral_constant<int, 0>{});
+        if (cc.pi >= npix) break;
+        step(std::integral_constant<int, 1>{});
+        if constexpr (NB == 3) {
+            if (cc.pi >= npix) break;
+            step(std::integral_constant<int, 2>{});
         }
     }
 }

@@ -117,7 +117,9 @@ size_t tcbnn_fc_weight_words(int in_features, int out_features) {
     return (size_t)pad32(out_features) * kw128(in_features);
 }
 size_t tcbnn_conv_filter_words(int r, int s, int in_ch, int out_ch) {
-    return (size_t)pad32(out_ch) * r * s * step32(in_ch);
+    const size_t bits = (size_t)pad32(out_ch) * r * s * step32(in_ch);
+    // 3x3 filters of the persistent matrix-core kernel carry an FP4-expanded copy (4 bits per weight)
+    return filter_has_fragments(r, s, in_ch) ? 5 * bits : bits;
 }
 size_t tcbnn_inconv_filter_words(int r, int s, int in_ch, int out_ch) {
     (void)in_ch;
