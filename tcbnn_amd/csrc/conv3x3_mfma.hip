@@ -46,8 +46,10 @@ constexpr int waves_hint(int spt, int rm, int nt) { return rm == RM_PLAIN && spt
 
 // SPT = k-steps (64 bits) per filter tap = Cin / 64; MT = 32-image tiles per wave (2 for plain
 // layers, 1 for residual layers); NT = 32-channel tiles per wave; R16 = the injected residual is
-// stored as int16 (half the registers hold it while it is in flight).
-template <int SPT, int RM, int MT, int NT, bool R16>
+// stored as int16 (half the registers hold it while it is in flight); POOL = 2x2 OR-pooling of the
+// output bits (kernel.cuh:797-816): a wave multiplies the four pixels of a window one after the
+// other and stores the OR of their words once.
+template <int SPT, int RM, int MT, int NT, bool R16, bool POOL>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(waves_hint(SPT, RM, NT)))) void
 conv3x3_mfma_f4_kernel(
     const BgemmParams p, const uint32_t* __restrict__ act, const uint32_t* __restrict__ wgt,
@@ -55,6 +57,7 @@ conv3x3_mfma_f4_kernel(
     int rin_fmt, int rout_fmt, unsigned act_bytes, unsigned rin_bytes, unsigned rout_bytes, unsigned bits_bytes,
     int n_groups, int b_groups, int pix_streams) {
     static_assert(RM == RM_NONE || MT == 1, "residual instantiations own one image tile per wave");
+    static_assert(RM == RM_NONE || !POOL, "residuals are defined for un-pooled layers only");
     constexpr int TPC = SPT >= 4 ? 3 : 9;  // taps per prefetch chunk (a filter row, or all of it)
     constexpr int NCH = 9 / TPC;           // chunks per tile
     constexpr int NQ = 9 * SPT;            // k-steps per tile
@@ -107,11 +110,13 @@ conv3x3_mfma_f4_kernel(
     }
     __syncthreads();
 
-    const int npix = p.PH * p.PW;
+    // a wave's work items: output pixels, or 2x2 windows of them (row width `roww`)
+    const int roww = POOL ? p.OW : p.PW;
+    const int npix = POOL ? p.OH * p.OW : p.PH * p.PW;
     int pi = stream * kWaves + wave;
     const int dpi = pix_streams * kWaves;
-    int y = pi / p.PW, x = pi % p.PW;
-    const int dy = dpi / p.PW, dx = dpi % p.PW;
+    int y = pi / roww, x = pi % roww;
+    const int dy = dpi / roww, dx = dpi % roww;
 
     int bimg[MT], bload[MT];
 #pragma unroll
@@ -289,8 +294,9 @@ conv3x3_mfma_f4_kernel(
 
     // One channel tile of the epilogue.  FAST (wave-uniform choice): all 32 channels exist and, with a
     // residual, all of them receive it, so no per-channel condition is evaluated at all.
-    auto epilogue_tile = [&](auto fast_tag, int nt, unsigned pix, unsigned bits_pix,
-                             int (*rv)[NW]) __attribute__((always_inline)) {
+    uint32_t poolw[MT][NT];  // POOL: OR of the window's words so far
+    auto epilogue_tile = [&](auto fast_tag, int nt, unsigned pix, unsigned bits_pix, int (*rv)[NW],
+                             int sub) __attribute__((always_inline)) {
         constexpr bool FAST = decltype(fast_tag)::value;
         const int cbase = n0 + nt * 32 + 16 * h;  // this lane's channels: cbase + v
         float thr[16];
@@ -396,16 +402,23 @@ conv3x3_mfma_f4_kernel(
                 }
             }
             const uint32_t other = (uint32_t)__shfl_xor((int)hw, 32);
+            uint32_t word = (hw << 16) | other;
+            if constexpr (POOL) {
+                word |= sub == 0 ? 0u : poolw[mt][nt];
+                poolw[mt][nt] = word;
+                if (sub != 3) continue;  // uniform: the window is not complete yet
+            }
             const int w = ng * NT + nt;
             if (w < p.bits_row_words)  // uniform
-                __builtin_amdgcn_raw_buffer_store_b32((int)((hw << 16) | other), r_bits,
+                __builtin_amdgcn_raw_buffer_store_b32((int)word, r_bits,
                                                       (int)(h == 0 && b_ok ? (unsigned)b * 4u : kOutOfRange),
                                                       (int)(bits_pix + (unsigned)w * row_b), 0);
         }
     };
 
-    auto epilogue = [&](int yy, int xx, int (*rv)[NW]) __attribute__((always_inline)) {
-        const unsigned pix = (unsigned)yy * (unsigned)p.PW + (unsigned)xx;
+    // (yy, xx): the output pixel, or the window when pooled (sub = pixel of the window, 3 = last)
+    auto epilogue = [&](int yy, int xx, int sub, int (*rv)[NW]) __attribute__((always_inline)) {
+        const unsigned pix = (unsigned)yy * (unsigned)roww + (unsigned)xx;
         const unsigned bits_pix = pix * (unsigned)p.bits_pix_stride * 4u;  // uniform
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
@@ -414,11 +427,11 @@ conv3x3_mfma_f4_kernel(
             // gets none at all holds zeros and is fast as well)
             const bool fast = cb + 32 <= p.N && (RM == RM_NONE || cb + 32 <= res_lim || cb >= res_lim);
             if (fast)
-                epilogue_tile(std::true_type{}, nt, pix, bits_pix, rv);
+                epilogue_tile(std::true_type{}, nt, pix, bits_pix, rv, sub);
             else
-                epilogue_tile(std::false_type{}, nt, pix, bits_pix, rv);
+                epilogue_tile(std::false_type{}, nt, pix, bits_pix, rv, sub);
         }
-        if (ng == n_groups - 1) {  // zero the pixel's padding words
+        if (ng == n_groups - 1 && (!POOL || sub == 3)) {  // zero the pixel's padding words
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
                 for (int w = max((p.N + 31) / 32, n_groups * NT); w < p.bits_row_words; ++w)
@@ -435,29 +448,36 @@ conv3x3_mfma_f4_kernel(
     constexpr int NB = kAhead ? 2 : (SPT >= 4 ? 3 : 2);
     constexpr int LOOK = NB - 1;
     struct Cursor {
-        int pi, y, x, chunk;
+        int pi, y, x, chunk, sub;  // item index and coordinates, chunk of the tile, pixel of the window
     };
     auto advance = [&](Cursor& c) __attribute__((always_inline)) {
         if (++c.chunk == NCH) {
             c.chunk = 0;
+            if constexpr (POOL) {
+                if (++c.sub < 4) return;
+                c.sub = 0;
+            }
             c.pi += dpi;
             c.x += dx;
             c.y += dy;
-            if (c.x >= p.PW) {
-                c.x -= p.PW;
+            if (c.x >= roww) {
+                c.x -= roww;
                 ++c.y;
             }
         }
     };
+    // output pixel a cursor stands on
+    auto pix_y = [&](const Cursor& c) __attribute__((always_inline)) { return POOL ? 2 * c.y + (c.sub >> 1) : c.y; };
+    auto pix_x = [&](const Cursor& c) __attribute__((always_inline)) { return POOL ? 2 * c.x + (c.sub & 1) : c.x; };
     uint32_t buf[NB][TPC * SPT][MT];
     uint32_t msk[NB];
     int rv[kAhead ? 2 : 1][NRV][NW];
-    Cursor cc = {pi, y, x, 0};  // chunk being multiplied
+    Cursor cc = {pi, y, x, 0, 0};  // chunk being multiplied
     Cursor lc = cc;             // chunk being requested (LOOK steps ahead)
 #pragma unroll
     for (int i = 0; i < LOOK; ++i) {
         msk[i] = 0;
-        if (lc.pi < npix) msk[i] = load_chunk(lc.y, lc.x, lc.chunk, buf[i]);
+        if (lc.pi < npix) msk[i] = load_chunk(pix_y(lc), pix_x(lc), lc.chunk, buf[i]);
         advance(lc);
     }
     if constexpr (kAhead) {
@@ -472,7 +492,7 @@ conv3x3_mfma_f4_kernel(
     auto step = [&](auto slot) __attribute__((always_inline)) {
         constexpr int I = decltype(slot)::value;
         constexpr int J = (I + LOOK) % NB;
-        if (lc.pi < npix) msk[J] = load_chunk(lc.y, lc.x, lc.chunk, buf[J]);
+        if (lc.pi < npix) msk[J] = load_chunk(pix_y(lc), pix_x(lc), lc.chunk, buf[J]);
         advance(lc);
         int (*rcur)[NW] = rv[kAhead ? I : 0];
         if constexpr (kAhead) {  // NCH == 1: the next chunk is the next tile
@@ -493,7 +513,7 @@ conv3x3_mfma_f4_kernel(
         }
         if (cc.chunk == NCH - 1) {
             if constexpr (!kAhead) finish_residual(rcur);
-            epilogue(cc.y, cc.x, rcur);
+            epilogue(cc.y, cc.x, cc.sub, rcur);
             zero_acc();
         }
         advance(cc);
@@ -522,18 +542,18 @@ TensorBytes tensor_bytes(const BgemmParams& p) {
     t.act = 4LL * p.H * p.W * p.cw * p.B;
     t.rin = p.res_in != nullptr ? 4 * res_words((long long)p.PH * p.PW * (p.res_pool ? 4 : 1), p.res_in_ch, p.res_in_fmt) : 0;
     t.rout = p.res_out != nullptr ? 4 * res_words((long long)p.PH * p.PW, p.N, p.res_out_fmt) : 0;
-    t.bits = 4LL * p.PH * p.PW * p.bits_pix_stride;
+    t.bits = 4LL * p.OH * p.OW * p.bits_pix_stride;
     return t;
 }
 
-template <int SPT, int RM, int MT, int NT, bool R16>
+template <int SPT, int RM, int MT, int NT, bool R16, bool POOL>
 int launch_t(const BgemmParams& p, hipStream_t stream) {
     constexpr int NQ = 9 * SPT;
     const size_t lds_bytes = (size_t)NQ * NT * 64 * 16 + NT * 32 * sizeof(float);
     static bool attr_set = false;  // per instantiation
     if (!attr_set) {
         if (int rc = check_hip(
-                hipFuncSetAttribute(reinterpret_cast<const void*>(&conv3x3_mfma_f4_kernel<SPT, RM, MT, NT, R16>),
+                hipFuncSetAttribute(reinterpret_cast<const void*>(&conv3x3_mfma_f4_kernel<SPT, RM, MT, NT, R16, POOL>),
                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes),
                 "hipFuncSetAttribute(MaxDynamicSharedMemorySize)"))
             return rc;
@@ -541,7 +561,7 @@ int launch_t(const BgemmParams& p, hipStream_t stream) {
     }
     const int n_groups = (p.N + 32 * NT - 1) / (32 * NT);
     const int b_groups = (p.B + 32 * MT - 1) / (32 * MT);
-    const int quads = (p.PH * p.PW + kWaves - 1) / kWaves;  // pixel quads (one pixel per wave)
+    const int quads = ((POOL ? p.OH * p.OW : p.PH * p.PW) + kWaves - 1) / kWaves;  // items of the four waves
     // Persistent workgroups: two per CU (four where only a quarter of the LDS is needed per workgroup,
     // Cin = 256 with one channel tile), fewer when their LDS does not fit.  Measured on every layer
     // of ResNet-18 at batch 256: more, shorter-lived workgroups stage the weights more often and lose.
@@ -564,7 +584,7 @@ int launch_t(const BgemmParams& p, hipStream_t stream) {
     const int res_lim = p.res_in != nullptr ? std::min(std::min(p.res_limit, p.res_in_ch), p.N) : 0;
     const long long blocks = (long long)best * n_groups * b_groups;
     const TensorBytes tb = tensor_bytes(p);
-    hipLaunchKernelGGL((conv3x3_mfma_f4_kernel<SPT, RM, MT, NT, R16>), dim3((unsigned)blocks), dim3(kThreads), lds_bytes,
+    hipLaunchKernelGGL((conv3x3_mfma_f4_kernel<SPT, RM, MT, NT, R16, POOL>), dim3((unsigned)blocks), dim3(kThreads), lds_bytes,
                        stream, p, p.act, p.wgt, p.bn, p.res_in, p.res_out, res_lim, p.res_in_fmt, p.res_out_fmt,
                        (unsigned)tb.act, (unsigned)tb.rin, (unsigned)tb.rout, (unsigned)tb.bits, n_groups, b_groups, best);
     TCBNN_LAUNCH_CHECK("conv3x3_mfma_f4_kernel");
@@ -577,7 +597,7 @@ int launch_t(const BgemmParams& p, hipStream_t stream) {
 // tile (each operand fragment feeds two MFMAs) until the weights of 64 channels no longer leave
 // room for a second workgroup (Cin = 512).
 struct Pick {
-    int rm, mt, nt, r16;
+    int rm, mt, nt, r16, pool;
 };
 constexpr int pick_nt(int spt, int rm) {
     return rm == RM_POOLED ? 1 : (rm == RM_PLAIN ? (spt >= 4 ? 1 : 2) : (spt >= 8 ? 1 : 2));
@@ -585,7 +605,8 @@ constexpr int pick_nt(int spt, int rm) {
 Pick pick(const BgemmParams& p) {
     const int rm = p.res_in == nullptr && p.res_out == nullptr ? RM_NONE
                                                                 : (p.res_in != nullptr && p.res_pool ? RM_POOLED : RM_PLAIN);
-    return {rm, rm == RM_NONE ? 2 : 1, pick_nt(p.cw / 2, rm), p.res_in != nullptr && p.res_in_fmt == TCBNN_RES_I16};
+    return {rm, rm == RM_NONE ? 2 : 1, pick_nt(p.cw / 2, rm), p.res_in != nullptr && p.res_in_fmt == TCBNN_RES_I16,
+            p.pool_h == 2};
 }
 
 template <int SPT>
@@ -593,13 +614,14 @@ int launch_m(const BgemmParams& p, hipStream_t stream) {
     const Pick k = pick(p);
     switch (k.rm) {
         case RM_NONE:
-            return launch_t<SPT, RM_NONE, 2, pick_nt(SPT, RM_NONE), false>(p, stream);
+            return k.pool ? launch_t<SPT, RM_NONE, 2, pick_nt(SPT, RM_NONE), false, true>(p, stream)
+                          : launch_t<SPT, RM_NONE, 2, pick_nt(SPT, RM_NONE), false, false>(p, stream);
         case RM_PLAIN:
-            return k.r16 ? launch_t<SPT, RM_PLAIN, 1, pick_nt(SPT, RM_PLAIN), true>(p, stream)
-                         : launch_t<SPT, RM_PLAIN, 1, pick_nt(SPT, RM_PLAIN), false>(p, stream);
+            return k.r16 ? launch_t<SPT, RM_PLAIN, 1, pick_nt(SPT, RM_PLAIN), true, false>(p, stream)
+                         : launch_t<SPT, RM_PLAIN, 1, pick_nt(SPT, RM_PLAIN), false, false>(p, stream);
         default:
-            return k.r16 ? launch_t<SPT, RM_POOLED, 1, pick_nt(SPT, RM_POOLED), true>(p, stream)
-                         : launch_t<SPT, RM_POOLED, 1, pick_nt(SPT, RM_POOLED), false>(p, stream);
+            return k.r16 ? launch_t<SPT, RM_POOLED, 1, pick_nt(SPT, RM_POOLED), true, false>(p, stream)
+                         : launch_t<SPT, RM_POOLED, 1, pick_nt(SPT, RM_POOLED), false, false>(p, stream);
     }
 }
 
@@ -613,15 +635,19 @@ static bool within_2gib(const BgemmParams& p) {
 }
 
 bool conv3x3_mfma_applicable(const BgemmParams& p) {
-    return p.R == 3 && p.S == 3 && p.pool_h == 1 && p.pool_w == 1 && p.mode == EPI_THRESH && p.nan_bit == 1 &&
+    // un-pooled, or 2x2 pooling of whole windows without residuals
+    const bool pool_ok = (p.pool_h == 1 && p.pool_w == 1) ||
+                         (p.pool_h == 2 && p.pool_w == 2 && p.PH % 2 == 0 && p.PW % 2 == 0 && p.res_in == nullptr &&
+                          p.res_out == nullptr);
+    return p.R == 3 && p.S == 3 && pool_ok && p.mode == EPI_THRESH && p.nan_bit == 1 &&
            p.ksplit <= 1 && (p.cw == 2 || p.cw == 4 || p.cw == 8 || p.cw == 16) && p.k_tap == 32 * p.cw &&
            (long long)p.PH * p.PW < (1 << 24) && within_2gib(p);
 }
 
 void conv3x3_mfma_kernel_name(const BgemmParams& p, char* buf, size_t len) {
     const Pick k = pick(p);
-    snprintf(buf, len, "conv3x3_mfma_f4_kernel<%d, %d, %d, %d, %s>", p.cw / 2, k.rm, k.mt, k.nt,
-             k.r16 ? "true" : "false");
+    snprintf(buf, len, "conv3x3_mfma_f4_kernel<%d, %d, %d, %d, %s, %s>", p.cw / 2, k.rm, k.mt, k.nt,
+             k.r16 ? "true" : "false", k.pool ? "true" : "false");
 }
 
 int launch_conv3x3_mfma(const BgemmParams& p, hipStream_t stream) {
