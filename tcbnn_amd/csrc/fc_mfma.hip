@@ -159,7 +159,7 @@ bool fc_mfma_applicable(const BgemmParams& p) {
     if (p.cw % 4 != 0 || p.k_tap > 32 * p.cw) return false;
     // larger problems fill the machine with one wave per tile and are served by the generic kernel
     const long long tiles = (long long)((p.B + 31) / 32) * ((p.N + 31) / 32);
-    return tiles <= 2048;
+    return tiles <= 16384;
 }
 
 void fc_mfma_kernel_name(const BgemmParams& p, char* buf, size_t len) {
