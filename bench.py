@@ -189,7 +189,7 @@ def main():
     groups = {}
     for L, layer in zip(spec, net.order):
         name = layer.kernel_name() if hasattr(layer, "kernel_name") else \
-            {"in": "pack_rows_kernel"}[L["kind"]]
+            {"in": "in128_kernel"}[L["kind"]]
         w = layer_work(L, spec, res_bytes)
         g = groups.setdefault(name, dict(bops=0.0, bytes=0.0, ms=0.0, launches=0))
         g["bops"] += w["bops"]

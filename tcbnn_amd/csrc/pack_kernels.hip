@@ -42,6 +42,32 @@ __global__ __launch_bounds__(kThreads) void pack_rows_kernel(const float* __rest
     }
 }
 
+// In128LayerFMT (kernel.cuh:153-172): fp32 [B][K] row major -> sign bits [KW128][B].  One thread per
+// (word, image): consecutive lanes are consecutive images, so the packed words are written as
+// contiguous runs, and each lane reads its own 128 contiguous bytes (one cache line) with four
+// 128-bit loads when the rows are 16-byte aligned.
+__global__ void in128_kernel(const float* __restrict__ x, uint32_t* __restrict__ out, int batch, int k, int kw) {
+    const long long idx = (long long)blockIdx.x * kThreads + threadIdx.x;
+    if (idx >= (long long)kw * batch) return;
+    const int b = (int)(idx % batch);
+    const int w = (int)(idx / batch);
+    const float* row = x + (size_t)b * k + 32 * w;
+    uint32_t word = 0;
+    if (32 * w + 32 <= k && k % 4 == 0) {
+        const float4* r4 = reinterpret_cast<const float4*>(row);
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            const float4 v = r4[q];
+            word = (word << 4) | (v.x >= 0.0f ? 8u : 0u) | (v.y >= 0.0f ? 4u : 0u) | (v.z >= 0.0f ? 2u : 0u) |
+                   (v.w >= 0.0f ? 1u : 0u);
+        }
+    } else {
+        for (int e = 0; e < 32; ++e)
+            if (32 * w + e < k && row[e] >= 0.0f) word |= 1u << (31 - e);
+    }
+    out[idx] = word;
+}
+
 // HWIO fp32 filter -> [opad32][R*S][cw]; one thread per output word.
 __global__ void pack_conv_filter_kernel(const float* __restrict__ f, uint32_t* __restrict__ dst,
                                         int taps, int in_ch, int out_ch, int cw, int opad) {
@@ -288,8 +314,12 @@ int tcbnn_in128_forward(const tcbnn_in128_desc* d, void* stream) {
     TCBNN_NOTNULL(d->input);
     TCBNN_NOTNULL(d->output);
     TCBNN_REQUIRE(d->input_height > 0 && d->input_width > 0, "in128: bad shape");
-    return tcbnn_pack_rows(d->input, d->output, d->input_height, d->input_width, d->input_width,
-                           kw128(d->input_width), stream);
+    const int kw = kw128(d->input_width);
+    const long long total = (long long)kw * d->input_height;
+    hipLaunchKernelGGL(in128_kernel, dim3(blocks_for(total)), dim3(kThreads), 0, (hipStream_t)stream, d->input,
+                       d->output, d->input_height, d->input_width, kw);
+    TCBNN_LAUNCH_CHECK("in128_kernel");
+    return TCBNN_OK;
 }
 
 int tcbnn_unpack_fc_output(const uint32_t* packed, float* out, int batch, int features,
