@@ -198,7 +198,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS ?
         const unsigned imgs_here = (unsigned)min(64, p.B - b0);
         const unsigned tile_bytes = imgs_here * 3u * (unsigned)plane * 4u;  // host checked: below 2 GiB
         const unsigned voff = lane_ok ? ((unsigned)seg0 * (unsigned)plane + (unsigned)sax) * 4u : kOutOfRange;
-        const int lds0 = ((seg0 % 3) * ncols + scol) * kLB + seg0 / 3;
+        const int lds0 = (scol * 3 + seg0 % 3) * kLB + seg0 / 3;  // LDS: [column][channel][image]
         // every pass of every lane inside the 192 segments and the batch (wave-uniform)?
         const bool all_in = NST * rp == 3 * 64 && b0 + 64 <= p.B;
         __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
@@ -251,7 +251,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS ?
                     const int e = tid + k * kThreads;
                     const int bc = (int)(((unsigned)e * (unsigned)div_magic) >> 16);
                     const int col = e - bc * ncols;
-                    if (e < n_stage) tile[((bc >> 6) * ncols + col) * kLB + (bc & 63)] = stg[k];
+                    if (e < n_stage) tile[(col * 3 + (bc >> 6)) * kLB + (bc & 63)] = stg[k];
                 }
             }
         };
@@ -268,10 +268,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS ?
                 // sign patterns of this tap's 32 channels, one per word (wide scalar loads)
                 const u16v* pw = reinterpret_cast<const u16v*>(pats + (size_t)(r * p.S + s) * p.opad + wi * 32);
                 const u16v i0 = pw[0], i1 = pw[1];
-                const v8f ca = sign_combos(tile[(0 * ncols + cola) * kLB + lane], tile[(1 * ncols + cola) * kLB + lane],
-                                           tile[(2 * ncols + cola) * kLB + lane]);
-                const v8f cb = sign_combos(tile[(0 * ncols + colb) * kLB + lane], tile[(1 * ncols + colb) * kLB + lane],
-                                           tile[(2 * ncols + colb) * kLB + lane]);
+                // the three channels of a column are kLB floats apart: one address per pixel, constant offsets
+                const float* ta = tile + cola * 3 * kLB + lane;
+                const float* tb = tile + colb * 3 * kLB + lane;
+                const v8f ca = sign_combos(ta[0], ta[kLB], ta[2 * kLB]);
+                const v8f cb = sign_combos(tb[0], tb[kLB], tb[2 * kLB]);
                 add_indexed8x2(&acca[0], &accb[0], ca, cb, i0[0], i0[1], i0[2], i0[3], i0[4], i0[5], i0[6], i0[7]);
                 add_indexed8x2(&acca[8], &accb[8], ca, cb, i0[8], i0[9], i0[10], i0[11], i0[12], i0[13], i0[14],
                                i0[15]);
@@ -288,10 +289,21 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS ?
                 const float* acc = px == 0 ? acca : accb;
                 const size_t pix = (size_t)y * p.PW + xa + px;
                 uint32_t word = 0;
+                if (wi * 32 + 32 <= p.O) {  // uniform: full channel tile
+                    // bit = !(acc < bn) = inverted sign of acc - bn (equal operands give +0; a NaN threshold
+                    // counts as -inf: the bit is 1 either way)
 #pragma unroll
-                for (int n = 0; n < 32; ++n) {
-                    const int ch = wi * 32 + n;
-                    if (ch < p.O) word |= (acc[n] < bn[ch] ? 0u : 1u) << (31 - n);
+                    for (int n = 0; n < 32; ++n) {
+                        const float t = bn[wi * 32 + n];
+                        word = __builtin_amdgcn_alignbit(word, __float_as_uint(acc[n] - (t != t ? -__builtin_huge_valf() : t)), 31);
+                    }
+                    word = ~word;
+                } else {
+#pragma unroll
+                    for (int n = 0; n < 32; ++n) {
+                        const int ch = wi * 32 + n;
+                        if (ch < p.O) word |= (acc[n] < bn[ch] ? 0u : 1u) << (31 - n);
+                    }
                 }
                 out[(pix * p.ow + wi) * p.B + b] = word;
                 if (res != nullptr) {

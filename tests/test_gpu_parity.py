@@ -361,6 +361,30 @@ def test_inconv128_layer(gpu, b, h, R, stride, cout, pool, save):
     layer.release()
 
 
+def test_inconv128_special_thresholds(gpu):
+    """NaN, +-inf and exactly met thresholds in the first layer (kernel.cuh:655: bit = !(acc < bn))."""
+    r = rng(321)
+    b, h, cout = 6, 16, 64
+    x = rm.pm1(r, (b, 3, h, h))  # +-1 input: sums are exact integers, ties can be constructed
+    f = rm.pm1(r, (7, 7, 3, cout))
+    _, res = orc.inconv128(x, f, np.zeros(cout, np.float32), 4, True, 1, True)
+    bn = r.normal(0, 8, cout).astype(np.float32)
+    bn[0:4] = np.nan
+    bn[4:6] = np.inf
+    bn[6:8] = -np.inf
+    bn[8:40] = res[1, 2, 3, 8:40]
+    want, wres = orc.inconv128(x, f, bn, 4, True, 1, True)
+    layer = gpu.InConv128LayerParam("Conv1", h, h, 7, 7, 3, cout, b, 4, 4, True, 1, 1, True)
+    layer.initialize(x, gpu.ArrayWeights([f, bn]))
+    layer.forward()
+    gpuops.sync()
+    np.testing.assert_array_equal(layer.download_packed(), want)
+    np.testing.assert_array_equal(layer.download_residual(), wres)
+    bits = orc.unpack_bits(want, cout)
+    assert (bits[..., 0:4] == 1).all() and (bits[..., 4:6] == -1).all() and (bits[..., 6:8] == 1).all()
+    layer.release()
+
+
 def test_inconv128_small_batch_is_repeatable(gpu):
     """Few waves per SIMD is the worst case for the register-indexed accumulation of the
     first layer (index write -> use needs wait states): every repeat must match the oracle."""
