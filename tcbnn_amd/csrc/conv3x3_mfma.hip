@@ -73,7 +73,9 @@ conv3x3_mfma_f4_kernel(
     const int j = lane & 31;
     const int h = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int ng = blockIdx.x % n_groups;
+    // The channel group is rotated by the workgroup's position, so that the workgroups an XCD receives
+    // (every 8th) cover all channel groups, those that inject a residual and those that do not alike.
+    const int ng = (blockIdx.x % n_groups + blockIdx.x / n_groups) % n_groups;
     const int bg = (blockIdx.x / n_groups) % b_groups;
     const int stream = blockIdx.x / (n_groups * b_groups);
     const int n0 = ng * (32 * NT);
