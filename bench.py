@@ -38,20 +38,21 @@ COMPUTE_PEAKS_TOPS = {
 # launches of a kernel name in one step of the default workload (ResNet-18, batch 256, FP4 engine); a kernel
 # name that is not listed (another network, batch or engine) reports null.
 MEASURED_TRAFFIC_BYTES = {
-    "inconv_tiled_kernel<16, true>": 381400712,
-    "conv3x3_mfma_f4_kernel<1, 0, 2, 2, false>": 16283847,
-    "conv3x3_mfma_f4_kernel<1, 1, 1, 2, true>": 228868160,
-    "conv3x3_mfma_f4_kernel<2, 2, 1, 1, true>": 186302646,
-    "conv3x3_mfma_f4_kernel<2, 0, 2, 2, false>": 12512218,
-    "conv3x3_mfma_f4_kernel<2, 1, 1, 2, true>": 116245214,
-    "conv3x3_mfma_f4_kernel<4, 2, 1, 1, true>": 95096837,
-    "conv3x3_mfma_f4_kernel<4, 0, 2, 2, false>": 11224199,
-    "conv3x3_mfma_f4_kernel<4, 1, 1, 1, true>": 66435010,
-    "conv3x3_mfma_f4_kernel<8, 2, 1, 1, true>": 47223952,
-    "conv3x3_mfma_f4_kernel<8, 0, 2, 1, false>": 7800695,
-    "conv3x3_mfma_f4_kernel<8, 1, 1, 1, true>": 20616829,
-    "fc_mfma_f4_kernel<0>": 8245599,
-    "fc_mfma_f4_kernel<1>": 1385636,
+    "expand_conv_filter_kernel": 705273,
+    "inconv_tiled_kernel<16, true>": 433093303,
+    "conv3x3_mfma_f4_kernel<1, 0, 2, 2, false, false>": 16359208,
+    "conv3x3_mfma_f4_kernel<1, 1, 1, 2, true, false>": 218881851,
+    "conv3x3_mfma_f4_kernel<2, 2, 1, 1, true, false>": 174685432,
+    "conv3x3_mfma_f4_kernel<2, 0, 2, 2, false, false>": 12835124,
+    "conv3x3_mfma_f4_kernel<2, 1, 1, 2, true, false>": 113083025,
+    "conv3x3_mfma_f4_kernel<4, 2, 1, 1, true, false>": 98999409,
+    "conv3x3_mfma_f4_kernel<4, 0, 2, 2, false, false>": 14066543,
+    "conv3x3_mfma_f4_kernel<4, 1, 1, 1, true, false>": 68383766,
+    "conv3x3_mfma_f4_kernel<8, 2, 1, 1, true, false>": 56525871,
+    "conv3x3_mfma_f4_kernel<8, 0, 2, 1, false, false>": 16985795,
+    "conv3x3_mfma_f4_kernel<8, 1, 1, 1, true, false>": 29776500,
+    "fc_mfma_f4_kernel<0>": 8223072,
+    "fc_mfma_f4_kernel<1>": 1381369,
 }
 
 
