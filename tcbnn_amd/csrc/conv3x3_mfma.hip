@@ -50,7 +50,7 @@ constexpr int waves_hint(int spt, int rm, int nt) { return rm == RM_PLAIN && spt
 // output bits (kernel.cuh:797-816): a wave multiplies the four pixels of a window one after the
 // other and stores the OR of their words once.
 template <int SPT, int RM, int MT, int NT, bool R16, bool POOL>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(waves_hint(SPT, RM, NT)))) void
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(waves_hint(SPT, RM, NT), waves_hint(SPT, RM, NT)))) void
 conv3x3_mfma_f4_kernel(
     const BgemmParams p, const uint32_t* __restrict__ act, const uint32_t* __restrict__ wgt,
     const float* __restrict__ bnp, const int32_t* __restrict__ rin, int32_t* __restrict__ rout, int res_lim,
@@ -106,11 +106,24 @@ conv3x3_mfma_f4_kernel(
     }
     // A NaN threshold always yields bit 1 (!(x < NaN)), exactly like -inf: staged as such, so that
     // the epilogue can take the bit from the sign of x - threshold.
+    // Without a residual the sum s is an integer with |s| <= 9 Cin <= 4608, so s < threshold is
+    // the same as s < ceil(threshold), and thresholds beyond +-8192 decide like +-8192.  The
+    // negated integer threshold is then what the accumulator STARTS from (operand C of the tile's
+    // first MFMA): the finished accumulator is s - ceil(threshold), exact in fp32, and its sign is
+    // the inverted output bit, with no per-value subtraction in the epilogue.
     if (tid < NT * 32) {
-        const float t = n0 + tid < p.N ? bnp[n0 + tid] : 0.0f;
-        lds_thr[tid] = t != t ? -__builtin_huge_valf() : t;
+        float t = n0 + tid < p.N ? bnp[n0 + tid] : 0.0f;
+        t = t != t ? -__builtin_huge_valf() : t;
+        if constexpr (RM == RM_NONE) t = 0.0f - fminf(fmaxf(ceilf(t), -8192.0f), 8192.0f);
+        lds_thr[tid] = t;
     }
     __syncthreads();
+    // start values of a lane's 16 channels per channel tile (zeros when a residual is added first)
+    v16f acc0[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc0[nt][v] = RM == RM_NONE ? lds_thr[nt * 32 + 16 * h + v] : 0.0f;
 
     // a wave's work items: output pixels, or 2x2 windows of them (row width `roww`)
     const int roww = POOL ? p.OW : p.PW;
@@ -139,22 +152,58 @@ conv3x3_mfma_f4_kernel(
     const __amdgpu_buffer_rsrc_t r_act = make_rsrc(act, act_bytes), r_rin = make_rsrc(rin, rin_bytes),
                                  r_rout = make_rsrc(rout, rout_bytes), r_bits = make_rsrc(p.out_bits, bits_bytes);
     const unsigned row_b = (unsigned)p.B * 4u;  // bytes between consecutive words / channels of an image
-    unsigned voff_act[MT];
+    unsigned voff_act[MT], voff_bits[MT];  // activation loads; output words (stored by lanes 0-31)
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) voff_act[mt] = ((unsigned)h * (unsigned)p.B + (unsigned)bload[mt]) * 4u;
+    for (int mt = 0; mt < MT; ++mt) {
+        voff_act[mt] = ((unsigned)h * (unsigned)p.B + (unsigned)bload[mt]) * 4u;
+        voff_bits[mt] = h == 0 && bimg[mt] < p.B ? (unsigned)bimg[mt] * 4u : kOutOfRange;
+    }
 
+    // The tile's first MFMA must belong to a tap that is never outside the frame (it brings in the
+    // accumulator's start value): the centre tap.  Chunks of one filter row therefore come in the
+    // order middle, top, bottom, and the taps of a chunk start with its middle one; the sums are
+    // exact integers, so the order does not change them.
+    auto chunk_row = [](int chunk) __attribute__((always_inline)) { return chunk == 0 ? 1 : (chunk == 1 ? 0 : 2); };
     // Requests the activation words of chunk `chunk` of the tile at pixel (yy, xx); returns the
     // wave-uniform mask of its in-frame taps.
+    const unsigned pix_b = (unsigned)p.cw * row_b;        // bytes of one input pixel
+    const unsigned pitch_b = (unsigned)p.W * pix_b;       // bytes of one input row
+    constexpr uint32_t kAllTaps = (1u << TPC) - 1u;
+    // Is every tap of the chunk inside the frame (the bulk of a layer)?  Then its loads need no
+    // tests and one scalar add per tap: `soff` = offset of the chunk's first tap.
+    auto chunk_interior = [&](int yy, int xx, int chunk, unsigned& soff) __attribute__((always_inline)) {
+        const int ay0 = yy * p.stride_h - p.pad_h, ax0 = xx * p.stride_w - p.pad_w;
+        const int r0 = TPC == 9 ? 0 : chunk_row(chunk), nr = TPC == 9 ? 3 : 1;  // filter rows of the chunk
+        soff = (unsigned)((ay0 + r0) * p.W + ax0) * pix_b;  // uniform
+        return ay0 + r0 >= 0 && ay0 + r0 + nr <= p.H && ax0 >= 0 && ax0 + 3 <= p.W;
+    };
+    // loads of k-step i (taps in raster order) of an interior chunk; moves `soff` on after a tap
+    auto load_step = [&](uint32_t (*buf)[MT], int i, unsigned& soff) __attribute__((always_inline)) {
+        const int tl = i / SPT, t = i % SPT;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt)
+            buf[i][mt] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(r_act, (int)voff_act[mt],
+                                                                       (int)(soff + (unsigned)(2 * t) * row_b), 0);
+        if (t == SPT - 1) soff += tl % 3 == 2 ? pitch_b - 2 * pix_b : pix_b;
+    };
     auto load_chunk = [&](int yy, int xx, int chunk, uint32_t (*buf)[MT]) __attribute__((always_inline)) {
+        const int ay0 = yy * p.stride_h - p.pad_h, ax0 = xx * p.stride_w - p.pad_w;
+        const int r0 = TPC == 9 ? 0 : chunk_row(chunk);
+        unsigned soff0;
+        if (chunk_interior(yy, xx, chunk, soff0)) {
+#pragma unroll
+            for (int i = 0; i < TPC * SPT; ++i) load_step(buf, i, soff0);
+            return kAllTaps;
+        }
         uint32_t mask = 0;
 #pragma unroll
         for (int tl = 0; tl < TPC; ++tl) {
-            const int r = TPC == 9 ? tl / 3 : (TPC == 3 ? chunk : chunk / 3);
-            const int s = TPC == 1 ? chunk % 3 : tl % 3;
-            const int ay = yy * p.stride_h - p.pad_h + r, ax = xx * p.stride_w - p.pad_w + s;
+            const int r = TPC == 9 ? tl / 3 : r0;
+            const int s = tl % 3;
+            const int ay = ay0 + r, ax = ax0 + s;
             if (ay >= 0 && ay < p.H && ax >= 0 && ax < p.W) {
                 mask |= 1u << tl;
-                const unsigned soff = (unsigned)(ay * p.W + ax) * (unsigned)p.cw * row_b;  // uniform
+                const unsigned soff = (unsigned)(ay * p.W + ax) * pix_b;  // uniform
 #pragma unroll
                 for (int t = 0; t < SPT; ++t)
 #pragma unroll
@@ -167,43 +216,106 @@ conv3x3_mfma_f4_kernel(
     };
 
     v16f acc[MT][NT];
-    auto zero_acc = [&]() __attribute__((always_inline)) {
-#pragma unroll
-        for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) acc[mt][nt][v] = 0.0f;
-    };
 
-    auto compute_tap = [&](int tap, int tl, uint32_t (*buf)[MT]) __attribute__((always_inline)) {
+    // One k-step (64 input channels of one tap): the expanded activation words `bfrag` times the NT
+    // weight fragments `a`.  FIRST: the accumulators start from acc0 instead of their old value.
+    auto expand_step = [&](v4i* bfrag, const uint32_t* words) __attribute__((always_inline)) {
 #pragma unroll
-        for (int t = 0; t < SPT; ++t) {
-            v4i bfrag[MT];
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) bfrag[mt] = expand_f4(buf[tl * SPT + t][mt]);
-#pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
-                const v4i afrag = lds_w[((tap * SPT + t) * NT + nt) * 64 + lane];
-#pragma unroll
-                for (int mt = 0; mt < MT; ++mt) acc[mt][nt] = Acc<FMT_F4>::mma(afrag, bfrag[mt], acc[mt][nt]);
-            }
-        }
+        for (int mt = 0; mt < MT; ++mt) bfrag[mt] = expand_f4(words[mt]);
     };
-    // For Cin <= 128, interior pixels (every tap of the chunk in the frame: the bulk of a layer) run one
-    // straight-line block, so that the weight fragments of the next step are read from LDS while
-    // the current MFMAs execute; border pixels test each tap.
-    auto compute_chunk = [&](int chunk, uint32_t (*buf)[MT], uint32_t mask) __attribute__((always_inline)) {
-        if (SPT <= 2 && mask == (1u << TPC) - 1u) {
+    auto mma_frag = [&](auto first_tag, const v4i* a, const v4i* bfrag) __attribute__((always_inline)) {
+        constexpr bool FIRST = decltype(first_tag)::value;
 #pragma unroll
-            for (int tl = 0; tl < TPC; ++tl) compute_tap(chunk * TPC + tl, tl, buf);
+        for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+                acc[mt][nt] = Acc<FMT_F4>::mma(a[nt], bfrag[mt], FIRST ? acc0[nt] : acc[mt][nt]);
+    };
+    auto mma_step = [&](auto first_tag, const v4i* a, const uint32_t* words) __attribute__((always_inline)) {
+        v4i bfrag[MT];
+        expand_step(bfrag, words);
+        mma_frag(first_tag, a, bfrag);
+    };
+    auto load_a = [&](v4i* a, int q) __attribute__((always_inline)) {
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) a[nt] = lds_w[(q * NT + nt) * 64 + lane];
+    };
+    // Everything but LDS reads may be moved across this point by the instruction scheduler: the
+    // fragment reads issued before it stay a whole k-step ahead of the MFMAs that use them.
+    constexpr int kAllButDsRead = 0x07ff & ~0x0180;
+    // order of the taps inside a chunk: the middle one first
+    auto tap_of = [](int i) __attribute__((always_inline)) {
+        return TPC == 9 ? (i == 0 ? 4 : (i <= 4 ? i - 1 : i)) : (i == 0 ? 1 : (i == 1 ? 0 : 2));
+    };
+    v4i a_first[2][NT];  // weight fragments of a tile's first two k-steps (interior path)
+    if constexpr (SPT <= 2) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i) load_a(a_first[i], tap_of(i / SPT) * SPT + i % SPT);
+    }
+    // For Cin <= 128, interior pixels (every tap of the chunk in the frame: the bulk of a layer) run one
+    // straight-line block with the weight fragments of step i+1 read from LDS before step i is
+    // multiplied; border pixels test each tap and read ahead inside a tap only.
+    // LOADS: the words of the next chunk (interior as well) are requested two per step, in the shadow of
+    // the MFMAs, instead of in one burst before the chunk.
+    auto compute_chunk_as = [&](auto first_tag, auto loads_tag, int chunk, uint32_t (*buf)[MT], uint32_t mask,
+                                uint32_t (*nbuf)[MT], unsigned nsoff) __attribute__((always_inline)) {
+        constexpr bool FIRST = decltype(first_tag)::value;
+        constexpr bool LOADS = decltype(loads_tag)::value;
+        const int tap0 = TPC == 9 ? 0 : chunk_row(chunk) * 3;
+        if (LOADS || (SPT <= 2 && mask == kAllTaps)) {
+            // The fragments of the first two steps are the same for every tile and stay in registers
+            // (a_first); those of step i + 2 are requested when step i starts, into a ring of three.
+            constexpr int NS = TPC * SPT;
+            auto q_of = [&](int i) __attribute__((always_inline)) { return (tap0 + tap_of(i / SPT)) * SPT + i % SPT; };
+            // Software pipeline, one scheduling region per step (nothing moves across the region
+            // boundaries): request the fragments of step i + 2, expand the activations of step i + 1,
+            // multiply step i.
+            auto words_of = [&](int i) __attribute__((always_inline)) { return buf[tap_of(i / SPT) * SPT + i % SPT]; };
+            v4i a[3][NT], b[2][MT];
+            expand_step(b[0], words_of(0));
+#pragma unroll
+            for (int i = 0; i < NS; ++i) {
+                if (i + 2 < NS) load_a(a[(i + 2) % 3], q_of(i + 2));
+                if constexpr (LOADS) load_step(nbuf, i, nsoff);
+                if (i + 1 < NS) expand_step(b[(i + 1) & 1], words_of(i + 1));
+                const v4i* ai = i < 2 ? a_first[i] : a[i % 3];
+                if (FIRST && i == 0)
+                    mma_frag(std::true_type{}, ai, b[0]);
+                else
+                    mma_frag(std::false_type{}, ai, b[i & 1]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         } else {
 #pragma unroll
-            for (int tl = 0; tl < TPC; ++tl) {
-                if (!((mask >> tl) & 1u)) continue;  // wave-uniform
-                compute_tap(chunk * TPC + tl, tl, buf);
+            for (int i = 0; i < TPC; ++i) {
+                const int tl = tap_of(i);
+                if (!((mask >> tl) & 1u)) continue;  // wave-uniform; never the middle tap
+                v4i a[2][NT];
+                load_a(a[0], (tap0 + tl) * SPT);
+#pragma unroll
+                for (int t = 0; t < SPT; ++t) {
+                    if (t + 1 < SPT) load_a(a[(t + 1) & 1], (tap0 + tl) * SPT + t + 1);
+                    __builtin_amdgcn_sched_barrier(kAllButDsRead);
+                    if (FIRST && i == 0 && t == 0)
+                        mma_step(std::true_type{}, a[0], buf[tl * SPT + t]);
+                    else
+                        mma_step(std::false_type{}, a[t & 1], buf[tl * SPT + t]);
+                }
             }
         }
+    };
+    auto compute_chunk = [&](int chunk, uint32_t (*buf)[MT], uint32_t mask, bool fused, uint32_t (*nbuf)[MT],
+                             unsigned nsoff) __attribute__((always_inline)) {
+        if constexpr (SPT <= 2) {
+            if (fused) {  // uniform; NCH == 1: the chunk is a whole tile
+                compute_chunk_as(std::true_type{}, std::true_type{}, chunk, buf, mask, nbuf, nsoff);
+                return;
+            }
+        }
+        if (NCH == 1 || chunk == 0)  // uniform: the tile starts here
+            compute_chunk_as(std::true_type{}, std::false_type{}, chunk, buf, mask, nbuf, nsoff);
+        else
+            compute_chunk_as(std::false_type{}, std::false_type{}, chunk, buf, mask, nbuf, nsoff);
     };
 
     // ---- residual operand (kernel.cuh:770-794).  A lane owns channels n0 + 32 nt + 16 h + v of
@@ -302,7 +414,7 @@ conv3x3_mfma_f4_kernel(
         constexpr bool FAST = decltype(fast_tag)::value;
         const int cbase = n0 + nt * 32 + 16 * h;  // this lane's channels: cbase + v
         float thr[16];
-        {
+        if constexpr (RM != RM_NONE) {
             const float4* t4 = reinterpret_cast<const float4*>(lds_thr + nt * 32 + 16 * h);
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
@@ -389,21 +501,24 @@ conv3x3_mfma_f4_kernel(
                     }
                 }
             } else {
-                // the accumulator is the exact integer sum: compare it directly
+                // the accumulator is the exact integer sum minus the integer threshold (never -0):
+                // its sign is the inverted bit
                 if constexpr (FAST) {
 #pragma unroll
                     for (int v = 0; v < 16; ++v)
-                        hw = __builtin_amdgcn_alignbit(hw, __float_as_uint(acc[mt][nt][v] - thr[v]), 31);
+                        hw = __builtin_amdgcn_alignbit(hw, __float_as_uint(acc[mt][nt][v]), 31);
                     hw = ~hw & 0xffffu;
                 } else {
 #pragma unroll
                     for (int v = 0; v < 16; ++v) {
-                        const uint32_t bit = (cbase + v < p.N && !(acc[mt][nt][v] < thr[v])) ? 1u : 0u;
+                        const uint32_t bit = (cbase + v < p.N && !(acc[mt][nt][v] < 0.0f)) ? 1u : 0u;
                         hw = hw + hw + bit;
                     }
                 }
             }
-            const uint32_t other = (uint32_t)__shfl_xor((int)hw, 32);
+            // the half word of lane + 32 (only the lower 32 lanes store a word): lanes 0-31 of the
+            // second result are lanes 32-63 of the first operand; one VALU op, no LDS round trip
+            const uint32_t other = __builtin_amdgcn_permlane32_swap(hw, hw, false, false)[1];
             uint32_t word = (hw << 16) | other;
             if constexpr (POOL) {
                 word |= sub == 0 ? 0u : poolw[mt][nt];
@@ -412,8 +527,7 @@ conv3x3_mfma_f4_kernel(
             }
             const int w = ng * NT + nt;
             if (w < p.bits_row_words)  // uniform
-                __builtin_amdgcn_raw_buffer_store_b32((int)word, r_bits,
-                                                      (int)(h == 0 && b_ok ? (unsigned)b * 4u : kOutOfRange),
+                __builtin_amdgcn_raw_buffer_store_b32((int)word, r_bits, (int)voff_bits[mt],
                                                       (int)(bits_pix + (unsigned)w * row_b), 0);
         }
     };
@@ -437,16 +551,15 @@ conv3x3_mfma_f4_kernel(
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
                 for (int w = max((p.N + 31) / 32, n_groups * NT); w < p.bits_row_words; ++w)
-                    __builtin_amdgcn_raw_buffer_store_b32(
-                        0, r_bits, (int)(h == 0 && bimg[mt] < p.B ? (unsigned)bimg[mt] * 4u : kOutOfRange),
-                        (int)(bits_pix + (unsigned)w * row_b), 0);
+                    __builtin_amdgcn_raw_buffer_store_b32(0, r_bits, (int)voff_bits[mt],
+                                                          (int)(bits_pix + (unsigned)w * row_b), 0);
         }
     };
 
     // ---- persistent loop over this wave's tiles.  The activation chunks rotate through NB register
     // buffers: the chunk that will be multiplied NB-1 steps from now is requested before the current
-    // one is multiplied (two steps of lookahead for Cin >= 256, where one chunk of MFMAs is shorter
-    // than the memory latency and few waves share a SIMD).
+    // one is multiplied (two or three steps of lookahead without a residual, where one chunk of MFMAs
+    // is much shorter than the memory latency and few waves share a SIMD).
     constexpr int NB = kAhead ? 2 : (SPT >= 4 ? 3 : 2);
     constexpr int LOOK = NB - 1;
     struct Cursor {
@@ -488,20 +601,30 @@ conv3x3_mfma_f4_kernel(
             if constexpr (RM == RM_POOLED) finish_residual(rv[0]);
         }
     }
-    zero_acc();
 
     // one step with compile-time buffer indices: multiply buffer I, request into buffer (I + LOOK) % NB
     auto step = [&](auto slot) __attribute__((always_inline)) {
         constexpr int I = decltype(slot)::value;
         constexpr int J = (I + LOOK) % NB;
-        if (lc.pi < npix) msk[J] = load_chunk(pix_y(lc), pix_x(lc), lc.chunk, buf[J]);
+        // Both this chunk and the next one interior (Cin <= 128): the next one's loads ride along with
+        // this one's MFMAs.
+        bool fused = false;
+        unsigned nsoff = 0;
+        if (lc.pi < npix) {
+            if (SPT <= 2 && msk[I] == kAllTaps && chunk_interior(pix_y(lc), pix_x(lc), lc.chunk, nsoff)) {
+                fused = true;
+                msk[J] = kAllTaps;
+            } else {
+                msk[J] = load_chunk(pix_y(lc), pix_x(lc), lc.chunk, buf[J]);
+            }
+        }
         advance(lc);
         int (*rcur)[NW] = rv[kAhead ? I : 0];
         if constexpr (kAhead) {  // NCH == 1: the next chunk is the next tile
             Cursor nt = cc;
             advance(nt);
             if (nt.pi < npix) request_residual(nt.y, nt.x, rv[1 - I]);
-            compute_chunk(cc.chunk, buf[I], msk[I]);
+            compute_chunk(cc.chunk, buf[I], msk[I], fused, buf[J], nsoff);
             // a pooled source is reduced as soon as its tile has been multiplied (frees the registers of
             // the window); otherwise the operand is left in flight until its own epilogue
             if constexpr (RM == RM_POOLED) {
@@ -511,12 +634,11 @@ conv3x3_mfma_f4_kernel(
             if constexpr (RM != RM_NONE) {
                 if (cc.chunk == 0) request_residual(cc.y, cc.x, rcur);
             }
-            compute_chunk(cc.chunk, buf[I], msk[I]);
+            compute_chunk(cc.chunk, buf[I], msk[I], fused, buf[J], nsoff);
         }
         if (cc.chunk == NCH - 1) {
             if constexpr (!kAhead) finish_residual(rcur);
             epilogue(cc.y, cc.x, cc.sub, rcur);
-            zero_acc();
         }
         advance(cc);
     };
@@ -525,9 +647,13 @@ conv3x3_mfma_f4_kernel(
         step(std::integral_constant<int, 0>{});
         if (cc.pi >= npix) break;
         step(std::integral_constant<int, 1>{});
-        if constexpr (NB == 3) {
+        if constexpr (NB >= 3) {
             if (cc.pi >= npix) break;
             step(std::integral_constant<int, 2>{});
+        }
+        if constexpr (NB >= 4) {
+            if (cc.pi >= npix) break;
+            step(std::integral_constant<int, 3>{});
         }
     }
 }
@@ -641,7 +767,10 @@ bool conv3x3_mfma_applicable(const BgemmParams& p) {
     const bool pool_ok = (p.pool_h == 1 && p.pool_w == 1) ||
                          (p.pool_h == 2 && p.pool_w == 2 && p.PH % 2 == 0 && p.PW % 2 == 0 && p.res_in == nullptr &&
                           p.res_out == nullptr);
-    return p.R == 3 && p.S == 3 && pool_ok && p.mode == EPI_THRESH && p.nan_bit == 1 &&
+    // the centre tap of every output pixel lies inside the frame (the kernel starts each tile with it)
+    const bool centre_ok = p.pad_h <= 1 && p.pad_w <= 1 && (p.PH - 1) * p.stride_h - p.pad_h + 1 < p.H &&
+                           (p.PW - 1) * p.stride_w - p.pad_w + 1 < p.W;
+    return p.R == 3 && p.S == 3 && pool_ok && centre_ok && p.mode == EPI_THRESH && p.nan_bit == 1 &&
            p.ksplit <= 1 && (p.cw == 2 || p.cw == 4 || p.cw == 8 || p.cw == 16) && p.k_tap == 32 * p.cw &&
            (long long)p.PH * p.PW < (1 << 24) && within_2gib(p);
 }

@@ -191,18 +191,23 @@ int tcbnn_out128_forward(const tcbnn_out128_desc* d, void* stream) {
     return run_bgemm(p, d->variant, (hipStream_t)stream);
 }
 
-int tcbnn_conv128_forward(const tcbnn_conv128_desc* d, void* stream) {
+// The bit-GEMM problem of a Conv128 layer.  `launch`: the pointers are required (forward);
+// otherwise only the shape is checked and nullness of the residual pointers follows the flags
+// (kernel name of the launch that forward would make).
+static int conv_problem(const tcbnn_conv128_desc* d, bool launch, BgemmParams* out) {
     TCBNN_NOTNULL(d);
-    TCBNN_NOTNULL(d->input);
-    TCBNN_NOTNULL(d->filter);
-    TCBNN_NOTNULL(d->bn);
-    TCBNN_NOTNULL(d->output);
+    if (launch) {
+        TCBNN_NOTNULL(d->input);
+        TCBNN_NOTNULL(d->filter);
+        TCBNN_NOTNULL(d->bn);
+        TCBNN_NOTNULL(d->output);
+    }
     TCBNN_REQUIRE(d->input_height > 0 && d->input_width > 0 && d->batch > 0 &&
                       d->input_channels > 0 && d->output_channels > 0 && d->filter_height > 0 &&
                       d->filter_width > 0 && d->stride_height > 0 && d->stride_width > 0 &&
                       d->pool_height > 0 && d->pool_width > 0,
                   "conv128: bad shape");
-    BgemmParams p;
+    BgemmParams& p = *out;
     memset(&p, 0, sizeof(p));
     p.act = d->input;
     p.wgt = d->filter;
@@ -235,11 +240,13 @@ int tcbnn_conv128_forward(const tcbnn_conv128_desc* d, void* stream) {
     p.bits_row_words = d->ahead_fc ? kw128(p.N) : ow;
     p.bits_pix_stride = (long long)p.bits_row_words * p.B;
     p.ksplit = 1;
+    // a stand-in for a residual pointer the name query does not need
+    int32_t* const some = reinterpret_cast<int32_t*>(const_cast<tcbnn_conv128_desc*>(d));
     if (d->inject_residual) {
-        TCBNN_NOTNULL(d->input_residual);
+        if (launch) TCBNN_NOTNULL(d->input_residual);
         TCBNN_REQUIRE(d->input_residual_channels > 0, "conv128: input_residual_channels unset");
         TCBNN_REQUIRE(d->residual_channels >= 0, "conv128: negative residual_channels");
-        p.res_in = d->input_residual;
+        p.res_in = launch ? d->input_residual : some;
         p.res_in_ch = d->input_residual_channels;
         p.res_limit = d->residual_channels;
         p.res_pool = d->residual_pool ? 1 : 0;
@@ -248,12 +255,18 @@ int tcbnn_conv128_forward(const tcbnn_conv128_desc* d, void* stream) {
         p.res_in_fmt = d->input_residual_format;
     }
     if (d->save_residual) {
-        TCBNN_NOTNULL(d->output_residual);
+        if (launch) TCBNN_NOTNULL(d->output_residual);
         TCBNN_REQUIRE(d->output_residual_format == TCBNN_RES_I32 || d->output_residual_format == TCBNN_RES_I16,
                       "conv128: unknown output_residual_format");
-        p.res_out = d->output_residual;
+        p.res_out = launch ? d->output_residual : some;
         p.res_out_fmt = d->output_residual_format;
     }
+    return TCBNN_OK;
+}
+
+int tcbnn_conv128_forward(const tcbnn_conv128_desc* d, void* stream) {
+    BgemmParams p;
+    if (int rc = conv_problem(d, true, &p)) return rc;
     return run_bgemm(p, d->variant, (hipStream_t)stream);
 }
 
@@ -269,32 +282,8 @@ static int kernel_name(const BgemmParams& p, int variant, char* buf, size_t len)
 }
 
 int tcbnn_conv128_kernel_name(const tcbnn_conv128_desc* d, char* buf, size_t len) {
-    TCBNN_NOTNULL(d);
     BgemmParams p;
-    memset(&p, 0, sizeof(p));
-    p.B = d->batch;
-    p.cw = step32(d->input_channels);
-    p.R = d->filter_height;
-    p.S = d->filter_width;
-    p.pool_h = d->pool_height;
-    p.pool_w = d->pool_width;
-    p.PH = tcbnn_conv_out(d->input_height, p.R, d->stride_height, d->padding, 1);
-    p.PW = tcbnn_conv_out(d->input_width, p.S, d->stride_width, d->padding, 1);
-    p.OH = (p.PH + p.pool_h - 1) / p.pool_h;
-    p.OW = (p.PW + p.pool_w - 1) / p.pool_w;
-    p.N = d->output_channels;
-    p.ksplit = 1;
-    p.mode = EPI_THRESH;
-    p.nan_bit = 1;
-    p.k_tap = d->input_channels;
-    p.stride_h = d->stride_height;
-    p.stride_w = d->stride_width;
-    p.res_pool = d->residual_pool;
-    p.res_in_fmt = d->input_residual_format;
-    p.res_out_fmt = d->output_residual_format;
-    // only nullness matters for the name
-    p.res_in = d->inject_residual ? reinterpret_cast<const int32_t*>(d) : nullptr;
-    p.res_out = d->save_residual ? reinterpret_cast<int32_t*>(const_cast<tcbnn_conv128_desc*>(d)) : nullptr;
+    if (int rc = conv_problem(d, false, &p)) return rc;
     return kernel_name(p, d->variant, buf, len);
 }
 int tcbnn_fc128_kernel_name(const tcbnn_fc128_desc* d, char* buf, size_t len) {
