@@ -50,7 +50,7 @@ constexpr int waves_hint(int spt, int rm, int nt) { return rm == RM_PLAIN && spt
 // output bits (kernel.cuh:797-816): a wave multiplies the four pixels of a window one after the
 // other and stores the OR of their words once.
 template <int SPT, int RM, int MT, int NT, bool R16, bool POOL>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(waves_hint(SPT, RM, NT), waves_hint(SPT, RM, NT)))) void
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(waves_hint(SPT, RM, NT)))) void
 conv3x3_mfma_f4_kernel(
     const BgemmParams p, const uint32_t* __restrict__ act, const uint32_t* __restrict__ wgt,
     const float* __restrict__ bnp, const int32_t* __restrict__ rin, int32_t* __restrict__ rout, int res_lim,
@@ -130,8 +130,11 @@ conv3x3_mfma_f4_kernel(
     const int npix = POOL ? p.OH * p.OW : p.PH * p.PW;
     int pi = stream * kWaves + wave;
     const int dpi = pix_streams * kWaves;
-    int y = pi / roww, x = pi % roww;
-    const int dy = dpi / roww, dx = dpi % roww;
+    // Item pi stands for row pi / roww and column (pi % roww + row) % roww.  The skew by the row keeps
+    // a wave from staying in one column when its stride is a multiple of the row width (then the waves
+    // that own a border column, whose tiles are slower, would finish long after the others).
+    const int y = pi / roww, xr = pi % roww;
+    const int dy = dpi / roww, dx = dpi % roww, dxs = (dx + dy) % roww;
 
     int bimg[MT], bload[MT];
 #pragma unroll
@@ -247,11 +250,6 @@ conv3x3_mfma_f4_kernel(
     auto tap_of = [](int i) __attribute__((always_inline)) {
         return TPC == 9 ? (i == 0 ? 4 : (i <= 4 ? i - 1 : i)) : (i == 0 ? 1 : (i == 1 ? 0 : 2));
     };
-    v4i a_first[2][NT];  // weight fragments of a tile's first two k-steps (interior path)
-    if constexpr (SPT <= 2) {
-#pragma unroll
-        for (int i = 0; i < 2; ++i) load_a(a_first[i], tap_of(i / SPT) * SPT + i % SPT);
-    }
     // For Cin <= 128, interior pixels (every tap of the chunk in the frame: the bulk of a layer) run one
     // straight-line block with the weight fragments of step i+1 read from LDS before step i is
     // multiplied; border pixels test each tap and read ahead inside a tap only.
@@ -263,22 +261,21 @@ conv3x3_mfma_f4_kernel(
         constexpr bool LOADS = decltype(loads_tag)::value;
         const int tap0 = TPC == 9 ? 0 : chunk_row(chunk) * 3;
         if (LOADS || (SPT <= 2 && mask == kAllTaps)) {
-            // The fragments of the first two steps are the same for every tile and stay in registers
-            // (a_first); those of step i + 2 are requested when step i starts, into a ring of three.
             constexpr int NS = TPC * SPT;
             auto q_of = [&](int i) __attribute__((always_inline)) { return (tap0 + tap_of(i / SPT)) * SPT + i % SPT; };
             // Software pipeline, one scheduling region per step (nothing moves across the region
-            // boundaries): request the fragments of step i + 2, expand the activations of step i + 1,
-            // multiply step i.
+            // boundaries): request the fragments and expand the activations of step i + 1, multiply
+            // step i.
             auto words_of = [&](int i) __attribute__((always_inline)) { return buf[tap_of(i / SPT) * SPT + i % SPT]; };
-            v4i a[3][NT], b[2][MT];
+            v4i a[2][NT], b[2][MT];
+            load_a(a[0], q_of(0));
             expand_step(b[0], words_of(0));
 #pragma unroll
             for (int i = 0; i < NS; ++i) {
-                if (i + 2 < NS) load_a(a[(i + 2) % 3], q_of(i + 2));
+                if (i + 1 < NS) load_a(a[(i + 1) & 1], q_of(i + 1));
                 if constexpr (LOADS) load_step(nbuf, i, nsoff);
                 if (i + 1 < NS) expand_step(b[(i + 1) & 1], words_of(i + 1));
-                const v4i* ai = i < 2 ? a_first[i] : a[i % 3];
+                const v4i* ai = a[i & 1];
                 if (FIRST && i == 0)
                     mma_frag(std::true_type{}, ai, b[0]);
                 else
@@ -563,7 +560,8 @@ conv3x3_mfma_f4_kernel(
     constexpr int NB = kAhead ? 2 : (SPT >= 4 ? 3 : 2);
     constexpr int LOOK = NB - 1;
     struct Cursor {
-        int pi, y, x, chunk, sub;  // item index and coordinates, chunk of the tile, pixel of the window
+        int pi, y, x, chunk, sub;  // item index, row and (skewed) column, chunk of the tile, pixel of the window
+        int xr;                    // pi % roww
     };
     auto advance = [&](Cursor& c) __attribute__((always_inline)) {
         if (++c.chunk == NCH) {
@@ -573,12 +571,15 @@ conv3x3_mfma_f4_kernel(
                 c.sub = 0;
             }
             c.pi += dpi;
-            c.x += dx;
+            c.xr += dx;
             c.y += dy;
-            if (c.x >= roww) {
-                c.x -= roww;
+            c.x += dxs;
+            if (c.xr >= roww) {
+                c.xr -= roww;
                 ++c.y;
+                ++c.x;
             }
+            if (c.x >= roww) c.x -= roww;
         }
     };
     // output pixel a cursor stands on
@@ -587,7 +588,7 @@ conv3x3_mfma_f4_kernel(
     uint32_t buf[NB][TPC * SPT][MT];
     uint32_t msk[NB];
     int rv[kAhead ? 2 : 1][NRV][NW];
-    Cursor cc = {pi, y, x, 0, 0};  // chunk being multiplied
+    Cursor cc = {pi, y, (xr + y) % roww, 0, 0, xr};  // chunk being multiplied
     Cursor lc = cc;             // chunk being requested (LOOK steps ahead)
 #pragma unroll
     for (int i = 0; i < LOOK; ++i) {
