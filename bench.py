@@ -122,7 +122,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--net", default="imagenet_resnet", choices=["imagenet_resnet", "cifar10_vgg", "mnist_mlp"])
+    ap.add_argument("--net", default="imagenet_resnet", choices=["imagenet_resnet", "cifar10_vgg", "mnist_mlp", "alexnet", "cifar10_resnet", "imagenet_vgg"])
     ap.add_argument("--batch", type=int, default=None)
     ap.add_argument("--variant", default="auto")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -146,7 +146,7 @@ def main():
         _lib.check(_lib.lib.tcbnn_set_default_variant(_lib.VARIANTS[args.variant]))
     variant = {v: k for k, v in _lib.VARIANTS.items()}[_lib.lib.tcbnn_get_default_variant()]
 
-    default_batch = {"imagenet_resnet": 256, "cifar10_vgg": 256, "mnist_mlp": 8192}[args.net]
+    default_batch = {"mnist_mlp": 8192}.get(args.net, 256)
     batch = args.batch or default_batch
     spec = nets.SPECS[args.net](batch=batch)
     weights = tcbnn_amd.synthetic_weights(spec, seed=0)
@@ -218,7 +218,8 @@ def main():
     cpu = None
     if not args.no_cpu:
         from oracle import nets as orc_nets, orc
-        cb = args.cpu_batch or {"imagenet_resnet": 16, "cifar10_vgg": 64, "mnist_mlp": 8192}[args.net]
+        cb = args.cpu_batch or {"imagenet_resnet": 16, "cifar10_vgg": 64, "mnist_mlp": 8192, "alexnet": 32,
+                                   "cifar10_resnet": 16, "imagenet_vgg": 8}[args.net]
         cb = min(cb, batch)
         cspec = nets.SPECS[args.net](batch=cb)
         xs = x[:cb]
@@ -253,7 +254,10 @@ def main():
         "config": {"workload": "%s, reference topology (%s), batch %d, seeded synthetic weights and input"
                                % (args.net, {"imagenet_resnet": "imagenet_resnet.cu:223-325",
                                              "cifar10_vgg": "cifar10_vgg.cu:162-199",
-                                             "mnist_mlp": "mnist_mlp.cu:111-124"}[args.net], batch),
+                                             "mnist_mlp": "mnist_mlp.cu:111-124",
+                                             "alexnet": "alexnet.cu:143-177",
+                                             "cifar10_resnet": "cifar10_resnet.cu:189-259",
+                                             "imagenet_vgg": "imagenet_vgg.cu:217-286"}[args.net], batch),
                    "variant": variant, "layers": len(spec),
                    "residual_storage": ("int16 where the bound of |residual| proves it exact (%d of %d tensors), "
                                         "else int32" % (sum(1 for v in res_bytes.values() if v == 2), len(res_bytes)))

@@ -19,6 +19,8 @@
 //   inconv_generic_kernel (any pooling): one lane per pooled output pixel.
 #include <stdlib.h>
 
+#include <type_traits>
+
 #include "common.h"
 
 namespace tcbnn {
@@ -125,7 +127,10 @@ typedef uint32_t u16v __attribute__((ext_vector_type(16)));
 //     LDS slot a constant plus an immediate: no per-element address arithmetic.  NST = passes =
 //     ceil(192 / (4 rpw)).
 //   ROWS = false: the elements are dealt to the threads linearly, NST = ceil(3 * 64 * ncols / 256).
-template <int NST, bool ROWS>
+// POOLED: blockIdx selects a row of the POOLED output; the workgroup runs the pool_h convolution rows
+// of it one after the other and ORs their words (kernel.cuh:646-664); with pool_w = 2 the two columns of
+// a wave are one window.  pool_w is 1 or 2 (the host checks), no residual is saved.
+template <int NST, bool ROWS, bool POOLED>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS ? 4 : 3))) void inconv_tiled_kernel(
     const InConvParams p, const float* __restrict__ in, const uint4* __restrict__ masks,
     const float* __restrict__ bn, uint32_t* __restrict__ out, int32_t* __restrict__ res, int b_tiles,
@@ -168,14 +173,18 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS ?
         reinterpret_cast<const uint32_t*>(masks) + (size_t)p.R * p.S * p.opad * 4;  // packed pattern table
 
     for (int g = 0; g < n_groups; ++g) {
+      uint32_t pooled[2] = {0u, 0u};  // POOLED: OR of the rows so far, per pixel column of the wave
+      const int wi = g * 2 + chh;                       // output word = channel tile of this wave
+      const bool work = xa_ok && wi * 32 < p.opad;      // uniform
+      for (int py = 0; py < (POOLED ? p.pool_h : 1); ++py) {
+        const int yc = POOLED ? y * p.pool_h + py : y;  // convolution row (uniform)
+        if (POOLED && yc >= p.PH) break;
         float acca[32], accb[32];  // this wave's 32 channels of pixels xa and xb
 #pragma unroll
         for (int n = 0; n < 32; ++n) acca[n] = accb[n] = 0.0f;
-        const int wi = g * 2 + chh;                       // output word = channel tile of this wave
-        const bool work = xa_ok && wi * 32 < p.opad;      // uniform
 
         // Filter rows inside the frame: r_lo <= r < r_hi (uniform for the whole workgroup).
-        const int ay0 = y * p.stride_h - p.pad_h;
+        const int ay0 = yc * p.stride_h - p.pad_h;
         const int r_lo = max(0, -ay0), r_hi = min(p.R, p.H - ay0);
         const int n_stage = 3 * 64 * ncols;
 
@@ -287,7 +296,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS ?
             for (int px = 0; px < 2; ++px) {
                 if (px == 1 && !xb_ok) continue;
                 const float* acc = px == 0 ? acca : accb;
-                const size_t pix = (size_t)y * p.PW + xa + px;
+                const size_t pix = (size_t)yc * p.PW + xa + px;
                 uint32_t word = 0;
                 if (wi * 32 + 32 <= p.O) {  // uniform: full channel tile
                     // bit = !(acc < bn) = inverted sign of acc - bn (equal operands give +0; a NaN threshold
@@ -304,6 +313,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS ?
                         const int ch = wi * 32 + n;
                         if (ch < p.O) word |= (acc[n] < bn[ch] ? 0u : 1u) << (31 - n);
                     }
+                }
+                if constexpr (POOLED) {
+                    pooled[px] |= word;
+                    continue;
                 }
                 out[(pix * p.ow + wi) * p.B + b] = word;
                 if (res != nullptr) {
@@ -333,6 +346,17 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS ?
                 }
             }
         }
+      }
+      if constexpr (POOLED) {
+          if (work && b < p.B && wi < p.ow) {
+              if (p.pool_w == 2) {
+                  out[(((size_t)y * p.OW + xa / 2) * p.ow + wi) * p.B + b] = pooled[0] | (xb_ok ? pooled[1] : 0u);
+              } else {
+                  out[(((size_t)y * p.OW + xa) * p.ow + wi) * p.B + b] = pooled[0];
+                  if (xb_ok) out[(((size_t)y * p.OW + xb) * p.ow + wi) * p.B + b] = pooled[1];
+              }
+          }
+      }
     }
 }
 
@@ -445,7 +469,9 @@ static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name
     p.OH = (p.PH + p.pool_h - 1) / p.pool_h;
     p.OW = (p.PW + p.pool_w - 1) / p.pool_w;
 
-    const bool tiled = p.pool_h == 1 && p.pool_w == 1 && (kXT - 1) * p.stride_w + p.S <= kMaxCols;
+    const bool pooled = p.pool_h != 1 || p.pool_w != 1;
+    const bool tiled = (p.pool_w == 1 || p.pool_w == 2) && (kXT - 1) * p.stride_w + p.S <= kMaxCols;
+    const int rows_out = pooled ? p.OH : p.PH;  // rows the workgroups are dealt
     if (name_buf != nullptr) {  // report the kernel instead of launching it
         if (!tiled) {
             snprintf(name_buf, name_len, "inconv_generic_kernel");
@@ -455,10 +481,11 @@ static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name
         const int rpw = (64 / ncols) / 3 * 3;
         if (rpw >= 3 && 64LL * 3 * p.H * p.W * 4 < (1LL << 31)) {
             const int passes = (3 * 64 + 4 * rpw - 1) / (4 * rpw);
-            snprintf(name_buf, name_len, "inconv_tiled_kernel<%d, true>", passes <= 4 ? 4 : (passes <= 8 ? 8 : 16));
+            snprintf(name_buf, name_len, "inconv_tiled_kernel<%d, true, %s>", passes <= 4 ? 4 : (passes <= 8 ? 8 : 16),
+                     pooled ? "true" : "false");
         } else {
-            snprintf(name_buf, name_len, "inconv_tiled_kernel<%d, false>",
-                     (3 * 64 * ncols + kThreads - 1) / kThreads <= 15 ? 15 : 24);
+            snprintf(name_buf, name_len, "inconv_tiled_kernel<%d, false, %s>",
+                     (3 * 64 * ncols + kThreads - 1) / kThreads <= 15 ? 15 : 24, pooled ? "true" : "false");
         }
         return TCBNN_OK;
     }
@@ -475,8 +502,8 @@ static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name
         static const bool plain_order = getenv("TCBNN_INCONV_ORDER") != nullptr;  // tuning switch
         const int y_phases = (!plain_order && 8 % b_tiles == 0) ? 8 / b_tiles : 0;
         const long long blocks = y_phases > 0
-                                     ? 8LL * ((x_groups + y_phases - 1) / y_phases) * p.PH
-                                     : (long long)b_tiles * x_groups * p.PH;
+                                     ? 8LL * ((x_groups + y_phases - 1) / y_phases) * rows_out
+                                     : (long long)b_tiles * x_groups * rows_out;
         TCBNN_REQUIRE(blocks <= 0x7fffffffLL, "inconv128: grid too large");
         // staging scheme (see the kernel): whole segments per wave when at least 3 fit its 64 lanes
         const int rpw = (64 / ncols) / 3 * 3;
@@ -484,20 +511,28 @@ static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name
             hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(kThreads), 0, (hipStream_t)stream, p, p.in,
                                p.masks, p.bn, p.out, p.res, b_tiles, x_groups, y_phases, div_magic, rpw);
         };
+        auto launch_nst = [&](auto nst_tag, auto rows_tag) {
+            constexpr int NST = decltype(nst_tag)::value;
+            constexpr bool ROWS = decltype(rows_tag)::value;
+            if (pooled)
+                launch(inconv_tiled_kernel<NST, ROWS, true>);
+            else
+                launch(inconv_tiled_kernel<NST, ROWS, false>);
+        };
         if (rpw >= 3 && 64LL * 3 * p.H * p.W * 4 < (1LL << 31)) {
             const int passes = (3 * 64 + 4 * rpw - 1) / (4 * rpw);
             if (passes <= 4)
-                launch(inconv_tiled_kernel<4, true>);
+                launch_nst(std::integral_constant<int, 4>{}, std::true_type{});
             else if (passes <= 8)
-                launch(inconv_tiled_kernel<8, true>);
+                launch_nst(std::integral_constant<int, 8>{}, std::true_type{});
             else
-                launch(inconv_tiled_kernel<16, true>);
+                launch_nst(std::integral_constant<int, 16>{}, std::true_type{});
         } else {
             const int nst = (3 * 64 * ncols + kThreads - 1) / kThreads;
             if (nst <= 15)
-                launch(inconv_tiled_kernel<15, false>);
+                launch_nst(std::integral_constant<int, 15>{}, std::false_type{});
             else
-                launch(inconv_tiled_kernel<24, false>);
+                launch_nst(std::integral_constant<int, 24>{}, std::false_type{});
         }
         TCBNN_LAUNCH_CHECK("inconv_tiled_kernel");
         return TCBNN_OK;

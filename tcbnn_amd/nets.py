@@ -1,5 +1,6 @@
-"""Network drivers: the layer wiring of the reference's mnist_mlp.cu, cifar10_vgg.cu and
-imagenet_resnet.cu mains, as host loops over layer.forward(stream).
+"""Network drivers: the layer wiring of the reference's mnist_mlp.cu, cifar10_vgg.cu,
+imagenet_resnet.cu, alexnet.cu, cifar10_resnet.cu and imagenet_vgg.cu mains, as host loops over
+layer.forward(stream).
 
 A network is described by a list of layer specs (plain dicts, constructor arguments in
 the reference's order) so the same description can drive other implementations of the
@@ -90,7 +91,73 @@ def imagenet_resnet_spec(batch=256, image=224, output_size=1000):
     return spec
 
 
-SPECS = {"mnist_mlp": mnist_mlp_spec, "cifar10_vgg": cifar10_vgg_spec, "imagenet_resnet": imagenet_resnet_spec}
+def alexnet_spec(batch=256, image=224, n_hidden=4096, output_size=1000):
+    """alexnet.cu:143-177: 11x11 stride-4 first layer with 2x2 pooling, a 5x5 layer, channel counts
+    that are not multiples of 128 (192, 384)."""
+    spec = [dict(kind="inconv", name="Conv1", h=image, w=image, r=11, s=11, cin=3, cout=64, batch=batch,
+                 stride=4, padding=True, pool=2, save_residual=False)]
+    h = _conv_out(image, 11, 4, pool=2)
+    spec.append(_conv("Conv2", h, 64, 192, batch, "Conv1", pool=2, r=5)); h = _conv_out(h, 5, 1, pool=2)
+    spec.append(_conv("Conv3", h, 192, 384, batch, "Conv2"))
+    spec.append(_conv("Conv4", h, 384, 256, batch, "Conv3"))
+    spec.append(_conv("Conv5", h, 256, 256, batch, "Conv4", pool=2, ahead_fc=True)); h = _conv_out(h, 3, 1, pool=2)
+    spec.append(dict(kind="fc", name="Fc1", batch=batch, inp=h * h * 256, out=n_hidden, src="Conv5"))
+    spec.append(dict(kind="fc", name="Fc2", batch=batch, inp=n_hidden, out=n_hidden, src="Fc1"))
+    spec.append(dict(kind="out", name="Fout", batch=batch, inp=n_hidden, out=output_size, src="Fc2"))
+    return spec
+
+
+def cifar10_resnet_spec(batch=256, image=32, output_size=10):
+    """cifar10_resnet.cu:189-259: 3x3 first layer with saved residual, three stages of two blocks
+    (128 / 256 / 512 channels), stage-entry shortcut = 2x2 maximum of the previous residual into the
+    first 128 / 256 channels."""
+    B = batch
+    spec = [dict(kind="inconv", name="Conv1", h=image, w=image, r=3, s=3, cin=3, cout=128, batch=B,
+                 stride=1, padding=True, pool=1, save_residual=True)]
+    h = image
+    spec.append(_conv("L1B1C1", h, 128, 128, B, "Conv1"))
+    spec.append(_conv("L1B1C2", h, 128, 128, B, "L1B1C1", save_residual=True, inject_residual=True,
+                      residual_channels=128, res_src="Conv1"))
+    spec.append(_conv("L1B2C1", h, 128, 128, B, "L1B1C2"))
+    spec.append(_conv("L1B2C2", h, 128, 128, B, "L1B2C1", save_residual=True, inject_residual=True,
+                      residual_channels=128, res_src="L1B1C2"))
+    prev, cin = "L1B2C2", 128
+    for stage, cout in ((2, 256), (3, 512)):
+        n1, n2, n3, n4 = ("L%dB%dC%d" % (stage, b, c) for b in (1, 2) for c in (1, 2))
+        spec.append(_conv(n1, h, cin, cout, B, prev, stride=2))
+        h = _conv_out(h, 3, 2)
+        spec.append(_conv(n2, h, cout, cout, B, n1, save_residual=True, inject_residual=True,
+                          residual_channels=cin, residual_pool=True, res_src=prev))
+        spec.append(_conv(n3, h, cout, cout, B, n2))
+        last = stage == 3
+        spec.append(_conv(n4, h, cout, cout, B, n3, ahead_fc=last, save_residual=not last,
+                          inject_residual=True, residual_channels=cout, res_src=n2))
+        prev, cin = n4, cout
+    spec.append(dict(kind="fc", name="Fc1", batch=B, inp=h * h * 512, out=512, src=prev))
+    spec.append(dict(kind="out", name="Fout", batch=B, inp=512, out=output_size, src="Fc1"))
+    return spec
+
+
+def imagenet_vgg_spec(batch=256, image=224, n_hidden=4096, output_size=1000):
+    """imagenet_vgg.cu:217-286: VGG-16, 2x2 pooling after layers 2, 4, 7, 10 and 13."""
+    spec = [dict(kind="inconv", name="Conv1", h=image, w=image, r=3, s=3, cin=3, cout=64, batch=batch,
+                 stride=1, padding=True, pool=1, save_residual=False)]
+    h, cin, prev = image, 64, "Conv1"
+    plan = [(64, 2), (128, 1), (128, 2), (256, 1), (256, 1), (256, 2), (512, 1), (512, 1), (512, 2),
+            (512, 1), (512, 1), (512, 2)]
+    for i, (cout, pool) in enumerate(plan):
+        name = "Conv%d" % (i + 2)
+        spec.append(_conv(name, h, cin, cout, batch, prev, pool=pool, ahead_fc=i == len(plan) - 1))
+        h = _conv_out(h, 3, 1, pool=pool)
+        prev, cin = name, cout
+    spec.append(dict(kind="fc", name="Fc1", batch=batch, inp=h * h * 512, out=n_hidden, src=prev))
+    spec.append(dict(kind="fc", name="Fc2", batch=batch, inp=n_hidden, out=n_hidden, src="Fc1"))
+    spec.append(dict(kind="out", name="Fout", batch=batch, inp=n_hidden, out=output_size, src="Fc2"))
+    return spec
+
+
+SPECS = {"mnist_mlp": mnist_mlp_spec, "cifar10_vgg": cifar10_vgg_spec, "imagenet_resnet": imagenet_resnet_spec,
+         "alexnet": alexnet_spec, "cifar10_resnet": cifar10_resnet_spec, "imagenet_vgg": imagenet_vgg_spec}
 
 
 def binary_ops(spec):

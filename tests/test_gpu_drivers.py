@@ -66,6 +66,23 @@ def test_imagenet_resnet_driver(gpu, tmp_path):
     _run_driver(tmp_path, "imagenet_resnet", spec, ["--image", "64", "--classes", "100"], 7, "mfma_f4")
 
 
+def test_alexnet_driver(gpu, tmp_path):
+    from tcbnn_amd import nets
+    spec = nets.alexnet_spec(batch=8, image=96, output_size=100)
+    _run_driver(tmp_path, "alexnet", spec, ["--image", "96", "--classes", "100"], 8, "mfma_f4")
+
+
+def test_cifar10_resnet_driver(gpu, tmp_path):
+    from tcbnn_amd import nets
+    _run_driver(tmp_path, "cifar10_resnet", nets.cifar10_resnet_spec(batch=8), [], 9, "mfma_f4")
+
+
+def test_imagenet_vgg_driver(gpu, tmp_path):
+    from tcbnn_amd import nets
+    spec = nets.imagenet_vgg_spec(batch=8, image=32, output_size=100)
+    _run_driver(tmp_path, "imagenet_vgg", spec, ["--image", "32", "--classes", "100"], 10, "popc")
+
+
 def test_driver_synthetic_mode_runs(gpu):
     exe = os.path.join(BIN, "imagenet_resnet")
     proc = subprocess.run([exe, "--batch", "8", "--image", "64", "--classes", "10", "--reps", "2"],

@@ -343,7 +343,12 @@ def test_conv128_rejects_residual_with_pooling(gpu):
                                                          # scheme), partial image tiles, whole tiles, odd channel counts
                                                          (70, 24, 11, 4, 64, 1, True), (66, 20, 7, 4, 40, 1, True),
                                                          (9, 17, 3, 2, 33, 1, True), (64, 16, 7, 4, 64, 1, True),
-                                                         (128, 10, 3, 1, 64, 1, True)])
+                                                         (128, 10, 3, 1, 64, 1, True),
+                                                         # pooled first layers (alexnet.cu:143-144): tiled kernel
+                                                         # with 2x2 windows, odd row / column counts, a 3x3 pool
+                                                         # (generic kernel)
+                                                         (70, 24, 11, 4, 64, 2, False), (8, 26, 3, 2, 64, 2, False),
+                                                         (9, 18, 7, 2, 40, 2, False), (5, 18, 3, 1, 64, 3, False)])
 def test_inconv128_layer(gpu, b, h, R, stride, cout, pool, save):
     r = rng(b + h + R + cout)
     x = r.standard_normal((b, 3, h, h)).astype(np.float32)
@@ -471,6 +476,29 @@ def test_imagenet_resnet18(gpu, variant, residual_format):
         net.release()
         assert fmts and all(f == 1 for f in fmts.values()), fmts
     _compare_network(gpu, spec, 3, variant, residual_format)
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+def test_alexnet(gpu, variant):
+    """alexnet.cu:143-177 at full image size: 11x11 stride-4 pooled first layer, 5x5 layer, 192 / 384
+    channels (words that are only partly used), three FC layers."""
+    from tcbnn_amd import nets
+    _compare_network(gpu, nets.alexnet_spec(batch=8), 11, variant)
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+def test_cifar10_resnet(gpu, variant):
+    """cifar10_resnet.cu:189-259 at full image size: 3x3 first layer with saved residual, pooled
+    residuals at both stage entries."""
+    from tcbnn_amd import nets
+    _compare_network(gpu, nets.cifar10_resnet_spec(batch=16), 12, variant)
+
+
+@pytest.mark.parametrize("variant", ["mfma_f4"])
+def test_imagenet_vgg(gpu, variant):
+    """imagenet_vgg.cu:217-286 (VGG-16) at full image size."""
+    from tcbnn_amd import nets
+    _compare_network(gpu, nets.imagenet_vgg_spec(batch=8), 13, variant)
 
 
 def test_imagenet_resnet18_batch256_every_image(gpu):
