@@ -58,7 +58,7 @@ conv3x3_mfma_f4_kernel(
     int n_groups, int b_groups, int pix_streams) {
     static_assert(RM == RM_NONE || MT == 1, "residual instantiations own one image tile per wave");
     static_assert(RM == RM_NONE || !POOL, "residuals are defined for un-pooled layers only");
-    constexpr int TPC = SPT >= 4 ? 3 : 9;  // taps per prefetch chunk (a filter row, or all of it)
+    constexpr int TPC = SPT >= 3 ? 3 : 9;  // taps per prefetch chunk (a filter row, or all of it)
     constexpr int NCH = 9 / TPC;           // chunks per tile
     constexpr int NQ = 9 * SPT;            // k-steps per tile
     // A tile of one chunk is shorter than the memory latency: its residual operand is then
@@ -557,7 +557,7 @@ conv3x3_mfma_f4_kernel(
     // buffers: the chunk that will be multiplied NB-1 steps from now is requested before the current
     // one is multiplied (two or three steps of lookahead without a residual, where one chunk of MFMAs
     // is much shorter than the memory latency and few waves share a SIMD).
-    constexpr int NB = kAhead ? 2 : (SPT >= 4 ? 3 : 2);
+    constexpr int NB = kAhead ? 2 : (SPT >= 3 ? 3 : 2);
     constexpr int LOOK = NB - 1;
     struct Cursor {
         int pi, y, x, chunk, sub;  // item index, row and (skewed) column, chunk of the tile, pixel of the window
@@ -729,7 +729,7 @@ struct Pick {
     int rm, mt, nt, r16, pool;
 };
 constexpr int pick_nt(int spt, int rm) {
-    return rm == RM_POOLED ? 1 : (rm == RM_PLAIN ? (spt >= 4 ? 1 : 2) : (spt >= 8 ? 1 : 2));
+    return rm == RM_POOLED ? 1 : (rm == RM_PLAIN ? (spt >= 4 ? 1 : 2) : (spt >= 6 ? 1 : 2));
 }
 Pick pick(const BgemmParams& p) {
     const int rm = p.res_in == nullptr && p.res_out == nullptr ? RM_NONE
@@ -772,7 +772,7 @@ bool conv3x3_mfma_applicable(const BgemmParams& p) {
     const bool centre_ok = p.pad_h <= 1 && p.pad_w <= 1 && (p.PH - 1) * p.stride_h - p.pad_h + 1 < p.H &&
                            (p.PW - 1) * p.stride_w - p.pad_w + 1 < p.W;
     return p.R == 3 && p.S == 3 && pool_ok && centre_ok && p.mode == EPI_THRESH && p.nan_bit == 1 &&
-           p.ksplit <= 1 && (p.cw == 2 || p.cw == 4 || p.cw == 8 || p.cw == 16) && p.k_tap == 32 * p.cw &&
+           p.ksplit <= 1 && filter_has_fragments(3, 3, 32 * p.cw) && p.k_tap == 32 * p.cw &&
            (long long)p.PH * p.PW < (1 << 24) && within_2gib(p);
 }
 
@@ -788,8 +788,12 @@ int launch_conv3x3_mfma(const BgemmParams& p, hipStream_t stream) {
             return launch_m<1>(p, stream);
         case 4:
             return launch_m<2>(p, stream);
+        case 6:
+            return launch_m<3>(p, stream);
         case 8:
             return launch_m<4>(p, stream);
+        case 12:
+            return launch_m<6>(p, stream);
         default:
             return launch_m<8>(p, stream);
     }

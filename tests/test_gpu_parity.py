@@ -178,6 +178,9 @@ CONV_CASES = [
     (8, 8, 128, 128, 1, 1, False), (70, 8, 128, 128, 1, 2, False), (8, 7, 64, 96, 1, 2, False),
     (130, 12, 64, 128, 2, 1, False), (8, 9, 256, 32, 1, 3, False), (24, 4, 512, 512, 1, 2, True),
     (8, 4, 64, 160, 1, 2, True), (256, 7, 128, 64, 1, 1, False),
+    # Cin = 192 / 384 (alexnet.cu:154-162) and 2x2 pooling with them
+    (40, 13, 192, 384, 1, 1, False), (72, 13, 384, 256, 1, 1, False), (8, 6, 192, 96, 1, 2, True),
+    (130, 9, 384, 64, 2, 1, False),
 ]
 
 
@@ -210,7 +213,7 @@ def test_conv128_layer(gpu, variant, b, h, cin, cout, stride, pool, ahead_fc):
 
 # (cin, cout): the persistent 3x3 kernel's instantiations (Cin 64 .. 512), a channel count that is not a
 # multiple of 32 and an odd one (half-filled last 16-bit pair); formats of the injected and saved tensors
-RES_SHAPES = [(64, 96), (128, 64), (256, 35), (512, 64)]
+RES_SHAPES = [(64, 96), (128, 64), (256, 35), (512, 64), (192, 64), (384, 40)]
 RES_FORMATS = [(0, 0), (1, 1), (0, 1), (1, 0)]
 
 
