@@ -117,6 +117,67 @@ def roofline_of(name, g, variant):
     return rec
 
 
+def sweep(args, np, _lib):
+    """Stand-alone kernels of the reference's benchmarks: BMMAS_new (tensorcore_kernel.cu:336-356) as
+    tcbnn_bmm, BTC_Conv2d_balance (bmma_kernel.cu:101-165) as tcbnn_bconv; operands resident, packed
+    once outside the timed launches; int32 outputs.  Binary operations: 2 per +-1 multiply-accumulate,
+    border taps included; bytes: packed operands + int32 output, each moved once."""
+    import ctypes as C
+    from tcbnn_amd.device import DeviceBuffer, Event, Stream
+    lib = _lib.lib
+    stream = Stream()
+    rng = np.random.default_rng(0)
+    reps = max(args.steps, 10)
+
+    def timed(launch):
+        for _ in range(args.warmup):
+            launch()
+        stream.synchronize()
+        ts = []
+        e0, e1 = Event(), Event()
+        for _ in range(reps):
+            e0.record(stream)
+            launch()
+            e1.record(stream)
+            stream.synchronize()
+            ts.append(e0.elapsed_ms(e1))
+        return float(np.median(ts))
+
+    rows = []
+    for name, v in (("popc", _lib.VARIANTS["popc"]), ("mfma_i8", _lib.VARIANTS["mfma_i8"]), ("mfma_f4", _lib.VARIANTS["mfma_f4"])):
+        for m, n, k in ((1024, 1024, 1024), (8192, 1024, 1024), (8192, 8192, 8192)):
+            a = DeviceBuffer.from_numpy(rng.integers(0, 2 ** 32, size=(k // 32, m), dtype=np.uint64).astype(np.uint32))
+            b = DeviceBuffer.from_numpy(rng.integers(0, 2 ** 32, size=(n, k // 32), dtype=np.uint64).astype(np.uint32))
+            c = DeviceBuffer(4 * m * n)
+            ms = timed(lambda: _lib.check(lib.tcbnn_bmm(a.ptr, b.ptr, c.ptr, m, n, k, v, stream.handle)))
+            ops, byts = 2.0 * m * n * k, (m + n) * k / 8 + 4.0 * m * n
+            rows.append(dict(case="bmm %dx%dx%d" % (m, n, k), engine=name, ms=round(ms, 4),
+                             binary_tops=round(ops / ms / 1e9, 1), hbm_gbs=round(byts / ms / 1e6, 1)))
+            for buf in (a, b, c):
+                buf.free()
+        for h, ch in ((32, 128), (16, 256), (8, 512), (56, 64), (28, 128), (14, 256), (7, 512)):
+            B = 256
+            inp = DeviceBuffer.from_numpy(rng.integers(0, 2 ** 32, size=h * h * (ch // 32) * B, dtype=np.uint64).astype(np.uint32))
+            f = DeviceBuffer.from_numpy((rng.integers(0, 2, size=(3, 3, ch, ch)) * 2 - 1).astype(np.float32))
+            filt = DeviceBuffer(4 * lib.tcbnn_conv_filter_words(3, 3, ch, ch))
+            _lib.check(lib.tcbnn_pack_conv_filter(f.ptr, filt.ptr, 3, 3, ch, ch, stream.handle))
+            out = DeviceBuffer(4 * B * h * h * ch)
+            ms = timed(lambda: _lib.check(lib.tcbnn_bconv(inp.ptr, filt.ptr, out.ptr, B, h, h, ch, ch, 3, 3, 1, 1, 1, 1,
+                                                          h, h, v, stream.handle)))
+            ops = 2.0 * B * h * h * ch * ch * 9
+            byts = B * h * h * ch / 8 + 9 * ch * ch / 8 + 4.0 * B * h * h * ch
+            rows.append(dict(case="bconv 3x3 %dx%d C=%d b256" % (h, h, ch), engine=name, ms=round(ms, 4),
+                             binary_tops=round(ops / ms / 1e9, 1), hbm_gbs=round(byts / ms / 1e6, 1)))
+            for buf in (inp, f, filt, out):
+                buf.free()
+    sys.stderr.write("%-28s %-8s %9s %12s %9s\n" % ("case", "engine", "ms", "binary TOP/s", "GB/s"))
+    for r in rows:
+        sys.stderr.write("%-28s %-8s %9.4f %12.1f %9.1f\n" % (r["case"], r["engine"], r["ms"], r["binary_tops"], r["hbm_gbs"]))
+    print(json.dumps({"metric": "binary TOP/s of the stand-alone bit-GEMM / 3x3 bit-convolution kernels (int32 outputs)",
+                      "unit": "TOP/s", "n_gpus": 1, "data": "synthetic", "rows": rows}))
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -128,6 +189,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-batch", type=int, default=None)
     ap.add_argument("--layers", action="store_true", help="also print a per-layer table to stderr")
+    ap.add_argument("--sweep", action="store_true",
+                    help="instead of a network: the stand-alone bit-GEMM and 3x3 bit-convolution shapes "
+                         "(int32 outputs), every engine; one JSON line with a row per case")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build drives one GPU (one process, one device); --gpus %d is not supported. "
@@ -145,6 +209,9 @@ def main():
     if args.variant != "auto":
         _lib.check(_lib.lib.tcbnn_set_default_variant(_lib.VARIANTS[args.variant]))
     variant = {v: k for k, v in _lib.VARIANTS.items()}[_lib.lib.tcbnn_get_default_variant()]
+
+    if args.sweep:
+        return sweep(args, np, _lib)
 
     default_batch = {"mnist_mlp": 8192}.get(args.net, 256)
     batch = args.batch or default_batch

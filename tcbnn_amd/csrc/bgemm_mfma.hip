@@ -253,10 +253,20 @@ __global__ __launch_bounds__(kThreads) void bgemm_mfma_kernel(
                                     __fmul_rn((float)A::to_int(acc[mt][nt][v]), bnp[c]), p.bn_bias[c]);
                         }
                     } else {
-                        int32_t* dst = p.out_i32 + pix * p.raw_pix_stride + (size_t)b * p.raw_b_stride;
+                        int32_t* dst = p.out_i32 + pix * p.raw_pix_stride + (size_t)b * p.raw_b_stride + cbase;
+                        // a lane's 16 values are consecutive in memory: four 128-bit stores where the
+                        // run is whole and aligned
+                        if (cbase + 16 <= p.N && (reinterpret_cast<uintptr_t>(dst) & 15) == 0) {
 #pragma unroll
-                        for (int v = 0; v < 16; ++v)
-                            if (cbase + v < p.N) dst[cbase + v] = A::to_int(acc[mt][nt][v]);
+                            for (int g = 0; g < 4; ++g)
+                                reinterpret_cast<int4*>(dst)[g] =
+                                    make_int4(A::to_int(acc[mt][nt][4 * g]), A::to_int(acc[mt][nt][4 * g + 1]),
+                                              A::to_int(acc[mt][nt][4 * g + 2]), A::to_int(acc[mt][nt][4 * g + 3]));
+                        } else {
+#pragma unroll
+                            for (int v = 0; v < 16; ++v)
+                                if (cbase + v < p.N) dst[v] = A::to_int(acc[mt][nt][v]);
+                        }
                     }
                 }
             }

@@ -39,6 +39,7 @@ constexpr int kThreads = 64 * kWaves;
 constexpr int RM_NONE = 0;    // threshold only
 constexpr int RM_PLAIN = 1;   // residual injected from a source of the same size and / or saved
 constexpr int RM_POOLED = 2;  // residual injected as the 2x2 max of a source twice the size
+constexpr int RM_RAW = 3;     // no threshold: the +-1 dot products are stored as int32 (tcbnn_bconv)
 
 // Waves per SIMD the register allocator is asked to make room for: the residual layers are
 // bound by HBM and want more memory requests in flight, the plain layers want registers.
@@ -56,14 +57,15 @@ conv3x3_mfma_f4_kernel(
     const float* __restrict__ bnp, const int32_t* __restrict__ rin, int32_t* __restrict__ rout, int res_lim,
     int rin_fmt, int rout_fmt, unsigned act_bytes, unsigned rin_bytes, unsigned rout_bytes, unsigned bits_bytes,
     int n_groups, int b_groups, int pix_streams) {
-    static_assert(RM == RM_NONE || MT == 1, "residual instantiations own one image tile per wave");
+    static_assert(RM == RM_NONE || RM == RM_RAW || MT == 1, "residual instantiations own one image tile per wave");
+    constexpr bool kRes = RM == RM_PLAIN || RM == RM_POOLED;  // a residual is injected and / or saved
     static_assert(RM == RM_NONE || !POOL, "residuals are defined for un-pooled layers only");
     constexpr int TPC = SPT >= 3 ? 3 : 9;  // taps per prefetch chunk (a filter row, or all of it)
     constexpr int NCH = 9 / TPC;           // chunks per tile
     constexpr int NQ = 9 * SPT;            // k-steps per tile
     // A tile of one chunk is shorter than the memory latency: its residual operand is then
     // requested a whole tile ahead (double-buffered); otherwise with the tile's first chunk.
-    constexpr bool kAhead = RM != RM_NONE && NCH == 1;
+    constexpr bool kAhead = kRes && NCH == 1;
     extern __shared__ v4i lds_dyn[];
     v4i* lds_w = lds_dyn;  // [NQ][NT][64] fragments
     float* lds_thr = reinterpret_cast<float*>(lds_dyn + NQ * NT * 64);  // [NT*32]
@@ -112,7 +114,7 @@ conv3x3_mfma_f4_kernel(
     // first MFMA): the finished accumulator is s - ceil(threshold), exact in fp32, and its sign is
     // the inverted output bit, with no per-value subtraction in the epilogue.
     if (tid < NT * 32) {
-        float t = n0 + tid < p.N ? bnp[n0 + tid] : 0.0f;
+        float t = RM != RM_RAW && n0 + tid < p.N ? bnp[n0 + tid] : 0.0f;
         t = t != t ? -__builtin_huge_valf() : t;
         if constexpr (RM == RM_NONE) t = 0.0f - fminf(fmaxf(ceilf(t), -8192.0f), 8192.0f);
         lds_thr[tid] = t;
@@ -155,6 +157,9 @@ conv3x3_mfma_f4_kernel(
     const __amdgpu_buffer_rsrc_t r_act = make_rsrc(act, act_bytes), r_rin = make_rsrc(rin, rin_bytes),
                                  r_rout = make_rsrc(rout, rout_bytes), r_bits = make_rsrc(p.out_bits, bits_bytes);
     const unsigned row_b = (unsigned)p.B * 4u;  // bytes between consecutive words / channels of an image
+    // RM_RAW: may a lane's 16 consecutive int32 outputs go out as 128-bit words?  (uniform)
+    const bool raw_aligned = RM == RM_RAW && p.raw_pix_stride % 4 == 0 && p.raw_b_stride % 4 == 0 &&
+                             (reinterpret_cast<uintptr_t>(rout) & 15) == 0;
     unsigned voff_act[MT], voff_bits[MT];  // activation loads; output words (stored by lanes 0-31)
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
@@ -319,7 +324,7 @@ conv3x3_mfma_f4_kernel(
     // image bload[0]; every load is a wave-uniform base plus this per-lane element offset.
     // A lane's 16 values arrive as 16 (int32) or 8 (int16 pairs) words; a plain operand stays in
     // that raw form until its epilogue, a pooled one is reduced to 16 ints by finish_residual.
-    constexpr int NRV = RM != RM_NONE ? NT : 1;
+    constexpr int NRV = kRes ? NT : 1;
     constexpr int NTMP = RM == RM_POOLED ? 3 : 1;
     constexpr int NRAW = R16 ? 8 : 16;                    // words loaded per channel tile
     constexpr int NW = RM == RM_POOLED ? 16 : NRAW;       // words kept per channel tile
@@ -330,7 +335,7 @@ conv3x3_mfma_f4_kernel(
     const unsigned grp_b = (unsigned)p.B * 16u;  // bytes between consecutive channel groups
 
     auto request_residual = [&](int yy, int xx, int (*rv)[NW]) __attribute__((always_inline)) {
-        if constexpr (RM != RM_NONE) {
+        if constexpr (kRes) {
             constexpr bool i16 = R16;
             // bytes per source pixel; per-lane offset; 128-bit loads per channel tile.  Groups past the
             // source's channels read the neighbouring pixel or (at the end of the tensor) zeros; their
@@ -411,7 +416,7 @@ conv3x3_mfma_f4_kernel(
         constexpr bool FAST = decltype(fast_tag)::value;
         const int cbase = n0 + nt * 32 + 16 * h;  // this lane's channels: cbase + v
         float thr[16];
-        if constexpr (RM != RM_NONE) {
+        if constexpr (kRes) {
             const float4* t4 = reinterpret_cast<const float4*>(lds_thr + nt * 32 + 16 * h);
 #pragma unroll
             for (int k = 0; k < 4; ++k) {
@@ -422,12 +427,40 @@ conv3x3_mfma_f4_kernel(
                 thr[4 * k + 3] = tv.w;
             }
         }
+        if constexpr (RM == RM_RAW) {
+            // int32 dot products, out_i32[pix * raw_pix_stride + b * raw_b_stride + channel]: a lane's 16
+            // channels are consecutive, stored as four 128-bit words (single words for a partial tile or an
+            // unaligned run); the kernel's `rout` descriptor covers this tensor
+            const unsigned so = (pix * (unsigned)p.raw_pix_stride + (unsigned)(n0 + nt * 32)) * 4u;  // uniform
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const unsigned vo = bimg[mt] < p.B ? ((unsigned)bimg[mt] * (unsigned)p.raw_b_stride + 16u * (unsigned)h) * 4u
+                                                   : kOutOfRange;
+                if (FAST && raw_aligned) {
+                    v4i q[4];
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        q[g] = v4i{(int)acc[mt][nt][4 * g], (int)acc[mt][nt][4 * g + 1], (int)acc[mt][nt][4 * g + 2],
+                                   (int)acc[mt][nt][4 * g + 3]};
+                        __builtin_amdgcn_raw_buffer_store_b128(q[g], r_rout, (int)vo, (int)(so + 16u * (unsigned)g), 0);
+                    }
+                    asm volatile("s_nop 4" ::"v"(q[0]), "v"(q[1]), "v"(q[2]), "v"(q[3]));  // see the residual stores
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v)
+                        __builtin_amdgcn_raw_buffer_store_b32((int)acc[mt][nt][v], r_rout,
+                                                              (int)(cbase + v < p.N ? vo : kOutOfRange),
+                                                              (int)(so + 4u * (unsigned)v), 0);
+                }
+            }
+            return;
+        }
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
             const int b = bimg[mt];
             const bool b_ok = b < p.B;
             uint32_t hw = 0;
-            if constexpr (RM != RM_NONE) {
+            if constexpr (kRes) {
                 int res[16];
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
@@ -538,13 +571,13 @@ conv3x3_mfma_f4_kernel(
             const int cb = n0 + nt * 32;
             // uniform: every channel of the tile exists, and gets a residual if any does (a tile that
             // gets none at all holds zeros and is fast as well)
-            const bool fast = cb + 32 <= p.N && (RM == RM_NONE || cb + 32 <= res_lim || cb >= res_lim);
+            const bool fast = cb + 32 <= p.N && (!kRes || cb + 32 <= res_lim || cb >= res_lim);
             if (fast)
                 epilogue_tile(std::true_type{}, nt, pix, bits_pix, rv, sub);
             else
                 epilogue_tile(std::false_type{}, nt, pix, bits_pix, rv, sub);
         }
-        if (ng == n_groups - 1 && (!POOL || sub == 3)) {  // zero the pixel's padding words
+        if (RM != RM_RAW && ng == n_groups - 1 && (!POOL || sub == 3)) {  // zero the pixel's padding words
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
                 for (int w = max((p.N + 31) / 32, n_groups * NT); w < p.bits_row_words; ++w)
@@ -632,7 +665,7 @@ conv3x3_mfma_f4_kernel(
                 if (nt.pi < npix) finish_residual(rv[1 - I]);
             }
         } else {
-            if constexpr (RM != RM_NONE) {
+            if constexpr (kRes) {
                 if (cc.chunk == 0) request_residual(cc.y, cc.x, rcur);
             }
             compute_chunk(cc.chunk, buf[I], msk[I], fused, buf[J], nsoff);
@@ -672,6 +705,11 @@ TensorBytes tensor_bytes(const BgemmParams& p) {
     t.rin = p.res_in != nullptr ? 4 * res_words((long long)p.PH * p.PW * (p.res_pool ? 4 : 1), p.res_in_ch, p.res_in_fmt) : 0;
     t.rout = p.res_out != nullptr ? 4 * res_words((long long)p.PH * p.PW, p.N, p.res_out_fmt) : 0;
     t.bits = 4LL * p.OH * p.OW * p.bits_pix_stride;
+    if (p.mode == EPI_RAW) {  // the int32 output takes the place of the saved residual
+        const long long last = ((long long)p.PH * p.PW - 1) * p.raw_pix_stride + (long long)(p.B - 1) * p.raw_b_stride + p.N;
+        t.rout = 4 * last;
+        t.bits = 0;
+    }
     return t;
 }
 
@@ -714,7 +752,8 @@ int launch_t(const BgemmParams& p, hipStream_t stream) {
     const long long blocks = (long long)best * n_groups * b_groups;
     const TensorBytes tb = tensor_bytes(p);
     hipLaunchKernelGGL((conv3x3_mfma_f4_kernel<SPT, RM, MT, NT, R16, POOL>), dim3((unsigned)blocks), dim3(kThreads), lds_bytes,
-                       stream, p, p.act, p.wgt, p.bn, p.res_in, p.res_out, res_lim, p.res_in_fmt, p.res_out_fmt,
+                       stream, p, p.act, p.wgt, p.bn, p.res_in, RM == RM_RAW ? p.out_i32 : p.res_out, res_lim, p.res_in_fmt,
+                       p.res_out_fmt,
                        (unsigned)tb.act, (unsigned)tb.rin, (unsigned)tb.rout, (unsigned)tb.bits, n_groups, b_groups, best);
     TCBNN_LAUNCH_CHECK("conv3x3_mfma_f4_kernel");
     return TCBNN_OK;
@@ -729,12 +768,14 @@ struct Pick {
     int rm, mt, nt, r16, pool;
 };
 constexpr int pick_nt(int spt, int rm) {
-    return rm == RM_POOLED ? 1 : (rm == RM_PLAIN ? (spt >= 4 ? 1 : 2) : (spt >= 6 ? 1 : 2));
+    return rm == RM_POOLED ? 1 : (rm == RM_PLAIN ? (spt >= 4 ? 1 : 2) : (spt >= 6 ? 1 : 2));  // RM_RAW as RM_NONE
 }
 Pick pick(const BgemmParams& p) {
-    const int rm = p.res_in == nullptr && p.res_out == nullptr ? RM_NONE
-                                                                : (p.res_in != nullptr && p.res_pool ? RM_POOLED : RM_PLAIN);
-    return {rm, rm == RM_NONE ? 2 : 1, pick_nt(p.cw / 2, rm), p.res_in != nullptr && p.res_in_fmt == TCBNN_RES_I16,
+    const int rm = p.mode == EPI_RAW ? RM_RAW
+                   : p.res_in == nullptr && p.res_out == nullptr
+                       ? RM_NONE
+                       : (p.res_in != nullptr && p.res_pool ? RM_POOLED : RM_PLAIN);
+    return {rm, rm == RM_NONE || rm == RM_RAW ? 2 : 1, pick_nt(p.cw / 2, rm), p.res_in != nullptr && p.res_in_fmt == TCBNN_RES_I16,
             p.pool_h == 2};
 }
 
@@ -745,6 +786,8 @@ int launch_m(const BgemmParams& p, hipStream_t stream) {
         case RM_NONE:
             return k.pool ? launch_t<SPT, RM_NONE, 2, pick_nt(SPT, RM_NONE), false, true>(p, stream)
                           : launch_t<SPT, RM_NONE, 2, pick_nt(SPT, RM_NONE), false, false>(p, stream);
+        case RM_RAW:
+            return launch_t<SPT, RM_RAW, 2, pick_nt(SPT, RM_RAW), false, false>(p, stream);
         case RM_PLAIN:
             return k.r16 ? launch_t<SPT, RM_PLAIN, 1, pick_nt(SPT, RM_PLAIN), true, false>(p, stream)
                          : launch_t<SPT, RM_PLAIN, 1, pick_nt(SPT, RM_PLAIN), false, false>(p, stream);
@@ -771,7 +814,11 @@ bool conv3x3_mfma_applicable(const BgemmParams& p) {
     // the centre tap of every output pixel lies inside the frame (the kernel starts each tile with it)
     const bool centre_ok = p.pad_h <= 1 && p.pad_w <= 1 && (p.PH - 1) * p.stride_h - p.pad_h + 1 < p.H &&
                            (p.PW - 1) * p.stride_w - p.pad_w + 1 < p.W;
-    return p.R == 3 && p.S == 3 && pool_ok && centre_ok && p.mode == EPI_THRESH && p.nan_bit == 1 &&
+    // threshold epilogue, or the int32 dot products of an un-pooled convolution without residuals
+    const bool mode_ok = (p.mode == EPI_THRESH && p.nan_bit == 1) ||
+                         (p.mode == EPI_RAW && p.pool_h == 1 && p.pool_w == 1 && p.res_in == nullptr &&
+                          p.res_out == nullptr && p.raw_pix_stride >= 0 && p.raw_b_stride >= 0);
+    return p.R == 3 && p.S == 3 && pool_ok && centre_ok && mode_ok &&
            p.ksplit <= 1 && filter_has_fragments(3, 3, 32 * p.cw) && p.k_tap == 32 * p.cw &&
            (long long)p.PH * p.PW < (1 << 24) && within_2gib(p);
 }
