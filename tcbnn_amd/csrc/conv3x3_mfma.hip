@@ -1,24 +1,28 @@
 // Persistent FP4 matrix-core kernel for the 3x3 bit convolutions that carry almost all of a
-// binarized ResNet / VGG (Conv128LayerFMT, kernel.cuh:676-827, pool 1x1, Cin = 64 .. 512).
+// binarized ResNet / VGG / AlexNet (Conv128LayerFMT, kernel.cuh:676-827; Cin = 64, 128, 192, 256, 384
+// or 512; un-pooled, or 2x2-pooled without residuals) and for the stand-alone 3x3 bit convolution
+// with int32 output (BTC_Conv2d_balance, bmma_kernel.cu:101-165).
 //
 // Same operand mapping as bgemm_mfma.hip (MFMA "A" = 32 output channels, "B" = 32 images, a lane
 // of the accumulator owns one image and 16 channels), plus what a short-K convolution needs to
 // keep the matrix cores fed on a machine whose memory latency (~1 us) is longer than the whole
-// K loop of one tile (9 taps x Cin = 576..2304 bits: 36..144 MFMAs):
-//   - persistent workgroups: the expanded FP4 weight fragments of a 64-channel group (18..72
-//     KiB) and its thresholds are staged in LDS ONCE, then every wave walks a strided list of
-//     (pixel, 64-image) tiles; no barrier after the staging;
+// K loop of one tile (9 taps x Cin = 576..4608 bits: 36..288 MFMAs):
+//   - persistent workgroups: the FP4 weight fragments of a channel group (18..72 KiB, expanded once
+//     when the filter was packed) and its thresholds are staged in LDS ONCE, then every wave walks a
+//     strided list of (pixel, 64-image) tiles; no barrier after the staging;
 //   - whole-chunk register prefetch: all activation words a wave needs for the next chunk of
-//     taps (the whole tile for Cin <= 128, one filter row for Cin = 256, one tap for Cin = 512)
-//     are requested while
-//     the current chunk is multiplied, double-buffered across tile boundaries, so the loads of
-//     tile i+1 fly under the MFMAs and the epilogue of tile i;
+//     taps (the whole tile for Cin <= 128, one filter row above) are requested while the current
+//     chunk is multiplied, across tile boundaries; for Cin <= 128 the requests are issued two per
+//     k-step between the MFMAs of an interior tile (issued in one burst they hold the wave back);
 //   - wave-uniform border handling: a tap outside the frame is a cleared bit in a scalar mask
-//     (its loads and MFMAs are skipped), which is exactly the reference's "exclude" rule;
-//   - epilogue straight from the accumulator: fp32 compare against the threshold (the
-//     accumulator is an exact integer), shift the bit into a 16-channel half-word, one lane^32
-//     swap, 128-byte stores of the batch-innermost layouts; int32 residual add / save as
-//     contiguous runs.
+//     (its loads and MFMAs are skipped), which is exactly the reference's "exclude" rule; pixel
+//     columns are skewed by the row so that every wave gets its share of the slower border tiles;
+//   - threshold folded into the accumulator: without a residual the accumulator starts from the
+//     negated integer threshold (operand C of the tile's first MFMA, always the centre tap), so the
+//     output bit is the sign of the finished accumulator;
+//   - epilogue straight from the accumulator: one funnel shift per channel into a 16-channel half
+//     word, one lane swap, 128-byte stores of the batch-innermost layouts; residual add / save as
+//     contiguous 16-byte runs per lane.
 #include <algorithm>
 #include <cmath>
 #include <cstdlib>
@@ -55,7 +59,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(waves_
 conv3x3_mfma_f4_kernel(
     const BgemmParams p, const uint32_t* __restrict__ act, const uint32_t* __restrict__ wgt,
     const float* __restrict__ bnp, const int32_t* __restrict__ rin, int32_t* __restrict__ rout, int res_lim,
-    int rin_fmt, int rout_fmt, unsigned act_bytes, unsigned rin_bytes, unsigned rout_bytes, unsigned bits_bytes,
+    int rout_fmt, unsigned act_bytes, unsigned rin_bytes, unsigned rout_bytes, unsigned bits_bytes,
     int n_groups, int b_groups, int pix_streams) {
     static_assert(RM == RM_NONE || RM == RM_RAW || MT == 1, "residual instantiations own one image tile per wave");
     constexpr bool kRes = RM == RM_PLAIN || RM == RM_POOLED;  // a residual is injected and / or saved
@@ -588,8 +592,8 @@ conv3x3_mfma_f4_kernel(
 
     // ---- persistent loop over this wave's tiles.  The activation chunks rotate through NB register
     // buffers: the chunk that will be multiplied NB-1 steps from now is requested before the current
-    // one is multiplied (two or three steps of lookahead without a residual, where one chunk of MFMAs
-    // is much shorter than the memory latency and few waves share a SIMD).
+    // one is multiplied (two steps of lookahead for Cin >= 192, where one chunk of MFMAs is shorter
+    // than the memory latency and few waves share a SIMD).
     constexpr int NB = kAhead ? 2 : (SPT >= 3 ? 3 : 2);
     constexpr int LOOK = NB - 1;
     struct Cursor {
@@ -752,8 +756,7 @@ int launch_t(const BgemmParams& p, hipStream_t stream) {
     const long long blocks = (long long)best * n_groups * b_groups;
     const TensorBytes tb = tensor_bytes(p);
     hipLaunchKernelGGL((conv3x3_mfma_f4_kernel<SPT, RM, MT, NT, R16, POOL>), dim3((unsigned)blocks), dim3(kThreads), lds_bytes,
-                       stream, p, p.act, p.wgt, p.bn, p.res_in, RM == RM_RAW ? p.out_i32 : p.res_out, res_lim, p.res_in_fmt,
-                       p.res_out_fmt,
+                       stream, p, p.act, p.wgt, p.bn, p.res_in, RM == RM_RAW ? p.out_i32 : p.res_out, res_lim, p.res_out_fmt,
                        (unsigned)tb.act, (unsigned)tb.rin, (unsigned)tb.rout, (unsigned)tb.bits, n_groups, b_groups, best);
     TCBNN_LAUNCH_CHECK("conv3x3_mfma_f4_kernel");
     return TCBNN_OK;
