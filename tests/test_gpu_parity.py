@@ -119,7 +119,11 @@ def test_bconv_sweep_shapes(gpu, variant, h, c):
 @pytest.mark.parametrize("variant", VARIANTS)
 @pytest.mark.parametrize("b,h,cin,cout,R,stride", [(70, 9, 32, 16, 3, 2), (3, 12, 160, 40, 5, 2),
                                                    (130, 6, 96, 24, 1, 2), (5, 16, 64, 8, 7, 4),
-                                                   (260, 5, 256, 64, 3, 1)])
+                                                   (260, 5, 256, 64, 3, 1),
+                                                   # 3x3 shapes of the persistent kernel's int32 epilogue: partial
+                                                   # channel tile, partial image tile, stride 2, one-pixel frame
+                                                   (70, 9, 64, 48, 3, 2), (33, 7, 192, 100, 3, 1), (8, 1, 128, 64, 3, 1),
+                                                   (40, 2, 384, 32, 3, 1)])
 def test_bconv_odd_shapes(gpu, variant, b, h, cin, cout, R, stride):
     r = rng(b + h + cin)
     x = rm.pm1(r, (b, h, h, cin))
@@ -181,6 +185,9 @@ CONV_CASES = [
     # Cin = 192 / 384 (alexnet.cu:154-162) and 2x2 pooling with them
     (40, 13, 192, 384, 1, 1, False), (72, 13, 384, 256, 1, 1, False), (8, 6, 192, 96, 1, 2, True),
     (130, 9, 384, 64, 2, 1, False),
+    # frames of one to three pixels (every tile is a border tile), odd sizes with stride 2
+    (8, 1, 64, 64, 1, 1, False), (40, 2, 128, 32, 1, 2, False), (40, 3, 64, 64, 2, 1, False),
+    (72, 5, 512, 40, 2, 1, True),
 ]
 
 
