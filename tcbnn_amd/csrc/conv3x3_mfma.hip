@@ -37,6 +37,9 @@ namespace {
 using namespace mfma;
 
 constexpr int kWaves = 4;
+// Residual layers run two image tiles per wave from this Cin / 64 on (Cin = 512: the layer is bound by
+// issue slots, not by HBM; measured slower for Cin = 256 and for pooled sources).
+constexpr int kResMt2From = 8;
 constexpr int kThreads = 64 * kWaves;
 
 // Residual mode of an instantiation.
@@ -47,7 +50,7 @@ constexpr int RM_RAW = 3;     // no threshold: the +-1 dot products are stored a
 
 // Waves per SIMD the register allocator is asked to make room for: the residual layers are
 // bound by HBM and want more memory requests in flight, the plain layers want registers.
-constexpr int waves_hint(int spt, int rm, int nt) { return rm == RM_PLAIN && spt == 4 && nt == 1 ? 4 : 2; }
+constexpr int waves_hint(int spt, int rm, int nt) { return rm == RM_PLAIN && spt == 4 && nt == 1 && kResMt2From > 4 ? 4 : 2; }
 
 // SPT = k-steps (64 bits) per filter tap = Cin / 64; MT = 32-image tiles per wave (2 for plain
 // layers, 1 for residual layers); NT = 32-channel tiles per wave; R16 = the injected residual is
@@ -61,7 +64,6 @@ conv3x3_mfma_f4_kernel(
     const float* __restrict__ bnp, const int32_t* __restrict__ rin, int32_t* __restrict__ rout, int res_lim,
     int rout_fmt, unsigned act_bytes, unsigned rin_bytes, unsigned rout_bytes, unsigned bits_bytes,
     int n_groups, int b_groups, int pix_streams) {
-    static_assert(RM == RM_NONE || RM == RM_RAW || MT == 1, "residual instantiations own one image tile per wave");
     constexpr bool kRes = RM == RM_PLAIN || RM == RM_POOLED;  // a residual is injected and / or saved
     static_assert(RM == RM_NONE || !POOL, "residuals are defined for un-pooled layers only");
     constexpr int TPC = SPT >= 3 ? 3 : 9;  // taps per prefetch chunk (a filter row, or all of it)
@@ -325,17 +327,19 @@ conv3x3_mfma_f4_kernel(
     };
 
     // ---- residual operand (kernel.cuh:770-794).  A lane owns channels n0 + 32 nt + 16 h + v of
-    // image bload[0]; every load is a wave-uniform base plus this per-lane element offset.
+    // images bload[mt] (slot mt * NT + nt); every load is a wave-uniform base plus a per-lane offset.
     // A lane's 16 values arrive as 16 (int32) or 8 (int16 pairs) words; a plain operand stays in
     // that raw form until its epilogue, a pooled one is reduced to 16 ints by finish_residual.
-    constexpr int NRV = kRes ? NT : 1;
+    constexpr int NRV = kRes ? MT * NT : 1;
     constexpr int NTMP = RM == RM_POOLED ? 3 : 1;
     constexpr int NRAW = R16 ? 8 : 16;                    // words loaded per channel tile
     constexpr int NW = RM == RM_POOLED ? 16 : NRAW;       // words kept per channel tile
     int tmp[NTMP][NRV][NRAW];  // pooled: the other three pixels of the 2x2 window
     // A lane's 16 channels are 4 groups of 4 (int32) or 2 groups of 8 (int16): 16 bytes each.
-    const unsigned lane_off = ((unsigned)(4 * h) * (unsigned)p.B + (unsigned)bload[0]) * 16u;
-    const unsigned lane_off16 = ((unsigned)(2 * h) * (unsigned)p.B + (unsigned)bload[0]) * 16u;
+    unsigned lane_off[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+        lane_off[mt] = ((unsigned)((R16 ? 2 : 4) * h) * (unsigned)p.B + (unsigned)bload[mt]) * 16u;
     const unsigned grp_b = (unsigned)p.B * 16u;  // bytes between consecutive channel groups
 
     auto request_residual = [&](int yy, int xx, int (*rv)[NW]) __attribute__((always_inline)) {
@@ -345,20 +349,21 @@ conv3x3_mfma_f4_kernel(
             // source's channels read the neighbouring pixel or (at the end of the tensor) zeros; their
             // values are cleared by finish_residual.
             const unsigned ch_b = (unsigned)(i16 ? (p.res_in_ch + 7) / 8 : (p.res_in_ch + 3) / 4) * grp_b;
-            const unsigned loff = i16 ? lane_off16 : lane_off;
             constexpr int nld = i16 ? 2 : 4;
             const unsigned pix = RM == RM_POOLED ? (unsigned)(2 * yy) * (unsigned)(2 * p.PW) + (unsigned)(2 * xx)
                                                  : (unsigned)yy * (unsigned)p.PW + (unsigned)xx;
             const unsigned ddy = (unsigned)(2 * p.PW) * ch_b;
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
+            for (int sl = 0; sl < MT * NT; ++sl) {
+                const int nt = sl % NT;
+                const unsigned loff = lane_off[sl / NT];
                 const int cb = n0 + nt * 32;
                 if (cb >= res_lim) {  // uniform: this channel tile receives no residual
 #pragma unroll
-                    for (int v = 0; v < NW; ++v) rv[nt][v] = 0;
+                    for (int v = 0; v < NW; ++v) rv[sl][v] = 0;
                     if constexpr (RM == RM_POOLED) {
 #pragma unroll
-                        for (int v = 0; v < NRAW; ++v) tmp[0][nt][v] = tmp[1][nt][v] = tmp[2][nt][v] = 0;
+                        for (int v = 0; v < NRAW; ++v) tmp[0][sl][v] = tmp[1][sl][v] = tmp[2][sl][v] = 0;
                     }
                     continue;
                 }
@@ -374,11 +379,11 @@ conv3x3_mfma_f4_kernel(
                 for (int g = 0; g < 4; ++g) {
                     if (g >= nld) continue;  // uniform
                     const unsigned so = base + (unsigned)g * grp_b;
-                    load4(&rv[nt][4 * g], so);
+                    load4(&rv[sl][4 * g], so);
                     if constexpr (RM == RM_POOLED) {
-                        load4(&tmp[0][nt][4 * g], so + ch_b);
-                        load4(&tmp[1][nt][4 * g], so + ddy);
-                        load4(&tmp[2][nt][4 * g], so + ddy + ch_b);
+                        load4(&tmp[0][sl][4 * g], so + ch_b);
+                        load4(&tmp[1][sl][4 * g], so + ddy);
+                        load4(&tmp[2][sl][4 * g], so + ddy + ch_b);
                     }
                 }
             }
@@ -388,7 +393,7 @@ conv3x3_mfma_f4_kernel(
     auto finish_residual = [&](int (*rv)[NW]) __attribute__((always_inline)) {
         if constexpr (RM == RM_POOLED) {
 #pragma unroll
-            for (int nt = 0; nt < NT; ++nt) {
+            for (int nt = 0; nt < MT * NT; ++nt) {  // every (image tile, channel tile) slot
                 if constexpr (R16) {
 #pragma unroll
                     for (int k = 7; k >= 0; --k) {  // downwards: slot k is read before 2k, 2k+1 are written
@@ -470,10 +475,10 @@ conv3x3_mfma_f4_kernel(
                 for (int v = 0; v < 16; ++v) {
                     int val;
                     if constexpr (RM == RM_PLAIN && R16) {
-                        const int w = rv[nt][v >> 1];
+                        const int w = rv[mt * NT + nt][v >> 1];
                         val = (v & 1) ? (w >> 16) : (int)(short)(w & 0xffff);
                     } else {
-                        val = rv[nt][v];
+                        val = rv[mt * NT + nt][v];
                     }
                     if constexpr (!FAST) {
                         if (cbase + v >= res_lim) val = 0;
@@ -594,7 +599,7 @@ conv3x3_mfma_f4_kernel(
     // buffers: the chunk that will be multiplied NB-1 steps from now is requested before the current
     // one is multiplied (two steps of lookahead for Cin >= 192, where one chunk of MFMAs is shorter
     // than the memory latency and few waves share a SIMD).
-    constexpr int NB = kAhead ? 2 : (SPT >= 3 ? 3 : 2);
+    constexpr int NB = kAhead ? 2 : (SPT >= 3 && !(kRes && MT == 2 && SPT >= 6) ? 3 : 2);  // (registers)
     constexpr int LOOK = NB - 1;
     struct Cursor {
         int pi, y, x, chunk, sub;  // item index, row and (skewed) column, chunk of the tile, pixel of the window
@@ -737,7 +742,7 @@ int launch_t(const BgemmParams& p, hipStream_t stream) {
     // Cin = 256 with one channel tile), fewer when their LDS does not fit.  Measured on every layer
     // of ResNet-18 at batch 256: more, shorter-lived workgroups stage the weights more often and lose.
     static const int wg_env = getenv("TCBNN_WG_PER_CU") ? atoi(getenv("TCBNN_WG_PER_CU")) : 0;  // tuning switch
-    const int wg_want = wg_env > 0 ? wg_env : (SPT == 4 && NT == 1 ? 4 : 2);
+    const int wg_want = wg_env > 0 ? wg_env : (SPT == 4 && NT == 1 && MT == 1 ? 4 : 2);
     const int wg_per_cu = std::max(1, std::min(wg_want, (int)(160 * 1024 / lds_bytes)));
     const int target = std::max(1, 256 * wg_per_cu / (n_groups * b_groups));
     int best = std::min(target, quads);
@@ -773,12 +778,16 @@ struct Pick {
 constexpr int pick_nt(int spt, int rm) {
     return rm == RM_POOLED ? 1 : (rm == RM_PLAIN ? (spt >= 4 ? 1 : 2) : (spt >= 6 ? 1 : 2));  // RM_RAW as RM_NONE
 }
+// image tiles per wave: two wherever the layer is bound by issue slots rather than by HBM
+constexpr int pick_mt(int spt, int rm) {
+    return rm == RM_NONE || rm == RM_RAW ? 2 : (rm == RM_PLAIN && spt >= kResMt2From ? 2 : 1);
+}
 Pick pick(const BgemmParams& p) {
     const int rm = p.mode == EPI_RAW ? RM_RAW
                    : p.res_in == nullptr && p.res_out == nullptr
                        ? RM_NONE
                        : (p.res_in != nullptr && p.res_pool ? RM_POOLED : RM_PLAIN);
-    return {rm, rm == RM_NONE || rm == RM_RAW ? 2 : 1, pick_nt(p.cw / 2, rm), p.res_in != nullptr && p.res_in_fmt == TCBNN_RES_I16,
+    return {rm, pick_mt(p.cw / 2, rm), pick_nt(p.cw / 2, rm), p.res_in != nullptr && p.res_in_fmt == TCBNN_RES_I16,
             p.pool_h == 2};
 }
 
@@ -792,11 +801,11 @@ int launch_m(const BgemmParams& p, hipStream_t stream) {
         case RM_RAW:
             return launch_t<SPT, RM_RAW, 2, pick_nt(SPT, RM_RAW), false, false>(p, stream);
         case RM_PLAIN:
-            return k.r16 ? launch_t<SPT, RM_PLAIN, 1, pick_nt(SPT, RM_PLAIN), true, false>(p, stream)
-                         : launch_t<SPT, RM_PLAIN, 1, pick_nt(SPT, RM_PLAIN), false, false>(p, stream);
+            return k.r16 ? launch_t<SPT, RM_PLAIN, pick_mt(SPT, RM_PLAIN), pick_nt(SPT, RM_PLAIN), true, false>(p, stream)
+                         : launch_t<SPT, RM_PLAIN, pick_mt(SPT, RM_PLAIN), pick_nt(SPT, RM_PLAIN), false, false>(p, stream);
         default:
-            return k.r16 ? launch_t<SPT, RM_POOLED, 1, pick_nt(SPT, RM_POOLED), true, false>(p, stream)
-                         : launch_t<SPT, RM_POOLED, 1, pick_nt(SPT, RM_POOLED), false, false>(p, stream);
+            return k.r16 ? launch_t<SPT, RM_POOLED, pick_mt(SPT, RM_POOLED), pick_nt(SPT, RM_POOLED), true, false>(p, stream)
+                         : launch_t<SPT, RM_POOLED, pick_mt(SPT, RM_POOLED), pick_nt(SPT, RM_POOLED), false, false>(p, stream);
     }
 }
 
