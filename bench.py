@@ -38,19 +38,18 @@ COMPUTE_PEAKS_TOPS = {
 # launches of a kernel name in one step of the default workload (ResNet-18, batch 256, FP4 engine); a kernel
 # name that is not listed (another network, batch or engine) reports null.
 MEASURED_TRAFFIC_BYTES = {
-    "expand_conv_filter_kernel": 705273,
-    "inconv_tiled_kernel<16, true>": 433093303,
-    "conv3x3_mfma_f4_kernel<1, 0, 2, 2, false, false>": 16359208,
-    "conv3x3_mfma_f4_kernel<1, 1, 1, 2, true, false>": 218881851,
-    "conv3x3_mfma_f4_kernel<2, 2, 1, 1, true, false>": 174685432,
-    "conv3x3_mfma_f4_kernel<2, 0, 2, 2, false, false>": 12835124,
-    "conv3x3_mfma_f4_kernel<2, 1, 1, 2, true, false>": 113083025,
-    "conv3x3_mfma_f4_kernel<4, 2, 1, 1, true, false>": 98999409,
-    "conv3x3_mfma_f4_kernel<4, 0, 2, 2, false, false>": 14066543,
-    "conv3x3_mfma_f4_kernel<4, 1, 1, 1, true, false>": 68383766,
-    "conv3x3_mfma_f4_kernel<8, 2, 1, 1, true, false>": 56525871,
-    "conv3x3_mfma_f4_kernel<8, 0, 2, 1, false, false>": 16985795,
-    "conv3x3_mfma_f4_kernel<8, 1, 1, 1, true, false>": 29776500,
+    "inconv_tiled_kernel<16, true, false>": 432886221,
+    "conv3x3_mfma_f4_kernel<1, 0, 2, 2, false, false>": 18619438,
+    "conv3x3_mfma_f4_kernel<1, 1, 1, 2, true, false>": 219005875,
+    "conv3x3_mfma_f4_kernel<2, 2, 1, 1, true, false>": 174967546,
+    "conv3x3_mfma_f4_kernel<2, 0, 2, 2, false, false>": 12883763,
+    "conv3x3_mfma_f4_kernel<2, 1, 1, 2, true, false>": 113232001,
+    "conv3x3_mfma_f4_kernel<4, 2, 1, 1, true, false>": 99248455,
+    "conv3x3_mfma_f4_kernel<4, 0, 2, 2, false, false>": 14088068,
+    "conv3x3_mfma_f4_kernel<4, 1, 1, 1, true, false>": 83556751,
+    "conv3x3_mfma_f4_kernel<8, 2, 1, 1, true, false>": 56636377,
+    "conv3x3_mfma_f4_kernel<8, 0, 2, 1, false, false>": 17012419,
+    "conv3x3_mfma_f4_kernel<8, 1, 2, 1, true, false>": 29928284,
     "fc_mfma_f4_kernel<0>": 8223072,
     "fc_mfma_f4_kernel<1>": 1381369,
 }

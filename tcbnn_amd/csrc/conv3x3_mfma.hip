@@ -356,34 +356,27 @@ conv3x3_mfma_f4_kernel(
 #pragma unroll
             for (int sl = 0; sl < MT * NT; ++sl) {
                 const int nt = sl % NT;
-                const unsigned loff = lane_off[sl / NT];
                 const int cb = n0 + nt * 32;
-                if (cb >= res_lim) {  // uniform: this channel tile receives no residual
-#pragma unroll
-                    for (int v = 0; v < NW; ++v) rv[sl][v] = 0;
-                    if constexpr (RM == RM_POOLED) {
-#pragma unroll
-                        for (int v = 0; v < NRAW; ++v) tmp[0][sl][v] = tmp[1][sl][v] = tmp[2][sl][v] = 0;
-                    }
-                    continue;
-                }
+                // a channel tile that receives no residual (uniform) reads zeros through an out-of-range
+                // offset: no branch, no memory traffic
+                const unsigned loff = cb < res_lim ? lane_off[sl / NT] : kOutOfRange;
                 const unsigned base = pix * ch_b + (unsigned)(i16 ? cb / 8 : cb / 4) * grp_b;  // uniform
-                auto load4 = [&](int* dst, unsigned so) __attribute__((always_inline)) {
-                    const v4i q = __builtin_amdgcn_raw_buffer_load_b128(r_rin, (int)loff, (int)so, 0);
-                    dst[0] = q[0];
-                    dst[1] = q[1];
-                    dst[2] = q[2];
-                    dst[3] = q[3];
-                };
 #pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    if (g >= nld) continue;  // uniform
+                for (int g = 0; g < nld; ++g) {
                     const unsigned so = base + (unsigned)g * grp_b;
-                    load4(&rv[sl][4 * g], so);
+                    const v4i q0 = __builtin_amdgcn_raw_buffer_load_b128(r_rin, (int)loff, (int)so, 0);
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) rv[sl][4 * g + k] = q0[k];
                     if constexpr (RM == RM_POOLED) {
-                        load4(&tmp[0][sl][4 * g], so + ch_b);
-                        load4(&tmp[1][sl][4 * g], so + ddy);
-                        load4(&tmp[2][sl][4 * g], so + ddy + ch_b);
+                        const v4i q1 = __builtin_amdgcn_raw_buffer_load_b128(r_rin, (int)loff, (int)(so + ch_b), 0);
+                        const v4i q2 = __builtin_amdgcn_raw_buffer_load_b128(r_rin, (int)loff, (int)(so + ddy), 0);
+                        const v4i q3 = __builtin_amdgcn_raw_buffer_load_b128(r_rin, (int)loff, (int)(so + ddy + ch_b), 0);
+#pragma unroll
+                        for (int k = 0; k < 4; ++k) {
+                            tmp[0][sl][4 * g + k] = q1[k];
+                            tmp[1][sl][4 * g + k] = q2[k];
+                            tmp[2][sl][4 * g + k] = q3[k];
+                        }
                     }
                 }
             }
