@@ -50,7 +50,7 @@ constexpr int RM_RAW = 3;     // no threshold: the +-1 dot products are stored a
 
 // Waves per SIMD the register allocator is asked to make room for: the residual layers are
 // bound by HBM and want more memory requests in flight, the plain layers want registers.
-constexpr int waves_hint(int spt, int rm, int nt) { return rm == RM_PLAIN && spt == 4 && nt == 1 && kResMt2From > 4 ? 4 : 2; }
+constexpr int waves_hint(int spt, int rm, int nt) { return rm == RM_PLAIN && spt == 4 && nt == 1 ? 3 : 2; }
 
 // SPT = k-steps (64 bits) per filter tap = Cin / 64; MT = 32-image tiles per wave (2 for plain
 // layers, 1 for residual layers); NT = 32-channel tiles per wave; R16 = the injected residual is
@@ -735,7 +735,7 @@ int launch_t(const BgemmParams& p, hipStream_t stream) {
     // Cin = 256 with one channel tile), fewer when their LDS does not fit.  Measured on every layer
     // of ResNet-18 at batch 256: more, shorter-lived workgroups stage the weights more often and lose.
     static const int wg_env = getenv("TCBNN_WG_PER_CU") ? atoi(getenv("TCBNN_WG_PER_CU")) : 0;  // tuning switch
-    const int wg_want = wg_env > 0 ? wg_env : (SPT == 4 && NT == 1 && MT == 1 ? 4 : 2);
+    const int wg_want = wg_env > 0 ? wg_env : (SPT == 4 && NT == 1 && MT == 1 ? 3 : 2);
     const int wg_per_cu = std::max(1, std::min(wg_want, (int)(160 * 1024 / lds_bytes)));
     const int target = std::max(1, 256 * wg_per_cu / (n_groups * b_groups));
     int best = std::min(target, quads);
