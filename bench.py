@@ -67,6 +67,13 @@ def layer_work(L, spec=(), res_bytes=None):
     B = L["batch"]
     if L["kind"] == "in":
         byts = B * L["features"] * 4 + B * L["features"] / 8
+    elif L["kind"] == "pool":  # bits in + out, residual in + out
+        oh = (L["h"] + 2 * L["pad"] - L["window"]) // L["stride"] + 1
+        rb = res_bytes.get(L.get("res_src"), 4) if L.get("res_src") else 0
+        byts = B * L["channels"] * (L["h"] * L["w"] + oh * oh) * (1 / 8 + rb)
+    elif L["kind"] == "avgfc":
+        byts = B * L["h"] * L["w"] * L["channels"] * res_bytes.get(L.get("res_src"), 4) + \
+            L["channels"] * L["out"] * 4 + B * L["out"] * 4
     elif L["kind"] in ("fc", "out"):
         byts = B * L["inp"] / 8 + L["inp"] * L["out"] / 8 + (B * L["out"] * 4 if L["kind"] == "out" else B * L["out"] / 8)
     else:
@@ -83,7 +90,7 @@ def layer_work(L, spec=(), res_bytes=None):
                 byts += B * oh * ow * L["cout"] * res_bytes.get(L["name"], 4)
             if L["inject_residual"]:
                 # channels actually injected: those the source layer saved, capped by residual_channels
-                src_ch = [S["cout"] for S in spec if S["name"] == L.get("res_src")]
+                src_ch = [S.get("cout", S.get("channels")) for S in spec if S["name"] == L.get("res_src")]
                 ch = min([L["residual_channels"], L["cout"]] + src_ch)
                 byts += B * oh * ow * (4 if L["residual_pool"] else 1) * ch * res_bytes.get(L.get("res_src"), 4)
     return dict(bops=bops, flops=flops, bytes=float(byts))
@@ -182,7 +189,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--net", default="imagenet_resnet", choices=["imagenet_resnet", "cifar10_vgg", "mnist_mlp", "alexnet", "cifar10_resnet", "imagenet_vgg"])
+    ap.add_argument("--net", default="imagenet_resnet", choices=["imagenet_resnet", "cifar10_vgg", "mnist_mlp", "alexnet", "cifar10_resnet", "imagenet_vgg",
+                                                                 "imagenet_resnet_textbook"])
     ap.add_argument("--batch", type=int, default=None)
     ap.add_argument("--variant", default="auto")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -251,7 +259,7 @@ def main():
 
     # width each saved residual is stored in (16 bits where its bound proves that exact)
     res_bytes = {L["name"]: (2 if net.layers[L["name"]].output_residual_gpu.format == _lib.RES_I16 else 4)
-                 for L in spec if L.get("save_residual")}
+                 for L in spec if L.get("save_residual") or (L["kind"] == "pool" and L.get("res_src"))}
     # group launches by device kernel, as a profiler does
     groups = {}
     for L, layer in zip(spec, net.order):
@@ -285,7 +293,7 @@ def main():
     if not args.no_cpu:
         from oracle import nets as orc_nets, orc
         cb = args.cpu_batch or {"imagenet_resnet": 16, "cifar10_vgg": 64, "mnist_mlp": 8192, "alexnet": 32,
-                                   "cifar10_resnet": 16, "imagenet_vgg": 8}[args.net]
+                                   "cifar10_resnet": 16, "imagenet_vgg": 8, "imagenet_resnet_textbook": 16}[args.net]
         cb = min(cb, batch)
         cspec = nets.SPECS[args.net](batch=cb)
         xs = x[:cb]
@@ -323,7 +331,8 @@ def main():
                                              "mnist_mlp": "mnist_mlp.cu:111-124",
                                              "alexnet": "alexnet.cu:143-177",
                                              "cifar10_resnet": "cifar10_resnet.cu:189-259",
-                                             "imagenet_vgg": "imagenet_vgg.cu:217-286"}[args.net], batch),
+                                             "imagenet_vgg": "imagenet_vgg.cu:217-286",
+                                             "imagenet_resnet_textbook": "no reference driver"}[args.net], batch),
                    "variant": variant, "layers": len(spec),
                    "residual_storage": ("int16 where the bound of |residual| proves it exact (%d of %d tensors), "
                                         "else int32" % (sum(1 for v in res_bytes.values() if v == 2), len(res_bytes)))

@@ -248,6 +248,43 @@ int tcbnn_fc128_kernel_name(const tcbnn_fc128_desc* d, char* buf, size_t len);
 int tcbnn_out128_kernel_name(const tcbnn_out128_desc* d, char* buf, size_t len);
 int tcbnn_inconv128_kernel_name(const tcbnn_inconv128_desc* d, char* buf, size_t len);
 
+/* ------------------------------------------------ layers of the textbook ResNet wiring */
+/* The reference wires ResNet-18 without a pooling layer after the first convolution, without
+ * convolutional shortcuts and without an average-pooling head (imagenet_resnet.cu:223-325).  The two
+ * layers below have NO counterpart in the reference; together with a Conv128 layer of filter 1x1,
+ * stride 2 and save_residual (the downsample shortcut) they let the same engine run the textbook wiring
+ * (7x7/2 first layer + 3x3/2 max-pool, 1x1/2 shortcut convolutions, global average pool + fp32 FC).
+ *
+ * Overlapping pooling on a packed activation tensor and, optionally, its residual: every output bit is
+ * the OR of the bits of its window (the maximum of the +-1 values), every output residual value the
+ * maximum of the window's values; taps outside the frame are ignored.  Output size per dimension:
+ * (in + 2*padding - window) / stride + 1.  The output residual has the input's format. */
+typedef struct tcbnn_pool128_desc {
+    const uint32_t* input;          /* device, conv activation layout [H][W][CW][B]                 */
+    uint32_t* output;               /* device, [OH][OW][CW][B]                                      */
+    const int32_t* input_residual;  /* device, residual layout with `channels` channels, or NULL    */
+    int32_t* output_residual;       /* device, residual layout [OH][OW]..., or NULL                 */
+    int input_height, input_width, channels, batch;
+    int window, stride, padding;    /* square window; padding < window                              */
+    int residual_format;            /* TCBNN_RES_* of both residual tensors                         */
+} tcbnn_pool128_desc;
+int tcbnn_pool_out(int in_size, int window, int stride, int padding);
+int tcbnn_pool128_forward(const tcbnn_pool128_desc* d, void* stream);
+
+/* Global average pool over the pixels of a residual tensor, then an fp32 fully connected layer:
+ * mean[b][c] = (float)(sum over pixels of residual[p][c][b]) / (float)(height*width) (the sum is an exact
+ * integer), out[b][n] = bias[n] + sum over c, in ascending order with fused multiply-add, of
+ * mean[b][c] * weight[c][n].  channels <= 512. */
+typedef struct tcbnn_avgpool_fc_desc {
+    const int32_t* input_residual;  /* device, residual layout [H][W]... with `channels` channels   */
+    const float* weight;            /* device, fp32 [channels][out_features] row major              */
+    const float* bias;              /* device, fp32 [out_features]                                  */
+    float* output;                  /* device, fp32 [batch][out_features] row major                 */
+    int input_height, input_width, channels, batch, out_features;
+    int residual_format;            /* TCBNN_RES_* of input_residual                                */
+} tcbnn_avgpool_fc_desc;
+int tcbnn_avgpool_fc_forward(const tcbnn_avgpool_fc_desc* d, void* stream);
+
 /* ------------------------------------------------ standalone GEMM / conv */
 /* C[m][n] = K - 2*popc(A[m,:] xor B[n,:]), int32 row major [M][N].  A: [K/32][M]
  * (tcbnn_pack_rows output), B: [N][K/32] (tcbnn_pack_cols output: each column of the

@@ -37,6 +37,14 @@ def run(spec, weights, x):
                                L["stride"], L["padding"], L["pool"], L["ahead_fc"], L["save_residual"],
                                L["inject_residual"], L["residual_channels"], L["residual_pool"], res_in)
             outs[L["name"]] = dict(out=o, res=r)
+        elif k == "pool":
+            res_in = outs[L["res_src"]]["res"] if L["res_src"] else None
+            o, r = orc.pool128(outs[L["src"]]["out"], L["channels"], L["window"], L["stride"], L["pad"], res_in)
+            outs[L["name"]] = dict(out=o, res=r)
+        elif k == "avgfc":
+            w, bias = next(it), next(it)
+            outs[L["name"]] = dict(out=orc.avgpool_fc(outs[L["res_src"]]["res"],
+                                                      w.reshape(L["channels"], L["out"]), bias))
         else:
             raise ValueError(k)
     return outs

@@ -46,6 +46,8 @@ _sig("orc_conv_to_fmt", [_vp, _vp] + [_i] * 4)
 _sig("orc_fc_weight_to_fmt", [_vp, _vp, _i, _i])
 _sig("orc_conv_filter_to_fmt", [_vp, _vp] + [_i] * 4)
 _sig("orc_residual_to_reference", [_vp, _vp] + [_i] * 4)
+_sig("orc_pool128", [_vp] * 4 + [_i] * 7)
+_sig("orc_avgpool_fc", [_vp] * 4 + [_i] * 5)
 
 
 def step32(x):
@@ -199,6 +201,34 @@ def inconv128(x, hwio, bn, stride=1, padding=True, pool=1, save_residual=False):
     _lib.orc_inconv128(_p(x), _p(f), _p(bn), _p(out), _p(res), h, w, cout, b, r, s, stride, stride,
                        int(padding), pool, pool)
     return out, res
+
+
+def pool128(inp, c, window, stride, padding, res_in=None):
+    """Overlapping OR / max pooling (no counterpart in the reference).  inp: [H][W][B][CW] words; res_in:
+    int32 [H][W][B][C] or None.  Returns (packed output, pooled residual or None)."""
+    inp = _u32(inp)
+    h, w, b, cw = inp.shape
+    oh, ow = (h + 2 * padding - window) // stride + 1, (w + 2 * padding - window) // stride + 1
+    out = np.empty((oh, ow, b, cw), np.uint32)
+    res_out = None
+    if res_in is not None:
+        res_in = np.ascontiguousarray(res_in, dtype=np.int32)
+        res_out = np.empty((oh, ow, b, c), np.int32)
+    _lib.orc_pool128(_p(inp), _p(out), _p(res_in) if res_in is not None else None,
+                     _p(res_out) if res_out is not None else None, h, w, c, b, window, stride, padding)
+    return out, res_out
+
+
+def avgpool_fc(res, weight, bias):
+    """Global average pool + fp32 FC head (no counterpart in the reference).  res: int32 [H][W][B][C];
+    weight fp32 [C][N]; bias [N].  Returns fp32 [B][N]."""
+    res = np.ascontiguousarray(res, dtype=np.int32)
+    weight, bias = _f32(weight), _f32(bias)
+    h, w, b, c = res.shape
+    n = weight.shape[1]
+    out = np.empty((b, n), np.float32)
+    _lib.orc_avgpool_fc(_p(res), _p(weight), _p(bias), _p(out), h, w, c, b, n)
+    return out
 
 
 def fc_to_fmt(logical, batch, k):

@@ -408,4 +408,62 @@ void orc_residual_to_reference(const int32_t* res, int32_t* ref, int h, int w, i
                 ref[(pix * b8 + b) * c128 + o] = res[(pix * batch + b) * c + o];
 }
 
+
+// ---- layers of the textbook ResNet wiring: NO counterpart in the reference (its ResNet has no
+// pooling layer, no convolutional shortcut and no average-pooling head, imagenet_resnet.cu:223-325).
+// Defined here as plain loops; pinned in the tests against torch.nn.functional.max_pool2d on the
+// unpacked +-1 values / the integer residual, and against fp64 mean + matmul.
+// Overlapping pooling: bit = OR over the window's in-frame taps, residual = their maximum.
+void orc_pool128(const uint32_t* in, uint32_t* out, const int32_t* res_in, int32_t* res_out, int h, int w,
+                 int c, int batch, int window, int stride, int padding) {
+    const int oh = (h + 2 * padding - window) / stride + 1, ow = (w + 2 * padding - window) / stride + 1;
+    const int cw = step32(c);
+#pragma omp parallel for collapse(2)
+    for (int oy = 0; oy < oh; ++oy)
+        for (int ox = 0; ox < ow; ++ox)
+            for (int b = 0; b < batch; ++b) {
+                for (int k = 0; k < cw; ++k) {
+                    uint32_t acc = 0;
+                    for (int r = 0; r < window; ++r)
+                        for (int s = 0; s < window; ++s) {
+                            const int y = oy * stride - padding + r, x = ox * stride - padding + s;
+                            if (y >= 0 && y < h && x >= 0 && x < w) acc |= in[(((size_t)y * w + x) * batch + b) * cw + k];
+                        }
+                    out[(((size_t)oy * ow + ox) * batch + b) * cw + k] = acc;
+                }
+                if (res_in == nullptr) continue;
+                for (int o = 0; o < c; ++o) {
+                    int m = INT_MIN;
+                    for (int r = 0; r < window; ++r)
+                        for (int s = 0; s < window; ++s) {
+                            const int y = oy * stride - padding + r, x = ox * stride - padding + s;
+                            if (y >= 0 && y < h && x >= 0 && x < w)
+                                m = std::max(m, res_in[(((size_t)y * w + x) * batch + b) * c + o]);
+                        }
+                    res_out[(((size_t)oy * ow + ox) * batch + b) * c + o] = m;
+                }
+            }
+}
+// Global average pool of an integer residual tensor + fp32 fully connected layer: the pixel sum is an
+// exact integer, mean = (float)sum / (float)pixels, out = bias + fma chain over the channels in
+// ascending order.
+void orc_avgpool_fc(const int32_t* res, const float* weight, const float* bias, float* out, int h, int w, int c,
+                    int batch, int n) {
+    const int pixels = h * w;
+#pragma omp parallel for
+    for (int b = 0; b < batch; ++b) {
+        std::vector<float> mean(c);
+        for (int o = 0; o < c; ++o) {
+            long long sum = 0;
+            for (int p = 0; p < pixels; ++p) sum += res[((size_t)p * batch + b) * c + o];
+            mean[o] = (float)(int)sum / (float)pixels;
+        }
+        for (int j = 0; j < n; ++j) {
+            float acc = 0.0f;
+            for (int o = 0; o < c; ++o) acc = fmaf(mean[o], weight[(size_t)o * n + j], acc);
+            out[(size_t)b * n + j] = acc + bias[j];
+        }
+    }
+}
+
 }  // extern "C"

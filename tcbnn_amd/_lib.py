@@ -67,6 +67,19 @@ class Conv128Desc(C.Structure):
                 ("input_residual_format", c_int), ("output_residual_format", c_int)]
 
 
+class Pool128Desc(C.Structure):
+    _fields_ = [("input", c_void_p), ("output", c_void_p), ("input_residual", c_void_p),
+                ("output_residual", c_void_p), ("input_height", c_int), ("input_width", c_int),
+                ("channels", c_int), ("batch", c_int), ("window", c_int), ("stride", c_int),
+                ("padding", c_int), ("residual_format", c_int)]
+
+
+class AvgPoolFcDesc(C.Structure):
+    _fields_ = [("input_residual", c_void_p), ("weight", c_void_p), ("bias", c_void_p), ("output", c_void_p),
+                ("input_height", c_int), ("input_width", c_int), ("channels", c_int), ("batch", c_int),
+                ("out_features", c_int), ("residual_format", c_int)]
+
+
 # name -> (restype, argtypes); the complete list of symbols include/tcbnn_hip.h declares.
 ABI = {
     "tcbnn_abi_version": (c_int, []),
@@ -75,6 +88,9 @@ ABI = {
     "tcbnn_get_default_variant": (c_int, []),
     "tcbnn_conv_pad": (c_int, [c_int] * 4),
     "tcbnn_conv_out": (c_int, [c_int] * 5),
+    "tcbnn_pool_out": (c_int, [c_int] * 4),
+    "tcbnn_pool128_forward": (c_int, [C.POINTER(Pool128Desc), c_void_p]),
+    "tcbnn_avgpool_fc_forward": (c_int, [C.POINTER(AvgPoolFcDesc), c_void_p]),
     "tcbnn_fc_act_words": (c_size_t, [c_int] * 2),
     "tcbnn_conv_act_words": (c_size_t, [c_int] * 4),
     "tcbnn_fc_weight_words": (c_size_t, [c_int] * 2),

@@ -219,19 +219,42 @@ __global__ __launch_bounds__(kThreads) void bgemm_mfma_kernel(
                     }
                     int32_t* __restrict__ rout = p.res_out;
                     uint32_t hw = 0;
+                    int resv[16];
 #pragma unroll
                     for (int v = 0; v < 16; ++v) {
                         const int c = cbase + v;
                         int res = A::to_int(acc[mt][nt][v]);
                         uint32_t bit = 0;
                         if (c < p.N) {
-                            if constexpr (MM == MM_THRESH_RES) {
-                                res += rv[v];
-                                if (rout != nullptr && b_ok) residual_store(rout, p.res_out_fmt, pix, p.N, c, p.B, b, res);
-                            }
+                            if constexpr (MM == MM_THRESH_RES) res += rv[v];
                             bit = thresh_bit(res, bnp[c], p.nan_bit);
                         }
+                        resv[v] = c < p.N ? res : 0;  // channels past N are stored as 0 inside a group
                         hw = (hw << 1) | bit;
+                    }
+                    if constexpr (MM == MM_THRESH_RES) {
+                        // a lane's 16 channels are whole 16-byte groups of the residual layouts: 128-bit stores
+                        if (rout != nullptr && b_ok && cbase < p.N) {
+                            int4* __restrict__ dst = reinterpret_cast<int4*>(rout);
+                            if (p.res_out_fmt == TCBNN_RES_I16) {
+                                const size_t g0 = (pix * (size_t)((p.N + 7) / 8) + cbase / 8) * p.B + b;
+#pragma unroll
+                                for (int g = 0; g < 2; ++g)
+                                    if (cbase + 8 * g < p.N)
+                                        dst[g0 + (size_t)g * p.B] = make_int4(
+                                            (resv[8 * g] & 0xffff) | (resv[8 * g + 1] << 16),
+                                            (resv[8 * g + 2] & 0xffff) | (resv[8 * g + 3] << 16),
+                                            (resv[8 * g + 4] & 0xffff) | (resv[8 * g + 5] << 16),
+                                            (resv[8 * g + 6] & 0xffff) | (resv[8 * g + 7] << 16));
+                            } else {
+                                const size_t g0 = (pix * (size_t)((p.N + 3) / 4) + cbase / 4) * p.B + b;
+#pragma unroll
+                                for (int g = 0; g < 4; ++g)
+                                    if (cbase + 4 * g < p.N)
+                                        dst[g0 + (size_t)g * p.B] =
+                                            make_int4(resv[4 * g], resv[4 * g + 1], resv[4 * g + 2], resv[4 * g + 3]);
+                            }
+                        }
                     }
                     const uint32_t other = (uint32_t)__shfl_xor((int)hw, 32);
                     outword[mt][nt] |= h == 0 ? (hw << 16) | other : (other << 16) | hw;

@@ -105,6 +105,14 @@ struct Synthetic {
                 thr[j] = -thr[j];
             }
     }
+    // fp32 head: weights N(0, 1/sqrt(fan_in)) [fan_in][nout], bias N(0, 1)
+    void fp32_layer(size_t fan_in, size_t nout) {
+        Rng r(seed ^ (0x1000ull + tensor++));
+        const size_t base = values.size();
+        values.resize(base + fan_in * nout + nout);
+        for (size_t i = 0; i < fan_in * nout; ++i) values[base + i] = (float)(r.normal() / sqrt((double)fan_in));
+        for (size_t j = 0; j < nout; ++j) values[base + fan_in * nout + j] = (float)r.normal();
+    }
     // output layer: +-1 weights, scale N(1, 0.1), bias N(0, 1)
     void output_layer(size_t fan_in, size_t nout) {
         Rng r(seed ^ (0x1000ull + tensor++));

@@ -760,3 +760,157 @@ class Conv128LayerParam {  // param.h:872-1065
     tcbnn_host::ResidualInfo input_residual_info;  // of input_residual_gpu
     int buf_height, buf_width;
 };
+
+// ======================================================================================
+// Layers of the textbook ResNet wiring.  NO counterpart among the reference's classes (its ResNet
+// has no pooling layer after the first convolution, no convolutional shortcut and a binarized FC
+// head, imagenet_resnet.cu:223-325); same conventions as the classes above.
+
+// Overlapping OR / max pooling of a packed activation tensor and, optionally, its residual.
+class Pool128LayerParam {
+   public:
+    Pool128LayerParam(const char* _name, int _input_height, int _input_width, int _channels, int _batch,
+                      int _window = 3, int _stride = 2, int _padding = 1, bool _pool_residual = false)
+        : input_gpu(NULL), input_residual_gpu(NULL), output_gpu(NULL), output_residual_gpu(NULL),
+          input_height(_input_height), input_width(_input_width), output_channels(_channels), batch(_batch),
+          window(_window), stride(_stride), padding(_padding), pool_residual(_pool_residual) {
+        strncpy(name, _name, 8);
+        output_height = buf_height = tcbnn_pool_out(input_height, window, stride, padding);
+        output_width = buf_width = tcbnn_pool_out(input_width, window, stride, padding);
+        residual_info.channels = 0;
+        residual_info.bound = 0;
+        residual_info.format = TCBNN_RES_I32;
+    }
+    ~Pool128LayerParam() { release(); }
+    Pool128LayerParam* initialize(uin32* prev_layer_gpu, int* _input_residual_gpu = NULL) {
+        CHECK_NULL_POINTER(prev_layer_gpu);
+        input_gpu = prev_layer_gpu;
+        SAFE_ALOC_GPU(output_gpu, 4 * tcbnn_conv_act_words(output_height, output_width, batch, output_channels));
+        if (pool_residual) {
+            CHECK_NULL_POINTER(_input_residual_gpu);
+            input_residual_gpu = _input_residual_gpu;
+            std::map<const void*, tcbnn_host::ResidualInfo>& reg = tcbnn_host::residual_registry();
+            std::map<const void*, tcbnn_host::ResidualInfo>::iterator it = reg.find(input_residual_gpu);
+            const tcbnn_host::ResidualInfo foreign = {output_channels, INT32_MAX, TCBNN_RES_I32};
+            residual_info = it != reg.end() ? it->second : foreign;  // a maximum keeps bound and format
+            residual_info.channels = output_channels;
+            SAFE_ALOC_GPU(output_residual_gpu, tcbnn_residual_bytes(output_height, output_width, output_channels,
+                                                                    batch, residual_info.format));
+            reg[output_residual_gpu] = residual_info;
+        }
+        return this;
+    }
+    uin32* get_output_gpu() { return this->output_gpu; }
+    int* get_output_residual_gpu() { return this->output_residual_gpu; }
+    void forward(hipStream_t stream = 0) {
+        tcbnn_pool128_desc d;
+        memset(&d, 0, sizeof(d));
+        d.input = input_gpu;
+        d.output = output_gpu;
+        d.input_residual = input_residual_gpu;
+        d.output_residual = output_residual_gpu;
+        d.input_height = input_height;
+        d.input_width = input_width;
+        d.channels = output_channels;
+        d.batch = batch;
+        d.window = window;
+        d.stride = stride;
+        d.padding = padding;
+        d.residual_format = residual_info.format;
+        TCBNN_SAFE_CALL(tcbnn_pool128_forward(&d, stream));
+    }
+    void release() {
+        if (output_residual_gpu != NULL) tcbnn_host::residual_registry().erase(output_residual_gpu);
+        SAFE_FREE_GPU(output_gpu);
+        SAFE_FREE_GPU(output_residual_gpu);
+    }
+
+   public:
+    uin32* input_gpu;
+    int* input_residual_gpu;
+    uin32* output_gpu;
+    int* output_residual_gpu;
+    int input_height, input_width, output_height, output_width, buf_height, buf_width;
+    int output_channels, batch, window, stride, padding;
+    bool pool_residual;
+    tcbnn_host::ResidualInfo residual_info;
+    char name[8];
+};
+
+// Global average pool over a residual tensor + fp32 fully connected layer.  Weight file order: the fp32
+// weight matrix [channels][out_features], then the bias.
+class AvgPoolFcLayerParam {
+   public:
+    AvgPoolFcLayerParam(const char* _name, int _input_height, int _input_width, int _channels, int _batch,
+                        int _out_features)
+        : input_residual_gpu(NULL), weight(NULL), weight_gpu(NULL), bias(NULL), bias_gpu(NULL), output(NULL),
+          output_gpu(NULL), input_height(_input_height), input_width(_input_width), channels(_channels),
+          batch(_batch), out_features(_out_features) {
+        strncpy(name, _name, 8);
+        input_residual_info.channels = channels;
+        input_residual_info.bound = INT32_MAX;
+        input_residual_info.format = TCBNN_RES_I32;
+    }
+    ~AvgPoolFcLayerParam() { release(); }
+    int weight_size() { return channels * out_features; }
+    int output_bytes() { return batch * out_features * (int)sizeof(float); }
+    AvgPoolFcLayerParam* initialize(tcbnn_host::ConfigSource config_file, int* _input_residual_gpu) {
+        CHECK_NULL_POINTER(_input_residual_gpu);
+        input_residual_gpu = _input_residual_gpu;
+        std::map<const void*, tcbnn_host::ResidualInfo>& reg = tcbnn_host::residual_registry();
+        std::map<const void*, tcbnn_host::ResidualInfo>::iterator it = reg.find(input_residual_gpu);
+        if (it != reg.end()) input_residual_info = it->second;
+        SAFE_ALOC_HOST(weight, weight_size() * sizeof(float));
+        config_file.read(weight, weight_size());
+        SAFE_ALOC_GPU(weight_gpu, weight_size() * sizeof(float));
+        HIP_SAFE_CALL(hipMemcpy(weight_gpu, weight, weight_size() * sizeof(float), hipMemcpyHostToDevice));
+        SAFE_ALOC_HOST(bias, out_features * sizeof(float));
+        config_file.read(bias, out_features);
+        SAFE_ALOC_GPU(bias_gpu, out_features * sizeof(float));
+        HIP_SAFE_CALL(hipMemcpy(bias_gpu, bias, out_features * sizeof(float), hipMemcpyHostToDevice));
+        SAFE_ALOC_GPU(output_gpu, output_bytes());
+        return this;
+    }
+    float* get_output_gpu() { return this->output_gpu; }
+    void forward(hipStream_t stream = 0) {
+        tcbnn_avgpool_fc_desc d;
+        memset(&d, 0, sizeof(d));
+        d.input_residual = input_residual_gpu;
+        d.weight = weight_gpu;
+        d.bias = bias_gpu;
+        d.output = output_gpu;
+        d.input_height = input_height;
+        d.input_width = input_width;
+        d.channels = channels;
+        d.batch = batch;
+        d.out_features = out_features;
+        d.residual_format = input_residual_info.format;
+        TCBNN_SAFE_CALL(tcbnn_avgpool_fc_forward(&d, stream));
+    }
+    float* download_output() {
+        if (output == NULL) SAFE_ALOC_HOST(output, output_bytes());
+        HIP_SAFE_CALL(hipMemcpy(output, output_gpu, output_bytes(), hipMemcpyDeviceToHost));
+        return this->output;
+    }
+    void release() {
+        SAFE_FREE_HOST(weight);
+        SAFE_FREE_HOST(bias);
+        SAFE_FREE_HOST(output);
+        SAFE_FREE_GPU(weight_gpu);
+        SAFE_FREE_GPU(bias_gpu);
+        SAFE_FREE_GPU(output_gpu);
+    }
+
+   public:
+    int* input_residual_gpu;
+    float* weight;
+    float* weight_gpu;
+    float* bias;
+    float* bias_gpu;
+    float* output;
+    float* output_gpu;
+    int input_height, input_width, channels, batch, out_features;
+    tcbnn_host::ResidualInfo input_residual_info;
+    char name[8];
+};
+

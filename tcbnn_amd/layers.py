@@ -562,3 +562,114 @@ class Conv128LayerParam(_ConvGeometry):
             if b is not None:
                 b.free()
         self.filter_gpu = self.bn_gpu = self.output_gpu = self.output_residual_gpu = None
+
+
+class Pool128LayerParam:
+    """Overlapping OR / max pooling of a packed activation tensor and, optionally, its residual (the
+    3x3 stride-2 max-pool of the textbook ResNet wiring).  No counterpart among the reference's layer
+    classes: its pooling is a non-overlapping window fused into the convolution (kernel.cuh:811-815)."""
+
+    def __init__(self, name, input_height, input_width, channels, batch, window=3, stride=2, padding=1,
+                 pool_residual=False):
+        self.name = name
+        self.input_height, self.input_width = input_height, input_width
+        self.output_channels = channels
+        self.batch = batch
+        self.window, self.stride, self.padding = window, stride, padding
+        self.pool_residual = pool_residual
+        self.output_height = self.buf_height = lib.tcbnn_pool_out(input_height, window, stride, padding)
+        self.output_width = self.buf_width = lib.tcbnn_pool_out(input_width, window, stride, padding)
+        self.input_gpu = self.input_residual_gpu = self.output_gpu = self.output_residual_gpu = None
+
+    def initialize(self, prev_layer_gpu, input_residual_gpu=None):
+        if prev_layer_gpu is None:
+            raise _lib.TcbnnError("Error: NULL pointer (input_gpu)")
+        self.input_gpu = prev_layer_gpu
+        self.output_gpu = DeviceBuffer(4 * lib.tcbnn_conv_act_words(self.output_height, self.output_width,
+                                                                    self.batch, self.output_channels))
+        if self.pool_residual:
+            if input_residual_gpu is None:
+                raise _lib.TcbnnError("Error: NULL pointer (input_residual_gpu)")
+            self.input_residual_gpu = input_residual_gpu
+            # a maximum never exceeds the bound of its operands: same bound, same format
+            self.output_residual_gpu = _residual_buffer(self.output_channels, self.output_height, self.output_width,
+                                                        self.batch, input_residual_gpu.bound,
+                                                        input_residual_gpu.format)
+        return self
+
+    def get_output_gpu(self):
+        return self.output_gpu
+
+    def get_output_residual_gpu(self):
+        return self.output_residual_gpu
+
+    def _desc(self):
+        rin, rout = self.input_residual_gpu, self.output_residual_gpu
+        return _lib.Pool128Desc(self.input_gpu.ptr, self.output_gpu.ptr, rin.ptr if rin is not None else None,
+                                rout.ptr if rout is not None else None, self.input_height, self.input_width,
+                                self.output_channels, self.batch, self.window, self.stride, self.padding,
+                                rin.format if rin is not None else 0)
+
+    def forward(self, stream=None):
+        d = self._desc()
+        check(lib.tcbnn_pool128_forward(C.byref(d), _stream_handle(stream)))
+
+    def kernel_name(self):
+        return "pool128_kernel"
+
+    download_packed = _ConvGeometry.download_packed
+    download_residual = _ConvGeometry.download_residual
+    _is_fc_ready = _ConvGeometry._is_fc_ready
+
+    def release(self):
+        for b in (self.output_gpu, self.output_residual_gpu):
+            if b is not None:
+                b.free()
+        self.output_gpu = self.output_residual_gpu = None
+
+
+class AvgPoolFcLayerParam:
+    """Global average pool over a residual tensor + fp32 fully connected layer (the head of the textbook
+    ResNet wiring; the reference's head is a binarized FC layer, imagenet_resnet.cu:320-325).  Weight file
+    order: the fp32 weight matrix [channels][out_features], then the bias."""
+
+    def __init__(self, name, input_height, input_width, channels, batch, out_features):
+        self.name = name
+        self.input_height, self.input_width = input_height, input_width
+        self.channels, self.batch, self.out_features = channels, batch, out_features
+        self.input_residual_gpu = self.weight_gpu = self.bias_gpu = self.output_gpu = None
+
+    def initialize(self, config_file, input_residual_gpu):
+        if input_residual_gpu is None:
+            raise _lib.TcbnnError("Error: NULL pointer (input_residual_gpu)")
+        self.input_residual_gpu = input_residual_gpu
+        self.weight = np.array(config_file.launch_array(self.channels * self.out_features), dtype=np.float32)
+        self.bias = np.array(config_file.launch_array(self.out_features), dtype=np.float32)
+        self.weight_gpu = DeviceBuffer.from_numpy(self.weight)
+        self.bias_gpu = DeviceBuffer.from_numpy(self.bias)
+        self.output_gpu = DeviceBuffer(4 * self.batch * self.out_features)
+        return self
+
+    def get_output_gpu(self):
+        return self.output_gpu
+
+    def _desc(self):
+        return _lib.AvgPoolFcDesc(self.input_residual_gpu.ptr, self.weight_gpu.ptr, self.bias_gpu.ptr,
+                                  self.output_gpu.ptr, self.input_height, self.input_width, self.channels,
+                                  self.batch, self.out_features, self.input_residual_gpu.format)
+
+    def forward(self, stream=None):
+        d = self._desc()
+        check(lib.tcbnn_avgpool_fc_forward(C.byref(d), _stream_handle(stream)))
+
+    def kernel_name(self):
+        return "avgpool_fc_kernel"
+
+    def download_output(self):
+        return self.output_gpu.to_numpy(np.float32, (self.batch, self.out_features))
+
+    def release(self):
+        for b in (self.weight_gpu, self.bias_gpu, self.output_gpu):
+            if b is not None:
+                b.free()
+        self.weight_gpu = self.bias_gpu = self.output_gpu = None

@@ -10,8 +10,8 @@ reference's weight file is consumed (utility.h:188-196).
 import numpy as np
 
 from . import _lib
-from .layers import (ArrayWeights, Conv128LayerParam, Fc128LayerParam, In128LayerParam,
-                     InConv128LayerParam, Out128LayerParam, PAD128)
+from .layers import (ArrayWeights, AvgPoolFcLayerParam, Conv128LayerParam, Fc128LayerParam, In128LayerParam,
+                     InConv128LayerParam, Out128LayerParam, PAD128, Pool128LayerParam)
 
 
 def _conv_out(h, r, s, padding=True, pool=1):
@@ -156,7 +156,42 @@ def imagenet_vgg_spec(batch=256, image=224, n_hidden=4096, output_size=1000):
     return spec
 
 
-SPECS = {"mnist_mlp": mnist_mlp_spec, "cifar10_vgg": cifar10_vgg_spec, "imagenet_resnet": imagenet_resnet_spec,
+def imagenet_resnet_textbook_spec(batch=256, image=224, output_size=1000):
+    """ResNet-18 BNN wired as the textbook network rather than as imagenet_resnet.cu:223-325 wires it:
+    7x7 stride-2 first layer + 3x3 stride-2 max-pool (bits OR-pooled, residual max-pooled), a 1x1 stride-2
+    binarized convolution as the shortcut at every stage entry (its pre-threshold sums are the injected
+    residual), global average pool of the last residual + fp32 FC.  The reference has no such driver; the
+    layers it needs beyond the reference's are Pool128 and AvgPoolFc."""
+    B = batch
+    spec = [dict(kind="inconv", name="Conv1", h=image, w=image, r=7, s=7, cin=3, cout=64, batch=B,
+                 stride=2, padding=True, pool=1, save_residual=True)]
+    h = _conv_out(image, 7, 2)
+    spec.append(dict(kind="pool", name="Pool1", h=h, w=h, channels=64, batch=B, window=3, stride=2, pad=1,
+                     src="Conv1", res_src="Conv1"))
+    h = (h + 2 - 3) // 2 + 1
+    spec.append(_conv("L1B1C1", h, 64, 64, B, "Pool1"))
+    spec.append(_conv("L1B1C2", h, 64, 64, B, "L1B1C1", save_residual=True, inject_residual=True,
+                      residual_channels=64, res_src="Pool1"))
+    spec.append(_conv("L1B2C1", h, 64, 64, B, "L1B1C2"))
+    spec.append(_conv("L1B2C2", h, 64, 64, B, "L1B2C1", save_residual=True, inject_residual=True,
+                      residual_channels=64, res_src="L1B1C2"))
+    prev, cin = "L1B2C2", 64
+    for stage, cout in ((2, 128), (3, 256), (4, 512)):
+        ds, n1, n2, n3, n4 = ["L%dDS" % stage] + ["L%dB%dC%d" % (stage, b, c) for b in (1, 2) for c in (1, 2)]
+        spec.append(_conv(ds, h, cin, cout, B, prev, stride=2, save_residual=True, r=1))  # shortcut
+        spec.append(_conv(n1, h, cin, cout, B, prev, stride=2))
+        h = _conv_out(h, 3, 2)
+        spec.append(_conv(n2, h, cout, cout, B, n1, save_residual=True, inject_residual=True,
+                          residual_channels=cout, res_src=ds))
+        spec.append(_conv(n3, h, cout, cout, B, n2))
+        spec.append(_conv(n4, h, cout, cout, B, n3, save_residual=True, inject_residual=True,
+                          residual_channels=cout, res_src=n2))
+        prev, cin = n4, cout
+    spec.append(dict(kind="avgfc", name="Fout", h=h, w=h, channels=512, batch=B, out=output_size, res_src=prev))
+    return spec
+
+
+SPECS = {"imagenet_resnet_textbook": imagenet_resnet_textbook_spec, "mnist_mlp": mnist_mlp_spec, "cifar10_vgg": cifar10_vgg_spec, "imagenet_resnet": imagenet_resnet_spec,
          "alexnet": alexnet_spec, "cifar10_resnet": cifar10_resnet_spec, "imagenet_vgg": imagenet_vgg_spec}
 
 
@@ -184,7 +219,11 @@ def synthetic_weights(spec, seed=0, fold_flips=True):
     arrays = []
     for L in spec:
         k = L["kind"]
-        if k == "in":
+        if k in ("in", "pool"):
+            continue
+        if k == "avgfc":  # fp32 head: weights N(0, 1/sqrt(C)), bias N(0, 1)
+            arrays += [rng.normal(0.0, 1.0 / np.sqrt(L["channels"]), (L["channels"], L["out"])).astype(np.float32),
+                       rng.normal(0.0, 1.0, L["out"]).astype(np.float32)]
             continue
         if k in ("fc", "out"):
             w = rng.integers(0, 2, size=(L["inp"], L["out"])).astype(np.float32) * 2 - 1
@@ -242,6 +281,14 @@ class Network:
                                           residual_format=residual_format)
                 res = self.layers[L["res_src"]].get_output_residual_gpu() if L["res_src"] else None
                 layer.initialize(src, self.layers[L["src"]].get_output_gpu(), res)
+            elif k == "pool":
+                layer = Pool128LayerParam(L["name"], L["h"], L["w"], L["channels"], L["batch"], L["window"],
+                                          L["stride"], L["pad"], pool_residual=L["res_src"] is not None)
+                res = self.layers[L["res_src"]].get_output_residual_gpu() if L["res_src"] else None
+                layer.initialize(self.layers[L["src"]].get_output_gpu(), res)
+            elif k == "avgfc":
+                layer = AvgPoolFcLayerParam(L["name"], L["h"], L["w"], L["channels"], L["batch"], L["out"])
+                layer.initialize(src, self.layers[L["res_src"]].get_output_residual_gpu())
             elif k == "fc":
                 layer = Fc128LayerParam(L["name"], L["batch"], L["inp"], L["out"], variant=variant)
                 layer.initialize(src, self.layers[L["src"]].get_output_gpu())

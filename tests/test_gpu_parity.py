@@ -449,6 +449,8 @@ def _compare_network(gpu, spec, seed, variant, residual_format=None):
         if L["kind"] == "out":
             np.testing.assert_allclose(logits, w["out"], rtol=1e-5, atol=0)
             np.testing.assert_array_equal(logits, w["out"])
+        elif L["kind"] == "avgfc":  # fp32 head: 1e-5 of the logits' scale
+            np.testing.assert_allclose(logits, w["out"], rtol=1e-5, atol=1e-5 * float(np.abs(w["out"]).max()))
         else:
             got = layer.download_packed()
             np.testing.assert_array_equal(got, w["out"].reshape(got.shape), err_msg=L["name"])
@@ -509,6 +511,52 @@ def test_imagenet_vgg(gpu, variant):
     """imagenet_vgg.cu:217-286 (VGG-16) at full image size."""
     from tcbnn_amd import nets
     _compare_network(gpu, nets.imagenet_vgg_spec(batch=8), 13, variant)
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+def test_imagenet_resnet18_textbook_wiring(gpu, variant):
+    """7x7/2 first layer + 3x3/2 max-pool, 1x1/2 shortcut convolutions, average-pool + fp32 FC head: no
+    reference driver exists for this wiring, the CPU oracle (pinned against torch) is the only check."""
+    from tcbnn_amd import nets
+    _compare_network(gpu, nets.imagenet_resnet_textbook_spec(batch=8), 14, variant)
+
+
+@pytest.mark.parametrize("fmt", [0, 1])
+@pytest.mark.parametrize("b,h,c,window,stride,pad", [(8, 12, 64, 3, 2, 1), (70, 7, 40, 3, 2, 1), (5, 9, 100, 2, 2, 0),
+                                                     (3, 5, 33, 3, 1, 1)])
+def test_pool128(gpu, b, h, c, window, stride, pad, fmt):
+    """Overlapping OR / max pooling: bits and residual against the oracle, both residual formats, odd shapes."""
+    from tcbnn_amd import layers
+    r = rng(b + h + c)
+    x = rm.pm1(r, (b, h, h, c))
+    res = r.integers(-30000, 30000, size=(h, h, b, c)).astype(np.int32)
+    inp = orc.pack_conv_input_nhwc(x)
+    want_bits, want_res = orc.pool128(inp, c, window, stride, pad, res)
+    layer = layers.Pool128LayerParam("p", h, h, c, b, window, stride, pad, pool_residual=True)
+    layer.initialize(gpuops.pack_conv_input(x), _residual_source(res, fmt))
+    layer.forward()
+    gpuops.sync()
+    np.testing.assert_array_equal(layer.download_packed(), want_bits)
+    np.testing.assert_array_equal(layer.download_residual(), want_res)
+    layer.release()
+
+
+@pytest.mark.parametrize("fmt", [0, 1])
+@pytest.mark.parametrize("b,h,c,n", [(8, 7, 512, 1000), (70, 3, 100, 37), (33, 1, 64, 10)])
+def test_avgpool_fc(gpu, b, h, c, n, fmt):
+    from tcbnn_amd import layers
+    r = rng(b + h + c + n)
+    res = r.integers(-20000, 20000, size=(h, h, b, c)).astype(np.int32)
+    w = r.standard_normal((c, n)).astype(np.float32)
+    bias = r.standard_normal(n).astype(np.float32)
+    want = orc.avgpool_fc(res, w, bias)
+    layer = layers.AvgPoolFcLayerParam("head", h, h, c, b, n)
+    layer.initialize(layers.ArrayWeights([w, bias]), _residual_source(res, fmt))
+    layer.forward()
+    gpuops.sync()
+    got = layer.download_output()
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-5 * float(np.abs(want).max()))
+    layer.release()
 
 
 def test_imagenet_resnet18_batch256_every_image(gpu):

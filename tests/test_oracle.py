@@ -360,3 +360,40 @@ def test_residual_reference_layout():
     assert ref.shape == (2, 3, 8, 128)
     np.testing.assert_array_equal(ref[:, :, :5, :64], res)
     assert not ref[:, :, 5:, :].any() and not ref[..., 64:].any()
+
+
+# --------------------------------------------------------------------------- layers of the textbook wiring
+@pytest.mark.parametrize("b,h,c,window,stride,pad", [(3, 11, 40, 3, 2, 1), (2, 8, 64, 3, 2, 1), (4, 9, 33, 2, 2, 0),
+                                                     (1, 5, 96, 3, 1, 1)])
+def test_pool128_is_max_pool_of_values_and_of_the_residual(b, h, c, window, stride, pad):
+    """OR of sign bits == sign of the maximum of the +-1 values; residual == integer max-pool
+    (torch.nn.functional.max_pool2d pads with -inf, i.e. ignores taps outside the frame)."""
+    import torch
+    r = np.random.default_rng(b + h + c)
+    x = rm.pm1(r, (b, h, h, c))
+    res = r.integers(-30000, 30000, size=(h, h, b, c)).astype(np.int32)
+    out, pooled = orc.pool128(orc.pack_conv_input_nhwc(x), c, window, stride, pad, res)
+    want = torch.nn.functional.max_pool2d(torch.tensor(x).permute(0, 3, 1, 2), window, stride, pad)
+    np.testing.assert_array_equal(orc.unpack_bits(out, c), want.permute(2, 3, 0, 1).numpy())
+    want_res = torch.nn.functional.max_pool2d(torch.tensor(res.astype(np.float64)).permute(2, 3, 0, 1), window, stride, pad)
+    np.testing.assert_array_equal(pooled, want_res.permute(2, 3, 0, 1).numpy().astype(np.int32))
+    # thresholding commutes with the maximum: pooling the bits of (res >= t) equals the bit of the pooled residual
+    t = 123
+    bits = (res >= t).astype(np.float32) * 2 - 1  # [H][W][B][C] -> NHWC
+    out2, _ = orc.pool128(orc.pack_conv_input_nhwc(np.ascontiguousarray(bits.transpose(2, 0, 1, 3))), c, window, stride, pad)
+    np.testing.assert_array_equal(orc.unpack_bits(out2, c) > 0, pooled >= t)
+
+
+@pytest.mark.parametrize("b,h,c,n", [(3, 7, 512, 10), (5, 2, 40, 7), (2, 1, 64, 3)])
+def test_avgpool_fc_against_fp64(b, h, c, n):
+    r = np.random.default_rng(b + h + c + n)
+    res = r.integers(-20000, 20000, size=(h, h, b, c)).astype(np.int32)
+    w = r.standard_normal((c, n)).astype(np.float32)
+    bias = r.standard_normal(n).astype(np.float32)
+    got = orc.avgpool_fc(res, w, bias)
+    want = res.astype(np.float64).mean(axis=(0, 1)) @ w.astype(np.float64) + bias
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=1e-5 * np.abs(want).max())
+    # a constant residual averages to itself exactly
+    const = np.full((h, h, b, c), 7, np.int32)
+    one = orc.avgpool_fc(const, np.ones((c, 1), np.float32), np.zeros(1, np.float32))
+    np.testing.assert_array_equal(one, np.full((b, 1), 7.0 * c, np.float32))
