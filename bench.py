@@ -196,6 +196,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-batch", type=int, default=None)
     ap.add_argument("--layers", action="store_true", help="also print a per-layer table to stderr")
+    ap.add_argument("--graph", action="store_true",
+                    help="time the steps as replays of one captured HIP graph instead of eager launches")
     ap.add_argument("--sweep", action="store_true",
                     help="instead of a network: the stand-alone bit-GEMM and 3x3 bit-convolution shapes "
                          "(int32 outputs), every engine; one JSON line with a row per case")
@@ -234,9 +236,16 @@ def main():
         net.forward(stream)
     stream.synchronize()
     _lib.device_synchronize()
+    step = lambda: net.forward(stream)
+    if args.graph:  # the forward allocates nothing and uses no memset: it can be captured whole
+        from tcbnn_amd.device import Graph
+        graph = Graph(stream, net.forward)
+        step = graph.launch
+        step()
+        stream.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        net.forward(stream)
+        step()
     stream.synchronize()
     _lib.device_synchronize()
     wall = time.perf_counter() - t0
@@ -333,7 +342,7 @@ def main():
                                              "cifar10_resnet": "cifar10_resnet.cu:189-259",
                                              "imagenet_vgg": "imagenet_vgg.cu:217-286",
                                              "imagenet_resnet_textbook": "no reference driver"}[args.net], batch),
-                   "variant": variant, "layers": len(spec),
+                   "variant": variant, "layers": len(spec), "launch": "hip graph replay" if args.graph else "eager",
                    "residual_storage": ("int16 where the bound of |residual| proves it exact (%d of %d tensors), "
                                         "else int32" % (sum(1 for v in res_bytes.values() if v == 2), len(res_bytes)))
                    if res_bytes else "none"},

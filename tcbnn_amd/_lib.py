@@ -164,6 +164,12 @@ _hip.hipEventDestroy.argtypes = [c_void_p]
 _hip.hipEventRecord.argtypes = [c_void_p, c_void_p]
 _hip.hipEventSynchronize.argtypes = [c_void_p]
 _hip.hipEventElapsedTime.argtypes = [C.POINTER(C.c_float), c_void_p, c_void_p]
+_hip.hipStreamBeginCapture.argtypes = [c_void_p, c_int]
+_hip.hipStreamEndCapture.argtypes = [c_void_p, C.POINTER(c_void_p)]
+_hip.hipGraphInstantiate.argtypes = [C.POINTER(c_void_p), c_void_p, c_void_p, c_void_p, c_size_t]
+_hip.hipGraphLaunch.argtypes = [c_void_p, c_void_p]
+_hip.hipGraphExecDestroy.argtypes = [c_void_p]
+_hip.hipGraphDestroy.argtypes = [c_void_p]
 
 H2D, D2H, D2D = 1, 2, 3
 

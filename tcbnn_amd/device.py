@@ -100,3 +100,35 @@ class Event:
                 hip.hipEventDestroy(self.handle)
         except Exception:
             pass
+
+
+class Graph:
+    """A HIP graph captured from the launches `record(stream)` makes on `stream` (the layers' forward
+    calls allocate nothing and clear nothing with memset, so a whole network can be captured); replay
+    with launch().  The caller warms the launches up once before capturing."""
+
+    def __init__(self, stream, record):
+        self.stream = stream
+        g = C.c_void_p(0)
+        hip_check(hip.hipStreamBeginCapture(stream.handle, 0), "hipStreamBeginCapture")  # global mode
+        try:
+            record(stream)
+        finally:
+            hip_check(hip.hipStreamEndCapture(stream.handle, C.byref(g)), "hipStreamEndCapture")
+        self.graph = g.value
+        e = C.c_void_p(0)
+        hip_check(hip.hipGraphInstantiate(C.byref(e), self.graph, None, None, 0), "hipGraphInstantiate")
+        self.exec = e.value
+
+    def launch(self):
+        hip_check(hip.hipGraphLaunch(self.exec, self.stream.handle), "hipGraphLaunch")
+
+    def __del__(self):
+        try:
+            if getattr(self, "exec", None):
+                hip.hipGraphExecDestroy(self.exec)
+            if getattr(self, "graph", None):
+                hip.hipGraphDestroy(self.graph)
+        except Exception:
+            pass
+

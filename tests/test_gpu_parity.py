@@ -559,6 +559,41 @@ def test_avgpool_fc(gpu, b, h, c, n, fmt):
     layer.release()
 
 
+def test_forward_captured_in_a_hip_graph(gpu):
+    """The whole forward (no allocation, no memset) is captured into a HIP graph and replayed several
+    times, with eager work and synchronisations between the replays and a new input before the last
+    one; every replay must reproduce the eager logits."""
+    from tcbnn_amd import nets
+    from tcbnn_amd.device import Graph, Stream
+    spec = nets.imagenet_resnet_spec(batch=16, image=64, output_size=100)
+    weights = gpu.synthetic_weights(spec, 21)
+    # the second input stays inside the magnitude bound the residual formats were chosen for
+    x0, x1 = gpu.synthetic_input(spec, 21), gpu.synthetic_input(spec, 22) * np.float32(0.9)
+    net = gpu.Network(spec, weights, x0)
+    stream = Stream()
+    net.forward(stream)
+    stream.synchronize()
+    eager0 = net.logits().copy()
+    graph = Graph(stream, net.forward)
+    for _ in range(3):
+        net.layers["Fout"].output_gpu.fill(0)  # eager work between the replays
+        gpuops.sync()
+        graph.launch()
+        stream.synchronize()
+        np.testing.assert_array_equal(net.logits(), eager0)
+    net.set_input(x1)
+    graph.launch()
+    stream.synchronize()
+    replay1 = net.logits().copy()
+    net.forward(stream)
+    stream.synchronize()
+    np.testing.assert_array_equal(replay1, net.logits())
+    assert not np.array_equal(replay1, eager0)
+    want = orc_nets.run(spec, weights, x1)["Fout"]["out"]
+    np.testing.assert_array_equal(replay1, want)
+    net.release()
+
+
 def test_imagenet_resnet18_batch256_every_image(gpu):
     """Full configured size on the default engine, every one of the 256 images and every layer against the
     oracle (packed activations and residuals bit for bit, logits to 1e-5 relative), three forward passes:
