@@ -123,7 +123,7 @@ def test_bconv_sweep_shapes(gpu, variant, h, c):
                                                    # 3x3 shapes of the persistent kernel's int32 epilogue: partial
                                                    # channel tile, partial image tile, stride 2, one-pixel frame
                                                    (70, 9, 64, 48, 3, 2), (33, 7, 192, 100, 3, 1), (8, 1, 128, 64, 3, 1),
-                                                   (40, 2, 384, 32, 3, 1)])
+                                                   (40, 2, 384, 32, 3, 1), (9, 6, 64, 33, 3, 1)])
 def test_bconv_odd_shapes(gpu, variant, b, h, cin, cout, R, stride):
     r = rng(b + h + cin)
     x = rm.pm1(r, (b, h, h, cin))
@@ -220,7 +220,7 @@ def test_conv128_layer(gpu, variant, b, h, cin, cout, stride, pool, ahead_fc):
 
 # (cin, cout): the persistent 3x3 kernel's instantiations (Cin 64 .. 512), a channel count that is not a
 # multiple of 32 and an odd one (half-filled last 16-bit pair); formats of the injected and saved tensors
-RES_SHAPES = [(64, 96), (128, 64), (256, 35), (512, 64), (192, 64), (384, 40)]
+RES_SHAPES = [(64, 96), (128, 64), (256, 35), (512, 64), (192, 64), (384, 40), (96, 35)]
 RES_FORMATS = [(0, 0), (1, 1), (0, 1), (1, 0)]
 
 
