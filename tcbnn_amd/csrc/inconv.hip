@@ -119,6 +119,7 @@ __device__ __forceinline__ void add_indexed8x2(float* a, float* b, v8f ca, v8f c
 // The read-only operands are separate __restrict__ kernel arguments so that the
 // wave-uniform mask / threshold loads become scalar loads (s_load) feeding v_xor directly.
 typedef uint32_t u16v __attribute__((ext_vector_type(16)));
+typedef int v4i_t __attribute__((ext_vector_type(4)));
 
 // Staging of one filter row: the 3 x 64 (channel, image) row segments of ncols floats each.
 //   ROWS = true (ncols <= 21): a wave takes rpw (a multiple of 3) segments at a time, lanes
@@ -324,24 +325,28 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS ?
                     int r32[32];
 #pragma unroll
                     for (int n = 0; n < 32; ++n) r32[n] = wi * 32 + n < p.O ? (int)acc[n] : 0;
-                    int4* __restrict__ dst = reinterpret_cast<int4*>(res);
+                    // streaming stores: the tensor (103 MB at batch 256) is far larger than the caches and is
+                    // read two launches later
+                    v4i_t* __restrict__ dst = reinterpret_cast<v4i_t*>(res);
                     if (p.res_fmt == TCBNN_RES_I16) {
                         const size_t g0 = (pix * ((p.O + 7) / 8) + wi * 4) * p.B + b;
 #pragma unroll
                         for (int g = 0; g < 4; ++g)
                             if (wi * 32 + 8 * g < p.O)
-                                dst[g0 + (size_t)g * p.B] =
-                                    make_int4((r32[8 * g] & 0xffff) | (r32[8 * g + 1] << 16),
-                                              (r32[8 * g + 2] & 0xffff) | (r32[8 * g + 3] << 16),
-                                              (r32[8 * g + 4] & 0xffff) | (r32[8 * g + 5] << 16),
-                                              (r32[8 * g + 6] & 0xffff) | (r32[8 * g + 7] << 16));
+                                __builtin_nontemporal_store(
+                                    v4i_t{(r32[8 * g] & 0xffff) | (r32[8 * g + 1] << 16),
+                                          (r32[8 * g + 2] & 0xffff) | (r32[8 * g + 3] << 16),
+                                          (r32[8 * g + 4] & 0xffff) | (r32[8 * g + 5] << 16),
+                                          (r32[8 * g + 6] & 0xffff) | (r32[8 * g + 7] << 16)},
+                                    dst + g0 + (size_t)g * p.B);
                     } else {
                         const size_t g0 = (pix * ((p.O + 3) / 4) + wi * 8) * p.B + b;
 #pragma unroll
                         for (int g = 0; g < 8; ++g)
                             if (wi * 32 + 4 * g < p.O)
-                                dst[g0 + (size_t)g * p.B] =
-                                    make_int4(r32[4 * g], r32[4 * g + 1], r32[4 * g + 2], r32[4 * g + 3]);
+                                __builtin_nontemporal_store(
+                                    v4i_t{r32[4 * g], r32[4 * g + 1], r32[4 * g + 2], r32[4 * g + 3]},
+                                    dst + g0 + (size_t)g * p.B);
                     }
                 }
             }
