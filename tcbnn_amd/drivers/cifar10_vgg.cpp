@@ -5,7 +5,7 @@
 int main(int argc, char** argv) {
     driver::Options o = driver::parse(argc, argv,
         "cifar10_vgg [--batch N] [--seed S] [--reps R] [--weights vgg_cifar10.csv] [--input x.f32] "
-        "[--out logits.f32] [--variant popc|mfma_i8|mfma_f4]");
+        "[--out logits.f32] [--labels y.u32] [--variant popc|mfma_i8|mfma_f4]");
     HIP_SAFE_CALL(hipSetDevice(0));
     const unsigned batch = o.batch ? o.batch : 256;
     const unsigned output_size = o.classes ? o.classes : 10;

@@ -13,6 +13,7 @@
 #include <string>
 #include <vector>
 
+#include "../host/tcbnn_data.hpp"
 #include "../host/tcbnn_layers.hpp"
 
 namespace driver {
@@ -27,6 +28,7 @@ struct Options {
     std::string weights;    // text weight file in the reference's format; empty = synthetic
     std::string input;      // raw float32 input file; empty = synthetic
     std::string out;        // raw float32 logits are written here if set
+    std::string labels;     // raw uint32 labels (read_dataset writes them): scores the logits against them
     std::string variant;    // popc | mfma_i8 | mfma_f4
 };
 
@@ -50,6 +52,7 @@ inline Options parse(int argc, char** argv, const char* usage) {
         else if (a == "--weights") o.weights = next();
         else if (a == "--input") o.input = next();
         else if (a == "--out") o.out = next();
+        else if (a == "--labels") o.labels = next();
         else if (a == "--variant") o.variant = next();
         else {
             fprintf(stderr, "unknown argument %s\n%s\n", a.c_str(), usage);
@@ -168,6 +171,13 @@ inline void report(const char* net, int batch, double ms, double binary_ops, con
            "\"binary_tops\": %.2f, \"logits0\": [%.6g, %.6g, %.6g]}\n",
            net, batch, ms, batch / (ms * 1e-3), binary_ops / (ms * 1e-3) / 1e12, logits[0],
            logits[classes > 1 ? 1 : 0], logits[classes > 2 ? 2 : 0]);
+    if (!o.labels.empty()) {  // the call every reference main carries, commented out (e.g. mnist_mlp.cu:156)
+        std::vector<unsigned> labels(batch);
+        FILE* f = tcbnn_data::open_or_die(o.labels, "label");
+        tcbnn_data::read_or_die(f, labels.data(), labels.size() * sizeof(unsigned), o.labels);
+        fclose(f);
+        validate_prediction(const_cast<float*>(logits), labels.data(), (unsigned)classes, (unsigned)batch);
+    }
     if (!o.out.empty()) {
         FILE* f = fopen(o.out.c_str(), "wb");
         if (f == NULL || fwrite(logits, sizeof(float), (size_t)batch * classes, f) != (size_t)batch * classes) {

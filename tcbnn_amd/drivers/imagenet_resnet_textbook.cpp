@@ -9,7 +9,7 @@
 int main(int argc, char** argv) {
     driver::Options o = driver::parse(argc, argv,
         "imagenet_resnet_textbook [--batch N] [--image 224] [--classes 1000] [--seed S] [--reps R] "
-        "[--weights FILE] [--input x.f32] [--out logits.f32] [--variant popc|mfma_i8|mfma_f4]");
+        "[--weights FILE] [--input x.f32] [--out logits.f32] [--labels y.u32] [--variant popc|mfma_i8|mfma_f4]");
     HIP_SAFE_CALL(hipSetDevice(0));
     const unsigned batch = o.batch ? o.batch : 256;
     const unsigned output_size = o.classes ? o.classes : 1000;

@@ -4,7 +4,7 @@
 
 int main(int argc, char** argv) {
     driver::Options o = driver::parse(argc, argv,
-        "mnist_mlp [--batch N] [--seed S] [--reps R] [--weights mlp_mnist.csv] [--input x.f32] [--out logits.f32] "
+        "mnist_mlp [--batch N] [--seed S] [--reps R] [--weights mlp_mnist.csv] [--input x.f32] [--out logits.f32] [--labels y.u32] "
         "[--variant popc|mfma_i8|mfma_f4]");
     HIP_SAFE_CALL(hipSetDevice(0));
     const unsigned batch = o.batch ? o.batch : 8192;

@@ -110,3 +110,41 @@ def test_driver_error_convention_is_print_and_exit(gpu):
     proc = subprocess.run([exe, "--weights", "/nonexistent.csv"], stdout=subprocess.PIPE, stderr=subprocess.PIPE,
                           text=True, timeout=60)
     assert proc.returncode != 0 and "NULL pointer" in proc.stderr
+
+
+def test_mnist_mlp_driver_on_a_dataset_file(gpu, tmp_path):
+    """idx files -> read_dataset -> mnist_mlp --input/--labels: the evaluation flow of the reference's main
+    (read_MNIST_normalized ... validate_prediction, mnist_mlp.cu:80-156), on synthetic idx files."""
+    import struct
+    import tcbnn_amd
+    from tcbnn_amd import data, nets
+    batch = 96
+    rng = np.random.default_rng(11)
+    px = rng.integers(0, 256, size=(batch, 28, 28), dtype=np.uint8)
+    lab = rng.integers(0, 10, size=batch, dtype=np.uint8)
+    fi, fl = str(tmp_path / "img-idx3"), str(tmp_path / "lab-idx1")
+    with open(fi, "wb") as f:
+        f.write(struct.pack(">4i", 2051, batch, 28, 28) + px.tobytes())
+    with open(fl, "wb") as f:
+        f.write(struct.pack(">2i", 2049, batch) + lab.tobytes())
+    xf, lf, wf, of = (str(tmp_path / n) for n in ("x.f32", "y.u32", "w.csv", "logits.f32"))
+    subprocess.check_call([os.path.join(BIN, "read_dataset"), "mnist", fi, fl, str(batch), xf, lf])
+    x, labels = data.read_MNIST_normalized(fi, fl, batch)
+    assert np.array_equal(np.fromfile(xf, np.float32), x.ravel())
+
+    spec = nets.mnist_mlp_spec(batch=batch)
+    weights = tcbnn_amd.synthetic_weights(spec, 12)
+    _write_weight_file(wf, weights)
+    proc = subprocess.run([os.path.join(BIN, "mnist_mlp"), "--batch", str(batch), "--weights", wf, "--input", xf,
+                           "--labels", lf, "--out", of, "--reps", "1", "--warmup", "0"],
+                          stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
+    assert proc.returncode == 0, proc.stdout
+    got = np.fromfile(of, np.float32).reshape(batch, 10)
+    want = orc_nets.run(spec, weights, x.reshape(batch, 784))[spec[-1]["name"]]["out"]
+    np.testing.assert_array_equal(got, want)
+    top1, top5, pos = data.score_prediction(want, labels)
+    lines = proc.stdout.splitlines()
+    i = lines.index("=====Predict=======")
+    assert lines[i + 1].split() == [str(v) for v in pos]
+    pct = lambda n: float(np.float32(n) / np.float32(batch) * np.float32(100))  # the reference prints float32
+    assert lines[i + 3] == "Top-1:%f%%" % pct(top1) and lines[i + 4] == "Top-5:%f%%" % pct(top5)
