@@ -324,6 +324,12 @@ int tcbnn_conv_from_reference_fmt(const uint32_t* fmt, uint32_t* packed, int hei
  * zero fill (kernel.cuh:666-668, 820-823). */
 int tcbnn_residual_to_reference(const int32_t* res, int32_t* ref, int height, int width,
                                 int batch, int ch, int format, void* stream);
+/* The reverse: a residual in the reference layout -> the engine layout `format`
+ * (tcbnn_residual_bytes(...) bytes), for a Conv128 layer that injects a residual a
+ * reference-layout producer saved (read at kernel.cuh:760-791).  TCBNN_RES_I16 keeps the low
+ * 16 bits: only for values the caller knows to fit. */
+int tcbnn_residual_from_reference(const int32_t* ref, int32_t* res, int height, int width,
+                                  int batch, int ch, int format, void* stream);
 
 #ifdef __cplusplus
 }

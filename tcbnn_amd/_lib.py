@@ -124,6 +124,7 @@ ABI = {
     "tcbnn_conv_to_reference_fmt": (c_int, [c_void_p, c_void_p] + [c_int] * 4 + [c_void_p]),
     "tcbnn_conv_from_reference_fmt": (c_int, [c_void_p, c_void_p] + [c_int] * 4 + [c_void_p]),
     "tcbnn_residual_to_reference": (c_int, [c_void_p, c_void_p] + [c_int] * 5 + [c_void_p]),
+    "tcbnn_residual_from_reference": (c_int, [c_void_p, c_void_p] + [c_int] * 5 + [c_void_p]),
 }
 
 for _name, (_res, _args) in ABI.items():

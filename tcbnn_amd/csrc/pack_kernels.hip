@@ -218,6 +218,30 @@ __global__ void residual_to_reference_kernel(const int32_t* __restrict__ res,
     ref[idx] = (b < batch && c < ch) ? residual_load(res, fmt, (size_t)pix, ch, c, batch, b) : 0;
 }
 
+// One thread per 16-byte group of the engine's layouts (4 int32 or 8 int16 channels of one image and pixel);
+// channels past `ch` are stored as 0, which is what the consumers of the padding lanes expect.
+__global__ void residual_from_reference_kernel(const int32_t* __restrict__ ref, int32_t* __restrict__ res,
+                                               long long pixels, int batch, int ch, int b8, int c128, int fmt) {
+    const int per = fmt == TCBNN_RES_I16 ? 8 : 4;
+    const int groups = (ch + per - 1) / per;
+    const long long idx = (long long)blockIdx.x * kThreads + threadIdx.x;
+    if (idx >= pixels * groups * batch) return;
+    const int b = (int)(idx % batch);
+    const int g = (int)((idx / batch) % groups);
+    const long long pix = idx / ((long long)batch * groups);
+    const int32_t* src = ref + ((size_t)pix * b8 + b) * c128 + (size_t)g * per;
+    int v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = (i < per && g * per + i < ch) ? src[i] : 0;
+    int4 o;
+    if (fmt == TCBNN_RES_I16)
+        o = make_int4((v[0] & 0xffff) | (v[1] << 16), (v[2] & 0xffff) | (v[3] << 16), (v[4] & 0xffff) | (v[5] << 16),
+                      (v[6] & 0xffff) | (v[7] << 16));
+    else
+        o = make_int4(v[0], v[1], v[2], v[3]);
+    reinterpret_cast<int4*>(res)[idx] = o;  // [pix][group][b] is the linear order of both layouts
+}
+
 }  // namespace
 }  // namespace tcbnn
 
@@ -400,6 +424,21 @@ int tcbnn_residual_to_reference(const int32_t* res, int32_t* ref, int height, in
     hipLaunchKernelGGL(residual_to_reference_kernel, dim3(blocks_for(total)), dim3(kThreads), 0,
                        (hipStream_t)stream, res, ref, pixels, batch, ch, pad8(batch), pad128(ch), format);
     TCBNN_LAUNCH_CHECK("residual_to_reference_kernel");
+    return TCBNN_OK;
+}
+
+int tcbnn_residual_from_reference(const int32_t* ref, int32_t* res, int height, int width, int batch,
+                                  int ch, int format, void* stream) {
+    TCBNN_NOTNULL(ref);
+    TCBNN_NOTNULL(res);
+    TCBNN_REQUIRE(batch > 0 && height > 0 && width > 0 && ch > 0, "residual_from_reference: bad shape");
+    TCBNN_REQUIRE(format == TCBNN_RES_I32 || format == TCBNN_RES_I16, "residual_from_reference: unknown format");
+    const long long pixels = (long long)height * width;
+    const int per = format == TCBNN_RES_I16 ? 8 : 4;
+    const long long total = pixels * ((ch + per - 1) / per) * batch;
+    hipLaunchKernelGGL(residual_from_reference_kernel, dim3(blocks_for(total)), dim3(kThreads), 0,
+                       (hipStream_t)stream, ref, res, pixels, batch, ch, pad8(batch), pad128(ch), format);
+    TCBNN_LAUNCH_CHECK("residual_from_reference_kernel");
     return TCBNN_OK;
 }
 

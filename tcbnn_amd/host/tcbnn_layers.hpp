@@ -185,6 +185,13 @@ class In128LayerParam {  // param.h:115-222
         SAFE_FREE_GPU(tmp);
         return this->output;
     }
+    // The output in the reference's own tile layout ON THE DEVICE (what get_output_gpu() of the reference
+    // holds, kernel.cuh:170): converted on `stream`, after forward(), into a buffer this layer owns.
+    uin32* get_output_gpu_reference_fmt(hipStream_t stream = 0) {
+        if (output_fmt_gpu == NULL) SAFE_ALOC_GPU(output_fmt_gpu, output_bit_bytes());
+        TCBNN_SAFE_CALL(tcbnn_fc_to_reference_fmt(output_gpu, output_fmt_gpu, output_height, output_width, stream));
+        return output_fmt_gpu;
+    }
     float* download_full_output() {  // +-1.0f [B][K] (UnPackFcOutput128FMT, param.h:87-104)
         float* full_output = NULL;
         SAFE_ALOC_HOST(full_output, output_bytes());
@@ -198,6 +205,7 @@ class In128LayerParam {  // param.h:115-222
     void release() {
         SAFE_FREE_GPU(input_gpu);
         SAFE_FREE_GPU(output_gpu);
+        SAFE_FREE_GPU(output_fmt_gpu);
         SAFE_FREE_HOST(output);
     }
     ~In128LayerParam() { release(); }
@@ -213,6 +221,7 @@ class In128LayerParam {  // param.h:115-222
     int output_height;
     In128LayerParam* gpu;
     char name[8];
+    uin32* output_fmt_gpu = NULL;  // reference-layout copy of the output (no counterpart in the reference)
 };
 
 // ======================================================================================
@@ -257,6 +266,20 @@ class Fc128LayerParam {  // param.h:224-385
         return this;
     }
     uin32* get_output_gpu() { return this->output_gpu; }
+    // Reference-layout neighbours (kernel.cuh:187-191 reads, :222-223 writes [B/8][K/128][8][4] tiles): the input
+    // is converted on `stream` from a device buffer in that layout into a buffer this layer owns (a copy, so call
+    // it again when the source changes), the output after forward() likewise into the reference layout.
+    void set_input_gpu_reference_fmt(const uin32* fmt_gpu, hipStream_t stream = 0) {
+        CHECK_NULL_POINTER(fmt_gpu);
+        if (input_own_gpu == NULL) SAFE_ALOC_GPU(input_own_gpu, 4 * tcbnn_fc_act_words(input_height, input_width));
+        TCBNN_SAFE_CALL(tcbnn_fc_from_reference_fmt(fmt_gpu, input_own_gpu, input_height, input_width, stream));
+        input_gpu = input_own_gpu;
+    }
+    uin32* get_output_gpu_reference_fmt(hipStream_t stream = 0) {
+        if (output_fmt_gpu == NULL) SAFE_ALOC_GPU(output_fmt_gpu, output_bit_bytes());
+        TCBNN_SAFE_CALL(tcbnn_fc_to_reference_fmt(output_gpu, output_fmt_gpu, output_height, output_width, stream));
+        return output_fmt_gpu;
+    }
     void forward(hipStream_t stream = 0) {
         tcbnn_fc128_desc d = {input_gpu, weight_gpu, bn_gpu,  output_gpu,    input_height,
                               input_width, weight_width, variant, workspace_gpu, workspace_words()};
@@ -289,6 +312,8 @@ class Fc128LayerParam {  // param.h:224-385
         SAFE_FREE_GPU(bn_gpu);
         SAFE_FREE_GPU(output_gpu);
         SAFE_FREE_GPU(workspace_gpu);
+        SAFE_FREE_GPU(input_own_gpu);
+        SAFE_FREE_GPU(output_fmt_gpu);
     }
     ~Fc128LayerParam() { release(); }
 
@@ -312,6 +337,8 @@ class Fc128LayerParam {  // param.h:224-385
     char name[8];
     int variant;             // TCBNN_VARIANT_* (no counterpart in the reference)
     int32_t* workspace_gpu;  // split-K scratch (no counterpart in the reference)
+    uin32* input_own_gpu = NULL;   // engine-layout copy of a reference-layout input
+    uin32* output_fmt_gpu = NULL;  // reference-layout copy of the output
 };
 
 // ======================================================================================
@@ -358,6 +385,13 @@ class Out128LayerParam {  // param.h:388-531
         CHECK_NULL_POINTER(input_gpu);
         return this;
     }
+    // input from a device buffer in the reference's tile layout (kernel.cuh:243-247): see Fc128LayerParam
+    void set_input_gpu_reference_fmt(const uin32* fmt_gpu, hipStream_t stream = 0) {
+        CHECK_NULL_POINTER(fmt_gpu);
+        if (input_own_gpu == NULL) SAFE_ALOC_GPU(input_own_gpu, 4 * tcbnn_fc_act_words(input_height, input_width));
+        TCBNN_SAFE_CALL(tcbnn_fc_from_reference_fmt(fmt_gpu, input_own_gpu, input_height, input_width, stream));
+        input_gpu = input_own_gpu;
+    }
     void forward(hipStream_t stream = 0) {
         tcbnn_out128_desc d = {input_gpu,    weight_gpu,  bn_scale_gpu, bn_bias_gpu, output_gpu,
                                input_height, input_width, weight_width, variant};
@@ -377,6 +411,7 @@ class Out128LayerParam {  // param.h:388-531
         SAFE_FREE_GPU(output_gpu);
         SAFE_FREE_GPU(bn_scale_gpu);
         SAFE_FREE_GPU(bn_bias_gpu);
+        SAFE_FREE_GPU(input_own_gpu);
     }
     ~Out128LayerParam() { release(); }
 
@@ -401,6 +436,7 @@ class Out128LayerParam {  // param.h:388-531
     Out128LayerParam* gpu;
     char name[8];
     int variant;
+    uin32* input_own_gpu = NULL;  // engine-layout copy of a reference-layout input
 };
 
 // ======================================================================================
@@ -489,6 +525,24 @@ class InConv128LayerParam {  // param.h:701-870
                                   pool_height,    pool_width,     save_residual ? 1 : 0, residual_info.format};
         TCBNN_SAFE_CALL(tcbnn_inconv128_forward(&d, stream));
     }
+    // Output and saved residual in the reference's own device layouts (kernel.cuh:650-668), converted on `stream`
+    // after forward() into buffers this layer owns: [OH][OW][PAD8(B)/8][STEP128(O)][8][4] words, and int32
+    // [P][Q][PAD8(B)][PAD128(O)].
+    uin32* get_output_gpu_reference_fmt(hipStream_t stream = 0) {
+        if (output_fmt_gpu == NULL) SAFE_ALOC_GPU(output_fmt_gpu, output_bit_bytes());
+        TCBNN_SAFE_CALL(tcbnn_conv_to_reference_fmt(output_gpu, output_fmt_gpu, output_height, output_width, batch,
+                                                    output_channels, stream));
+        return output_fmt_gpu;
+    }
+    int* get_output_residual_gpu_reference(hipStream_t stream = 0) {
+        CHECK_NULL_POINTER(output_residual_gpu);
+        if (output_residual_ref_gpu == NULL)
+            SAFE_ALOC_GPU(output_residual_ref_gpu,
+                          (size_t)buf_height * buf_width * PAD8(batch) * PAD128(output_channels) * sizeof(int));
+        TCBNN_SAFE_CALL(tcbnn_residual_to_reference(output_residual_gpu, output_residual_ref_gpu, buf_height,
+                                                    buf_width, batch, output_channels, residual_info.format, stream));
+        return output_residual_ref_gpu;
+    }
     unsigned* download_output() {
         if (output == NULL) SAFE_ALOC_HOST(output, output_bit_bytes());
         uin32* tmp = NULL;
@@ -520,6 +574,8 @@ class InConv128LayerParam {  // param.h:701-870
         SAFE_FREE_GPU(bn_gpu);
         if (output_residual_gpu != NULL) tcbnn_host::residual_registry().erase(output_residual_gpu);
         SAFE_FREE_GPU(output_residual_gpu);
+        SAFE_FREE_GPU(output_fmt_gpu);
+        SAFE_FREE_GPU(output_residual_ref_gpu);
     }
     ~InConv128LayerParam() { release(); }
 
@@ -554,6 +610,8 @@ class InConv128LayerParam {  // param.h:701-870
     InConv128LayerParam* gpu;
     char name[8];
     int buf_height, buf_width;  // conv output size before pooling
+    uin32* output_fmt_gpu = NULL;        // reference-layout copies of the output and the saved residual
+    int* output_residual_ref_gpu = NULL;
 };
 
 // ======================================================================================
@@ -679,6 +737,51 @@ class Conv128LayerParam {  // param.h:872-1065
         d.output_residual_format = residual_info.format;
         TCBNN_SAFE_CALL(tcbnn_conv128_forward(&d, stream));
     }
+    // Reference-layout neighbours.  Input bits [H][W][PAD8(B)/8][STEP128(C)][8][4] (read at kernel.cuh:741-749) and
+    // an injected residual int32 [Hr][Wr][PAD8(B)][PAD128(residual_channels)] (kernel.cuh:770-791; Hr x Wr is the
+    // convolution's output size, twice that with residual_pool) are converted on `stream` from device buffers in
+    // those layouts into buffers this layer owns: copies, so call again when the source changes.  Nothing is
+    // known about a foreign residual's values: it is kept as int32 with an unknown bound, and a layer that also
+    // saves a residual must have been initialized with it, so that its own residual is sized for that.
+    void set_input_gpu_reference_fmt(const uin32* fmt_gpu, hipStream_t stream = 0) {
+        CHECK_NULL_POINTER(fmt_gpu);
+        if (input_own_gpu == NULL)
+            SAFE_ALOC_GPU(input_own_gpu, 4 * tcbnn_conv_act_words(input_height, input_width, batch, input_channels));
+        TCBNN_SAFE_CALL(tcbnn_conv_from_reference_fmt(fmt_gpu, input_own_gpu, input_height, input_width, batch,
+                                                      input_channels, stream));
+        input_gpu = input_own_gpu;
+    }
+    void set_input_residual_gpu_reference(const int* ref_gpu, hipStream_t stream = 0) {
+        CHECK_NULL_POINTER(ref_gpu);
+        const int scale = residual_pool ? 2 : 1;
+        const int rh = buf_height * scale, rw = buf_width * scale;
+        if (input_residual_own_gpu == NULL)
+            SAFE_ALOC_GPU(input_residual_own_gpu, tcbnn_residual_bytes(rh, rw, residual_channels, batch, TCBNN_RES_I32));
+        TCBNN_SAFE_CALL(tcbnn_residual_from_reference(ref_gpu, input_residual_own_gpu, rh, rw, batch,
+                                                      residual_channels, TCBNN_RES_I32, stream));
+        set_input_residual_gpu(input_residual_own_gpu);  // not in the registry: int32, unknown bound
+    }
+    // Output (conv tiles, or FC tiles for an FC-ready layer: kernel.cuh:798-815) and saved residual
+    // (kernel.cuh:818-824) in the reference's device layouts, converted on `stream` after forward().
+    uin32* get_output_gpu_reference_fmt(hipStream_t stream = 0) {
+        if (output_fmt_gpu == NULL) SAFE_ALOC_GPU(output_fmt_gpu, output_bit_bytes());
+        if (ahead_fc)
+            TCBNN_SAFE_CALL(tcbnn_fc_to_reference_fmt(output_gpu, output_fmt_gpu, batch,
+                                                      output_height * output_width * PAD128(output_channels), stream));
+        else
+            TCBNN_SAFE_CALL(tcbnn_conv_to_reference_fmt(output_gpu, output_fmt_gpu, output_height, output_width,
+                                                        batch, output_channels, stream));
+        return output_fmt_gpu;
+    }
+    int* get_output_residual_gpu_reference(hipStream_t stream = 0) {
+        CHECK_NULL_POINTER(output_residual_gpu);
+        if (output_residual_ref_gpu == NULL)
+            SAFE_ALOC_GPU(output_residual_ref_gpu,
+                          (size_t)buf_height * buf_width * PAD8(batch) * PAD128(output_channels) * sizeof(int));
+        TCBNN_SAFE_CALL(tcbnn_residual_to_reference(output_residual_gpu, output_residual_ref_gpu, buf_height,
+                                                    buf_width, batch, output_channels, residual_info.format, stream));
+        return output_residual_ref_gpu;
+    }
     unsigned* download_output() {
         if (output == NULL) SAFE_ALOC_HOST(output, output_bit_bytes());
         uin32* tmp = NULL;
@@ -717,6 +820,10 @@ class Conv128LayerParam {  // param.h:872-1065
         SAFE_FREE_GPU(bn_gpu);
         if (output_residual_gpu != NULL) tcbnn_host::residual_registry().erase(output_residual_gpu);
         SAFE_FREE_GPU(output_residual_gpu);
+        SAFE_FREE_GPU(input_own_gpu);
+        SAFE_FREE_GPU(input_residual_own_gpu);
+        SAFE_FREE_GPU(output_fmt_gpu);
+        SAFE_FREE_GPU(output_residual_ref_gpu);
     }
     ~Conv128LayerParam() { release(); }
 
@@ -759,6 +866,10 @@ class Conv128LayerParam {  // param.h:872-1065
     int input_residual_channels;
     tcbnn_host::ResidualInfo input_residual_info;  // of input_residual_gpu
     int buf_height, buf_width;
+    uin32* input_own_gpu = NULL;         // engine-layout copies of a reference-layout input / injected residual
+    int* input_residual_own_gpu = NULL;
+    uin32* output_fmt_gpu = NULL;        // reference-layout copies of the output and the saved residual
+    int* output_residual_ref_gpu = NULL;
 };
 
 // ======================================================================================

@@ -90,7 +90,84 @@ def _residual_buffer(channels, height, width, batch, bound, force_format=None):
     return buf
 
 
-class In128LayerParam:
+class _ReferenceLayoutIO:
+    """Device buffers in the reference's own tile layouts at a layer's edges, for a neighbour that is a
+    layer of the reference (FC tiles [B/8][K/128][8][4], kernel.cuh:170,187-191,222-223; conv tiles
+    [H][W][B/8][C/128][8][4], kernel.cuh:650-660,741-749,811-815; residuals int32
+    [P][Q][PAD8(B)][PAD128(O)], kernel.cuh:666-668,770-791,820-823).  Every accessor enqueues a conversion
+    on `stream` between such a buffer and one in the engine's layout that the layer owns: copies, not
+    views, so imports are repeated when the source changes and exports after every forward()."""
+
+    def _ref_buf(self, key, nbytes):
+        bufs = self.__dict__.setdefault("_ref_bufs", {})
+        if key not in bufs:
+            bufs[key] = DeviceBuffer(nbytes)
+        return bufs[key]
+
+    def _release_ref_bufs(self):
+        for b in self.__dict__.pop("_ref_bufs", {}).values():
+            b.free()
+
+    # how this layer's input / output bits are tiled: ("fc", batch, features) or ("conv", h, w, batch, channels)
+    def _input_tiling(self):
+        if hasattr(self, "input_channels"):
+            return ("conv", self.input_height, self.input_width, self.batch, self.input_channels)
+        return ("fc", self.input_height, self.input_width)
+
+    def _output_tiling(self):
+        if hasattr(self, "output_channels"):
+            if getattr(self, "ahead_fc", False):
+                return ("fc", self.batch, self.output_height * self.output_width * PAD128(self.output_channels))
+            return ("conv", self.output_height, self.output_width, self.batch, self.output_channels)
+        return ("fc", self.output_height, self.output_width)
+
+    def set_input_gpu_reference_fmt(self, fmt_gpu, stream=None):
+        t = self._input_tiling()
+        if t[0] == "fc":
+            own = self._ref_buf("in", 4 * lib.tcbnn_fc_act_words(t[1], t[2]))
+            check(lib.tcbnn_fc_from_reference_fmt(fmt_gpu.ptr, own.ptr, t[1], t[2], _stream_handle(stream)))
+        else:
+            own = self._ref_buf("in", 4 * lib.tcbnn_conv_act_words(t[1], t[2], t[3], t[4]))
+            check(lib.tcbnn_conv_from_reference_fmt(fmt_gpu.ptr, own.ptr, t[1], t[2], t[3], t[4],
+                                                    _stream_handle(stream)))
+        self.input_gpu = own
+
+    def get_output_gpu_reference_fmt(self, stream=None):
+        t = self._output_tiling()
+        fmt = self._ref_buf("out", 16 * self.output_bit_size())
+        if t[0] == "fc":
+            check(lib.tcbnn_fc_to_reference_fmt(self.output_gpu.ptr, fmt.ptr, t[1], t[2], _stream_handle(stream)))
+        else:
+            check(lib.tcbnn_conv_to_reference_fmt(self.output_gpu.ptr, fmt.ptr, t[1], t[2], t[3], t[4],
+                                                  _stream_handle(stream)))
+        return fmt
+
+    def get_output_residual_gpu_reference(self, stream=None):
+        src = self.output_residual_gpu
+        if src is None:
+            raise _lib.TcbnnError("Error: NULL pointer (output_residual_gpu)")
+        ref = self._ref_buf("res_out", 4 * self.buf_height * self.buf_width * PAD8(self.batch)
+                            * PAD128(self.output_channels))
+        check(lib.tcbnn_residual_to_reference(src.ptr, ref.ptr, self.buf_height, self.buf_width, self.batch,
+                                              self.output_channels, src.format, _stream_handle(stream)))
+        return ref
+
+    def set_input_residual_gpu_reference(self, ref_gpu, stream=None):
+        """Nothing is known about a foreign residual's values: it is kept as int32 with an unknown bound, so a
+        layer that also saves a residual must have been initialized with an equally unbounded source."""
+        scale = 2 if self.residual_pool else 1
+        rh, rw = self.buf_height * scale, self.buf_width * scale
+        bufs = self.__dict__.setdefault("_ref_bufs", {})
+        if "res_in" not in bufs:
+            bufs["res_in"] = _residual_buffer(self.residual_channels, rh, rw, self.batch, _lib.INT32_MAX,
+                                              _lib.RES_I32)
+        own = bufs["res_in"]
+        check(lib.tcbnn_residual_from_reference(ref_gpu.ptr, own.ptr, rh, rw, self.batch, self.residual_channels,
+                                                _lib.RES_I32, _stream_handle(stream)))
+        self.set_input_residual_gpu(own)
+
+
+class In128LayerParam(_ReferenceLayoutIO):
     """param.h:115-222; forward = In128LayerFMT (kernel.cuh:153-172)."""
 
     def __init__(self, name, input_height, input_width):
@@ -134,6 +211,7 @@ class In128LayerParam:
         return _fc_download_full(self.output_gpu, self.output_height, self.output_width)
 
     def release(self):
+        self._release_ref_bufs()
         for b in (self.input_gpu, self.output_gpu):
             if b is not None:
                 b.free()
@@ -155,7 +233,7 @@ def _fc_download_full(buf, batch, features):
     return tmp.to_numpy(np.float32, (batch, features))
 
 
-class Fc128LayerParam:
+class Fc128LayerParam(_ReferenceLayoutIO):
     """param.h:224-385; forward = Fc128LayerFMT (kernel.cuh:174-226)."""
 
     def __init__(self, name, input_height, input_width, weight_width, variant=_lib.VARIANT_AUTO):
@@ -227,13 +305,14 @@ class Fc128LayerParam:
         return _fc_download_full(self.output_gpu, self.output_height, self.output_width)
 
     def release(self):
+        self._release_ref_bufs()
         for b in (self.weight_gpu, self.bn_gpu, self.output_gpu, getattr(self, "workspace_gpu", None)):
             if b is not None:
                 b.free()
         self.weight_gpu = self.bn_gpu = self.output_gpu = self.workspace_gpu = None
 
 
-class Out128LayerParam:
+class Out128LayerParam(_ReferenceLayoutIO):
     """param.h:388-531; forward = Out128LayerFMT (kernel.cuh:230-280)."""
 
     def __init__(self, name, input_height, input_width, weight_width, variant=_lib.VARIANT_AUTO):
@@ -293,13 +372,14 @@ class Out128LayerParam:
         return self.output_gpu.to_numpy(np.float32, (self.output_height, self.output_width))
 
     def release(self):
+        self._release_ref_bufs()
         for b in (self.weight_gpu, self.bn_scale_gpu, self.bn_bias_gpu, self.output_gpu):
             if b is not None:
                 b.free()
         self.weight_gpu = self.bn_scale_gpu = self.bn_bias_gpu = self.output_gpu = None
 
 
-class _ConvGeometry:
+class _ConvGeometry(_ReferenceLayoutIO):
     """Derived geometry shared by both conv constructors (param.h:719-728, 897-906)."""
 
     def _derive(self):
@@ -461,6 +541,7 @@ class InConv128LayerParam(_ConvGeometry):
         return buf.value.decode()
 
     def release(self):
+        self._release_ref_bufs()
         for b in (self.input_gpu, self.filter_gpu, self.bn_gpu, self.output_gpu, self.output_residual_gpu):
             if b is not None:
                 b.free()
@@ -493,6 +574,11 @@ class Conv128LayerParam(_ConvGeometry):
         self.input_gpu = input_gpu
 
     def set_input_residual_gpu(self, input_residual_gpu):
+        if input_residual_gpu is not None and not hasattr(input_residual_gpu, "bound"):
+            # a residual that no layer of this library produced: int32 with the consumer's channel limit and
+            # no known bound
+            input_residual_gpu.channels, input_residual_gpu.format = self.residual_channels, _lib.RES_I32
+            input_residual_gpu.bound = _lib.INT32_MAX
         out = self.output_residual_gpu
         if out is not None and input_residual_gpu is not None and self.inject_residual and \
                 lib.tcbnn_conv_residual_bound(self.input_channels, self.filter_height, self.filter_width,
@@ -558,6 +644,7 @@ class Conv128LayerParam(_ConvGeometry):
         return buf.value.decode()
 
     def release(self):
+        self._release_ref_bufs()
         for b in (self.filter_gpu, self.bn_gpu, self.output_gpu, self.output_residual_gpu):
             if b is not None:
                 b.free()

@@ -148,3 +148,15 @@ def test_mnist_mlp_driver_on_a_dataset_file(gpu, tmp_path):
     assert lines[i + 1].split() == [str(v) for v in pos]
     pct = lambda n: float(np.float32(n) / np.float32(batch) * np.float32(100))  # the reference prints float32
     assert lines[i + 3] == "Top-1:%f%%" % pct(top1) and lines[i + 4] == "Top-5:%f%%" % pct(top5)
+
+
+@pytest.mark.parametrize("variant", ["popc", "mfma_f4"])
+def test_reference_layout_accessors_of_the_cpp_classes(gpu, tmp_path, variant):
+    """drivers/reference_fmt_interop.cpp: the same small residual network with engine-layout and with
+    reference-layout buffers between the C++ layer objects; the binary compares the two itself."""
+    exe = os.path.join(BIN, "reference_fmt_interop")
+    assert os.path.exists(exe), "%s is not built (run __graft_entry__.build())" % exe
+    proc = subprocess.run([exe, "--batch", "12", "--seed", "3", "--variant", variant], stdout=subprocess.PIPE,
+                          stderr=subprocess.STDOUT, text=True, timeout=120)
+    assert proc.returncode == 0, proc.stdout
+    assert '"ok": true' in proc.stdout and '"c2_residual_nonzero": 0,' not in proc.stdout

@@ -436,6 +436,111 @@ def test_inconv128_presigned_input_is_exact_integer_conv(gpu):
 
 
 # --------------------------------------------------------------------------- whole networks
+@pytest.mark.parametrize("fmt", [0, 1])
+@pytest.mark.parametrize("h,b,c", [(5, 9, 64), (3, 70, 35), (2, 8, 130)])
+def test_residual_from_reference(gpu, h, b, c, fmt):
+    """Reference layout int32 [P][Q][PAD8(B)][PAD128(C)] -> engine layouts: against a host transpose, and back
+    through the existing converter (whose oracle twin is pinned on the CPU)."""
+    from tcbnn_amd import _lib
+    from tcbnn_amd.device import DeviceBuffer
+    r = rng(h * 100 + b + c + fmt)
+    res = r.integers(-30000, 30000, size=(h, h, b, c)).astype(np.int32)
+    ref_host = orc.residual_to_reference(res)
+    ref_host[:, :, b:, :] = 0x5A5A5A5A  # padding images / channels of a foreign buffer hold anything
+    ref_host[:, :, :, c:] = 0x5A5A5A5A
+    ref = gpuops.dev(ref_host)
+    own = DeviceBuffer(_lib.lib.tcbnn_residual_bytes(h, h, c, b, fmt))
+    own.fill(0xCD)
+    gpuops.check(_lib.lib.tcbnn_residual_from_reference(ref.ptr, own.ptr, h, h, b, c, fmt, None))
+    gpuops.sync()
+    want = _residual_source(res, fmt)  # the engine layout by host transpose, channels past c zero
+    grp, dt = (8, np.int16) if fmt == 1 else (4, np.int32)
+    shape = (h, h, (c + grp - 1) // grp, b, grp)
+    np.testing.assert_array_equal(own.to_numpy(dt, shape), want.to_numpy(dt, shape))
+    back = DeviceBuffer(ref_host.nbytes)
+    gpuops.check(_lib.lib.tcbnn_residual_to_reference(own.ptr, back.ptr, h, h, b, c, fmt, None))
+    gpuops.sync()
+    np.testing.assert_array_equal(back.to_numpy(np.int32, ref_host.shape), orc.residual_to_reference(res))
+
+
+@pytest.mark.parametrize("variant", ["popc", "mfma_f4"])
+def test_reference_layout_between_layers(gpu, variant):
+    """Every hand-over through device buffers in the reference's tile layouts (as if each neighbour were a layer
+    of the reference): stem (saves a residual) -> conv (injects it, saves its own) -> stride-2 conv -> FC-ready
+    conv (injects through the 2x2 max) -> FC -> output, against the oracle run on the plain tensors."""
+    r = rng(77)
+    b, h, ch, hid, classes = 12, 8, 64, 256, 10
+    v = _variant(gpu, variant)
+    x = r.standard_normal((b, 3, h, h)).astype(np.float32)
+    f0, f1, f2 = rm.pm1(r, (3, 3, 3, ch)), rm.pm1(r, (3, 3, ch, ch)), rm.pm1(r, (3, 3, ch, 2 * ch))
+    f3 = rm.pm1(r, (3, 3, 2 * ch, 2 * ch))
+    bn0 = r.normal(0, 5, ch).astype(np.float32)
+    bn1, bn2 = r.normal(0, 24, ch).astype(np.float32), r.normal(0, 24, 2 * ch).astype(np.float32)
+    bn3 = r.normal(0, 34, 2 * ch).astype(np.float32)
+    feats = (h // 2) * (h // 2) * 2 * ch
+    wfc, bnfc = rm.pm1(r, (feats, hid)), r.normal(0, 30, hid).astype(np.float32)
+    wout, sc, bi = rm.pm1(r, (hid, classes)), r.normal(1, 0.1, classes).astype(np.float32), \
+        r.normal(0, 1, classes).astype(np.float32)
+
+    # oracle on plain tensors
+    o0, r0 = orc.inconv128(x, f0, bn0, 1, True, 1, True)
+    o1, r1 = orc.conv128(o0, orc.pack_conv_filter(f1), bn1, ch, ch, 3, 3, save_residual=True, inject_residual=True,
+                         residual_channels=ch, res_in=r0)
+    o2, _ = orc.conv128(o1, orc.pack_conv_filter(f2), bn2, ch, 2 * ch, 3, 3, stride=2)
+    o3, _ = orc.conv128(o2, orc.pack_conv_filter(f3), bn3, 2 * ch, 2 * ch, 3, 3, ahead_fc=True, inject_residual=True,
+                        residual_channels=ch, residual_pool=True, res_in=r1)
+    o4 = orc.fc128(o3, orc.pack_fc_weight(wfc), bnfc, feats, hid)
+    want = orc.out128(o4, orc.pack_fc_weight(wout), sc, bi, hid, classes)
+
+    stem = gpu.InConv128LayerParam("Conv1", h, h, 3, 3, 3, ch, b, 1, 1, True, 1, 1, True)
+    stem.initialize(x, gpu.ArrayWeights([f0, bn0]))
+    stem.forward()
+    t0, q0 = stem.get_output_gpu_reference_fmt(), stem.get_output_residual_gpu_reference()
+    c1 = gpu.Conv128LayerParam("C1", h, h, 3, 3, ch, ch, b, 1, 1, True, 1, 1, False, True, True, ch, variant=v)
+    c1.initialize(gpu.ArrayWeights([f1, bn1]), t0, q0)
+    c1.set_input_gpu_reference_fmt(t0)
+    c1.set_input_residual_gpu_reference(q0)
+    c1.forward()
+    t1, q1 = c1.get_output_gpu_reference_fmt(), c1.get_output_residual_gpu_reference()
+    c2 = gpu.Conv128LayerParam("C2", h, h, 3, 3, ch, 2 * ch, b, 2, 2, variant=v)
+    c2.initialize(gpu.ArrayWeights([f2, bn2]), t1)
+    c2.set_input_gpu_reference_fmt(t1)
+    c2.forward()
+    t2 = c2.get_output_gpu_reference_fmt()
+    c3 = gpu.Conv128LayerParam("C3", h // 2, h // 2, 3, 3, 2 * ch, 2 * ch, b, 1, 1, True, 1, 1, True, False, True, ch,
+                               True, variant=v)
+    c3.initialize(gpu.ArrayWeights([f3, bn3]), t2, q1)
+    c3.set_input_gpu_reference_fmt(t2)
+    c3.set_input_residual_gpu_reference(q1)
+    c3.forward()
+    t3 = c3.get_output_gpu_reference_fmt()
+    fc = gpu.Fc128LayerParam("Fc1", b, feats, hid, variant=v)
+    fc.initialize(gpu.ArrayWeights([wfc, bnfc]), t3)
+    fc.set_input_gpu_reference_fmt(t3)
+    fc.forward()
+    t4 = fc.get_output_gpu_reference_fmt()
+    out = gpu.Out128LayerParam("Fout", b, hid, classes, variant=v)
+    out.initialize(gpu.ArrayWeights([wout, sc, bi]), t4)
+    out.set_input_gpu_reference_fmt(t4)
+    out.forward()
+    gpuops.sync()
+
+    words = lambda buf: buf.to_numpy(np.uint32, (buf.nbytes // 4,))
+    np.testing.assert_array_equal(words(t0), orc.conv_to_fmt(o0, ch))
+    np.testing.assert_array_equal(q0.to_numpy(np.int32, (h, h, orc.pad8(b), orc.pad128(ch))),
+                                  orc.residual_to_reference(r0))
+    np.testing.assert_array_equal(words(t1), orc.conv_to_fmt(o1, ch))
+    np.testing.assert_array_equal(q1.to_numpy(np.int32, (h, h, orc.pad8(b), orc.pad128(ch))),
+                                  orc.residual_to_reference(r1))
+    np.testing.assert_array_equal(words(t2), orc.conv_to_fmt(o2, 2 * ch))
+    np.testing.assert_array_equal(words(t3), orc.fc_to_fmt(o3, b, feats))
+    np.testing.assert_array_equal(words(t4), orc.fc_to_fmt(o4, b, hid))
+    got = out.download_output()
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=0)  # fp32 logits: 1e-5 relative
+    for layer in (stem, c1, c2, c3, fc, out):
+        layer.release()
+
+
 def _compare_network(gpu, spec, seed, variant, residual_format=None):
     weights = gpu.synthetic_weights(spec, seed)
     x = gpu.synthetic_input(spec, seed)
