@@ -122,17 +122,19 @@ typedef uint32_t u16v __attribute__((ext_vector_type(16)));
 typedef int v4i_t __attribute__((ext_vector_type(4)));
 
 // Staging of one filter row: the 3 x 64 (channel, image) row segments of ncols floats each.
-//   ROWS = true (ncols <= 21): a wave takes rpw (a multiple of 3) segments at a time, lanes
+//   ROWS = true: a wave takes rpw segments at a time (a multiple of 3 for ncols <= 21, else 2), lanes
 //     running along the segment; segments are numbered in memory order (image * 3 + channel),
 //     so that the address of pass k is a wave-uniform base plus a per-lane constant and the
-//     LDS slot a constant plus an immediate: no per-element address arithmetic.  NST = passes =
-//     ceil(192 / (4 rpw)).
-//   ROWS = false: the elements are dealt to the threads linearly, NST = ceil(3 * 64 * ncols / 256).
+//     LDS slot a per-lane constant plus an immediate: no per-element address arithmetic.  NST =
+//     passes = ceil(192 / (4 rpw)).  With rpw = 2 (NST = 24) the channel of a lane's segment
+//     changes from pass to pass with period 3, so the LDS slot has three per-lane constants.
+//   ROWS = false: the elements are dealt to the threads linearly, NST = ceil(3 * 64 * ncols / 256)
+//     (only for images too large for 32-bit buffer offsets).
 // POOLED: blockIdx selects a row of the POOLED output; the workgroup runs the pool_h convolution rows
 // of it one after the other and ORs their words (kernel.cuh:646-664); with pool_w = 2 the two columns of
 // a wave are one window.  pool_w is 1 or 2 (the host checks), no residual is saved.
 template <int NST, bool ROWS, bool POOLED>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS ? 4 : 3))) void inconv_tiled_kernel(
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS && NST <= 16 ? 4 : 3))) void inconv_tiled_kernel(
     const InConvParams p, const float* __restrict__ in, const uint4* __restrict__ masks,
     const float* __restrict__ bn, uint32_t* __restrict__ out, int32_t* __restrict__ res, int b_tiles,
     int x_groups, int y_phases, int div_magic, int rpw) {
@@ -209,6 +211,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS ?
         const unsigned tile_bytes = imgs_here * 3u * (unsigned)plane * 4u;  // host checked: below 2 GiB
         const unsigned voff = lane_ok ? ((unsigned)seg0 * (unsigned)plane + (unsigned)sax) * 4u : kOutOfRange;
         const int lds0 = (scol * 3 + seg0 % 3) * kLB + seg0 / 3;  // LDS: [column][channel][image]
+        // rp not a multiple of 3 (NST = 24): pass k = 3m + i holds segment seg0 + rp i + 3 rp m, i.e. the channel
+        // and image of segment seg0 + rp i, rp m images further on
+        constexpr bool kThirds = ROWS && NST == 24;
+        const int lds1 = (scol * 3 + (seg0 + rp) % 3) * kLB + (seg0 + rp) / 3;
+        const int lds2 = (scol * 3 + (seg0 + 2 * rp) % 3) * kLB + (seg0 + 2 * rp) / 3;
         // every pass of every lane inside the 192 segments and the batch (wave-uniform)?
         const bool all_in = NST * rp == 3 * 64 && b0 + 64 <= p.B;
         __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
@@ -253,7 +260,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS ?
                 if (sub < rpw) {
 #pragma unroll
                     for (int k = 0; k < NST; ++k)
-                        if (all_in || seg0 + k * rp < 3 * 64) tile[lds0 + k * (rp / 3)] = stg[k];
+                        if (all_in || seg0 + k * rp < 3 * 64) {
+                            if constexpr (kThirds)
+                                tile[(k % 3 == 0 ? lds0 : (k % 3 == 1 ? lds1 : lds2)) + (k / 3) * rp] = stg[k];
+                            else
+                                tile[lds0 + k * (rp / 3)] = stg[k];
+                        }
                 }
             } else {
 #pragma unroll
@@ -483,11 +495,11 @@ static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name
             return TCBNN_OK;
         }
         const int ncols = (kXT - 1) * p.stride_w + p.S;
-        const int rpw = (64 / ncols) / 3 * 3;
-        if (rpw >= 3 && 64LL * 3 * p.H * p.W * 4 < (1LL << 31)) {
+        const int rpw = 64 / ncols >= 3 ? (64 / ncols) / 3 * 3 : 2;
+        if (64LL * 3 * p.H * p.W * 4 < (1LL << 31)) {
             const int passes = (3 * 64 + 4 * rpw - 1) / (4 * rpw);
-            snprintf(name_buf, name_len, "inconv_tiled_kernel<%d, true, %s>", passes <= 4 ? 4 : (passes <= 8 ? 8 : 16),
-                     pooled ? "true" : "false");
+            snprintf(name_buf, name_len, "inconv_tiled_kernel<%d, true, %s>",
+                     passes <= 4 ? 4 : (passes <= 8 ? 8 : (passes <= 16 ? 16 : 24)), pooled ? "true" : "false");
         } else {
             snprintf(name_buf, name_len, "inconv_tiled_kernel<%d, false, %s>",
                      (3 * 64 * ncols + kThreads - 1) / kThreads <= 15 ? 15 : 24, pooled ? "true" : "false");
@@ -510,8 +522,9 @@ static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name
                                      ? 8LL * ((x_groups + y_phases - 1) / y_phases) * rows_out
                                      : (long long)b_tiles * x_groups * rows_out;
         TCBNN_REQUIRE(blocks <= 0x7fffffffLL, "inconv128: grid too large");
-        // staging scheme (see the kernel): whole segments per wave when at least 3 fit its 64 lanes
-        const int rpw = (64 / ncols) / 3 * 3;
+        // staging scheme (see the kernel): whole segments per wave, a multiple of 3 of them when 3 fit its 64
+        // lanes, else 2 (ncols <= kMaxCols = 32)
+        const int rpw = 64 / ncols >= 3 ? (64 / ncols) / 3 * 3 : 2;
         auto launch = [&](auto kernel) {
             hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(kThreads), 0, (hipStream_t)stream, p, p.in,
                                p.masks, p.bn, p.out, p.res, b_tiles, x_groups, y_phases, div_magic, rpw);
@@ -524,14 +537,16 @@ static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name
             else
                 launch(inconv_tiled_kernel<NST, ROWS, false>);
         };
-        if (rpw >= 3 && 64LL * 3 * p.H * p.W * 4 < (1LL << 31)) {
+        if (64LL * 3 * p.H * p.W * 4 < (1LL << 31)) {
             const int passes = (3 * 64 + 4 * rpw - 1) / (4 * rpw);
             if (passes <= 4)
                 launch_nst(std::integral_constant<int, 4>{}, std::true_type{});
             else if (passes <= 8)
                 launch_nst(std::integral_constant<int, 8>{}, std::true_type{});
-            else
+            else if (passes <= 16)
                 launch_nst(std::integral_constant<int, 16>{}, std::true_type{});
+            else
+                launch_nst(std::integral_constant<int, 24>{}, std::true_type{});
         } else {
             const int nst = (3 * 64 * ncols + kThreads - 1) / kThreads;
             if (nst <= 15)
