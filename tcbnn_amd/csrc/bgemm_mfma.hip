@@ -40,8 +40,10 @@ constexpr int kThreads = 64 * kWaves;
 constexpr int kNT = 2;    // 32-channel tiles per wave
 constexpr int kQB = 24;   // k-steps of weights staged in LDS at a time (24 * kNT KiB)
 
+// Without an occupancy target the compiler schedules the unrolled epilogue across up to 512 registers (one wave
+// per SIMD); most launches of this kernel are many short workgroups, which need several resident at a time.
 template <int FMT, int MT, int MM>
-__global__ __launch_bounds__(kThreads) void bgemm_mfma_kernel(
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(MT == 4 || MM == MM_THRESH_RES ? 2 : 3))) void bgemm_mfma_kernel(
     const BgemmParams p, const uint32_t* __restrict__ act, const uint32_t* __restrict__ wgt,
     const float* __restrict__ bnp, const int32_t* __restrict__ rin, int n_groups, int row_waves,
     int b_groups, int row_blocks) {
@@ -189,32 +191,75 @@ __global__ __launch_bounds__(kThreads) void bgemm_mfma_kernel(
         // ---------------- epilogue for pre-pool pixel (y, x) ----------------
         const size_t pix = (size_t)y * p.PW + x;
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-            const int b = bimg[mt];
-            const bool b_ok = b < p.B;
-            const int bb = bload[mt];
+        for (int nt = 0; nt < kNT; ++nt) {
+            const int cbase = n0 + nt * 32 + 16 * h;  // this lane's channels: cbase + v
+            // the lane's 16 thresholds, requested together and shared by its image tiles (a load per use, each
+            // under its own bounds test, was a chain of 16 * MT * kNT memory round trips)
+            float thr[16];
+            if constexpr (MM == MM_THRESH || MM == MM_THRESH_RES) {
 #pragma unroll
-            for (int nt = 0; nt < kNT; ++nt) {
-                const int cbase = n0 + nt * 32 + 16 * h;  // this lane's channels: cbase + v
+                for (int v = 0; v < 16; ++v) thr[v] = bnp[min(cbase + v, p.N - 1)];
+            }
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const int b = bimg[mt];
+                const bool b_ok = b < p.B;
+                const int bb = bload[mt];
                 if constexpr (MM == MM_THRESH || MM == MM_THRESH_RES) {
                     int rv[16];
                     if constexpr (MM == MM_THRESH_RES) {
 #pragma unroll
-                        for (int v = 0; v < 16; ++v) {
-                            const int c = cbase + v;
-                            int val = 0;
-                            if (rin != nullptr && c < p.res_limit && c < p.res_in_ch && c < p.N) {
-                                if (p.res_pool) {
-                                    const size_t rw2 = 2 * (size_t)p.PW, p00 = (size_t)(2 * y) * rw2 + 2 * x;
-                                    auto at = [&](size_t sp) {
-                                        return residual_load(rin, p.res_in_fmt, sp, p.res_in_ch, c, p.B, bb);
-                                    };
-                                    val = max(max(at(p00), at(p00 + 1)), max(at(p00 + rw2), at(p00 + rw2 + 1)));
+                        for (int v = 0; v < 16; ++v) rv[v] = 0;
+                        if (rin != nullptr && cbase < p.res_in_ch) {  // wave-uniform but for the channel half
+                            // the lane's 16 channels are whole 16-byte groups of the source: 128-bit loads
+                            const bool r16 = p.res_in_fmt == TCBNN_RES_I16;
+                            const size_t ngrp = r16 ? (p.res_in_ch + 7) / 8 : (p.res_in_ch + 3) / 4;
+                            const int4* __restrict__ src = reinterpret_cast<const int4*>(rin);
+                            auto fetch = [&](size_t sp, int* dst) {
+                                if (r16) {
+                                    const size_t g0 = (sp * ngrp + cbase / 8) * p.B + bb;
+#pragma unroll
+                                    for (int g = 0; g < 2; ++g) {
+                                        int4 q = make_int4(0, 0, 0, 0);
+                                        if (cbase + 8 * g < p.res_in_ch) q = src[g0 + (size_t)g * p.B];
+                                        const int w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+                                        for (int e = 0; e < 4; ++e) {
+                                            dst[8 * g + 2 * e] = (w[e] << 16) >> 16;
+                                            dst[8 * g + 2 * e + 1] = w[e] >> 16;
+                                        }
+                                    }
                                 } else {
-                                    val = residual_load(rin, p.res_in_fmt, pix, p.res_in_ch, c, p.B, bb);
+                                    const size_t g0 = (sp * ngrp + cbase / 4) * p.B + bb;
+#pragma unroll
+                                    for (int g = 0; g < 4; ++g) {
+                                        int4 q = make_int4(0, 0, 0, 0);
+                                        if (cbase + 4 * g < p.res_in_ch) q = src[g0 + (size_t)g * p.B];
+                                        dst[4 * g] = q.x;
+                                        dst[4 * g + 1] = q.y;
+                                        dst[4 * g + 2] = q.z;
+                                        dst[4 * g + 3] = q.w;
+                                    }
                                 }
+                            };
+                            if (p.res_pool) {
+                                const size_t rw2 = 2 * (size_t)p.PW, p00 = (size_t)(2 * y) * rw2 + 2 * x;
+                                fetch(p00, rv);
+                                const size_t others[3] = {p00 + 1, p00 + rw2, p00 + rw2 + 1};
+                                for (int k = 0; k < 3; ++k) {
+                                    int t[16];
+                                    fetch(others[k], t);
+#pragma unroll
+                                    for (int v = 0; v < 16; ++v) rv[v] = max(rv[v], t[v]);
+                                }
+                            } else {
+                                fetch(pix, rv);
                             }
-                            rv[v] = val;
+#pragma unroll
+                            for (int v = 0; v < 16; ++v) {
+                                const int c = cbase + v;
+                                if (!(c < p.res_limit && c < p.res_in_ch && c < p.N)) rv[v] = 0;
+                            }
                         }
                     }
                     int32_t* __restrict__ rout = p.res_out;
@@ -227,7 +272,7 @@ __global__ __launch_bounds__(kThreads) void bgemm_mfma_kernel(
                         uint32_t bit = 0;
                         if (c < p.N) {
                             if constexpr (MM == MM_THRESH_RES) res += rv[v];
-                            bit = thresh_bit(res, bnp[c], p.nan_bit);
+                            bit = thresh_bit(res, thr[v], p.nan_bit);
                         }
                         resv[v] = c < p.N ? res : 0;  // channels past N are stored as 0 inside a group
                         hw = (hw << 1) | bit;
@@ -258,6 +303,8 @@ __global__ __launch_bounds__(kThreads) void bgemm_mfma_kernel(
                     }
                     const uint32_t other = (uint32_t)__shfl_xor((int)hw, 32);
                     outword[mt][nt] |= h == 0 ? (hw << 16) | other : (other << 16) | hw;
+                    // one tile's epilogue at a time: interleaving them multiplies the live temporaries
+                    __builtin_amdgcn_sched_barrier(0);
                 } else {
                     if (!b_ok) continue;
                     if (p.ksplit > 1) {  // partial dot products; the finishing kernel does the rest
@@ -317,7 +364,9 @@ __global__ __launch_bounds__(kThreads) void bgemm_mfma_kernel(
 int images_per_wave_tiles(const BgemmParams& p) {
     const long long pix = (long long)p.OH * p.OW;
     const int n_groups = (p.N + 32 * kNT - 1) / (32 * kNT);
-    for (int mt = 4; mt > 1; mt >>= 1) {
+    // the residual epilogue does not fit 256 registers next to the accumulators of four image tiles
+    const int mt_max = (p.res_in != nullptr || p.res_out != nullptr) ? 2 : 4;
+    for (int mt = mt_max; mt > 1; mt >>= 1) {
         if (p.B <= 32 * (mt / 2)) continue;
         const long long waves = pix * ((p.B + 32 * mt - 1) / (32 * mt)) * n_groups * p.ksplit;
         if (waves >= 2048) return mt;
