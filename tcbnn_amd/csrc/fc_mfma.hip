@@ -123,14 +123,22 @@ __global__ __launch_bounds__(64 * kMaxWaves) void fc_mfma_f4_kernel(
         for (int v = 0; v < 16; ++v) dot[v] = red[v * 64 + lane];
     }
 
-    // ---- epilogue: the lane holds neurons n0 + 16h + v of image b
+    // ---- epilogue (wave 0): the lane holds neurons cbase + v of image b.  Its 16 thresholds (or scales and
+    // biases) are requested together, without bounds tests around the loads (neurons past N read the last valid
+    // entry and are discarded): a load under each test would be a chain of memory round trips.
     const int cbase = n0 + 16 * h;
+    float thr[16], bia[MODE == FC_AFFINE ? 16 : 1];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+        thr[v] = bnp[min(cbase + v, p.N - 1)];
+        if constexpr (MODE == FC_AFFINE) bia[v] = bias[min(cbase + v, p.N - 1)];
+    }
     if constexpr (MODE == FC_THRESH) {
         uint32_t hw = 0;
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const int c = cbase + v;
-            const uint32_t bit = c < p.N ? thresh_bit(dot[v], bnp[min(c, p.N - 1)], p.nan_bit) : 0u;
+            const uint32_t bit = c < p.N ? thresh_bit(dot[v], thr[v], p.nan_bit) : 0u;
             hw = hw + hw + bit;
         }
         const uint32_t other = (uint32_t)__shfl_xor((int)hw, 32);
@@ -145,7 +153,7 @@ __global__ __launch_bounds__(64 * kMaxWaves) void fc_mfma_f4_kernel(
             for (int v = 0; v < 16; ++v) {
                 const int c = cbase + v;
                 // the +-1 dot product equals (float)K - (float)popc*2.0f exactly (kernel.cuh:258-270)
-                if (c < p.N) p.out_f32[(size_t)b * p.N + c] = __fadd_rn(__fmul_rn((float)dot[v], bnp[c]), bias[c]);
+                if (c < p.N) p.out_f32[(size_t)b * p.N + c] = __fadd_rn(__fmul_rn((float)dot[v], thr[v]), bia[v]);
             }
         }
     }
