@@ -90,20 +90,28 @@ __global__ __launch_bounds__(kThreads) void avgpool_fc_kernel(const HeadParams p
         const int g = u / kHeadImages, i = u % kHeadImages;  // image fastest: 128-byte runs
         const int bb = min(b0 + i, p.B - 1);
         int sum[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-        for (int pix = 0; pix < p.P; ++pix) {
-            const int4 v = src[((size_t)pix * p.groups + g) * p.B + bb];
-            if (p.fmt == TCBNN_RES_I16) {
-                const int wv[4] = {v.x, v.y, v.z, v.w};
+        // eight pixels requested at a time (a load per loop pass waits for each one in turn); integer sums, so
+        // the order does not matter
+        for (int pix0 = 0; pix0 < p.P; pix0 += 8) {
+            int4 v[8];
 #pragma unroll
-                for (int k = 0; k < 4; ++k) {
-                    sum[2 * k] += (int)(short)(wv[k] & 0xffff);
-                    sum[2 * k + 1] += wv[k] >> 16;
+            for (int q = 0; q < 8; ++q) v[q] = src[((size_t)min(pix0 + q, p.P - 1) * p.groups + g) * p.B + bb];
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                if (pix0 + q >= p.P) continue;
+                if (p.fmt == TCBNN_RES_I16) {
+                    const int wv[4] = {v[q].x, v[q].y, v[q].z, v[q].w};
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        sum[2 * k] += (int)(short)(wv[k] & 0xffff);
+                        sum[2 * k + 1] += wv[k] >> 16;
+                    }
+                } else {
+                    sum[0] += v[q].x;
+                    sum[1] += v[q].y;
+                    sum[2] += v[q].z;
+                    sum[3] += v[q].w;
                 }
-            } else {
-                sum[0] += v.x;
-                sum[1] += v.y;
-                sum[2] += v.z;
-                sum[3] += v.w;
             }
         }
         for (int k = 0; k < p.per_group; ++k) {
@@ -117,18 +125,32 @@ __global__ __launch_bounds__(kThreads) void avgpool_fc_kernel(const HeadParams p
     float acc[kHeadImages];
 #pragma unroll
     for (int i = 0; i < kHeadImages; ++i) acc[i] = 0.0f;
-    for (int c = 0; c < p.C; ++c) {
-        const float wv = p.w[(size_t)c * p.N + n];
-        const float4 m0 = *reinterpret_cast<const float4*>(&mean[c][0]);
-        const float4 m1 = *reinterpret_cast<const float4*>(&mean[c][4]);
-        acc[0] = __fmaf_rn(m0.x, wv, acc[0]);
-        acc[1] = __fmaf_rn(m0.y, wv, acc[1]);
-        acc[2] = __fmaf_rn(m0.z, wv, acc[2]);
-        acc[3] = __fmaf_rn(m0.w, wv, acc[3]);
-        acc[4] = __fmaf_rn(m1.x, wv, acc[4]);
-        acc[5] = __fmaf_rn(m1.y, wv, acc[5]);
-        acc[6] = __fmaf_rn(m1.z, wv, acc[6]);
-        acc[7] = __fmaf_rn(m1.w, wv, acc[7]);
+    // weights of the next 16 channels are requested while the current 16 are used; the additions stay in ascending
+    // channel order
+    float wn[16];
+#pragma unroll
+    for (int q = 0; q < 16; ++q) wn[q] = p.w[(size_t)min(q, p.C - 1) * p.N + n];
+    for (int c0 = 0; c0 < p.C; c0 += 16) {
+        float wv[16];
+#pragma unroll
+        for (int q = 0; q < 16; ++q) wv[q] = wn[q];
+#pragma unroll
+        for (int q = 0; q < 16; ++q) wn[q] = p.w[(size_t)min(c0 + 16 + q, p.C - 1) * p.N + n];
+#pragma unroll
+        for (int q = 0; q < 16; ++q) {
+            const int c = min(c0 + q, p.C - 1);
+            const bool on = c0 + q < p.C;  // a channel past C leaves the sums as they are
+            const float4 m0 = *reinterpret_cast<const float4*>(&mean[c][0]);
+            const float4 m1 = *reinterpret_cast<const float4*>(&mean[c][4]);
+            acc[0] = on ? __fmaf_rn(m0.x, wv[q], acc[0]) : acc[0];
+            acc[1] = on ? __fmaf_rn(m0.y, wv[q], acc[1]) : acc[1];
+            acc[2] = on ? __fmaf_rn(m0.z, wv[q], acc[2]) : acc[2];
+            acc[3] = on ? __fmaf_rn(m0.w, wv[q], acc[3]) : acc[3];
+            acc[4] = on ? __fmaf_rn(m1.x, wv[q], acc[4]) : acc[4];
+            acc[5] = on ? __fmaf_rn(m1.y, wv[q], acc[5]) : acc[5];
+            acc[6] = on ? __fmaf_rn(m1.z, wv[q], acc[6]) : acc[6];
+            acc[7] = on ? __fmaf_rn(m1.w, wv[q], acc[7]) : acc[7];
+        }
     }
     const float bias = p.bias[n];
 #pragma unroll
