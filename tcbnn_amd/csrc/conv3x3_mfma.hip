@@ -92,49 +92,9 @@ conv3x3_mfma_f4_kernel(
     const int n0 = ng * (32 * NT);
     const int kw_tot = 9 * p.cw;
 
-    // ---- stage this channel group's weight fragments (already expanded when the filter was packed)
-    // and thresholds
-    {
-        const v4i* __restrict__ frag = reinterpret_cast<const v4i*>(wgt + (size_t)((p.N + 31) / 32) * 32 * kw_tot);
-        // all requests of a batch are in flight together (a loop of load-then-store would pay the
-        // memory latency once per fragment)
-        constexpr int kPerWave = (NQ * NT + kWaves - 1) / kWaves, kBatch = kPerWave < 9 ? kPerWave : 9;
-#pragma unroll
-        for (int i0 = 0; i0 < kPerWave; i0 += kBatch) {
-            v4i tmp[kBatch];
-#pragma unroll
-            for (int i = 0; i < kBatch; ++i) {
-                const int f = wave + (i0 + i) * kWaves;
-                const int q = f / NT, nt = f % NT;
-                tmp[i] = f < NQ * NT ? frag[((size_t)(ng * NT + nt) * NQ + q) * 64 + lane] : v4i{0, 0, 0, 0};
-            }
-#pragma unroll
-            for (int i = 0; i < kBatch; ++i) {
-                const int f = wave + (i0 + i) * kWaves;
-                if (f < NQ * NT) lds_w[f * 64 + lane] = tmp[i];
-            }
-        }
-    }
-    // A NaN threshold always yields bit 1 (!(x < NaN)), exactly like -inf: staged as such, so that
-    // the epilogue can take the bit from the sign of x - threshold.
-    // Without a residual the sum s is an integer with |s| <= 9 Cin <= 4608, so s < threshold is
-    // the same as s < ceil(threshold), and thresholds beyond +-8192 decide like +-8192.  The
-    // negated integer threshold is then what the accumulator STARTS from (operand C of the tile's
-    // first MFMA): the finished accumulator is s - ceil(threshold), exact in fp32, and its sign is
-    // the inverted output bit, with no per-value subtraction in the epilogue.
-    if (tid < NT * 32) {
-        float t = RM != RM_RAW && n0 + tid < p.N ? bnp[n0 + tid] : 0.0f;
-        t = t != t ? -__builtin_huge_valf() : t;
-        if constexpr (RM == RM_NONE) t = 0.0f - fminf(fmaxf(ceilf(t), -8192.0f), 8192.0f);
-        lds_thr[tid] = t;
-    }
-    __syncthreads();
-    // start values of a lane's 16 channels per channel tile (zeros when a residual is added first)
+    // start values of a lane's 16 channels per channel tile (zeros when a residual is added first); filled once
+    // the thresholds are staged
     v16f acc0[NT];
-#pragma unroll
-    for (int nt = 0; nt < NT; ++nt)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) acc0[nt][v] = RM == RM_NONE ? lds_thr[nt * 32 + 16 * h + v] : 0.0f;
 
     // a wave's work items: output pixels, or 2x2 windows of them (row width `roww`)
     const int roww = POOL ? p.OW : p.PW;
@@ -635,10 +595,54 @@ conv3x3_mfma_f4_kernel(
         advance(lc);
     }
     if constexpr (kAhead) {
-        if (cc.pi < npix) {
-            request_residual(cc.y, cc.x, rv[0]);
-            if constexpr (RM == RM_POOLED) finish_residual(rv[0]);
+        if (cc.pi < npix) request_residual(cc.y, cc.x, rv[0]);
+    }
+
+    // The first activation (and residual) requests are on their way: their latency now runs while the weights
+    // are staged.
+    // ---- stage this channel group's weight fragments (already expanded when the filter was packed)
+    // and thresholds
+    {
+        const v4i* __restrict__ frag = reinterpret_cast<const v4i*>(wgt + (size_t)((p.N + 31) / 32) * 32 * kw_tot);
+        // all requests of a batch are in flight together (a loop of load-then-store would pay the
+        // memory latency once per fragment)
+        constexpr int kPerWave = (NQ * NT + kWaves - 1) / kWaves, kBatch = kPerWave < 9 ? kPerWave : 9;
+#pragma unroll
+        for (int i0 = 0; i0 < kPerWave; i0 += kBatch) {
+            v4i tmp[kBatch];
+#pragma unroll
+            for (int i = 0; i < kBatch; ++i) {
+                const int f = wave + (i0 + i) * kWaves;
+                const int q = f / NT, nt = f % NT;
+                tmp[i] = f < NQ * NT ? frag[((size_t)(ng * NT + nt) * NQ + q) * 64 + lane] : v4i{0, 0, 0, 0};
+            }
+#pragma unroll
+            for (int i = 0; i < kBatch; ++i) {
+                const int f = wave + (i0 + i) * kWaves;
+                if (f < NQ * NT) lds_w[f * 64 + lane] = tmp[i];
+            }
         }
+    }
+    // A NaN threshold always yields bit 1 (!(x < NaN)), exactly like -inf: staged as such, so that
+    // the epilogue can take the bit from the sign of x - threshold.
+    // Without a residual the sum s is an integer with |s| <= 9 Cin <= 4608, so s < threshold is
+    // the same as s < ceil(threshold), and thresholds beyond +-8192 decide like +-8192.  The
+    // negated integer threshold is then what the accumulator STARTS from (operand C of the tile's
+    // first MFMA): the finished accumulator is s - ceil(threshold), exact in fp32, and its sign is
+    // the inverted output bit, with no per-value subtraction in the epilogue.
+    if (tid < NT * 32) {
+        float t = RM != RM_RAW && n0 + tid < p.N ? bnp[n0 + tid] : 0.0f;
+        t = t != t ? -__builtin_huge_valf() : t;
+        if constexpr (RM == RM_NONE) t = 0.0f - fminf(fmaxf(ceilf(t), -8192.0f), 8192.0f);
+        lds_thr[tid] = t;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc0[nt][v] = RM == RM_NONE ? lds_thr[nt * 32 + 16 * h + v] : 0.0f;
+    if constexpr (kAhead && RM == RM_POOLED) {
+        if (cc.pi < npix) finish_residual(rv[0]);
     }
 
     // one step with compile-time buffer indices: multiply buffer I, request into buffer (I + LOOK) % NB
