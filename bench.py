@@ -120,6 +120,14 @@ def roofline_of(name, g, variant):
         "ops_per_byte": round(intensity, 1) if g["bytes"] else None,
         "binary_tops": round(tops, 2), "hbm_gbs": round(gbs, 1),
     }
+    if g.get("flops"):
+        # The fp32 first layer is far from the HBM roof because its additions bind it: one dependent fp32 add per
+        # (tap, output channel, pixel, image) is the least the reference's summation order allows (its 2 flops per
+        # input value and tap are 6 per such add).  Peak: the published 157.3 TFLOP/s counts packed FMAs; plain adds
+        # issue at a quarter of that (64 lanes per CU and clock).
+        adds = g["flops"] / 6.0
+        rec["valu_fp32"] = {"adds_per_launch": round(adds / g["launches"]), "achieved": round(adds / secs / 1e12, 2),
+                            "peak": round(157.3 / 4, 1), "unit": "Tadd/s", "frac": round(adds / secs / 1e12 / (157.3 / 4), 4)}
     return rec
 
 
@@ -275,8 +283,9 @@ def main():
         name = layer.kernel_name() if hasattr(layer, "kernel_name") else \
             {"in": "in128_kernel"}[L["kind"]]
         w = layer_work(L, spec, res_bytes)
-        g = groups.setdefault(name, dict(bops=0.0, bytes=0.0, ms=0.0, launches=0))
+        g = groups.setdefault(name, dict(bops=0.0, flops=0.0, bytes=0.0, ms=0.0, launches=0))
         g["bops"] += w["bops"]
+        g["flops"] += w["flops"]
         g["bytes"] += w["bytes"]
         g["ms"] += layer_ms[L["name"]]
         g["launches"] += 1
