@@ -18,6 +18,7 @@
 //     contiguous 256-byte runs of the batch-innermost output layouts.
 //   inconv_generic_kernel (any pooling): one lane per pooled output pixel.
 #include <stdlib.h>
+#include <string.h>
 
 #include <type_traits>
 
@@ -489,6 +490,11 @@ static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name
     const bool pooled = p.pool_h != 1 || p.pool_w != 1;
     const bool tiled = (p.pool_w == 1 || p.pool_w == 2) && (kXT - 1) * p.stride_w + p.S <= kMaxCols;
     const int rows_out = pooled ? p.OH : p.PH;  // rows the workgroups are dealt
+    // Row-wise staging needs 32-bit buffer offsets over a workgroup's 64 images; larger images (above 2.7 M pixels)
+    // take the linear staging, which TCBNN_INCONV_STAGING=linear also selects (so that tests can reach it).
+    static const bool force_linear = getenv("TCBNN_INCONV_STAGING") != nullptr &&
+                                     strcmp(getenv("TCBNN_INCONV_STAGING"), "linear") == 0;
+    const bool row_staging = !force_linear && 64LL * 3 * p.H * p.W * 4 < (1LL << 31);
     if (name_buf != nullptr) {  // report the kernel instead of launching it
         if (!tiled) {
             snprintf(name_buf, name_len, "inconv_generic_kernel");
@@ -496,7 +502,7 @@ static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name
         }
         const int ncols = (kXT - 1) * p.stride_w + p.S;
         const int rpw = 64 / ncols >= 3 ? (64 / ncols) / 3 * 3 : 2;
-        if (64LL * 3 * p.H * p.W * 4 < (1LL << 31)) {
+        if (row_staging) {
             const int passes = (3 * 64 + 4 * rpw - 1) / (4 * rpw);
             snprintf(name_buf, name_len, "inconv_tiled_kernel<%d, true, %s>",
                      passes <= 4 ? 4 : (passes <= 8 ? 8 : (passes <= 16 ? 16 : 24)), pooled ? "true" : "false");
@@ -537,7 +543,7 @@ static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name
             else
                 launch(inconv_tiled_kernel<NST, ROWS, false>);
         };
-        if (64LL * 3 * p.H * p.W * 4 < (1LL << 31)) {
+        if (row_staging) {
             const int passes = (3 * 64 + 4 * rpw - 1) / (4 * rpw);
             if (passes <= 4)
                 launch_nst(std::integral_constant<int, 4>{}, std::true_type{});

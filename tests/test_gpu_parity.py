@@ -376,6 +376,43 @@ def test_inconv128_layer(gpu, b, h, R, stride, cout, pool, save):
     layer.release()
 
 
+_LINEAR_STAGING_CHECK = """
+import numpy as np
+import tcbnn_amd
+from tcbnn_amd import _lib
+from oracle import orc
+_lib.set_device(0)
+r = np.random.default_rng(3)
+for (b, h, R, stride, cout, pool, save) in [(70, 24, 11, 4, 64, 2, False), (9, 20, 7, 4, 40, 1, True), (64, 12, 3, 1, 64, 1, True)]:
+    x = r.standard_normal((b, 3, h, h)).astype(np.float32)
+    f = (r.integers(0, 2, size=(R, R, 3, cout)) * 2 - 1).astype(np.float32)
+    bn = r.normal(0, np.sqrt(3 * R * R), cout).astype(np.float32)
+    want, wres = orc.inconv128(x, f, bn, stride, True, pool, save)
+    layer = tcbnn_amd.InConv128LayerParam("Conv1", h, h, R, R, 3, cout, b, stride, stride, True, pool, pool, save)
+    layer.initialize(x, tcbnn_amd.ArrayWeights([f, bn]))
+    assert ", false, " in layer.kernel_name(), layer.kernel_name()
+    layer.forward()
+    _lib.device_synchronize()
+    assert np.array_equal(layer.download_packed(), want)
+    if save:
+        assert np.array_equal(layer.download_residual(), wres)
+print("linear staging ok")
+"""
+
+
+def test_inconv128_linear_staging(gpu):
+    """The staging scheme for images too large for 32-bit buffer offsets, selected here by its switch (the
+    library reads it once per process, hence the child process)."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, TCBNN_INCONV_STAGING="linear", PYTHONPATH=root)
+    proc = subprocess.run([sys.executable, "-c", _LINEAR_STAGING_CHECK], env=env, cwd=root, stdout=subprocess.PIPE,
+                          stderr=subprocess.STDOUT, text=True, timeout=120)
+    assert proc.returncode == 0 and "linear staging ok" in proc.stdout, proc.stdout
+
+
 def test_inconv128_special_thresholds(gpu):
     """NaN, +-inf and exactly met thresholds in the first layer (kernel.cuh:655: bit = !(acc < bn))."""
     r = rng(321)
