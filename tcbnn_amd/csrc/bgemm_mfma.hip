@@ -38,7 +38,7 @@ using namespace mfma;
 constexpr int kWaves = 4;
 constexpr int kThreads = 64 * kWaves;
 constexpr int kNT = 2;    // 32-channel tiles per wave
-constexpr int kQB = 24;   // k-steps of weights staged in LDS at a time (24 * kNT KiB)
+constexpr int kQB = 24;   // k-steps of weights staged in LDS at a time (24 * kNT KiB); a multiple of 4
 
 // Without an occupancy target the compiler schedules the unrolled epilogue across up to 512 registers (one wave
 // per SIMD); most launches of this kernel are many short workgroups, which need several resident at a time.
@@ -143,46 +143,107 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(MT == 
             return in_frame;
         };
 
-        int tr = (q_begin / steps) / p.S, ts = (q_begin / steps) % p.S, t = q_begin % steps;
-        uint32_t cur[MT], nxt[MT];
-        bool cur_ok = q_begin < q_end ? load_step(tr, ts, t, cur) : false;
-        for (int q0 = q_begin; q0 < q_end; q0 += kQB) {
-            if (!single_block) {
-                __syncthreads();
-                stage_weights(q0);
-                __syncthreads();
+        if constexpr (MM == MM_OTHER) {
+            // Activation words are requested kAhead k-steps before they are multiplied, through a ring of kAhead
+            // register slots (slot d is asked for step q + kAhead as soon as step q has been expanded from it): one
+            // step of 2-8 MFMAs is far shorter than a memory round trip, and with a prefetch distance of one step every
+            // step waited for it.
+            constexpr int kAhead = 4;  // divides kQB
+            int ltr = (q_begin / steps) / p.S, lts = (q_begin / steps) % p.S, lt = q_begin % steps;  // next step to request
+            int lq = q_begin;
+            uint32_t ring[kAhead][MT];
+            bool ring_ok[kAhead];
+            auto request = [&](uint32_t* dst) {
+                bool ok = false;
+                if (lq < q_end) {
+                    ok = load_step(ltr, lts, lt, dst);
+                    ++lq;
+                    if (++lt == steps) {
+                        lt = 0;
+                        if (++lts == p.S) {
+                            lts = 0;
+                            ++ltr;
+                        }
+                    }
+                }
+                return ok;
+            };
+    #pragma unroll
+            for (int d = 0; d < kAhead; ++d) ring_ok[d] = request(ring[d]);
+            for (int q0 = q_begin; q0 < q_end; q0 += kQB) {
+                if (!single_block) {
+                    __syncthreads();
+                    stage_weights(q0);
+                    __syncthreads();
+                }
+                const int cnt = min(kQB, q_end - q0);  // a multiple of kAhead except in the last block
+                for (int ql = 0; ql < cnt; ql += kAhead) {
+    #pragma unroll
+                    for (int d = 0; d < kAhead; ++d) {
+                        if (ql + d >= cnt) break;  // past the last step: nothing was requested into these slots
+                        v4i bfrag[MT];
+                        const bool ok = ring_ok[d];
+                        if (ok) {
+    #pragma unroll
+                            for (int mt = 0; mt < MT; ++mt)
+                                bfrag[mt] = FMT == FMT_F4 ? expand_f4(ring[d][mt]) : expand_i8(ring[d][mt], h);
+                        }
+                        ring_ok[d] = request(ring[d]);
+                        if (ok) {
+    #pragma unroll
+                            for (int nt = 0; nt < kNT; ++nt) {
+                                const v4i afrag = lds_w[((ql + d) * kNT + nt) * 64 + lane];
+    #pragma unroll
+                                for (int mt = 0; mt < MT; ++mt)
+                                    acc[mt][nt] = A::mma(afrag, bfrag[mt], acc[mt][nt]);
+                            }
+                        }
+                    }
+                }
             }
-            const int cnt = min(kQB, q_end - q0);
-            for (int ql = 0; ql < cnt; ++ql) {
-                // advance the (tap, step) counters and prefetch the next step's words
-                int ntr = tr, nts = ts, nt_ = t + 1;
-                if (nt_ == steps) {
-                    nt_ = 0;
-                    if (++nts == p.S) {
-                        nts = 0;
-                        ++ntr;
-                    }
+        } else {
+            // one step ahead: the threshold epilogues leave no registers for a ring (it spilled and was slower)
+            int tr = (q_begin / steps) / p.S, ts = (q_begin / steps) % p.S, t = q_begin % steps;
+            uint32_t cur[MT], nxt[MT];
+            bool cur_ok = q_begin < q_end ? load_step(tr, ts, t, cur) : false;
+            for (int q0 = q_begin; q0 < q_end; q0 += kQB) {
+                if (!single_block) {
+                    __syncthreads();
+                    stage_weights(q0);
+                    __syncthreads();
                 }
-                const bool nxt_ok = (q0 + ql + 1 < q_end) ? load_step(ntr, nts, nt_, nxt) : false;
-                if (cur_ok) {
-                    v4i bfrag[MT];
-#pragma unroll
-                    for (int mt = 0; mt < MT; ++mt)
-                        bfrag[mt] = FMT == FMT_F4 ? expand_f4(cur[mt]) : expand_i8(cur[mt], h);
-#pragma unroll
-                    for (int nt = 0; nt < kNT; ++nt) {
-                        const v4i afrag = lds_w[(ql * kNT + nt) * 64 + lane];
-#pragma unroll
+                const int cnt = min(kQB, q_end - q0);
+                for (int ql = 0; ql < cnt; ++ql) {
+                    // advance the (tap, step) counters and prefetch the next step's words
+                    int ntr = tr, nts = ts, nt_ = t + 1;
+                    if (nt_ == steps) {
+                        nt_ = 0;
+                        if (++nts == p.S) {
+                            nts = 0;
+                            ++ntr;
+                        }
+                    }
+                    const bool nxt_ok = (q0 + ql + 1 < q_end) ? load_step(ntr, nts, nt_, nxt) : false;
+                    if (cur_ok) {
+                        v4i bfrag[MT];
+    #pragma unroll
                         for (int mt = 0; mt < MT; ++mt)
-                            acc[mt][nt] = A::mma(afrag, bfrag[mt], acc[mt][nt]);
+                            bfrag[mt] = FMT == FMT_F4 ? expand_f4(cur[mt]) : expand_i8(cur[mt], h);
+    #pragma unroll
+                        for (int nt = 0; nt < kNT; ++nt) {
+                            const v4i afrag = lds_w[(ql * kNT + nt) * 64 + lane];
+    #pragma unroll
+                            for (int mt = 0; mt < MT; ++mt)
+                                acc[mt][nt] = A::mma(afrag, bfrag[mt], acc[mt][nt]);
+                        }
                     }
+                    tr = ntr;
+                    ts = nts;
+                    t = nt_;
+                    cur_ok = nxt_ok;
+    #pragma unroll
+                    for (int mt = 0; mt < MT; ++mt) cur[mt] = nxt[mt];
                 }
-                tr = ntr;
-                ts = nts;
-                t = nt_;
-                cur_ok = nxt_ok;
-#pragma unroll
-                for (int mt = 0; mt < MT; ++mt) cur[mt] = nxt[mt];
             }
         }
 
