@@ -76,11 +76,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(MT == 
     const int bg = active ? rw % b_groups : 0;
     const int oy = opix / p.OW, ox = opix % p.OW;
 
-    int bimg[MT], bload[MT];
+    int bimg[MT], bload[MT], voff[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         bimg[mt] = (bg * MT + mt) * 32 + j;
         bload[mt] = min(bimg[mt], p.B - 1);
+        voff[mt] = ((FMT == FMT_F4 ? h * p.B : 0) + bload[mt]) * 4;  // byte offset inside a pixel's [cw][B] words
     }
 
     // stage k-steps [q0, q0+cnt) of this channel group, expanded, in fragment order
@@ -130,15 +131,23 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(MT == 
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[mt][nt][v] = 0;
 
-        // activation word this lane needs for k-step (tap row tr, tap col ts, step t)
+        // Activation words this lane needs for k-step (tap row tr, tap col ts, step t).  The words of one input
+        // pixel ([cw][B]) are addressed as a buffer: the pixel and the step are wave-uniform (descriptor base and
+        // scalar offset, computed on the scalar unit), the lane contributes one constant offset per image tile,
+        // so a step costs no vector address arithmetic (it was ~45 of the ~75 VALU instructions per step).  With
+        // an odd cw the upper half-wave's word of the last step lies past the pixel's range and reads 0; the
+        // weight side of a pad word is 0 anyway.
         auto load_step = [&](int tr, int ts, int t, uint32_t* dst) {
             const int ay = ay0 + tr, ax = ax0 + ts;
             const bool in_frame = valid && ay >= 0 && ay < p.H && ax >= 0 && ax < p.W;
             if (in_frame) {
-                const int word = FMT == FMT_F4 ? min(2 * t + h, p.cw - 1) : t;
-                const uint32_t* src = act + ((size_t)(ay * p.W + ax) * p.cw + word) * p.B;
+                const uint32_t* pixel = act + (size_t)(ay * p.W + ax) * p.cw * p.B;
+                const __amdgpu_buffer_rsrc_t r = __builtin_amdgcn_make_buffer_rsrc(
+                    const_cast<uint32_t*>(pixel), 0, p.cw * p.B * 4, 0x00020000);
+                const int soff = (FMT == FMT_F4 ? 2 * t : t) * p.B * 4;
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt) dst[mt] = src[bload[mt]];
+                for (int mt = 0; mt < MT; ++mt)
+                    dst[mt] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(r, voff[mt], soff, 0);
             }
             return in_frame;
         };
@@ -168,7 +177,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(MT == 
                 }
                 return ok;
             };
-    #pragma unroll
+#pragma unroll
             for (int d = 0; d < kAhead; ++d) ring_ok[d] = request(ring[d]);
             for (int q0 = q_begin; q0 < q_end; q0 += kQB) {
                 if (!single_block) {
@@ -178,22 +187,22 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(MT == 
                 }
                 const int cnt = min(kQB, q_end - q0);  // a multiple of kAhead except in the last block
                 for (int ql = 0; ql < cnt; ql += kAhead) {
-    #pragma unroll
+#pragma unroll
                     for (int d = 0; d < kAhead; ++d) {
                         if (ql + d >= cnt) break;  // past the last step: nothing was requested into these slots
                         v4i bfrag[MT];
                         const bool ok = ring_ok[d];
                         if (ok) {
-    #pragma unroll
+#pragma unroll
                             for (int mt = 0; mt < MT; ++mt)
                                 bfrag[mt] = FMT == FMT_F4 ? expand_f4(ring[d][mt]) : expand_i8(ring[d][mt], h);
                         }
                         ring_ok[d] = request(ring[d]);
                         if (ok) {
-    #pragma unroll
+#pragma unroll
                             for (int nt = 0; nt < kNT; ++nt) {
                                 const v4i afrag = lds_w[((ql + d) * kNT + nt) * 64 + lane];
-    #pragma unroll
+#pragma unroll
                                 for (int mt = 0; mt < MT; ++mt)
                                     acc[mt][nt] = A::mma(afrag, bfrag[mt], acc[mt][nt]);
                             }
@@ -226,13 +235,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(MT == 
                     const bool nxt_ok = (q0 + ql + 1 < q_end) ? load_step(ntr, nts, nt_, nxt) : false;
                     if (cur_ok) {
                         v4i bfrag[MT];
-    #pragma unroll
+#pragma unroll
                         for (int mt = 0; mt < MT; ++mt)
                             bfrag[mt] = FMT == FMT_F4 ? expand_f4(cur[mt]) : expand_i8(cur[mt], h);
-    #pragma unroll
+#pragma unroll
                         for (int nt = 0; nt < kNT; ++nt) {
                             const v4i afrag = lds_w[(ql * kNT + nt) * 64 + lane];
-    #pragma unroll
+#pragma unroll
                             for (int mt = 0; mt < MT; ++mt)
                                 acc[mt][nt] = A::mma(afrag, bfrag[mt], acc[mt][nt]);
                         }
@@ -241,7 +250,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(MT == 
                     ts = nts;
                     t = nt_;
                     cur_ok = nxt_ok;
-    #pragma unroll
+#pragma unroll
                     for (int mt = 0; mt < MT; ++mt) cur[mt] = nxt[mt];
                 }
             }
@@ -512,6 +521,8 @@ int launch_bgemm_mfma(const BgemmParams& p_in, int variant, hipStream_t stream) 
     if (variant == TCBNN_VARIANT_MFMA_F4 && conv3x3_mfma_applicable(p_in))
         return launch_conv3x3_mfma(p_in, stream);
     if (variant == TCBNN_VARIANT_MFMA_F4 && fc_mfma_applicable(p_in)) return launch_fc_mfma(p_in, stream);
+    if ((long long)p_in.cw * p_in.B * 4 >= (1LL << 31))
+        return fail(TCBNN_EUNSUPPORTED, "bgemm: one pixel's activation words must stay below 2 GiB");
     BgemmParams p = p_in;
     p.ksplit = mfma_ksplit(p, variant);
     p.ws_is_dot = 1;
