@@ -506,6 +506,10 @@ void bgemm_mfma_kernel_name(const BgemmParams& p, int variant, char* buf, size_t
         conv3x3_mfma_kernel_name(p, buf, len);
         return;
     }
+    if (variant == TCBNN_VARIANT_MFMA_F4 && gemm_mfma_applicable(p)) {
+        gemm_mfma_kernel_name(p, buf, len);
+        return;
+    }
     if (variant == TCBNN_VARIANT_MFMA_F4 && fc_mfma_applicable(p)) {
         fc_mfma_kernel_name(p, buf, len);
         return;
@@ -520,6 +524,7 @@ int launch_bgemm_mfma(const BgemmParams& p_in, int variant, hipStream_t stream) 
     if (int rc = validate_bgemm(p_in)) return rc;
     if (variant == TCBNN_VARIANT_MFMA_F4 && conv3x3_mfma_applicable(p_in))
         return launch_conv3x3_mfma(p_in, stream);
+    if (variant == TCBNN_VARIANT_MFMA_F4 && gemm_mfma_applicable(p_in)) return launch_gemm_mfma(p_in, stream);
     if (variant == TCBNN_VARIANT_MFMA_F4 && fc_mfma_applicable(p_in)) return launch_fc_mfma(p_in, stream);
     if ((long long)p_in.cw * p_in.B * 4 >= (1LL << 31))
         return fail(TCBNN_EUNSUPPORTED, "bgemm: one pixel's activation words must stay below 2 GiB");

@@ -134,6 +134,10 @@ bool conv3x3_mfma_applicable(const BgemmParams& p);
 int launch_conv3x3_mfma(const BgemmParams& p, hipStream_t stream);
 void conv3x3_mfma_kernel_name(const BgemmParams& p, char* buf, size_t len);
 // FP4 matrix-core kernel for small fully connected layers (K split over the waves of a workgroup)
+// large unmasked bit-GEMMs (stand-alone product, FC layers at large batch)
+bool gemm_mfma_applicable(const BgemmParams& p);
+int launch_gemm_mfma(const BgemmParams& p, hipStream_t stream);
+void gemm_mfma_kernel_name(const BgemmParams& p, char* buf, size_t len);
 bool fc_mfma_applicable(const BgemmParams& p);
 int launch_fc_mfma(const BgemmParams& p, hipStream_t stream);
 void fc_mfma_kernel_name(const BgemmParams& p, char* buf, size_t len);

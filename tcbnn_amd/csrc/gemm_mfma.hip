@@ -1,0 +1,242 @@
+// FP4 matrix-core kernel for LARGE bit-GEMMs: the stand-alone bit matrix product (BMMAS_new,
+// tensorcore_kernel.cu:336-356: C = K - 2 popc(A xor B)) and fully connected layers at large batch
+// (Fc128LayerFMT / Out128LayerFMT, kernel.cuh:174-280; e.g. the 1024 -> 1024 layers of the MLP at batch
+// 8192), where K is a whole number of 64-bit k-steps and nothing needs masking.  The generic implicit-GEMM
+// kernel serves the same problems, but pays for its generality in every k-step (tap bookkeeping, frame and
+// range tests, weights expanded with masks behind two barriers per block).
+//
+//   workgroup = 4 waves = (4 x MT x 32 rows of the batch / of A) x 64 output columns;
+//   wave      = MT image tiles x 2 column tiles: 2 MT MFMAs (32 x 32 x 64, FP4) per k-step;
+//   weights   : the 64 columns' words are expanded to MFMA "A" fragments in LDS, 16 k-steps at a time,
+//               double-buffered: the words of the next block are requested before the current block is
+//               multiplied and expanded into the other buffer after it, one barrier per block;
+//   rows      : a lane's words come straight from memory through buffer addressing (one per-lane constant
+//               offset per image tile, the k-step in the scalar offset), four k-steps ahead of their use.
+// Operand roles, fragment order and the accumulator layout are those of bgemm_mfma.hip.
+#include "common.h"
+#include "mfma_util.h"
+
+namespace tcbnn {
+namespace {
+
+using namespace mfma;
+
+constexpr int kWaves = 4;
+constexpr int kThreads = 64 * kWaves;
+constexpr int kNT = 2;     // 32-column tiles per wave
+constexpr int kBlk = 16;   // k-steps of weights per LDS buffer (16 * kNT KiB)
+constexpr int kAhead = 4;  // k-steps a row word is requested ahead of its use; divides kBlk
+constexpr int kFrags = kBlk * kNT / kWaves;  // fragments a wave stages per block
+
+template <int MT, int EPI>
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) void gemm_mfma_f4_kernel(
+    const BgemmParams p, const uint32_t* __restrict__ act, const uint32_t* __restrict__ wgt,
+    const float* __restrict__ bnp, const float* __restrict__ bias, int n_groups) {
+    __shared__ v4i lds_w[2][kBlk * kNT * 64];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int j = lane & 31;  // image within a 32-image tile
+    const int h = lane >> 5;  // k half (operands) / column half (accumulator)
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int ng = blockIdx.x % n_groups, rb = blockIdx.x / n_groups;
+    const int n0 = ng * (32 * kNT);
+    const int b0 = (rb * kWaves + wave) * (32 * MT);
+    const int steps = p.cw / 2;  // 64-bit k-steps; cw is even and every bit is a true input (host checked)
+
+    // ---- weights: this wave stages fragments f = wave + 4 i = (k-step ql = wave/2 + 2 i, column tile wave % 2)
+    const int snt = wave & 1, sq = wave >> 1;
+    // a row past N (stand-alone product: the rows do not exist) reads the last row; its results are discarded
+    const uint32_t* __restrict__ wrow = wgt + (size_t)min(n0 + snt * 32 + row_to_channel(j), p.N - 1) * p.cw + h;
+    uint32_t wx[kFrags];
+    auto stage_load = [&](int q0) {
+#pragma unroll
+        for (int i = 0; i < kFrags; ++i) {
+            const int q = q0 + sq + 2 * i;
+            wx[i] = q < steps ? wrow[2 * q] : 0u;
+        }
+    };
+    auto stage_store = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < kFrags; ++i) lds_w[buf][((sq + 2 * i) * kNT + snt) * 64 + lane] = expand_f4(wx[i]);
+    };
+
+    // ---- rows: words [cw][B]; lane (j, h) of image tile mt reads word 2 q + h of image b0 + 32 mt + j
+    int bimg[MT], voff[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        bimg[mt] = b0 + mt * 32 + j;
+        voff[mt] = (h * p.B + min(bimg[mt], p.B - 1)) * 4;
+    }
+    const __amdgpu_buffer_rsrc_t r_act =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<uint32_t*>(act), 0, p.cw * p.B * 4, 0x00020000);
+    const int step_bytes = 2 * p.B * 4;
+    uint32_t ring[kAhead][MT];
+    int lq = 0;  // next k-step to request
+    auto request = [&](uint32_t* dst) {
+        if (lq < steps) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+                dst[mt] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(r_act, voff[mt], lq * step_bytes, 0);
+        }
+        ++lq;
+    };
+
+    v16f acc[MT][kNT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < kNT; ++nt)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[mt][nt][v] = 0.0f;
+
+#pragma unroll
+    for (int d = 0; d < kAhead; ++d) request(ring[d]);
+    stage_load(0);
+    stage_store(0);
+    __syncthreads();
+
+    int buf = 0;
+    for (int q0 = 0; q0 < steps; q0 += kBlk) {
+        const bool more = q0 + kBlk < steps;  // uniform
+        if (more) stage_load(q0 + kBlk);
+        const int cnt = min(kBlk, steps - q0);
+        const v4i* __restrict__ wl = lds_w[buf];
+        for (int ql = 0; ql < cnt; ql += kAhead) {
+#pragma unroll
+            for (int d = 0; d < kAhead; ++d) {
+                if (ql + d >= cnt) break;
+                v4i bfrag[MT];
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) bfrag[mt] = expand_f4(ring[d][mt]);
+                request(ring[d]);
+#pragma unroll
+                for (int nt = 0; nt < kNT; ++nt) {
+                    const v4i afrag = wl[((ql + d) * kNT + nt) * 64 + lane];
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt)
+                        acc[mt][nt] = Acc<FMT_F4>::mma(afrag, bfrag[mt], acc[mt][nt]);
+                }
+            }
+        }
+        // the other buffer was last read in the previous block, which every wave left before the barrier below
+        if (more) stage_store(buf ^ 1);
+        __syncthreads();
+        buf ^= 1;
+    }
+
+    // ---- epilogue: the lane holds columns cbase + v of image bimg[mt]
+#pragma unroll
+    for (int nt = 0; nt < kNT; ++nt) {
+        const int cbase = n0 + nt * 32 + 16 * h;
+        float thr[16], bia[EPI == EPI_AFFINE ? 16 : 1];
+        if constexpr (EPI != EPI_RAW) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                thr[v] = bnp[min(cbase + v, p.N - 1)];
+                if constexpr (EPI == EPI_AFFINE) bia[v] = bias[min(cbase + v, p.N - 1)];
+            }
+        }
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int b = bimg[mt];
+            const bool b_ok = b < p.B;
+            if constexpr (EPI == EPI_THRESH) {
+                uint32_t hw = 0;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const uint32_t bit = cbase + v < p.N ? thresh_bit((int)acc[mt][nt][v], thr[v], p.nan_bit) : 0u;
+                    hw = hw + hw + bit;
+                }
+                const uint32_t other = (uint32_t)__shfl_xor((int)hw, 32);
+                const int w = ng * kNT + nt;
+                if (h == 0 && b_ok) {
+                    if (w < p.bits_row_words) p.out_bits[(size_t)w * p.B + b] = (hw << 16) | other;
+                    if (ng == n_groups - 1 && nt == kNT - 1)  // padding words of the 128-padded feature axis
+                        for (int z = max((p.N + 31) / 32, n_groups * kNT); z < p.bits_row_words; ++z)
+                            p.out_bits[(size_t)z * p.B + b] = 0;
+                }
+            } else if constexpr (EPI == EPI_AFFINE) {
+                if (b_ok) {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v)
+                        // the +-1 dot product equals (float)K - (float)popc*2.0f exactly (kernel.cuh:258-270)
+                        if (cbase + v < p.N)
+                            p.out_f32[(size_t)b * p.N + cbase + v] =
+                                __fadd_rn(__fmul_rn((float)(int)acc[mt][nt][v], thr[v]), bia[v]);
+                }
+            } else {
+                if (b_ok) {
+                    int32_t* dst = p.out_i32 + (size_t)b * p.raw_b_stride + cbase;
+                    // a lane's 16 values are consecutive in memory: four 128-bit stores where the run is whole
+                    // and aligned
+                    if (cbase + 16 <= p.N && (reinterpret_cast<uintptr_t>(dst) & 15) == 0) {
+#pragma unroll
+                        for (int g = 0; g < 4; ++g)
+                            reinterpret_cast<int4*>(dst)[g] =
+                                make_int4((int)acc[mt][nt][4 * g], (int)acc[mt][nt][4 * g + 1],
+                                          (int)acc[mt][nt][4 * g + 2], (int)acc[mt][nt][4 * g + 3]);
+                    } else {
+#pragma unroll
+                        for (int v = 0; v < 16; ++v)
+                            if (cbase + v < p.N) dst[v] = (int)acc[mt][nt][v];
+                    }
+                }
+            }
+        }
+    }
+}
+
+// image tiles per wave: 4 when that still gives every CU two workgroups
+int gemm_mt(const BgemmParams& p) {
+    const long long n_groups = (p.N + 32 * kNT - 1) / (32 * kNT);
+    return ((p.B + 32 * 4 * kWaves - 1) / (32 * 4 * kWaves)) * n_groups >= 512 ? 4 : 2;
+}
+
+}  // namespace
+
+bool gemm_mfma_applicable(const BgemmParams& p) {
+    if (p.PH * p.PW != 1 || p.R * p.S != 1 || p.pool_h * p.pool_w != 1) return false;
+    if (p.res_in != nullptr || p.res_out != nullptr) return false;
+    if (p.mode != EPI_THRESH && p.mode != EPI_AFFINE && p.mode != EPI_RAW) return false;
+    if (p.cw % 2 != 0 || p.k_tap != 32 * p.cw) return false;           // whole unmasked k-steps only
+    if ((long long)p.cw * p.B * 4 >= (1LL << 31)) return false;          // 32-bit buffer offsets
+    // large enough to give every CU a workgroup with two image tiles per wave; smaller problems are bound by
+    // launch and fill and stay with the kernels written for them
+    const long long wgs = (long long)((p.B + 32 * 2 * kWaves - 1) / (32 * 2 * kWaves)) * ((p.N + 32 * kNT - 1) / (32 * kNT));
+    return wgs >= 256;
+}
+
+void gemm_mfma_kernel_name(const BgemmParams& p, char* buf, size_t len) {
+    snprintf(buf, len, "gemm_mfma_f4_kernel<%d, %d>", gemm_mt(p), p.mode);
+}
+
+template <int MT>
+static int launch_gemm_mt(const BgemmParams& p, hipStream_t stream) {
+    const int n_groups = (p.N + 32 * kNT - 1) / (32 * kNT);
+    const long long row_blocks = (p.B + 32 * MT * kWaves - 1) / (32 * MT * kWaves);
+    const long long blocks = row_blocks * n_groups;
+    if (blocks <= 0 || blocks > 0x7fffffffLL) return fail(TCBNN_EINVAL, "gemm grid too large");
+    const dim3 grid((unsigned)blocks), block(kThreads);
+    switch (p.mode) {
+        case EPI_THRESH:
+            hipLaunchKernelGGL((gemm_mfma_f4_kernel<MT, EPI_THRESH>), grid, block, 0, stream, p, p.act, p.wgt, p.bn,
+                               p.bn, n_groups);
+            break;
+        case EPI_AFFINE:
+            hipLaunchKernelGGL((gemm_mfma_f4_kernel<MT, EPI_AFFINE>), grid, block, 0, stream, p, p.act, p.wgt,
+                               p.bn_scale, p.bn_bias, n_groups);
+            break;
+        default:
+            hipLaunchKernelGGL((gemm_mfma_f4_kernel<MT, EPI_RAW>), grid, block, 0, stream, p, p.act, p.wgt, p.bn,
+                               p.bn, n_groups);
+    }
+    TCBNN_LAUNCH_CHECK("gemm_mfma_f4_kernel");
+    return TCBNN_OK;
+}
+
+int launch_gemm_mfma(const BgemmParams& p, hipStream_t stream) {
+    return gemm_mt(p) == 4 ? launch_gemm_mt<4>(p, stream) : launch_gemm_mt<2>(p, stream);
+}
+
+}  // namespace tcbnn
