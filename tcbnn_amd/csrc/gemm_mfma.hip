@@ -42,7 +42,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) v
     const int ng = blockIdx.x % n_groups, rb = blockIdx.x / n_groups;
     const int n0 = ng * (32 * kNT);
     const int b0 = (rb * kWaves + wave) * (32 * MT);
-    const int steps = p.cw / 2;  // 64-bit k-steps; cw is even and every bit is a true input (host checked)
+    const int steps = p.cw / 2;  // 64-bit k-steps: a multiple of kAhead, every bit a true input (host checked)
 
     // ---- weights: this wave stages fragments f = wave + 4 i = (k-step ql = wave/2 + 2 i, column tile wave % 2)
     const int snt = wave & 1, sq = wave >> 1;
@@ -73,12 +73,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) v
     const int step_bytes = 2 * p.B * 4;
     uint32_t ring[kAhead][MT];
     int lq = 0;  // next k-step to request
+    // no test for the end of K: a request past it lies outside the descriptor's range, touches no memory and
+    // returns 0 (such words are never multiplied), and the k-steps stay free of branches
     auto request = [&](uint32_t* dst) {
-        if (lq < steps) {
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
-                dst[mt] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(r_act, voff[mt], lq * step_bytes, 0);
-        }
+        for (int mt = 0; mt < MT; ++mt)
+            dst[mt] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(r_act, voff[mt], lq * step_bytes, 0);
         ++lq;
     };
 
@@ -96,27 +96,53 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) v
     stage_store(0);
     __syncthreads();
 
+    // Software pipeline, one k-step deep: while step q is multiplied, the weight fragments of step q + 1 are on
+    // their way from LDS and its row words are expanded (their ring slot is then asked for step q + 5).  Step q's
+    // words sit in ring slot q % kAhead; kBlk is a multiple of kAhead, so the slot of step ql + d of a block is d.
+    v4i anext[kNT], bnext[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) bnext[mt] = expand_f4(ring[0][mt]);
+    request(ring[0]);
+
     int buf = 0;
     for (int q0 = 0; q0 < steps; q0 += kBlk) {
         const bool more = q0 + kBlk < steps;  // uniform
         if (more) stage_load(q0 + kBlk);
-        const int cnt = min(kBlk, steps - q0);
+        const int cnt = min(kBlk, steps - q0);  // a multiple of kAhead (host checked)
         const v4i* __restrict__ wl = lds_w[buf];
+#pragma unroll
+        for (int nt = 0; nt < kNT; ++nt) anext[nt] = wl[nt * 64 + lane];
         for (int ql = 0; ql < cnt; ql += kAhead) {
 #pragma unroll
             for (int d = 0; d < kAhead; ++d) {
-                if (ql + d >= cnt) break;
-                v4i bfrag[MT];
+                v4i acur[kNT], bcur[MT];
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt) bfrag[mt] = expand_f4(ring[d][mt]);
-                request(ring[d]);
+                for (int nt = 0; nt < kNT; ++nt) acur[nt] = anext[nt];
 #pragma unroll
-                for (int nt = 0; nt < kNT; ++nt) {
-                    const v4i afrag = wl[((ql + d) * kNT + nt) * 64 + lane];
+                for (int mt = 0; mt < MT; ++mt) bcur[mt] = bnext[mt];
+                const int qn = min(ql + d + 1, kBlk - 1);  // after a block's last step: read again, not used
+#pragma unroll
+                for (int nt = 0; nt < kNT; ++nt) anext[nt] = wl[(qn * kNT + nt) * 64 + lane];
+                const int dn = (d + 1) % kAhead;  // a constant once the loop over d is unrolled
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt) bnext[mt] = expand_f4(ring[dn][mt]);
+                request(ring[dn]);
+#pragma unroll
+                for (int nt = 0; nt < kNT; ++nt)
 #pragma unroll
                     for (int mt = 0; mt < MT; ++mt)
-                        acc[mt][nt] = Acc<FMT_F4>::mma(afrag, bfrag[mt], acc[mt][nt]);
+                        acc[mt][nt] = Acc<FMT_F4>::mma(acur[nt], bcur[mt], acc[mt][nt]);
+                // issue order of the step: fragment reads first, then each MFMA followed by a few of the next
+                // step's expansion instructions (they run while the matrix pipeline is busy), the row requests
+                // in the middle
+                __builtin_amdgcn_sched_group_barrier(0x100, kNT, 0);  // LDS reads
+#pragma unroll
+                for (int i = 0; i < kNT * MT; ++i) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+                    __builtin_amdgcn_sched_group_barrier(0x002, (7 * MT + kNT * MT - 1) / (kNT * MT), 0);  // VALU
+                    if (i == kNT * MT / 2) __builtin_amdgcn_sched_group_barrier(0x020, MT, 0);  // row requests
                 }
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
         // the other buffer was last read in the previous block, which every wave left before the barrier below
@@ -199,7 +225,7 @@ bool gemm_mfma_applicable(const BgemmParams& p) {
     if (p.PH * p.PW != 1 || p.R * p.S != 1 || p.pool_h * p.pool_w != 1) return false;
     if (p.res_in != nullptr || p.res_out != nullptr) return false;
     if (p.mode != EPI_THRESH && p.mode != EPI_AFFINE && p.mode != EPI_RAW) return false;
-    if (p.cw % 2 != 0 || p.k_tap != 32 * p.cw) return false;           // whole unmasked k-steps only
+    if (p.cw % (2 * kAhead) != 0 || p.k_tap != 32 * p.cw) return false;  // whole unmasked groups of k-steps only
     if ((long long)p.cw * p.B * 4 >= (1LL << 31)) return false;          // 32-bit buffer offsets
     // large enough to give every CU a workgroup with two image tiles per wave; smaller problems are bound by
     // launch and fill and stay with the kernels written for them

@@ -26,8 +26,8 @@ def _variant(gpu, name):
 @pytest.mark.parametrize("m,n,k", [(1024, 1024, 1024), (8, 32, 32), (100, 64, 96), (77, 160, 1056),
                                    (300, 32, 4096), (64, 32, 64),
                                    # large products (the FP4 engine's large-GEMM kernel): ragged rows and columns,
-                                   # fewer k-steps than the prefetch depth, a last weight block of one k-step
-                                   (4100, 992, 192), (9000, 2048, 1088), (8192, 1024, 1024)])
+                                   # a single group of k-steps, a last weight block of one group, a K the kernel does not take
+                                   (4100, 992, 192), (4100, 992, 256), (9000, 2048, 1280), (8192, 1024, 1024)])
 def test_bmm(gpu, variant, m, n, k):
     r = rng(m + n + k)
     a = r.integers(0, 2 ** 32, size=(m, k // 32), dtype=np.uint64).astype(np.uint32)
@@ -88,7 +88,7 @@ def test_fc128_nan_threshold(gpu, variant):
 
 @pytest.mark.parametrize("variant", VARIANTS)
 @pytest.mark.parametrize("b,k,n", [(8, 1024, 10), (256, 512, 1000), (70, 300, 33), (8192, 1024, 10),
-                                   (4100, 1152, 1000)])
+                                   (4100, 1280, 1000)])
 def test_out128(gpu, variant, b, k, n):
     r = rng(b + k + n)
     x = r.standard_normal((b, k)).astype(np.float32)
