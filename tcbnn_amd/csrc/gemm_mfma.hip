@@ -25,7 +25,7 @@ constexpr int kWaves = 4;
 constexpr int kThreads = 64 * kWaves;
 constexpr int kNT = 2;     // 32-column tiles per wave
 constexpr int kBlk = 16;   // k-steps of weights per LDS buffer (16 * kNT KiB)
-constexpr int kAhead = 4;  // k-steps a row word is requested ahead of its use; divides kBlk
+constexpr int kAhead = 8;  // k-steps a row word is requested ahead of its use; divides kBlk
 constexpr int kFrags = kBlk * kNT / kWaves;  // fragments a wave stages per block
 
 template <int MT, int EPI>
