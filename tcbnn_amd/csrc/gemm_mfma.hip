@@ -1,7 +1,7 @@
 // FP4 matrix-core kernel for LARGE bit-GEMMs: the stand-alone bit matrix product (BMMAS_new,
 // tensorcore_kernel.cu:336-356: C = K - 2 popc(A xor B)) and fully connected layers at large batch
 // (Fc128LayerFMT / Out128LayerFMT, kernel.cuh:174-280; e.g. the 1024 -> 1024 layers of the MLP at batch
-// 8192), where K is a whole number of 64-bit k-steps and nothing needs masking.  The generic implicit-GEMM
+// 8192), where K is a whole number of 64-bit words per row.  The generic implicit-GEMM
 // kernel serves the same problems, but pays for its generality in every k-step (tap bookkeeping, frame and
 // range tests, weights expanded with masks behind two barriers per block).
 //
@@ -42,7 +42,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) v
     const int ng = blockIdx.x % n_groups, rb = blockIdx.x / n_groups;
     const int n0 = ng * (32 * kNT);
     const int b0 = (rb * kWaves + wave) * (32 * MT);
-    const int steps = p.cw / 2;  // 64-bit k-steps: a multiple of kAhead, every bit a true input (host checked)
+    // 64-bit k-steps (cw is even, host checked), run in whole groups of kAhead.  Nothing is masked: a pad bit is 0 in
+    // both operands (the layouts' convention), and so is every bit of a step past K (rows: outside the descriptor's
+    // range; weights: staged as 0).  A 0 bit expands to +1.0 on both sides, so each such position adds exactly +1
+    // to the dot product, and the known count is taken off in the epilogue.
+    const int true_steps = p.cw / 2;
+    const int steps = (true_steps + kAhead - 1) / kAhead * kAhead;
+    const int corr = 32 * p.cw - p.k_tap + 64 * (steps - true_steps);
 
     // ---- weights: this wave stages fragments f = wave + 4 i = (k-step ql = wave/2 + 2 i, column tile wave % 2)
     const int snt = wave & 1, sq = wave >> 1;
@@ -53,7 +59,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) v
 #pragma unroll
         for (int i = 0; i < kFrags; ++i) {
             const int q = q0 + sq + 2 * i;
-            wx[i] = q < steps ? wrow[2 * q] : 0u;
+            wx[i] = q < true_steps ? wrow[2 * q] : 0u;
         }
     };
     auto stage_store = [&](int buf) {
@@ -108,7 +114,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) v
     for (int q0 = 0; q0 < steps; q0 += kBlk) {
         const bool more = q0 + kBlk < steps;  // uniform
         if (more) stage_load(q0 + kBlk);
-        const int cnt = min(kBlk, steps - q0);  // a multiple of kAhead (host checked)
+        const int cnt = min(kBlk, steps - q0);  // a multiple of kAhead
         const v4i* __restrict__ wl = lds_w[buf];
 #pragma unroll
         for (int nt = 0; nt < kNT; ++nt) anext[nt] = wl[nt * 64 + lane];
@@ -171,7 +177,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) v
                 uint32_t hw = 0;
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
-                    const uint32_t bit = cbase + v < p.N ? thresh_bit((int)acc[mt][nt][v], thr[v], p.nan_bit) : 0u;
+                    const uint32_t bit = cbase + v < p.N ? thresh_bit((int)acc[mt][nt][v] - corr, thr[v], p.nan_bit) : 0u;
                     hw = hw + hw + bit;
                 }
                 const uint32_t other = (uint32_t)__shfl_xor((int)hw, 32);
@@ -189,7 +195,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) v
                         // the +-1 dot product equals (float)K - (float)popc*2.0f exactly (kernel.cuh:258-270)
                         if (cbase + v < p.N)
                             p.out_f32[(size_t)b * p.N + cbase + v] =
-                                __fadd_rn(__fmul_rn((float)(int)acc[mt][nt][v], thr[v]), bia[v]);
+                                __fadd_rn(__fmul_rn((float)((int)acc[mt][nt][v] - corr), thr[v]), bia[v]);
                 }
             } else {
                 if (b_ok) {
@@ -200,12 +206,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) v
 #pragma unroll
                         for (int g = 0; g < 4; ++g)
                             reinterpret_cast<int4*>(dst)[g] =
-                                make_int4((int)acc[mt][nt][4 * g], (int)acc[mt][nt][4 * g + 1],
-                                          (int)acc[mt][nt][4 * g + 2], (int)acc[mt][nt][4 * g + 3]);
+                                make_int4((int)acc[mt][nt][4 * g] - corr, (int)acc[mt][nt][4 * g + 1] - corr,
+                                          (int)acc[mt][nt][4 * g + 2] - corr, (int)acc[mt][nt][4 * g + 3] - corr);
                     } else {
 #pragma unroll
                         for (int v = 0; v < 16; ++v)
-                            if (cbase + v < p.N) dst[v] = (int)acc[mt][nt][v];
+                            if (cbase + v < p.N) dst[v] = (int)acc[mt][nt][v] - corr;
                     }
                 }
             }
@@ -225,7 +231,7 @@ bool gemm_mfma_applicable(const BgemmParams& p) {
     if (p.PH * p.PW != 1 || p.R * p.S != 1 || p.pool_h * p.pool_w != 1) return false;
     if (p.res_in != nullptr || p.res_out != nullptr) return false;
     if (p.mode != EPI_THRESH && p.mode != EPI_AFFINE && p.mode != EPI_RAW) return false;
-    if (p.cw % (2 * kAhead) != 0 || p.k_tap != 32 * p.cw) return false;  // whole unmasked groups of k-steps only
+    if (p.cw % 2 != 0 || p.k_tap > 32 * p.cw) return false;               // whole 64-bit k-steps
     if ((long long)p.cw * p.B * 4 >= (1LL << 31)) return false;          // 32-bit buffer offsets
     // large enough to give every CU a workgroup with two image tiles per wave; smaller problems are bound by
     // launch and fill and stay with the kernels written for them

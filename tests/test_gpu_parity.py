@@ -26,7 +26,7 @@ def _variant(gpu, name):
 @pytest.mark.parametrize("m,n,k", [(1024, 1024, 1024), (8, 32, 32), (100, 64, 96), (77, 160, 1056),
                                    (300, 32, 4096), (64, 32, 64),
                                    # large products (the FP4 engine's large-GEMM kernel): ragged rows and columns,
-                                   # a single group of k-steps, a last weight block of one group, a K the kernel does not take
+                                   # K of 3, 8 and 24 k-steps (groups of 8, weight blocks of 16)
                                    (4100, 992, 192), (4100, 992, 512), (9000, 2048, 1536), (8192, 1024, 1024)])
 def test_bmm(gpu, variant, m, n, k):
     r = rng(m + n + k)
@@ -54,7 +54,7 @@ def test_in128(gpu, b, k):
 @pytest.mark.parametrize("b,k,n", [(8, 128, 128), (64, 784, 1024), (100, 1024, 1024), (13, 300, 100),
                                    (256, 2048, 160), (130, 25088, 64), (1000, 1024, 32),
                                    # large batches: the large-GEMM kernel with the threshold epilogue
-                                   (8192, 1024, 1024), (4100, 512, 1000)])
+                                   (8192, 1024, 1024), (4100, 512, 1000), (4100, 300, 1000)])
 def test_fc128(gpu, variant, b, k, n):
     r = rng(b + k + n)
     x = r.standard_normal((b, k)).astype(np.float32)
@@ -88,7 +88,7 @@ def test_fc128_nan_threshold(gpu, variant):
 
 @pytest.mark.parametrize("variant", VARIANTS)
 @pytest.mark.parametrize("b,k,n", [(8, 1024, 10), (256, 512, 1000), (70, 300, 33), (8192, 1024, 10),
-                                   (4100, 1536, 1000)])
+                                   (4100, 1536, 1000), (4100, 1000, 72)])
 def test_out128(gpu, variant, b, k, n):
     r = rng(b + k + n)
     x = r.standard_normal((b, k)).astype(np.float32)
