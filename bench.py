@@ -38,18 +38,18 @@ COMPUTE_PEAKS_TOPS = {
 # launches of a kernel name in one step of the default workload (ResNet-18, batch 256, FP4 engine); a kernel
 # name that is not listed (another network, batch or engine) reports null.
 MEASURED_TRAFFIC_BYTES = {
-    "inconv_tiled_kernel<16, true, false>": 421054264,
-    "conv3x3_mfma_f4_kernel<1, 0, 2, 2, false, false>": 18636853,
-    "conv3x3_mfma_f4_kernel<1, 1, 1, 2, true, false>": 218914670,
-    "conv3x3_mfma_f4_kernel<2, 2, 1, 1, true, false>": 170883846,
+    "inconv_tiled_kernel<16, true, false>": 421060721,
+    "conv3x3_mfma_f4_kernel<1, 0, 2, 2, false, false>": 18636995,
+    "conv3x3_mfma_f4_kernel<1, 1, 1, 2, true, false>": 218917234,
+    "conv3x3_mfma_f4_kernel<2, 2, 1, 1, true, false>": 170880131,
     "conv3x3_mfma_f4_kernel<2, 0, 2, 2, false, false>": 12886323,
-    "conv3x3_mfma_f4_kernel<2, 1, 1, 2, true, false>": 113163716,
-    "conv3x3_mfma_f4_kernel<4, 2, 1, 1, true, false>": 94092964,
-    "conv3x3_mfma_f4_kernel<4, 0, 2, 2, false, false>": 14064485,
-    "conv3x3_mfma_f4_kernel<4, 1, 1, 1, true, false>": 68396806,
-    "conv3x3_mfma_f4_kernel<8, 2, 1, 1, true, false>": 55501197,
+    "conv3x3_mfma_f4_kernel<2, 1, 1, 2, true, false>": 113163606,
+    "conv3x3_mfma_f4_kernel<4, 2, 1, 1, true, false>": 94092878,
+    "conv3x3_mfma_f4_kernel<4, 0, 2, 2, false, false>": 14064388,
+    "conv3x3_mfma_f4_kernel<4, 1, 1, 1, true, false>": 68397807,
+    "conv3x3_mfma_f4_kernel<8, 2, 1, 1, true, false>": 55501495,
     "conv3x3_mfma_f4_kernel<8, 0, 2, 1, false, false>": 17022659,
-    "conv3x3_mfma_f4_kernel<8, 1, 2, 1, true, false>": 29919239,
+    "conv3x3_mfma_f4_kernel<8, 1, 2, 1, true, false>": 29919004,
     "fc_mfma_f4_kernel<0>": 8235359,
     "fc_mfma_f4_kernel<1>": 1386489,
 }
