@@ -28,6 +28,45 @@ constexpr int kBlk = 16;   // k-steps of weights per LDS buffer (16 * kNT KiB)
 constexpr int kAhead = 8;  // k-steps a row word is requested ahead of its use; divides kBlk
 constexpr int kFrags = kBlk * kNT / kWaves;  // fragments a wave stages per block
 
+// Row words are expanded WITHOUT shifts.  FP4 E2M1 has, for every bit position j of a nibble, two values that
+// differ in that bit alone and by exactly 2:  bit 3: +1.0 / -1.0 (0010 / 1010),  bit 2: 0 / 2 (0000 / 0100),
+// bit 1: 2 / 4 (0100 / 0110),  bit 0: 4 / 6 (0110 / 0111).  So dword j of the operand is (x & 0x1111.. << j) | c_j:
+// the bits of class j (positions 4p + j) stay where they are, one instruction per dword, four per word instead of
+// seven (three shifts + four bit-field inserts); VALU instructions and MFMAs of a SIMD do not overlap, so this is
+// matrix-pipeline time.  With s = +-1 the value of the row bit, the operand holds -s (class 3) or a_j + s with
+// a_2 = 1, a_1 = 3, a_0 = 5.  The weight side (expanded once per block, off the critical path) holds -w for class 3
+// and +w for the others, so a product is  w s  (class 3)  or  w s + a_j w:  the accumulator ends as the dot product
+// plus  C = sum over classes of a_j (sum of the column's w over the class), a per-column constant that the staging
+// lanes count as they go and the epilogue takes off.  All products and sums are small integers: exact.
+// one v_bfi_b32 each, D = (mask & x) | (~mask & c); written as asm because the compiler otherwise emits an AND and
+// an OR (two 32-bit constants do not fit one VOP3 instruction unless one sits in a vector register)
+__device__ __forceinline__ int bfi_keep(uint32_t mask, uint32_t x, uint32_t c) {
+    int d;
+    asm("v_bfi_b32 %0, %1, %2, %3" : "=v"(d) : "s"(mask), "v"(x), "v"(c));
+    return d;
+}
+__device__ __forceinline__ v4i expand_rows_f4(uint32_t x) {
+    v4i r;
+    r[0] = bfi_keep(0x11111111u, x, 0x66666666u);
+    r[1] = bfi_keep(0x22222222u, x, 0x44444444u);
+    r[2] = (int)(x & 0x44444444u);
+    r[3] = bfi_keep(0x88888888u, x, 0x22222222u);
+    return r;
+}
+// weight word -> fragment dwords in the same class order: the sign code of bit 4p + j, flipped for class 3 only
+__device__ __forceinline__ v4i expand_weights_f4(uint32_t x) {
+    v4i r;
+    r[0] = bfi_sign_nibbles(~x << 3);
+    r[1] = bfi_sign_nibbles(~x << 2);
+    r[2] = bfi_sign_nibbles(~x << 1);
+    r[3] = bfi_sign_nibbles(x);
+    return r;
+}
+// a_j-weighted sum of w = +-1 (bit set: +1) over the 24 class-0..2 positions of one weight word
+__device__ __forceinline__ int class_sum(uint32_t x) {
+    return 2 * (5 * __popc(x & 0x11111111u) + 3 * __popc(x & 0x22222222u) + __popc(x & 0x44444444u)) - 8 * (5 + 3 + 1);
+}
+
 template <int MT, int EPI>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) void gemm_mfma_f4_kernel(
     const BgemmParams p, const uint32_t* __restrict__ act, const uint32_t* __restrict__ wgt,
@@ -62,9 +101,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) v
             wx[i] = q < true_steps ? wrow[2 * q] : 0u;
         }
     };
-    auto stage_store = [&](int buf) {
+    int csum = 0;  // this lane's share of its column's constant C: the words it stages, pad steps included
+    auto stage_store = [&](int buf, int q0) {
 #pragma unroll
-        for (int i = 0; i < kFrags; ++i) lds_w[buf][((sq + 2 * i) * kNT + snt) * 64 + lane] = expand_f4(wx[i]);
+        for (int i = 0; i < kFrags; ++i) {
+            lds_w[buf][((sq + 2 * i) * kNT + snt) * 64 + lane] = expand_weights_f4(wx[i]);
+            if (q0 + sq + 2 * i < steps) csum += class_sum(wx[i]);
+        }
     };
 
     // ---- rows: words [cw][B]; lane (j, h) of image tile mt reads word 2 q + h of image b0 + 32 mt + j
@@ -99,7 +142,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) v
 #pragma unroll
     for (int d = 0; d < kAhead; ++d) request(ring[d]);
     stage_load(0);
-    stage_store(0);
+    stage_store(0, 0);
     __syncthreads();
 
     // Software pipeline, one k-step deep: while step q is multiplied, the weight fragments of step q + 1 are on
@@ -107,7 +150,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) v
     // words sit in ring slot q % kAhead; kBlk is a multiple of kAhead, so the slot of step ql + d of a block is d.
     v4i anext[kNT], bnext[MT];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) bnext[mt] = expand_f4(ring[0][mt]);
+    for (int mt = 0; mt < MT; ++mt) bnext[mt] = expand_rows_f4(ring[0][mt]);
     request(ring[0]);
 
     int buf = 0;
@@ -131,7 +174,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) v
                 for (int nt = 0; nt < kNT; ++nt) anext[nt] = wl[(qn * kNT + nt) * 64 + lane];
                 const int dn = (d + 1) % kAhead;  // a constant once the loop over d is unrolled
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt) bnext[mt] = expand_f4(ring[dn][mt]);
+                for (int mt = 0; mt < MT; ++mt) bnext[mt] = expand_rows_f4(ring[dn][mt]);
                 request(ring[dn]);
 #pragma unroll
                 for (int nt = 0; nt < kNT; ++nt)
@@ -145,22 +188,33 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) v
 #pragma unroll
                 for (int i = 0; i < kNT * MT; ++i) {
                     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
-                    __builtin_amdgcn_sched_group_barrier(0x002, (7 * MT + kNT * MT - 1) / (kNT * MT), 0);  // VALU
+                    __builtin_amdgcn_sched_group_barrier(0x002, (4 * MT + kNT * MT - 1) / (kNT * MT), 0);  // VALU
                     if (i == kNT * MT / 2) __builtin_amdgcn_sched_group_barrier(0x020, MT, 0);  // row requests
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
         // the other buffer was last read in the previous block, which every wave left before the barrier below
-        if (more) stage_store(buf ^ 1);
+        if (more) stage_store(buf ^ 1, q0 + kBlk);
         __syncthreads();
         buf ^= 1;
     }
+
+    // ---- the columns' constants: four lanes (two k-halves of two waves) staged each column's words.  The weight
+    // buffers are free now (every wave has passed the loop's last barrier).
+    int* colc = reinterpret_cast<int*>(&lds_w[0][0]);  // [kNT * 32]
+    if (tid < kNT * 32) colc[tid] = 0;
+    __syncthreads();
+    atomicAdd(&colc[snt * 32 + row_to_channel(j)], csum);
+    __syncthreads();
 
     // ---- epilogue: the lane holds columns cbase + v of image bimg[mt]
 #pragma unroll
     for (int nt = 0; nt < kNT; ++nt) {
         const int cbase = n0 + nt * 32 + 16 * h;
+        int off[16];  // what the accumulator holds beyond the dot product
+#pragma unroll
+        for (int v = 0; v < 16; ++v) off[v] = corr + colc[nt * 32 + 16 * h + v];
         float thr[16], bia[EPI == EPI_AFFINE ? 16 : 1];
         if constexpr (EPI != EPI_RAW) {
 #pragma unroll
@@ -177,7 +231,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) v
                 uint32_t hw = 0;
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
-                    const uint32_t bit = cbase + v < p.N ? thresh_bit((int)acc[mt][nt][v] - corr, thr[v], p.nan_bit) : 0u;
+                    const uint32_t bit = cbase + v < p.N ? thresh_bit((int)acc[mt][nt][v] - off[v], thr[v], p.nan_bit) : 0u;
                     hw = hw + hw + bit;
                 }
                 const uint32_t other = (uint32_t)__shfl_xor((int)hw, 32);
@@ -195,7 +249,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) v
                         // the +-1 dot product equals (float)K - (float)popc*2.0f exactly (kernel.cuh:258-270)
                         if (cbase + v < p.N)
                             p.out_f32[(size_t)b * p.N + cbase + v] =
-                                __fadd_rn(__fmul_rn((float)((int)acc[mt][nt][v] - corr), thr[v]), bia[v]);
+                                __fadd_rn(__fmul_rn((float)((int)acc[mt][nt][v] - off[v]), thr[v]), bia[v]);
                 }
             } else {
                 if (b_ok) {
@@ -206,12 +260,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) v
 #pragma unroll
                         for (int g = 0; g < 4; ++g)
                             reinterpret_cast<int4*>(dst)[g] =
-                                make_int4((int)acc[mt][nt][4 * g] - corr, (int)acc[mt][nt][4 * g + 1] - corr,
-                                          (int)acc[mt][nt][4 * g + 2] - corr, (int)acc[mt][nt][4 * g + 3] - corr);
+                                make_int4((int)acc[mt][nt][4 * g] - off[4 * g], (int)acc[mt][nt][4 * g + 1] - off[4 * g + 1],
+                                          (int)acc[mt][nt][4 * g + 2] - off[4 * g + 2],
+                                          (int)acc[mt][nt][4 * g + 3] - off[4 * g + 3]);
                     } else {
 #pragma unroll
                         for (int v = 0; v < 16; ++v)
-                            if (cbase + v < p.N) dst[v] = (int)acc[mt][nt][v] - corr;
+                            if (cbase + v < p.N) dst[v] = (int)acc[mt][nt][v] - off[v];
                     }
                 }
             }
