@@ -28,45 +28,8 @@ constexpr int kBlk = 16;   // k-steps of weights per LDS buffer (16 * kNT KiB)
 constexpr int kAhead = 8;  // k-steps a row word is requested ahead of its use; divides kBlk
 constexpr int kFrags = kBlk * kNT / kWaves;  // fragments a wave stages per block
 
-// Row words are expanded WITHOUT shifts.  FP4 E2M1 has, for every bit position j of a nibble, two values that
-// differ in that bit alone and by exactly 2:  bit 3: +1.0 / -1.0 (0010 / 1010),  bit 2: 0 / 2 (0000 / 0100),
-// bit 1: 2 / 4 (0100 / 0110),  bit 0: 4 / 6 (0110 / 0111).  So dword j of the operand is (x & 0x1111.. << j) | c_j:
-// the bits of class j (positions 4p + j) stay where they are, one instruction per dword, four per word instead of
-// seven (three shifts + four bit-field inserts); VALU instructions and MFMAs of a SIMD do not overlap, so this is
-// matrix-pipeline time.  With s = +-1 the value of the row bit, the operand holds -s (class 3) or a_j + s with
-// a_2 = 1, a_1 = 3, a_0 = 5.  The weight side (expanded once per block, off the critical path) holds -w for class 3
-// and +w for the others, so a product is  w s  (class 3)  or  w s + a_j w:  the accumulator ends as the dot product
-// plus  C = sum over classes of a_j (sum of the column's w over the class), a per-column constant that the staging
-// lanes count as they go and the epilogue takes off.  All products and sums are small integers: exact.
-// one v_bfi_b32 each, D = (mask & x) | (~mask & c); written as asm because the compiler otherwise emits an AND and
-// an OR (two 32-bit constants do not fit one VOP3 instruction unless one sits in a vector register)
-__device__ __forceinline__ int bfi_keep(uint32_t mask, uint32_t x, uint32_t c) {
-    int d;
-    asm("v_bfi_b32 %0, %1, %2, %3" : "=v"(d) : "s"(mask), "v"(x), "v"(c));
-    return d;
-}
-__device__ __forceinline__ v4i expand_rows_f4(uint32_t x) {
-    v4i r;
-    r[0] = bfi_keep(0x11111111u, x, 0x66666666u);
-    r[1] = bfi_keep(0x22222222u, x, 0x44444444u);
-    r[2] = (int)(x & 0x44444444u);
-    r[3] = bfi_keep(0x88888888u, x, 0x22222222u);
-    return r;
-}
-// weight word -> fragment dwords in the same class order: the sign code of bit 4p + j, flipped for class 3 only
-__device__ __forceinline__ v4i expand_weights_f4(uint32_t x) {
-    v4i r;
-    r[0] = bfi_sign_nibbles(~x << 3);
-    r[1] = bfi_sign_nibbles(~x << 2);
-    r[2] = bfi_sign_nibbles(~x << 1);
-    r[3] = bfi_sign_nibbles(x);
-    return r;
-}
-// a_j-weighted sum of w = +-1 (bit set: +1) over the 24 class-0..2 positions of one weight word
-__device__ __forceinline__ int class_sum(uint32_t x) {
-    return 2 * (5 * __popc(x & 0x11111111u) + 3 * __popc(x & 0x22222222u) + __popc(x & 0x44444444u)) - 8 * (5 + 3 + 1);
-}
-
+// Row words are expanded without shifts (expand_rows_f4 in mfma_util.h): the accumulator ends as the dot product
+// plus a per-column constant, which the staging lanes count as they go and the epilogue takes off.
 template <int MT, int EPI>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) void gemm_mfma_f4_kernel(
     const BgemmParams p, const uint32_t* __restrict__ act, const uint32_t* __restrict__ wgt,
