@@ -192,6 +192,18 @@ def sweep(args, np, _lib):
     return 0
 
 
+def cpu_model():
+    """Model name of the host processor (first entry of /proc/cpuinfo), for the CPU baseline record."""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -330,7 +342,7 @@ def main():
         cpu = {"value": round(cb / cpu_s, 2), "unit": "images/s", "cores": orc.num_threads(), "kind": "port",
                "sample": "%s forward, batch %d, mean of %d reps after 1 warm-up, OpenMP XOR/popcount "
                          "(64-bit words), same seeds" % (args.net, cb, reps),
-               "binary_tops": round(nets.binary_ops(cspec)[0] / cpu_s / 1e12, 4)}
+               "binary_tops": round(nets.binary_ops(cspec)[0] / cpu_s / 1e12, 4), "cpu_model": cpu_model()}
 
     out = {
         "metric": "images/sec ResNet-18 BNN 224x224 batch 256 on 1 MI355X" if args.net == "imagenet_resnet"

@@ -42,6 +42,13 @@ __global__ __launch_bounds__(kThreads) void pack_rows_kernel(const float* __rest
     }
 }
 
+// Clears n words.  A kernel rather than a memset call: memset nodes recorded into a captured HIP graph
+// have misbehaved on replay, and a caller may capture its set-up.
+__global__ __launch_bounds__(kThreads) void clear_words_kernel(uint32_t* __restrict__ dst, long long n) {
+    const long long idx = (long long)blockIdx.x * kThreads + threadIdx.x;
+    if (idx < n) dst[idx] = 0u;
+}
+
 // In128LayerFMT (kernel.cuh:153-172): fp32 [B][K] row major -> sign bits [KW128][B].  One thread per
 // (word, image): consecutive lanes are consecutive images, so the packed words are written as
 // contiguous runs, and each lane reads its own 128 contiguous bytes (one cache line) with four
@@ -281,9 +288,13 @@ int tcbnn_pack_fc_weight(const float* weight_kn, uint32_t* packed, int in_featur
     TCBNN_REQUIRE(in_features > 0 && out_features > 0, "pack_fc_weight: bad shape");
     const int kw = kw128(in_features);
     const int npad = pad32(out_features);
-    if (int rc = check_hip(hipMemsetAsync(packed, 0, (size_t)npad * kw * 4, (hipStream_t)stream),
-                           "hipMemsetAsync"))
-        return rc;
+    // rows of the padding neurons (the rest is written by the packing kernel)
+    const long long pad_words = (long long)(npad - out_features) * kw;
+    if (pad_words > 0) {
+        hipLaunchKernelGGL(clear_words_kernel, dim3(blocks_for(pad_words)), dim3(kThreads), 0, (hipStream_t)stream,
+                           packed + (size_t)out_features * kw, pad_words);
+        TCBNN_LAUNCH_CHECK("clear_words_kernel");
+    }
     return tcbnn_pack_cols(weight_kn, packed, in_features, out_features, kw, stream);
 }
 
