@@ -614,7 +614,10 @@ conv3x3_mfma_f4_kernel(
             for (int i = 0; i < kBatch; ++i) {
                 const int f = wave + (i0 + i) * kWaves;
                 const int q = f / NT, nt = f % NT;
-                tmp[i] = f < NQ * NT ? frag[((size_t)(ng * NT + nt) * NQ + q) * 64 + lane] : v4i{0, 0, 0, 0};
+                // (the second channel tile of the last group may lie past the padded filter: no fragments there)
+                tmp[i] = f < NQ * NT && (ng * NT + nt) * 32 < p.N
+                             ? frag[((size_t)(ng * NT + nt) * NQ + q) * 64 + lane]
+                             : v4i{0, 0, 0, 0};
             }
 #pragma unroll
             for (int i = 0; i < kBatch; ++i) {
