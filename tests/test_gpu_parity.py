@@ -52,7 +52,7 @@ def test_in128(gpu, b, k):
 
 @pytest.mark.parametrize("variant", VARIANTS)
 @pytest.mark.parametrize("b,k,n", [(8, 128, 128), (64, 784, 1024), (100, 1024, 1024), (13, 300, 100),
-                                   (256, 2048, 160), (130, 25088, 64), (1000, 1024, 32),
+                                   (256, 2048, 160), (130, 25088, 64), (1000, 1024, 32), (1, 512, 64), (3, 96, 40),
                                    # large batches: the large-GEMM kernel with the threshold epilogue
                                    (8192, 1024, 1024), (4100, 512, 1000), (4100, 300, 1000)])
 def test_fc128(gpu, variant, b, k, n):
@@ -87,7 +87,7 @@ def test_fc128_nan_threshold(gpu, variant):
 
 
 @pytest.mark.parametrize("variant", VARIANTS)
-@pytest.mark.parametrize("b,k,n", [(8, 1024, 10), (256, 512, 1000), (70, 300, 33), (8192, 1024, 10),
+@pytest.mark.parametrize("b,k,n", [(8, 1024, 10), (256, 512, 1000), (70, 300, 33), (1, 512, 1000), (8192, 1024, 10),
                                    (4100, 1536, 1000), (4100, 1000, 72)])
 def test_out128(gpu, variant, b, k, n):
     r = rng(b + k + n)
@@ -194,6 +194,8 @@ CONV_CASES = [
     # frames of one to three pixels (every tile is a border tile), odd sizes with stride 2
     (8, 1, 64, 64, 1, 1, False), (40, 2, 128, 32, 1, 2, False), (40, 3, 64, 64, 2, 1, False),
     (72, 5, 512, 40, 2, 1, True),
+    # a single image, an odd handful, one more than a tile
+    (1, 6, 64, 64, 1, 1, False), (3, 5, 128, 96, 2, 1, False), (33, 4, 256, 64, 1, 2, True),
 ]
 
 
