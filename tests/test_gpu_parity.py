@@ -238,8 +238,19 @@ RES_FORMATS = [(0, 0), (1, 1), (0, 1), (1, 0)]
 def test_conv128_residual_modes(gpu, variant, cin, cout, in_fmt, out_fmt):
     if variant != "mfma_f4" and cin > 128:
         pytest.skip("the other engines share one residual epilogue for every Cin")
-    r = rng(41 + cin + cout)
-    b, h = 72, 6
+    _residual_modes(gpu, variant, cin, cout, in_fmt, out_fmt, 72)
+
+
+@pytest.mark.parametrize("b", [1, 5, 33])
+@pytest.mark.parametrize("cin,cout", [(64, 64), (256, 96), (512, 64)])
+def test_conv128_residual_modes_small_batch(gpu, b, cin, cout):
+    """Batches below and just above one 32-image tile: lanes without an image must neither load nor store."""
+    _residual_modes(gpu, "mfma_f4", cin, cout, 1, 1, b)
+
+
+def _residual_modes(gpu, variant, cin, cout, in_fmt, out_fmt, b):
+    r = rng(41 + cin + cout + b)
+    h = 6
     x = rm.pm1(r, (b, h, h, cin))
     f = rm.pm1(r, (3, 3, cin, cout))
     bn = r.normal(0, 20, cout).astype(np.float32)
