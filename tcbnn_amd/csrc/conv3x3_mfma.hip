@@ -738,26 +738,30 @@ int launch_t(const BgemmParams& p, hipStream_t stream) {
             return rc;
         attr_set = true;
     }
+    // workgroups of this instantiation a CU can hold at once (registers and LDS)
+    static int resident = 0;
+    if (resident == 0) {
+        int n = 0;
+        if (int rc = check_hip(hipOccupancyMaxActiveBlocksPerMultiprocessor(
+                                   &n, reinterpret_cast<const void*>(&conv3x3_mfma_f4_kernel<SPT, RM, MT, NT, R16, POOL>),
+                                   kThreads, lds_bytes),
+                               "hipOccupancyMaxActiveBlocksPerMultiprocessor"))
+            return rc;
+        resident = std::max(1, n);
+    }
     const int n_groups = (p.N + 32 * NT - 1) / (32 * NT);
     const int b_groups = (p.B + 32 * MT - 1) / (32 * MT);
     const int quads = ((POOL ? p.OH * p.OW : p.PH * p.PW) + kWaves - 1) / kWaves;  // items of the four waves
-    // Persistent workgroups: two per CU (four where only a quarter of the LDS is needed per workgroup,
-    // Cin = 256 with one channel tile), fewer when their LDS does not fit.  Measured on every layer
-    // of ResNet-18 at batch 256: more, shorter-lived workgroups stage the weights more often and lose.
+    // Persistent workgroups, all resident at once: two per CU (three for Cin = 256 with one tile per wave), fewer
+    // when registers or LDS hold fewer.  Measured on every layer of ResNet-18 at batch 256: more, shorter-lived
+    // workgroups stage the weights more often and lose; and a grid even slightly larger than the resident slots
+    // loses more (its last workgroups start, stage and ramp up only when the first ones have finished: the 14 x 14
+    // and 7 x 7 layers ran 10-18 % longer with 1.5 rounds than with one round of workgroups that each take two
+    // items per wave).  So: as many pixel streams as fit in one round, never more.
     static const int wg_env = getenv("TCBNN_WG_PER_CU") ? atoi(getenv("TCBNN_WG_PER_CU")) : 0;  // tuning switch
     const int wg_want = wg_env > 0 ? wg_env : (SPT == 4 && NT == 1 && MT == 1 ? 3 : 2);
-    const int wg_per_cu = std::max(1, std::min(wg_want, (int)(160 * 1024 / lds_bytes)));
-    const int target = std::max(1, 256 * wg_per_cu / (n_groups * b_groups));
-    int best = std::min(target, quads);
-    double best_waste = 1e30;
-    for (int ps = std::max(1, target / 2); ps <= std::min(quads, target * 2); ++ps) {
-        const int per = (quads + ps - 1) / ps;
-        const double waste = (double)per * ps / quads + 0.02 * std::abs(ps - target) / (double)target;
-        if (waste < best_waste) {
-            best_waste = waste;
-            best = ps;
-        }
-    }
+    const int wg_per_cu = std::max(1, std::min(wg_want, resident));
+    const int best = std::max(1, std::min(256 * wg_per_cu / (n_groups * b_groups), quads));
     // channels that receive an injected residual: o < residual_channels, and only those the
     // source tensor holds (kernel.cuh:770)
     const int res_lim = p.res_in != nullptr ? std::min(std::min(p.res_limit, p.res_in_ch), p.N) : 0;
