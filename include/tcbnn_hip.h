@@ -94,9 +94,9 @@ int tcbnn_conv_out(int in_size, int filter, int stride, int padding, int pool);
 size_t tcbnn_fc_act_words(int batch, int features);                    /* B*KW128          */
 size_t tcbnn_conv_act_words(int height, int width, int batch, int ch); /* H*W*B*CW         */
 size_t tcbnn_fc_weight_words(int in_features, int out_features);       /* NPAD32*KW128     */
-size_t tcbnn_conv_filter_words(int r, int s, int in_ch, int out_ch);   /* NPAD32*R*S*CW, x5 for 3x3 filters with
-                                                                           Cin = 64/128/192/256/384/512: they carry an
-                                                                           FP4-expanded copy after the bit rows */
+size_t tcbnn_conv_filter_words(int r, int s, int in_ch, int out_ch);   /* NPAD32*R*S*CW, x2 for 3x3 filters with
+                                                                           Cin = 64/128/192/256/384/512: they carry a
+                                                                           copy in MFMA lane order after the bit rows */
 size_t tcbnn_inconv_filter_words(int r, int s, int in_ch, int out_ch); /* R*S*OPAD32*5     */
 /* bytes of a residual tensor of `channels` channels in the given TCBNN_RES_* format */
 size_t tcbnn_residual_bytes(int height, int width, int channels, int batch, int format);

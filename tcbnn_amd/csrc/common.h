@@ -123,8 +123,8 @@ int launch_splitk_finish(const BgemmParams& p, hipStream_t stream);
 void bgemm_popc_kernel_name(const BgemmParams& p, char* buf, size_t len);
 void bgemm_mfma_kernel_name(const BgemmParams& p, int variant, char* buf, size_t len);
 // A packed 3x3 filter with Cin = 64 / 128 / 192 / 256 / 384 / 512 carries, after its [OPAD32][9*cw] sign-bit rows, the
-// same weights expanded to FP4 MFMA fragments: v4i [OPAD32/32][9*cw/2][64 lanes] (written once by
-// tcbnn_pack_conv_filter, copied into LDS by the persistent kernel without any arithmetic).
+// same words in MFMA fragment order: uint32 [OPAD32/32][9*cw/2][64 lanes] (written once by tcbnn_pack_conv_filter;
+// the persistent kernel loads a fragment's 64 words with one contiguous request and expands them on the way to LDS).
 inline bool filter_has_fragments(int r, int s, int in_ch) {
     return r == 3 && s == 3 &&
            (in_ch == 64 || in_ch == 128 || in_ch == 192 || in_ch == 256 || in_ch == 384 || in_ch == 512);

@@ -7,8 +7,8 @@
 // of the accumulator owns one image and 16 channels), plus what a short-K convolution needs to
 // keep the matrix cores fed on a machine whose memory latency (~1 us) is longer than the whole
 // K loop of one tile (9 taps x Cin = 576..4608 bits: 36..288 MFMAs):
-//   - persistent workgroups: the FP4 weight fragments of a channel group (18..72 KiB, expanded once
-//     when the filter was packed) and its thresholds are staged in LDS ONCE, then every wave walks a
+//   - persistent workgroups: the FP4 weight fragments of a channel group (18..72 KiB, expanded from the
+//     filter's words in fragment order) and its thresholds are staged in LDS ONCE, then every wave walks a
 //     strided list of (pixel, 64-image) tiles; no barrier after the staging;
 //   - whole-chunk register prefetch: all activation words a wave needs for the next chunk of
 //     taps (the whole tile for Cin <= 128, one filter row above) are requested while the current
@@ -600,30 +600,28 @@ conv3x3_mfma_f4_kernel(
 
     // The first activation (and residual) requests are on their way: their latency now runs while the weights
     // are staged.
-    // ---- stage this channel group's weight fragments (already expanded when the filter was packed)
-    // and thresholds
+    // ---- stage this channel group's weight fragments and thresholds.  The filter holds the weight words in
+    // fragment order (64 consecutive words per fragment): all of a wave's words are requested at once, then
+    // expanded to FP4 on the way into LDS (7 VALU instructions per fragment and lane, once per workgroup;
+    // fetching fragments expanded at pack time moved four times the bytes and took longer).
     {
-        const v4i* __restrict__ frag = reinterpret_cast<const v4i*>(wgt + (size_t)((p.N + 31) / 32) * 32 * kw_tot);
-        // all requests of a batch are in flight together (a loop of load-then-store would pay the
-        // memory latency once per fragment)
-        constexpr int kPerWave = (NQ * NT + kWaves - 1) / kWaves, kBatch = kPerWave < 9 ? kPerWave : 9;
+        const uint32_t* __restrict__ fbits = wgt + (size_t)((p.N + 31) / 32) * 32 * kw_tot;
+        constexpr int kPerWave = (NQ * NT + kWaves - 1) / kWaves;
+        uint32_t tmp[kPerWave];
 #pragma unroll
-        for (int i0 = 0; i0 < kPerWave; i0 += kBatch) {
-            v4i tmp[kBatch];
+        for (int i = 0; i < kPerWave; ++i) {
+            const int f = wave + i * kWaves;
+            const int q = f / NT, nt = f % NT;
+            // (the second channel tile of the last group may lie past the padded filter: nothing to read there)
+            tmp[i] = f < NQ * NT && (ng * NT + nt) * 32 < p.N ? fbits[((size_t)(ng * NT + nt) * NQ + q) * 64 + lane] : 0u;
+        }
 #pragma unroll
-            for (int i = 0; i < kBatch; ++i) {
-                const int f = wave + (i0 + i) * kWaves;
-                const int q = f / NT, nt = f % NT;
-                // (the second channel tile of the last group may lie past the padded filter: no fragments there)
-                tmp[i] = f < NQ * NT && (ng * NT + nt) * 32 < p.N
-                             ? frag[((size_t)(ng * NT + nt) * NQ + q) * 64 + lane]
-                             : v4i{0, 0, 0, 0};
-            }
-#pragma unroll
-            for (int i = 0; i < kBatch; ++i) {
-                const int f = wave + (i0 + i) * kWaves;
-                if (f < NQ * NT) lds_w[f * 64 + lane] = tmp[i];
-            }
+        for (int i = 0; i < kPerWave; ++i) {
+            const int f = wave + i * kWaves;
+            const int nt = f % NT;
+            // channels past N multiply by FP4 zeros
+            const bool exists = (ng * NT + nt) * 32 + row_to_channel(j) < p.N;
+            if (f < NQ * NT) lds_w[f * 64 + lane] = expand_f4_masked(tmp[i], exists ? 0xffffffffu : 0u);
         }
     }
     // A NaN threshold always yields bit 1 (!(x < NaN)), exactly like -inf: staged as such, so that

@@ -118,8 +118,8 @@ size_t tcbnn_fc_weight_words(int in_features, int out_features) {
 }
 size_t tcbnn_conv_filter_words(int r, int s, int in_ch, int out_ch) {
     const size_t bits = (size_t)pad32(out_ch) * r * s * step32(in_ch);
-    // 3x3 filters of the persistent matrix-core kernel carry an FP4-expanded copy (4 bits per weight)
-    return filter_has_fragments(r, s, in_ch) ? 5 * bits : bits;
+    // 3x3 filters of the persistent matrix-core kernel carry a second copy in the order its lanes expand them
+    return filter_has_fragments(r, s, in_ch) ? 2 * bits : bits;
 }
 size_t tcbnn_inconv_filter_words(int r, int s, int in_ch, int out_ch) {
     (void)in_ch;

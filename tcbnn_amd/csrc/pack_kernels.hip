@@ -93,11 +93,12 @@ __global__ void pack_conv_filter_kernel(const float* __restrict__ f, uint32_t* _
     dst[idx] = word;
 }
 
-// Sign-bit rows [opad32][9*cw] of a 3x3 filter -> FP4 MFMA "A" fragments, v4i [opad32/32][9*cw/2][64]:
-// lane (j = lane % 32, h = lane / 32) of step q = tap * cw/2 + t holds word tap*cw + 2t + h of channel
-// 32*tile + row_to_channel(j), expanded; channels >= out_ch are FP4 zeros.
-__global__ void expand_conv_filter_kernel(const uint32_t* __restrict__ bits, mfma::v4i* __restrict__ frag,
-                                          int cw, int out_ch, long long total) {
+// Sign-bit rows [opad32][9*cw] of a 3x3 filter -> the same words in the order the persistent kernel's lanes expand
+// them into FP4 MFMA "A" fragments, uint32 [opad32/32][9*cw/2][64]: lane (j = lane % 32, h = lane / 32) of step
+// q = tap * cw/2 + t holds word tap*cw + 2t + h of channel 32*tile + row_to_channel(j), so that a wave stages a
+// fragment with one contiguous 256-byte load.
+__global__ void permute_conv_filter_kernel(const uint32_t* __restrict__ bits, uint32_t* __restrict__ frag_bits,
+                                           int cw, long long total) {
     const long long idx = (long long)blockIdx.x * kThreads + threadIdx.x;
     if (idx >= total) return;
     const int lane = (int)(idx & 63);
@@ -107,8 +108,7 @@ __global__ void expand_conv_filter_kernel(const uint32_t* __restrict__ bits, mfm
     const int j = lane & 31, h = lane >> 5;
     const int tap = q / (cw / 2), t = q % (cw / 2);
     const int c = tile * 32 + mfma::row_to_channel(j);
-    const uint32_t x = bits[(size_t)c * 9 * cw + tap * cw + 2 * t + h];
-    frag[idx] = mfma::expand_f4_masked(x, c < out_ch ? 0xffffffffu : 0u);
+    frag_bits[idx] = bits[(size_t)c * 9 * cw + tap * cw + 2 * t + h];
 }
 
 // HWIO fp32 [R*S][3][O] -> two tables:
@@ -309,10 +309,10 @@ int tcbnn_pack_conv_filter(const float* filter_hwio, uint32_t* packed, int r, in
                        (hipStream_t)stream, filter_hwio, packed, r * s, in_ch, out_ch, cw, opad);
     TCBNN_LAUNCH_CHECK("pack_conv_filter_kernel");
     if (filter_has_fragments(r, s, in_ch)) {
-        const long long frags = (long long)(opad / 32) * (9 * cw / 2) * 64;
-        hipLaunchKernelGGL(expand_conv_filter_kernel, dim3(blocks_for(frags)), dim3(kThreads), 0, (hipStream_t)stream,
-                           packed, reinterpret_cast<mfma::v4i*>(packed + total), cw, out_ch, frags);
-        TCBNN_LAUNCH_CHECK("expand_conv_filter_kernel");
+        const long long frags = (long long)(opad / 32) * (9 * cw / 2) * 64;  // == total
+        hipLaunchKernelGGL(permute_conv_filter_kernel, dim3(blocks_for(frags)), dim3(kThreads), 0, (hipStream_t)stream,
+                           packed, packed + total, cw, frags);
+        TCBNN_LAUNCH_CHECK("permute_conv_filter_kernel");
     }
     return TCBNN_OK;
 }

@@ -44,7 +44,7 @@ def test_size_helpers():
     assert L.tcbnn_fc_act_words(8192, 784) == 8192 * 28
     assert L.tcbnn_conv_act_words(56, 56, 256, 64) == 56 * 56 * 256 * 2
     assert L.tcbnn_fc_weight_words(784, 10) == 32 * 28
-    assert L.tcbnn_conv_filter_words(3, 3, 64, 64) == 64 * 9 * 2 * 5   # sign bits + FP4 fragment copy
+    assert L.tcbnn_conv_filter_words(3, 3, 64, 64) == 64 * 9 * 2 * 2   # sign bits + a copy in MFMA lane order
     assert L.tcbnn_conv_filter_words(3, 3, 96, 64) == 64 * 9 * 3       # sign bits only
     assert L.tcbnn_conv_filter_words(5, 5, 64, 40) == 64 * 25 * 2
     assert L.tcbnn_inconv_filter_words(7, 7, 3, 64) == 49 * 64 * 5
