@@ -38,18 +38,18 @@ COMPUTE_PEAKS_TOPS = {
 # launches of a kernel name in one step of the default workload (ResNet-18, batch 256, FP4 engine); a kernel
 # name that is not listed (another network, batch or engine) reports null.
 MEASURED_TRAFFIC_BYTES = {
-    "inconv_tiled_kernel<16, true, false>": 421164594,
-    "conv3x3_mfma_f4_kernel<1, 0, 2, 2, false, false>": 18636853,
-    "conv3x3_mfma_f4_kernel<1, 1, 1, 2, true, false>": 218918421,
-    "conv3x3_mfma_f4_kernel<2, 2, 1, 1, true, false>": 170881668,
-    "conv3x3_mfma_f4_kernel<2, 0, 2, 2, false, false>": 12886323,
-    "conv3x3_mfma_f4_kernel<2, 1, 1, 2, true, false>": 113162967,
-    "conv3x3_mfma_f4_kernel<4, 2, 1, 1, true, false>": 94092857,
-    "conv3x3_mfma_f4_kernel<4, 0, 2, 2, false, false>": 14064506,
-    "conv3x3_mfma_f4_kernel<4, 1, 1, 1, true, false>": 68696553,
-    "conv3x3_mfma_f4_kernel<8, 2, 1, 1, true, false>": 55501197,
-    "conv3x3_mfma_f4_kernel<8, 0, 2, 1, false, false>": 17022659,
-    "conv3x3_mfma_f4_kernel<8, 1, 2, 1, true, false>": 29919303,
+    "inconv_tiled_kernel<16, true, false>": 420951375,
+    "conv3x3_mfma_f4_kernel<1, 0, 2, 2, false, false>": 18525737,
+    "conv3x3_mfma_f4_kernel<1, 1, 1, 2, true, false>": 218836612,
+    "conv3x3_mfma_f4_kernel<2, 2, 1, 1, true, false>": 170652170,
+    "conv3x3_mfma_f4_kernel<2, 0, 2, 2, false, false>": 12667191,
+    "conv3x3_mfma_f4_kernel<2, 1, 1, 2, true, false>": 112945544,
+    "conv3x3_mfma_f4_kernel<4, 2, 1, 1, true, false>": 92339953,
+    "conv3x3_mfma_f4_kernel<4, 0, 2, 2, false, false>": 11900772,
+    "conv3x3_mfma_f4_kernel<4, 1, 1, 1, true, false>": 66646696,
+    "conv3x3_mfma_f4_kernel<8, 2, 1, 1, true, false>": 48450135,
+    "conv3x3_mfma_f4_kernel<8, 0, 2, 1, false, false>": 9972557,
+    "conv3x3_mfma_f4_kernel<8, 1, 2, 1, true, false>": 22938191,
     "fc_mfma_f4_kernel<0>": 8235359,
     "fc_mfma_f4_kernel<1>": 1386489,
 }
