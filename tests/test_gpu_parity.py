@@ -778,6 +778,27 @@ def test_imagenet_resnet18_batch256_every_image(gpu):
     net.release()
 
 
+def test_imagenet_resnet18_ragged_batch_above_256(gpu):
+    """Batch 328 (five full groups of 64 images and a group of 8) at full image size, every image and every
+    layer against the oracle: the last image group of each kernel is only partly filled, and element offsets
+    go beyond the ones a batch of 256 reaches."""
+    from tcbnn_amd import nets
+    spec = nets.imagenet_resnet_spec(batch=328)
+    weights = gpu.synthetic_weights(spec, 5)
+    x = gpu.synthetic_input(spec, 5)
+    want = orc_nets.run(spec, weights, x)
+    net = gpu.Network(spec, weights, x)
+    net.forward()
+    np.testing.assert_allclose(net.logits(), want["Fout"]["out"], rtol=1e-5, atol=0)
+    for L in spec[:-1]:
+        layer, w = net.layers[L["name"]], want[L["name"]]
+        got = layer.download_packed()
+        np.testing.assert_array_equal(got, w["out"].reshape(got.shape), err_msg=L["name"])
+        if w.get("res") is not None:
+            np.testing.assert_array_equal(layer.download_residual(), w["res"], err_msg=L["name"])
+    net.release()
+
+
 @pytest.mark.parametrize("variant", VARIANTS)
 def test_imagenet_resnet18_batch256_properties(gpu, variant):
     """Full configured size: images are independent, so the first 8 images of a batch-256 run
