@@ -322,7 +322,7 @@ def main():
     cpu = None
     if not args.no_cpu:
         from oracle import nets as orc_nets, orc
-        cb = args.cpu_batch or {"imagenet_resnet": 16, "cifar10_vgg": 64, "mnist_mlp": 8192, "alexnet": 32,
+        cb = args.cpu_batch or {"imagenet_resnet": 64, "cifar10_vgg": 64, "mnist_mlp": 8192, "alexnet": 32,
                                    "cifar10_resnet": 16, "imagenet_vgg": 8, "imagenet_resnet_textbook": 16}[args.net]
         cb = min(cb, batch)
         cspec = nets.SPECS[args.net](batch=cb)
@@ -333,15 +333,15 @@ def main():
         while True:
             cpu_out = orc_nets.run(cspec, weights, xs)
             reps += 1
-            if time.perf_counter() - t0 > 10.0 or reps >= 10:
+            if time.perf_counter() - t0 > 10.0 or reps >= 1000:  # about 10 s of CPU work
                 break
         cpu_s = (time.perf_counter() - t0) / reps
         # the GPU result of the same images must agree with what the CPU leg just computed
         got = net.logits()[:cb]
         np.testing.assert_allclose(got, cpu_out[spec[-1]["name"]]["out"], rtol=1e-5, atol=0)
         cpu = {"value": round(cb / cpu_s, 2), "unit": "images/s", "cores": orc.num_threads(), "kind": "port",
-               "sample": "%s forward, batch %d, mean of %d reps after 1 warm-up, OpenMP XOR/popcount "
-                         "(64-bit words), same seeds" % (args.net, cb, reps),
+               "sample": "%s forward, batch %d, mean of %d reps (%.1f s) after 1 warm-up, OpenMP XOR/popcount "
+                         "(64-bit words), same seeds" % (args.net, cb, reps, cpu_s * reps),
                "binary_tops": round(nets.binary_ops(cspec)[0] / cpu_s / 1e12, 4), "cpu_model": cpu_model()}
 
     out = {
