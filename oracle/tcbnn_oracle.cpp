@@ -228,6 +228,13 @@ void orc_bconv(const uint32_t* in, const uint32_t* filt, int32_t* out, int batch
 //     source channels >= res_in_ch read 0 (zero-filled padding, param.h:979-980)
 //   bit = (float)res < bn[o] ? 0 : 1                                        l.795-796
 //   OR into pooled pixel (y/pool_h, x/pool_w)                               l.811-815
+//   the pixels walked are pool_h*output_height x pool_w*output_width          l.685-690
+//     (NOT the pre-pool size): when the pooled size is rounded up, the last windows hold pixels past
+//     the convolution's own output; those are computed like any other, from the taps that still lie
+//     inside the frame (l.720-757), and their bits are ORed in.  With no tap left the sum is 0.
+//     Residuals on such pixels: the reference indexes buffers of output_height*output_width pixels
+//     (param.h:925-927) with pre-pool coordinates, i.e. out of bounds whenever pool > 1; here they
+//     neither receive nor save a residual (the GPU library rejects residuals on pooled layers).
 //   ahead_fc: FC feature index ((y/ph)*OW + x/pw)*PAD128(O) + o             l.798-808
 //   save_residual: Rout[y][x][b][o] = res                                   l.818-824
 void orc_conv128(const uint32_t* in, const uint32_t* filt, const float* bn, uint32_t* out,
@@ -249,7 +256,7 @@ void orc_conv128(const uint32_t* in, const uint32_t* filt, const float* bn, uint
             for (int py = 0; py < pool_h; ++py)
                 for (int px = 0; px < pool_w; ++px) {
                     const int y = oy * pool_h + py, x = ox * pool_w + px;
-                    if (y >= ph || x >= pw) continue;
+                    const bool past = y >= ph || x >= pw;  // beyond the convolution's own output
                     const int ay0 = y * stride_h - pad_h, ax0 = x * stride_w - pad_w;
                     for (int b = 0; b < batch; ++b)
                         for (int o = 0; o < cout; ++o) {
@@ -264,7 +271,7 @@ void orc_conv128(const uint32_t* in, const uint32_t* filt, const float* bn, uint
                                         ++exclude;
                                 }
                             int res = cin * r * s - exclude * cin - 2 * c;
-                            if (inject_residual && o < residual_channels) {
+                            if (inject_residual && o < residual_channels && !past) {
                                 int v = 0;
                                 if (o < res_in_ch) {
                                     if (residual_pool) {
@@ -284,7 +291,7 @@ void orc_conv128(const uint32_t* in, const uint32_t* filt, const float* bn, uint
                                 ahead_fc ? out + (size_t)b * oh * ow * ocw128 + ((size_t)oy * ow + ox) * ocw128 + (o >> 5)
                                          : out + (((size_t)oy * ow + ox) * batch + b) * ocw + (o >> 5);
                             *word |= bit << (31 - (o & 31));
-                            if (res_out) res_out[(((size_t)y * pw + x) * batch + b) * cout + o] = res;
+                            if (res_out && !past) res_out[(((size_t)y * pw + x) * batch + b) * cout + o] = res;
                         }
                 }
 }
@@ -293,6 +300,9 @@ void orc_conv128(const uint32_t* in, const uint32_t* filt, const float* bn, uint
 //   acc = 0; for r, s in-frame: acc += ((+-f0) + (+-f1)) + (+-f2)           l.609-643
 //     sign = filter bit (weight >= 0 -> +f, else -f)    param.h:626-628, kernel.cuh:636-638
 //   bit = (float)acc < bn[o] ? 0 : 1; OR-pool                                l.646-661
+//   pixels walked: pool_h*output_height x pool_w*output_width (l.587-596), so windows of a rounded-up
+//     pooled size include pixels past the convolution's own output: computed from the taps still in
+//     the frame (acc stays 0 when none is), bit ORed in; no residual is saved for them
 //   residual[y][x][b][o] = (int)acc                                          l.662-669
 // The three-term sum and the running sum are separate fp32 roundings in this order.
 void orc_inconv128(const float* x, const float* hwio, const float* bn, uint32_t* out,
@@ -313,7 +323,7 @@ void orc_inconv128(const float* x, const float* hwio, const float* bn, uint32_t*
             for (int py = 0; py < pool_h; ++py)
                 for (int px = 0; px < pool_w; ++px) {
                     const int y = oy * pool_h + py, xx = ox * pool_w + px;
-                    if (y >= ph || xx >= pw) continue;
+                    const bool past = y >= ph || xx >= pw;
                     const int ay0 = y * stride_h - pad_h, ax0 = xx * stride_w - pad_w;
                     for (int b = 0; b < batch; ++b) {
                         const float* img = x + (size_t)b * 3 * plane;
@@ -341,7 +351,7 @@ void orc_inconv128(const float* x, const float* hwio, const float* bn, uint32_t*
                         for (int o = 0; o < cout; ++o) {
                             const uint32_t bit = (acc[o] < bn[o]) ? 0u : 1u;
                             out[(((size_t)oy * ow + ox) * batch + b) * ocw + (o >> 5)] |= bit << (31 - (o & 31));
-                            if (res_out)
+                            if (res_out && !past)
                                 res_out[(((size_t)y * pw + xx) * batch + b) * cout + o] = f2i_rz_sat(acc[o]);
                         }
                     }

@@ -161,7 +161,10 @@ __global__ __launch_bounds__(kThreads)
     for (int pp = 0; pp < pool_n; ++pp) {
         const int y = oy * p.pool_h + pp / p.pool_w;
         const int x = ox * p.pool_w + pp % p.pool_w;
-        const bool valid = active && y < p.PH && x < p.PW;  // wave-uniform
+        // Every pixel of the pool window is computed, also those past the convolution's own output when the
+        // pooled size is rounded up (kernel.cuh:685-690 walks pool * output rows and columns): such a pixel sums
+        // the taps that still lie inside the frame (all others count as excluded) and its bit is ORed in.
+        const bool valid = active;  // wave-uniform
         const int ay0 = y * p.stride_h - p.pad_h;
         const int ax0 = x * p.stride_w - p.pad_w;
 

@@ -166,7 +166,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS &
     const int pp = wave & 1;    // which pair of the workgroup's four columns
     const int chh = wave >> 1;  // which 32 of the pass's 64 channels
     const int xa = x0 + 2 * pp, xb = xa + 1;
-    const bool xa_ok = xa < p.PW, xb_ok = xb < p.PW;  // wave-uniform
+    // columns of the launch: the convolution's own, or all columns of the pool windows (pooled width rounded up)
+    const int xcols = POOLED ? p.pool_w * p.OW : p.PW;
+    const bool xa_ok = xa < xcols, xb_ok = xb < xcols;  // wave-uniform
     const int b0 = bt * 64;
     const int b = b0 + lane;
     const int ncols = (kXT - 1) * p.stride_w + p.S;
@@ -182,7 +184,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS &
       const bool work = xa_ok && wi * 32 < p.opad;      // uniform
       for (int py = 0; py < (POOLED ? p.pool_h : 1); ++py) {
         const int yc = POOLED ? y * p.pool_h + py : y;  // convolution row (uniform)
-        if (POOLED && yc >= p.PH) break;
+        // (rows past the convolution's own output, when the pooled height is rounded up, are computed like any
+        // other from the filter rows still inside the frame: kernel.cuh:587-596 walks pool * output rows)
         float acca[32], accb[32];  // this wave's 32 channels of pixels xa and xb
 #pragma unroll
         for (int n = 0; n < 32; ++n) acca[n] = accb[n] = 0.0f;
@@ -393,7 +396,9 @@ __global__ __launch_bounds__(kThreads) void inconv_generic_kernel(const InConvPa
         for (int py = 0; py < p.pool_h; ++py) {
             for (int px = 0; px < p.pool_w; ++px) {
                 const int y = oy * p.pool_h + py, x = ox * p.pool_w + px;
-                if (y >= p.PH || x >= p.PW) continue;
+                // pixels of the window past the convolution's own output (pooled size rounded up) are computed
+                // like any other, from the taps still inside the frame (kernel.cuh:587-596 walks pool * output
+                // rows and columns); with no tap left the sum is 0
                 const int ay0 = y * p.stride_h - p.pad_h, ax0 = x * p.stride_w - p.pad_w;
                 float acc[32];
 #pragma unroll
@@ -514,7 +519,7 @@ static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name
     }
     if (tiled) {
         const int b_tiles = (p.B + 63) / 64;
-        const int x_groups = (p.PW + kXT - 1) / kXT;
+        const int x_groups = ((pooled ? p.pool_w * p.OW : p.PW) + kXT - 1) / kXT;
         // e / ncols == (e * magic) >> 16 for every e the staging loop uses
         const int ncols = (kXT - 1) * p.stride_w + p.S;
         const int div_magic = 65536 / ncols + 1;

@@ -122,6 +122,23 @@ def test_bconv_sweep_shapes(gpu, variant, h, c):
     np.testing.assert_array_equal(got, want)
 
 
+@pytest.mark.parametrize("h,c", SWEEP)
+def test_bconv_sweep_shapes_batch256(gpu, h, c):
+    """The sweep at its configured batch of 256 on the default engine (the persistent kernel's int32 epilogue
+    with every image group, pixel stream and channel group of the full-size launch), bit for bit."""
+    b = 256
+    r = rng(1000 + h + c)
+    x = rm.pm1(r, (b, h, h, c))
+    f = rm.pm1(r, (3, 3, c, c))
+    pad, buf, _ = orc.conv_geometry(h, 3, 1)
+    want = orc.bconv(orc.pack_conv_input_nhwc(x), orc.pack_conv_filter(f), c, c, 3, 3, 1, pad, buf, buf)
+    got = gpuops.bconv(gpuops.pack_conv_input(x), gpuops.pack_conv_filter(f), b, h, h, c, c, 3, 3, 1, pad, buf, buf,
+                       _variant(gpu, "mfma_f4"))
+    np.testing.assert_array_equal(got, want)
+    # the zero-padded cross-correlation it must equal (benchmark-bconv.cu:126-135), on a few images
+    np.testing.assert_array_equal(got[:3], rm.xcorr_pm1(x[:3], f, 1, pad, pad, buf, buf))
+
+
 @pytest.mark.parametrize("variant", VARIANTS)
 @pytest.mark.parametrize("b,h,cin,cout,R,stride", [(70, 9, 32, 16, 3, 2), (3, 12, 160, 40, 5, 2),
                                                    (130, 6, 96, 24, 1, 2), (5, 16, 64, 8, 7, 4),
@@ -196,6 +213,11 @@ CONV_CASES = [
     (72, 5, 512, 40, 2, 1, True),
     # a single image, an odd handful, one more than a tile
     (1, 6, 64, 64, 1, 1, False), (3, 5, 128, 96, 2, 1, False), (33, 4, 256, 64, 1, 2, True),
+    # pooled sizes that are rounded up: the last windows hold pixels past the convolution's own output, which
+    # the reference computes from the taps still in the frame and ORs in (kernel.cuh:685-690); with a 4x4 pool
+    # on 5 rows the windows' last two rows have no tap left (sum 0, decided by the sign of the threshold)
+    (8, 5, 64, 64, 1, 4, False), (40, 7, 128, 96, 1, 2, True), (8, 11, 64, 40, 2, 2, False),
+    (8, 3, 256, 64, 1, 2, False),
 ]
 
 
@@ -209,6 +231,7 @@ def test_conv128_layer(gpu, variant, b, h, cin, cout, stride, pool, ahead_fc):
     inp, filt = orc.pack_conv_input_nhwc(x), orc.pack_conv_filter(f)
     _, res = orc.conv128(inp, filt, bn, cin, cout, 3, 3, stride, True, 1, save_residual=True)
     bn[:4] = res[0, 0, 0, :4]  # ties on a border pixel
+    bn[4:8] = [0.0, -0.0, 0.5, -0.5]  # decide pixels whose window has no tap in the frame (sum 0)
     want, _ = orc.conv128(inp, filt, bn, cin, cout, 3, 3, stride, True, pool, ahead_fc)
     layer = _run_conv_layer(gpu, variant, x, f, bn, stride, pool, ahead_fc)
     np.testing.assert_array_equal(layer.download_packed(), want)
@@ -236,8 +259,6 @@ RES_FORMATS = [(0, 0), (1, 1), (0, 1), (1, 0)]
 @pytest.mark.parametrize("in_fmt,out_fmt", RES_FORMATS)
 @pytest.mark.parametrize("cin,cout", RES_SHAPES)
 def test_conv128_residual_modes(gpu, variant, cin, cout, in_fmt, out_fmt):
-    if variant != "mfma_f4" and cin > 128:
-        pytest.skip("the other engines share one residual epilogue for every Cin")
     _residual_modes(gpu, variant, cin, cout, in_fmt, out_fmt, 72)
 
 
@@ -377,12 +398,18 @@ def test_conv128_rejects_residual_with_pooling(gpu):
                                                          # with 2x2 windows, odd row / column counts, a 3x3 pool
                                                          # (generic kernel)
                                                          (70, 24, 11, 4, 64, 2, False), (8, 26, 3, 2, 64, 2, False),
-                                                         (9, 18, 7, 2, 40, 2, False), (5, 18, 3, 1, 64, 3, False)])
+                                                         (9, 18, 7, 2, 40, 2, False), (5, 18, 3, 1, 64, 3, False),
+                                                         # pooled sizes that are rounded up (kernel.cuh:587-596
+                                                         # walks pool * output pixels): generic and tiled kernels,
+                                                         # windows whose last rows have no tap in the frame
+                                                         (5, 17, 3, 1, 64, 3, False), (6, 5, 3, 1, 40, 4, False),
+                                                         (70, 7, 3, 1, 64, 2, False), (9, 21, 7, 4, 64, 2, False)])
 def test_inconv128_layer(gpu, b, h, R, stride, cout, pool, save):
     r = rng(b + h + R + cout)
     x = r.standard_normal((b, 3, h, h)).astype(np.float32)
     f = rm.pm1(r, (R, R, 3, cout))
     bn = r.normal(0, np.sqrt(3 * R * R), cout).astype(np.float32)
+    bn[:4] = [0.0, -0.0, 1e-30, -1e-30]  # decide pixels whose window has no tap in the frame (sum 0)
     want, wres = orc.inconv128(x, f, bn, stride, True, pool, save)
     layer = gpu.InConv128LayerParam("Conv1", h, h, R, R, 3, cout, b, stride, stride, True, pool, pool, save)
     layer.initialize(x, gpu.ArrayWeights([f, bn]))
@@ -634,6 +661,35 @@ def test_mnist_mlp_full_batch(gpu, variant):
 def test_cifar10_vgg(gpu, variant):
     from tcbnn_amd import nets
     _compare_network(gpu, nets.cifar10_vgg_spec(batch=16), 2, variant)
+
+
+def test_cifar10_vgg_batch256(gpu):
+    """cifar10_vgg.cu:162-199 at its configured batch of 256, every layer and image against the oracle."""
+    from tcbnn_amd import nets
+    _compare_network(gpu, nets.cifar10_vgg_spec(batch=256), 2, "mfma_f4")
+
+
+def test_cifar10_vgg_batch256_presigned_input(gpu):
+    """The same network on an input binarized by sign beforehand (+-1.0f): the first layer's sums are then exact
+    small integers whatever the order of the additions, every layer is compared, and the first layer's bits
+    are checked against the integer cross-correlation as well."""
+    from tcbnn_amd import nets
+    spec = nets.cifar10_vgg_spec(batch=256)
+    weights = gpu.synthetic_weights(spec, 4)
+    x = np.where(gpu.synthetic_input(spec, 4) >= 0, np.float32(1.0), np.float32(-1.0))
+    want = orc_nets.run(spec, weights, x)
+    net = gpu.Network(spec, weights, x)
+    net.forward()
+    np.testing.assert_allclose(net.logits(), want["Fout"]["out"], rtol=1e-5, atol=0)
+    for L in spec[:-1]:
+        got = net.layers[L["name"]].download_packed()
+        np.testing.assert_array_equal(got, want[L["name"]]["out"].reshape(got.shape), err_msg=L["name"])
+    first = spec[0]
+    f, bn = weights[0], weights[1]  # weight-file order: the first layer's filter (HWIO) and thresholds
+    sums = rm.xcorr_pm1(np.transpose(x[:4], (0, 2, 3, 1)), f, 1, 1, 1, 32, 32)  # [4][32][32][128]
+    bits = orc.unpack_bits(net.layers[first["name"]].download_packed(), 128)[:, :, :4] > 0  # [32][32][4][128]
+    np.testing.assert_array_equal(np.transpose(bits, (2, 0, 1, 3)), ~(sums.astype(np.float32) < bn))
+    net.release()
 
 
 @pytest.mark.parametrize("residual_format", [None, 0], ids=["narrowest", "int32"])

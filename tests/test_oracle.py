@@ -165,13 +165,18 @@ def test_bconv_brute_force_tiny():
 
 def _conv128_numpy(x, f, bn, stride, pool, res_in=None, residual_channels=0, residual_pool=False):
     """Independent statement of Conv128LayerFMT on unpacked tensors:
-    res = xcorr (+ residual rule); bit = !(res < bn); pooled bit = max over window."""
+    res = xcorr (+ residual rule); bit = !(res < bn); pooled bit = max over window.
+    The reference walks pool*output_height x pool*output_width pixels (kernel.cuh:685-690), not the
+    pre-pool size: the zero-padded cross-correlation is therefore evaluated on that larger grid (a pixel
+    past the convolution's own output sums the taps still inside the frame), and the windows are whole."""
     b, h, w, cin = x.shape
     R, S, _, cout = f.shape
     pad_h, ph, oh = rm.conv_pad_out(h, R, stride, True, pool)
     pad_w, pw, ow = rm.conv_pad_out(w, S, stride, True, pool)
-    res = rm.xcorr_pm1(x, f, stride, pad_h, pad_w, ph, pw)  # [B][ph][pw][O]
+    full = rm.xcorr_pm1(x, f, stride, pad_h, pad_w, pool * oh, pool * ow)  # [B][pool*oh][pool*ow][O]
+    res = full[:, :ph, :pw, :].copy()
     if res_in is not None:
+        assert pool == 1
         src = np.transpose(res_in, (2, 0, 1, 3)).astype(np.int64)  # [B][Hr][Wr][Cr]
         if residual_pool:
             src = rm.maxpool_nhwc(src.astype(np.float64), 2, 2).astype(np.int64)
@@ -179,9 +184,80 @@ def _conv128_numpy(x, f, bn, stride, pool, res_in=None, residual_channels=0, res
         lim = min(residual_channels, src.shape[-1], cout)
         add[..., :lim] = src[:, :ph, :pw, :lim]
         res = res + add
-    bits = ~(res.astype(np.float32) < bn[None, None, None, :])
+        full = res
+    bits = ~(full.astype(np.float32) < bn[None, None, None, :])
     pooled = rm.maxpool_nhwc(bits.astype(np.float64), pool, pool) > 0.5
     return res, pooled  # residual [B][ph][pw][O], bits [B][oh][ow][O]
+
+
+@pytest.mark.parametrize("h,pool,stride,R", [(7, 2, 1, 3), (9, 3, 1, 3), (3, 2, 1, 3), (7, 4, 1, 3), (11, 2, 2, 3),
+                                              (5, 2, 1, 5)])
+def test_conv128_rounded_up_pool_walks_pool_times_output_pixels(h, pool, stride, R):
+    """Brute force, straight from the reference's loop bounds: by in [0, pool*output_height), bx likewise
+    (kernel.cuh:685-690, 703-711); per pixel the in-frame taps only, `exclude` for the others (l.720-757);
+    res = Cin*R*S - exclude*Cin - 2*popc (l.766-768); bit ORed into (by/pool, bx/pool) (l.811-815).
+    H=7 / pool 2 and H=9 / pool 3 have pooled sizes that are rounded up: their last windows hold pixels
+    past the convolution's own 7 or 9 rows."""
+    r = rng(1000 * h + 10 * pool + stride)
+    b, cin, cout = 2, 64, 40
+    x, f = _rand_conv(r, b, h, h, cin, cout, R, R)
+    bn = r.normal(0, 6, cout).astype(np.float32)
+    bn[:5] = [0.0, -0.0, 0.5, -1e-30, 1e-30]  # a pixel with no tap in the frame has res = 0: decided here
+    pad, buf, oh = rm.conv_pad_out(h, R, stride, True, pool)
+    assert oh * pool >= buf
+    want = np.zeros((oh, oh, b, cout), bool)
+    seen_past = False
+    for by in range(pool * oh):
+        for bx in range(pool * oh):
+            ay0, ax0 = by * stride - pad, bx * stride - pad
+            seen_past |= by >= buf or bx >= buf
+            for n in range(b):
+                for o in range(cout):
+                    exclude, popc = 0, 0
+                    for i in range(R):
+                        for j in range(R):
+                            ay, ax = ay0 + i, ax0 + j
+                            if 0 <= ay < h and 0 <= ax < h:
+                                popc += int(np.sum((x[n, ay, ax] >= 0) != (f[i, j, :, o] >= 0)))
+                            else:
+                                exclude += 1
+                    res = cin * R * R - exclude * cin - 2 * popc
+                    if not (np.float32(res) < bn[o]):
+                        want[by // pool, bx // pool, n, o] = True
+    assert seen_past == (buf % pool != 0)
+    out, _ = orc.conv128(orc.pack_conv_input_nhwc(x), orc.pack_conv_filter(f), bn, cin, cout, R, R, stride,
+                         True, pool)
+    np.testing.assert_array_equal(out, rm.packbits_msb(want, orc.step32(cout)))
+
+
+@pytest.mark.parametrize("h,pool,stride,R", [(7, 2, 1, 3), (9, 3, 1, 3), (13, 2, 4, 7), (6, 4, 1, 3)])
+def test_inconv128_rounded_up_pool_walks_pool_times_output_pixels(h, pool, stride, R):
+    """The same for the first layer (kernel.cuh:587-596, 604-643): pixels past the convolution's own output
+    accumulate the in-frame taps in the reference's order, 0 when there is none.  Pre-signed +-1 inputs keep
+    every sum an exact small integer, so the expected bits need no care about the order."""
+    r = rng(77 * h + pool)
+    b, cout = 2, 40
+    f = rm.pm1(r, (R, R, 3, cout))
+    x = rm.pm1(r, (b, 3, h, h))
+    bn = np.round(r.normal(0, 4, cout)).astype(np.float32)
+    bn[:5] = [0.0, -0.0, 0.5, -1e-30, 1e-30]
+    pad, buf, oh = rm.conv_pad_out(h, R, stride, True, pool)
+    want = np.zeros((oh, oh, b, cout), bool)
+    for by in range(pool * oh):
+        for bx in range(pool * oh):
+            ay0, ax0 = by * stride - pad, bx * stride - pad
+            for n in range(b):
+                acc = np.zeros(cout, np.float32)
+                for i in range(R):
+                    for j in range(R):
+                        ay, ax = ay0 + i, ax0 + j
+                        if 0 <= ay < h and 0 <= ax < h:
+                            t = [np.where(f[i, j, c] >= 0, x[n, c, ay, ax], -x[n, c, ay, ax]).astype(np.float32)
+                                 for c in range(3)]
+                            acc = (acc + ((t[0] + t[1]) + t[2])).astype(np.float32)
+                want[by // pool, bx // pool, n] |= ~(acc < bn)
+    out, _ = orc.inconv128(x, f, bn, stride, True, pool)
+    np.testing.assert_array_equal(out, rm.packbits_msb(want, orc.step32(cout)))
 
 
 @pytest.mark.parametrize("b,h,cin,cout,stride,pool", [
@@ -265,11 +341,13 @@ def test_inconv128_against_fp64_and_exact_integers(h, R, stride, cout, pool):
     # (1) pre-signed +-1.0 input: every partial sum is a small integer, so the result is
     # order-free and must be exact.
     xs = rm.pm1(r, (b, 3, h, h))
-    want = rm.xcorr_pm1(np.transpose(xs, (0, 2, 3, 1)), f, stride, pad, pad, ph, ph)  # [B][ph][pw][O]
+    # evaluated on the pool*output grid the reference walks (kernel.cuh:587-596)
+    full = rm.xcorr_pm1(np.transpose(xs, (0, 2, 3, 1)), f, stride, pad, pad, pool * oh, pool * oh)
+    want = full[:, :ph, :ph, :]  # [B][ph][pw][O]
     bn_i = np.round(bn).astype(np.float32)
     bn_i[:4] = want[0, 0, 0, :4]  # ties
     out, res = orc.inconv128(xs, f, bn_i, stride, True, pool, save_residual=(pool == 1))
-    bits = ~(want.astype(np.float32) < bn_i[None, None, None, :])
+    bits = ~(full.astype(np.float32) < bn_i[None, None, None, :])
     pooled = rm.maxpool_nhwc(bits.astype(np.float64), pool, pool) > 0.5
     np.testing.assert_array_equal(out, rm.packbits_msb(np.transpose(pooled, (1, 2, 0, 3)), orc.step32(cout)))
     if pool == 1:
