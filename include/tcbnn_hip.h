@@ -167,6 +167,16 @@ typedef struct tcbnn_fc128_desc {
     size_t workspace_words;
 } tcbnn_fc128_desc;
 int tcbnn_fc128_forward(const tcbnn_fc128_desc* d, void* stream);
+/* The same layer for callers that can neither allocate device memory nor hand over a workspace (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  NO counterpart in the
+ * reference.  The split-K partial sums go to a buffer built into the library's code object (4 MiB of device
+ * memory per GPU, held until the process ends); d->workspace and d->workspace_words are ignored.  The call
+ * allocates and frees nothing, clears what it accumulates into with a fill kernel (no memset node), and gives
+ * the same bits as tcbnn_fc128_forward.  Limits: PAD32(weight_width) * input_height <= 1048576 words, else
+ * TCBNN_EINVAL; all calls on one GPU share the one buffer, so calls that overlap in time on one GPU (different
+ * streams or threads) race - serialise them.  The buffer's device address is looked up on the first call per
+ * device (hipGetSymbolAddress, which allocates nothing): make that first call outside a stream capture. */
+int tcbnn_fc128_forward_static_scratch(const tcbnn_fc128_desc* d, void* stream);
 
 /* Out128LayerFMT (kernel.cuh:230-280), fields of Out128LayerParam (param.h:506-530):
  * y[b][n] = ((float)K - (float)popc*2.0f)*bn_scale[n] + bn_bias[n], fp32 row major. */

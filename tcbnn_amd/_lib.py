@@ -108,6 +108,7 @@ ABI = {
     "tcbnn_pack_conv_input_nhwc": (c_int, [c_void_p, c_void_p] + [c_int] * 4 + [c_void_p]),
     "tcbnn_in128_forward": (c_int, [C.POINTER(In128Desc), c_void_p]),
     "tcbnn_fc128_forward": (c_int, [C.POINTER(Fc128Desc), c_void_p]),
+    "tcbnn_fc128_forward_static_scratch": (c_int, [C.POINTER(Fc128Desc), c_void_p]),
     "tcbnn_out128_forward": (c_int, [C.POINTER(Out128Desc), c_void_p]),
     "tcbnn_inconv128_forward": (c_int, [C.POINTER(InConv128Desc), c_void_p]),
     "tcbnn_conv128_forward": (c_int, [C.POINTER(Conv128Desc), c_void_p]),

@@ -16,6 +16,33 @@ namespace tcbnn {
 static thread_local char g_err[512] = "";
 static std::atomic<int> g_default_variant{-1};
 
+// ---- split-K scratch of tcbnn_fc128_forward_static_scratch -------------------------------------------------
+// Device memory that belongs to the loaded code object, not to an allocation: int32 [NPAD32][B] partial sums of
+// a split-K fully connected layer.  Every GPU the library runs on holds its own copy at its own address until the
+// process ends.  In host code the array's NAME is only a handle for hipGetSymbolAddress: it is never passed to a
+// kernel or a copy; the address that call returns for the current device is.
+constexpr size_t kStaticScratchWords = size_t(1) << 20;  // 4 MiB per GPU
+static __device__ __align__(256) int32_t scratch[kStaticScratchWords];
+constexpr int kMaxDevices = 64;
+static std::atomic<int32_t*> g_scratch_ptr[kMaxDevices];
+
+// Address of `scratch` on the current device, resolved once per device with that device current.
+static int static_scratch(int32_t** out) {
+    int dev = -1;
+    if (int rc = check_hip(hipGetDevice(&dev), "hipGetDevice")) return rc;
+    if (dev < 0 || dev >= kMaxDevices) return fail(TCBNN_EUNSUPPORTED, "static scratch: device ordinal %d", dev);
+    int32_t* ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (ptr == nullptr) {
+        void* sym = nullptr;
+        if (int rc = check_hip(hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)")) return rc;
+        if (sym == nullptr) return fail(TCBNN_EHIP, "static scratch: no device address on device %d", dev);
+        ptr = static_cast<int32_t*>(sym);
+        g_scratch_ptr[dev].store(ptr, std::memory_order_release);  // the same value from whichever thread gets here
+    }
+    *out = ptr;
+    return TCBNN_OK;
+}
+
 int fail(int code, const char* fmt, ...) {
     va_list ap;
     va_start(ap, fmt);
@@ -171,6 +198,22 @@ int tcbnn_fc128_forward(const tcbnn_fc128_desc* d, void* stream) {
         d->workspace_words >= (size_t)pad32(d->weight_width) * d->input_height)
         p.workspace = d->workspace;
     return run_bgemm(p, d->variant, (hipStream_t)stream);
+}
+
+int tcbnn_fc128_forward_static_scratch(const tcbnn_fc128_desc* d, void* stream) {
+    TCBNN_NOTNULL(d);
+    TCBNN_REQUIRE(d->input_height > 0 && d->input_width > 0 && d->weight_width > 0, "fc128: bad shape");
+    const size_t need = (size_t)pad32(d->weight_width) * (size_t)d->input_height;
+    TCBNN_REQUIRE(need <= kStaticScratchWords,
+                  "fc128 (static scratch): PAD32(weight_width) * input_height = %zu words exceeds the built-in "
+                  "scratch of %zu words; use tcbnn_fc128_forward with a workspace of the caller",
+                  need, kStaticScratchWords);
+    int32_t* ws = nullptr;
+    if (int rc = static_scratch(&ws)) return rc;
+    tcbnn_fc128_desc own = *d;  // the caller's workspace fields are ignored
+    own.workspace = ws;         // the device address, never the array's name
+    own.workspace_words = kStaticScratchWords;
+    return tcbnn_fc128_forward(&own, stream);
 }
 
 int tcbnn_out128_forward(const tcbnn_out128_desc* d, void* stream) {
