@@ -24,6 +24,7 @@
 //     word, one lane swap, 128-byte stores of the batch-innermost layouts; residual add / save as
 //     contiguous 16-byte runs per lane.
 #include <algorithm>
+#include <atomic>
 #include <cmath>
 #include <cstdlib>
 #include <type_traits>
@@ -59,14 +60,17 @@ constexpr int waves_hint(int spt, int rm, int nt) { return rm == RM_PLAIN && spt
 // layers, 1 for residual layers); NT = 32-channel tiles per wave; R16 = the injected residual is
 // stored as int16 (half the registers hold it while it is in flight); POOL = 2x2 OR-pooling of the
 // output bits (kernel.cuh:797-816): a wave multiplies the four pixels of a window one after the
-// other and stores the OR of their words once.
-template <int SPT, int RM, int MT, int NT, bool R16, bool POOL>
+// other and stores the OR of their words once.  FULLT = every 32-channel tile of the launch exists in full
+// and, with an injected residual, lies entirely below or entirely above the channel limit: the per-channel
+// tests of partial tiles are then not even compiled (they cost scalar registers and set-up instructions in
+// every launch, and the networks' channel counts are multiples of 64).
+template <int SPT, int RM, int MT, int NT, bool R16, bool POOL, bool FULLT>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(waves_hint(SPT, RM, NT)))) void
 conv3x3_mfma_f4_kernel(
     const BgemmParams p, const uint32_t* __restrict__ act, const uint32_t* __restrict__ wgt,
     const float* __restrict__ bnp, const int32_t* __restrict__ rin, int32_t* __restrict__ rout, int res_lim,
     int rout_fmt, unsigned act_bytes, unsigned rin_bytes, unsigned rout_bytes, unsigned bits_bytes,
-    int n_groups, int b_groups, int pix_streams) {
+    int n_groups, int b_groups, int pix_streams, int dy, int dx, int dxs) {
     constexpr bool kRes = RM == RM_PLAIN || RM == RM_POOLED;  // a residual is injected and / or saved
     static_assert(RM == RM_NONE || !POOL, "residuals are defined for un-pooled layers only");
     constexpr int TPC = SPT >= 3 ? 3 : 9;  // taps per prefetch chunk (a filter row, or all of it)
@@ -86,9 +90,10 @@ conv3x3_mfma_f4_kernel(
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     // The channel group is rotated by the workgroup's position, so that the workgroups an XCD receives
     // (every 8th) cover all channel groups, those that inject a residual and those that do not alike.
-    const int ng = (blockIdx.x % n_groups + blockIdx.x / n_groups) % n_groups;
-    const int bg = (blockIdx.x / n_groups) % b_groups;
-    const int stream = blockIdx.x / (n_groups * b_groups);
+    // (grid = channel groups x image groups x pixel streams, launched in that order)
+    const int bg = blockIdx.y;
+    const int stream = blockIdx.z;
+    const int ng = (blockIdx.x + bg + stream * b_groups) % n_groups;
     const int n0 = ng * (32 * NT);
     const int kw_tot = 9 * p.cw;
 
@@ -105,7 +110,7 @@ conv3x3_mfma_f4_kernel(
     // a wave from staying in one column when its stride is a multiple of the row width (then the waves
     // that own a border column, whose tiles are slower, would finish long after the others).
     const int y = pi / roww, xr = pi % roww;
-    const int dy = dpi / roww, dx = dpi % roww, dxs = (dx + dy) % roww;
+    // (dy = dpi / roww, dx = dpi % roww, dxs = (dx + dy) % roww come from the host)
 
     int bimg[MT], bload[MT];
 #pragma unroll
@@ -536,8 +541,8 @@ conv3x3_mfma_f4_kernel(
             const int cb = n0 + nt * 32;
             // uniform: every channel of the tile exists, and gets a residual if any does (a tile that
             // gets none at all holds zeros and is fast as well)
-            const bool fast = cb + 32 <= p.N && (!kRes || cb + 32 <= res_lim || cb >= res_lim);
-            if (fast)
+            const bool fast = FULLT || (cb + 32 <= p.N && (!kRes || cb + 32 <= res_lim || cb >= res_lim));
+            if (FULLT || fast)
                 epilogue_tile(std::true_type{}, nt, pix, bits_pix, rv, sub);
             else
                 epilogue_tile(std::false_type{}, nt, pix, bits_pix, rv, sub);
@@ -604,6 +609,10 @@ conv3x3_mfma_f4_kernel(
     // fragment order (64 consecutive words per fragment): all of a wave's words are requested at once, then
     // expanded to FP4 on the way into LDS (7 VALU instructions per fragment and lane, once per workgroup;
     // fetching fragments expanded at pack time moved four times the bytes and took longer).
+    // The thresholds are requested first, so that their latency runs together with the weights' (requested after
+    // the weights had been stored, they were a second memory round trip in every launch).
+    float thr_stage = 0.0f;
+    if (tid < NT * 32) thr_stage = RM != RM_RAW && (FULLT || n0 + tid < p.N) ? bnp[n0 + tid] : 0.0f;
     {
         const uint32_t* __restrict__ fbits = wgt + (size_t)((p.N + 31) / 32) * 32 * kw_tot;
         constexpr int kPerWave = (NQ * NT + kWaves - 1) / kWaves;
@@ -613,15 +622,21 @@ conv3x3_mfma_f4_kernel(
             const int f = wave + i * kWaves;
             const int q = f / NT, nt = f % NT;
             // (the second channel tile of the last group may lie past the padded filter: nothing to read there)
-            tmp[i] = f < NQ * NT && (ng * NT + nt) * 32 < p.N ? fbits[((size_t)(ng * NT + nt) * NQ + q) * 64 + lane] : 0u;
+            tmp[i] = f < NQ * NT && (FULLT || (ng * NT + nt) * 32 < p.N) ? fbits[((size_t)(ng * NT + nt) * NQ + q) * 64 + lane] : 0u;
         }
 #pragma unroll
         for (int i = 0; i < kPerWave; ++i) {
             const int f = wave + i * kWaves;
             const int nt = f % NT;
-            // channels past N multiply by FP4 zeros
-            const bool exists = (ng * NT + nt) * 32 + row_to_channel(j) < p.N;
-            if (f < NQ * NT) lds_w[f * 64 + lane] = expand_f4_masked(tmp[i], exists ? 0xffffffffu : 0u);
+            if (f < NQ * NT) {
+                if constexpr (FULLT) {
+                    lds_w[f * 64 + lane] = expand_f4(tmp[i]);
+                } else {
+                    // channels past N multiply by FP4 zeros
+                    const bool exists = (ng * NT + nt) * 32 + row_to_channel(j) < p.N;
+                    lds_w[f * 64 + lane] = expand_f4_masked(tmp[i], exists ? 0xffffffffu : 0u);
+                }
+            }
         }
     }
     // A NaN threshold always yields bit 1 (!(x < NaN)), exactly like -inf: staged as such, so that
@@ -632,7 +647,7 @@ conv3x3_mfma_f4_kernel(
     // first MFMA): the finished accumulator is s - ceil(threshold), exact in fp32, and its sign is
     // the inverted output bit, with no per-value subtraction in the epilogue.
     if (tid < NT * 32) {
-        float t = RM != RM_RAW && n0 + tid < p.N ? bnp[n0 + tid] : 0.0f;
+        float t = thr_stage;
         t = t != t ? -__builtin_huge_valf() : t;
         if constexpr (RM == RM_NONE) t = 0.0f - fminf(fmaxf(ceilf(t), -8192.0f), 8192.0f);
         lds_thr[tid] = t;
@@ -702,6 +717,24 @@ conv3x3_mfma_f4_kernel(
     }
 }
 
+// The current device and its number of compute units (looked up once per device).
+constexpr int kMaxDevices = 64;
+int device_info(int* dev, int* cus) {
+    static std::atomic<int> cu_count[kMaxDevices];
+    if (int rc = check_hip(hipGetDevice(dev), "hipGetDevice")) return rc;
+    if (*dev < 0 || *dev >= kMaxDevices) return fail(TCBNN_EUNSUPPORTED, "conv3x3: device ordinal %d", *dev);
+    int n = cu_count[*dev].load(std::memory_order_acquire);
+    if (n == 0) {
+        if (int rc = check_hip(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, *dev),
+                               "hipDeviceGetAttribute(MultiprocessorCount)"))
+            return rc;
+        n = std::max(1, n);
+        cu_count[*dev].store(n, std::memory_order_release);
+    }
+    *cus = n;
+    return TCBNN_OK;
+}
+
 // Sizes in bytes of the tensors the kernel addresses through buffer descriptors.
 struct TensorBytes {
     long long act, rin, rout, bits;
@@ -723,29 +756,28 @@ TensorBytes tensor_bytes(const BgemmParams& p) {
     return t;
 }
 
-template <int SPT, int RM, int MT, int NT, bool R16, bool POOL>
-int launch_t(const BgemmParams& p, hipStream_t stream) {
+template <int SPT, int RM, int MT, int NT, bool R16, bool POOL, bool FULLT>
+int launch_f(const BgemmParams& p, hipStream_t stream) {
     constexpr int NQ = 9 * SPT;
     const size_t lds_bytes = (size_t)NQ * NT * 64 * 16 + NT * 32 * sizeof(float);
-    static bool attr_set = false;  // per instantiation
-    if (!attr_set) {
-        if (int rc = check_hip(
-                hipFuncSetAttribute(reinterpret_cast<const void*>(&conv3x3_mfma_f4_kernel<SPT, RM, MT, NT, R16, POOL>),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes),
-                "hipFuncSetAttribute(MaxDynamicSharedMemorySize)"))
-            return rc;
-        attr_set = true;
-    }
-    // workgroups of this instantiation a CU can hold at once (registers and LDS)
-    static int resident = 0;
+    // Per instantiation and device, set up by the first launch there: the dynamic LDS limit, and how many of its
+    // workgroups a CU holds at once (registers and LDS).  Atomics only so that two host threads that both find the
+    // entry empty do no harm (both store the same value).
+    static std::atomic<int> resident_on[kMaxDevices];
+    int dev = 0, cus = 0;
+    if (int rc = device_info(&dev, &cus)) return rc;
+    int resident = resident_on[dev].load(std::memory_order_acquire);
     if (resident == 0) {
+        const void* fn = reinterpret_cast<const void*>(&conv3x3_mfma_f4_kernel<SPT, RM, MT, NT, R16, POOL, FULLT>);
+        if (int rc = check_hip(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes),
+                               "hipFuncSetAttribute(MaxDynamicSharedMemorySize)"))
+            return rc;
         int n = 0;
-        if (int rc = check_hip(hipOccupancyMaxActiveBlocksPerMultiprocessor(
-                                   &n, reinterpret_cast<const void*>(&conv3x3_mfma_f4_kernel<SPT, RM, MT, NT, R16, POOL>),
-                                   kThreads, lds_bytes),
+        if (int rc = check_hip(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, fn, kThreads, lds_bytes),
                                "hipOccupancyMaxActiveBlocksPerMultiprocessor"))
             return rc;
         resident = std::max(1, n);
+        resident_on[dev].store(resident, std::memory_order_release);
     }
     const int n_groups = (p.N + 32 * NT - 1) / (32 * NT);
     const int b_groups = (p.B + 32 * MT - 1) / (32 * MT);
@@ -759,17 +791,31 @@ int launch_t(const BgemmParams& p, hipStream_t stream) {
     static const int wg_env = getenv("TCBNN_WG_PER_CU") ? atoi(getenv("TCBNN_WG_PER_CU")) : 0;  // tuning switch
     const int wg_want = wg_env > 0 ? wg_env : (SPT == 4 && NT == 1 && MT == 1 ? 3 : 2);
     const int wg_per_cu = std::max(1, std::min(wg_want, resident));
-    const int best = std::max(1, std::min(256 * wg_per_cu / (n_groups * b_groups), quads));
+    const int best = std::max(1, std::min(cus * wg_per_cu / (n_groups * b_groups), quads));
     // channels that receive an injected residual: o < residual_channels, and only those the
     // source tensor holds (kernel.cuh:770)
     const int res_lim = p.res_in != nullptr ? std::min(std::min(p.res_limit, p.res_in_ch), p.N) : 0;
     const long long blocks = (long long)best * n_groups * b_groups;
     const TensorBytes tb = tensor_bytes(p);
-    hipLaunchKernelGGL((conv3x3_mfma_f4_kernel<SPT, RM, MT, NT, R16, POOL>), dim3((unsigned)blocks), dim3(kThreads), lds_bytes,
+    if (blocks > 0x7fffffffLL || b_groups > 65535 || best > 65535) return fail(TCBNN_EINVAL, "conv3x3: grid too large");
+    // a wave's stride over the work items, split into rows and columns once here instead of in every wave
+    const int roww = POOL ? p.OW : p.PW, dpi = best * kWaves;
+    const int dy = dpi / roww, dx = dpi % roww, dxs = (dx + dy) % roww;
+    hipLaunchKernelGGL((conv3x3_mfma_f4_kernel<SPT, RM, MT, NT, R16, POOL, FULLT>),
+                       dim3((unsigned)n_groups, (unsigned)b_groups, (unsigned)best), dim3(kThreads), lds_bytes,
                        stream, p, p.act, p.wgt, p.bn, p.res_in, RM == RM_RAW ? p.out_i32 : p.res_out, res_lim, p.res_out_fmt,
-                       (unsigned)tb.act, (unsigned)tb.rin, (unsigned)tb.rout, (unsigned)tb.bits, n_groups, b_groups, best);
+                       (unsigned)tb.act, (unsigned)tb.rin, (unsigned)tb.rout, (unsigned)tb.bits, n_groups, b_groups, best,
+                       dy, dx, dxs);
     TCBNN_LAUNCH_CHECK("conv3x3_mfma_f4_kernel");
     return TCBNN_OK;
+}
+
+// Every channel tile of the launch full, and the residual limit on a tile boundary?  (see FULLT at the kernel)
+template <int SPT, int RM, int MT, int NT, bool R16, bool POOL>
+int launch_t(const BgemmParams& p, hipStream_t stream) {
+    const int res_lim = p.res_in != nullptr ? std::min(std::min(p.res_limit, p.res_in_ch), p.N) : 0;
+    if (p.N % (32 * NT) == 0 && res_lim % 32 == 0) return launch_f<SPT, RM, MT, NT, R16, POOL, true>(p, stream);
+    return launch_f<SPT, RM, MT, NT, R16, POOL, false>(p, stream);
 }
 
 // Which instantiation serves a layer.  Measured on ResNet-18 at batch 256: the HBM-bound residual
@@ -842,8 +888,10 @@ bool conv3x3_mfma_applicable(const BgemmParams& p) {
 
 void conv3x3_mfma_kernel_name(const BgemmParams& p, char* buf, size_t len) {
     const Pick k = pick(p);
-    snprintf(buf, len, "conv3x3_mfma_f4_kernel<%d, %d, %d, %d, %s, %s>", p.cw / 2, k.rm, k.mt, k.nt,
-             k.r16 ? "true" : "false", k.pool ? "true" : "false");
+    const int res_lim = p.res_in != nullptr ? std::min(std::min(p.res_limit, p.res_in_ch), p.N) : 0;
+    const bool full = p.N % (32 * k.nt) == 0 && res_lim % 32 == 0;
+    snprintf(buf, len, "conv3x3_mfma_f4_kernel<%d, %d, %d, %d, %s, %s, %s>", p.cw / 2, k.rm, k.mt, k.nt,
+             k.r16 ? "true" : "false", k.pool ? "true" : "false", full ? "true" : "false");
 }
 
 int launch_conv3x3_mfma(const BgemmParams& p, hipStream_t stream) {
