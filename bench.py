@@ -32,27 +32,39 @@ COMPUTE_PEAKS_TOPS = {
     "mfma_f4": ("mfma", 10100.0),                         # dense fp4
 }
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch,
-# scaled by what the same counters read for a plain device-to-device copy of known size); the
-# runs and the scale factors (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0) are recorded in profiles/.  Average over the
-# launches of a kernel name in one step of the default workload (ResNet-18, batch 256, FP4 engine); a kernel
-# name that is not listed (another network, batch or engine) reports null.
-MEASURED_TRAFFIC_BYTES = {
-    "inconv_tiled_kernel<16, true, false>": 420951375,
-    "conv3x3_mfma_f4_kernel<1, 0, 2, 2, false, false>": 18525737,
-    "conv3x3_mfma_f4_kernel<1, 1, 1, 2, true, false>": 218836612,
-    "conv3x3_mfma_f4_kernel<2, 2, 1, 1, true, false>": 170652170,
-    "conv3x3_mfma_f4_kernel<2, 0, 2, 2, false, false>": 12667191,
-    "conv3x3_mfma_f4_kernel<2, 1, 1, 2, true, false>": 112945544,
-    "conv3x3_mfma_f4_kernel<4, 2, 1, 1, true, false>": 92339953,
-    "conv3x3_mfma_f4_kernel<4, 0, 2, 2, false, false>": 11900772,
-    "conv3x3_mfma_f4_kernel<4, 1, 1, 1, true, false>": 66646696,
-    "conv3x3_mfma_f4_kernel<8, 2, 1, 1, true, false>": 48450135,
-    "conv3x3_mfma_f4_kernel<8, 0, 2, 1, false, false>": 9972557,
-    "conv3x3_mfma_f4_kernel<8, 1, 2, 1, true, false>": 22938191,
-    "fc_mfma_f4_kernel<0>": 8235359,
-    "fc_mfma_f4_kernel<1>": 1386489,
-}
+# HBM bytes per launch (roofline.traffic) are not measured in this process: hardware counters need a profiler run
+# of their own.  They are read from a data file under profiles/ that records the rocprofv3 commands, the commit
+# and a digest of the kernel sources it was measured on.  When the kernel sources have changed since (or the file
+# is missing, or names no figure for a kernel), traffic is null and traffic_stale says why.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "hbm_traffic_resnet18_b256_fp4.json")
+
+
+def kernel_source_digest():
+    """sha256 over the device sources and headers the library is built from (names and contents, sorted)."""
+    import hashlib
+    h = hashlib.sha256()
+    src = os.path.join(ROOT, "tcbnn_amd", "csrc")
+    for name in sorted(os.listdir(src)):
+        if name.endswith((".hip", ".h")) and name != "hbm_copy_probe.hip":
+            h.update(name.encode())
+            with open(os.path.join(src, name), "rb") as f:
+                h.update(f.read())
+    return h.hexdigest()
+
+
+def load_measured_traffic():
+    """(bytes per launch by kernel name, stale flag, note)."""
+    try:
+        with open(TRAFFIC_FILE) as f:
+            rec = json.load(f)
+    except (OSError, ValueError):
+        return {}, True, "no traffic file"
+    if rec.get("kernel_source_sha256") != kernel_source_digest():
+        return {}, True, "kernel sources changed since the counters were read (commit %s)" % rec.get("git_commit")
+    return rec.get("bytes_per_launch", {}), False, "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE at commit %s" % rec.get("git_commit")
+
+
+MEASURED_TRAFFIC_BYTES, TRAFFIC_STALE, TRAFFIC_NOTE = {}, True, "not loaded"
 
 
 def layer_work(L, spec=(), res_bytes=None):
@@ -113,6 +125,7 @@ def roofline_of(name, g, variant):
         "unit": "GB/s" if hbm_bound else ("TFLOP/s" if variant == "mfma_f4" else "TOP/s"),
         "frac": round((gbs / HBM_PEAK_GBS) if hbm_bound else (tops / peak_c), 4),
         "traffic": MEASURED_TRAFFIC_BYTES.get(name),
+        "traffic_stale": TRAFFIC_STALE or name not in MEASURED_TRAFFIC_BYTES, "traffic_source": TRAFFIC_NOTE,
         "kernel": name, "launches_per_step": g["launches"],
         "avg_launch_ms": round(g["ms"] / g["launches"], 4),
         "algorithmic_bytes_per_launch": round(g["bytes"] / g["launches"]),
@@ -302,6 +315,11 @@ def main():
         g["ms"] += layer_ms[L["name"]]
         g["launches"] += 1
     by_time = sorted(groups.items(), key=lambda kv: -kv[1]["ms"])
+    global MEASURED_TRAFFIC_BYTES, TRAFFIC_STALE, TRAFFIC_NOTE
+    if args.net == "imagenet_resnet" and batch == 256 and variant == "mfma_f4":  # the workload the file covers
+        MEASURED_TRAFFIC_BYTES, TRAFFIC_STALE, TRAFFIC_NOTE = load_measured_traffic()
+    else:
+        MEASURED_TRAFFIC_BYTES, TRAFFIC_STALE, TRAFFIC_NOTE = {}, True, "no counter run covers this workload"
     roofline = roofline_of(by_time[0][0], by_time[0][1], variant)
     roofline_all = [roofline_of(n, g, variant) for n, g in by_time]
     bit = [g for n, g in groups.items() if g["bops"] > 0]

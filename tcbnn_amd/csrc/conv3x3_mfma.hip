@@ -97,6 +97,44 @@ conv3x3_mfma_f4_kernel(
     const int n0 = ng * (32 * NT);
     const int kw_tot = 9 * p.cw;
 
+    // Kernel arguments that are only used further down are fetched now, together with the first ones: left to
+    // the compiler, each is a scalar load placed right before its first use, i.e. one more exposed round trip
+    // to memory in the set-up of every launch.
+    auto fetch_now = [](auto v) __attribute__((always_inline)) { asm volatile("" ::"s"(v)); };
+    fetch_now(p.out_bits);
+    fetch_now(p.bits_pix_stride);
+    fetch_now(p.bits_row_words);
+    fetch_now(bnp);
+    fetch_now(p.PH);
+    fetch_now(p.OH);
+    if constexpr (RM == RM_RAW) {
+        fetch_now(p.raw_pix_stride);
+        fetch_now(p.raw_b_stride);
+    }
+
+    // ---- the first requests of a workgroup: its channel group's thresholds and weight words.  The filter holds
+    // the weight words in fragment order (64 consecutive words per fragment): all of a wave's words are requested
+    // at once, here, before anything else is worked out, so that their latency runs during the set-up of the tile
+    // loop; they are expanded to FP4 on the way into LDS further down (7 VALU instructions per fragment and lane,
+    // once per workgroup; fetching fragments expanded at pack time moved four times the bytes and took longer).
+    // (Thresholds requested after the weights had been stored were a second memory round trip in every launch.)
+    constexpr int kStagePerWave = (9 * SPT * NT + kWaves - 1) / kWaves;
+    float thr_stage = 0.0f;
+    uint32_t wstage[kStagePerWave];
+    {
+        if (tid < NT * 32) thr_stage = RM != RM_RAW && (FULLT || n0 + tid < p.N) ? bnp[n0 + tid] : 0.0f;
+        const uint32_t* __restrict__ fbits = wgt + (size_t)((p.N + 31) / 32) * 32 * kw_tot;
+#pragma unroll
+        for (int i = 0; i < kStagePerWave; ++i) {
+            const int f = wave + i * kWaves;
+            const int q = f / NT, nt = f % NT;
+            // (the second channel tile of the last group may lie past the padded filter: nothing to read there)
+            wstage[i] = f < 9 * SPT * NT && (FULLT || (ng * NT + nt) * 32 < p.N)
+                            ? fbits[((size_t)(ng * NT + nt) * (9 * SPT) + q) * 64 + lane]
+                            : 0u;
+        }
+    }
+
     // start values of a lane's 16 channels per channel tile (zeros when a residual is added first); filled once
     // the thresholds are staged
     v16f acc0[NT];
@@ -603,27 +641,11 @@ conv3x3_mfma_f4_kernel(
         if (cc.pi < npix) request_residual(cc.y, cc.x, rv[0]);
     }
 
-    // The first activation (and residual) requests are on their way: their latency now runs while the weights
-    // are staged.
-    // ---- stage this channel group's weight fragments and thresholds.  The filter holds the weight words in
-    // fragment order (64 consecutive words per fragment): all of a wave's words are requested at once, then
-    // expanded to FP4 on the way into LDS (7 VALU instructions per fragment and lane, once per workgroup;
-    // fetching fragments expanded at pack time moved four times the bytes and took longer).
-    // The thresholds are requested first, so that their latency runs together with the weights' (requested after
-    // the weights had been stored, they were a second memory round trip in every launch).
-    float thr_stage = 0.0f;
-    if (tid < NT * 32) thr_stage = RM != RM_RAW && (FULLT || n0 + tid < p.N) ? bnp[n0 + tid] : 0.0f;
+    // The first activation (and residual) requests are on their way as well.
+    // ---- expand the weight words into LDS
     {
-        const uint32_t* __restrict__ fbits = wgt + (size_t)((p.N + 31) / 32) * 32 * kw_tot;
-        constexpr int kPerWave = (NQ * NT + kWaves - 1) / kWaves;
-        uint32_t tmp[kPerWave];
-#pragma unroll
-        for (int i = 0; i < kPerWave; ++i) {
-            const int f = wave + i * kWaves;
-            const int q = f / NT, nt = f % NT;
-            // (the second channel tile of the last group may lie past the padded filter: nothing to read there)
-            tmp[i] = f < NQ * NT && (FULLT || (ng * NT + nt) * 32 < p.N) ? fbits[((size_t)(ng * NT + nt) * NQ + q) * 64 + lane] : 0u;
-        }
+        constexpr int kPerWave = kStagePerWave;
+        const uint32_t* tmp = wstage;
 #pragma unroll
         for (int i = 0; i < kPerWave; ++i) {
             const int f = wave + i * kWaves;

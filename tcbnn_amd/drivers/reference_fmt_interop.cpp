@@ -15,7 +15,7 @@ static std::vector<T> to_host(const T* dev, size_t n) {
 }
 
 int main(int argc, char** argv) {
-    driver::Options o = driver::parse(argc, argv, "reference_fmt_interop [--batch N] [--seed S] [--variant V]");
+    driver::Options o = driver::parse(argc, argv, "reference_fmt_interop [--batch N] [--seed S] [--variant V] [--oversize-input]");
     HIP_SAFE_CALL(hipSetDevice(0));
     const unsigned batch = o.batch ? o.batch : 12, image = 16, ch = 64, n_hidden = 256, classes = 10;
 
@@ -112,6 +112,38 @@ int main(int argc, char** argv) {
                 logits[0] == logits[1] ? "same" : "DIFFER", tiles[0] == tiles[1] ? "same" : "DIFFER",
                 resid[0] == resid[1] ? "same" : "DIFFER");
         return 1;
+    }
+    // A second batch through the same first-layer object: set_input() must give what a freshly initialized layer
+    // gives on that batch, and must refuse (print + exit(-1)) a batch beyond the bound the 16-bit residual format
+    // was chosen for at initialize().
+    {
+        const float* cursor = syn.values.data();
+        tcbnn_host::ConfigSource cfg(&cursor, syn.values.data() + syn.values.size());
+        InConv128LayerParam stem("Conv1", image, image, 3, 3, 3, ch, batch, 1, 1, true, 1, 1, true);
+        stem.initialize(images.data(), cfg);
+        std::vector<float> half(images);
+        for (float& v : half) v *= 0.5f;
+        stem.set_input(half.data());
+        stem.forward(stream);
+        uin32* t = stem.download_output();
+        std::vector<uin32> got(t, t + (size_t)stem.output_bit_size() * 4);
+        const float* cursor2 = syn.values.data();
+        tcbnn_host::ConfigSource cfg2(&cursor2, syn.values.data() + syn.values.size());
+        InConv128LayerParam fresh("Conv1", image, image, 3, 3, 3, ch, batch, 1, 1, true, 1, 1, true);
+        fresh.initialize(half.data(), cfg2);
+        fresh.forward(stream);
+        uin32* t2 = fresh.download_output();
+        if (got != std::vector<uin32>(t2, t2 + (size_t)fresh.output_bit_size() * 4)) {
+            fprintf(stderr, "Conv1: set_input() and a fresh initialize() disagree on the same batch\n");
+            return 1;
+        }
+        if (o.oversize_input) {
+            std::vector<float> big(images);
+            for (float& v : big) v *= 1000.0f;
+            stem.set_input(big.data());  // must not return
+            fprintf(stderr, "Conv1: set_input() accepted a batch beyond the residual bound\n");
+            return 1;
+        }
     }
     long long nz = 0;
     for (int v : resid[0]) nz += v != 0;

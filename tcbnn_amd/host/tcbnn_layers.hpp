@@ -516,6 +516,28 @@ class InConv128LayerParam {  // param.h:701-870
         }
         return this;
     }
+    // A new batch for the same layer objects (the reference's objects are single-shot, this engine's are not):
+    // uploads `input` into input_gpu.  The format of the saved residual, and of every residual downstream of it,
+    // was chosen at initialize() from the largest |value| of the first batch; a batch that exceeds the bound the
+    // format was proven for would wrap in 16 bits, so it is refused (print + exit, like every error here).
+    void set_input(float* input) {
+        CHECK_NULL_POINTER(input);
+        CHECK_NULL_POINTER(input_gpu);
+        if (save_residual) {
+            float input_abs_max = 0.0f;
+            for (int i = 0; i < input_size(); ++i) {
+                const float a = input[i] < 0 ? -input[i] : input[i];
+                if (!(a <= input_abs_max)) input_abs_max = a;  // also catches NaN
+            }
+            if (tcbnn_inconv_residual_bound(filter_height, filter_width, input_abs_max) > residual_info.bound) {
+                fprintf(stderr, "Error: set_input: |input| exceeds the bound the residual formats were chosen for "
+                                "(initialize the layers with the batch of largest magnitude).\n");
+                exit(-1);
+            }
+        }
+        this->input = input;
+        HIP_SAFE_CALL(hipMemcpy(input_gpu, input, input_bytes(), hipMemcpyHostToDevice));
+    }
     uin32* get_output_gpu() { return this->output_gpu; }
     int* get_output_residual_gpu() { return this->output_residual_gpu; }
     void forward(hipStream_t stream = 0) {

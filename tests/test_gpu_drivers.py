@@ -160,3 +160,14 @@ def test_reference_layout_accessors_of_the_cpp_classes(gpu, tmp_path, variant):
                           stderr=subprocess.STDOUT, text=True, timeout=120)
     assert proc.returncode == 0, proc.stdout
     assert '"ok": true' in proc.stdout and '"c2_residual_nonzero": 0,' not in proc.stdout
+
+
+def test_first_layer_set_input_refuses_a_batch_beyond_its_residual_bound(gpu):
+    """The C++ first layer picks 16-bit residual storage from the first batch's largest |value|; a later batch
+    that exceeds that bound must end in the reference's error convention (message + exit(-1)), not in wrapped
+    residuals.  (The same binary, without the flag, checks that an admissible second batch gives what a fresh
+    layer gives: the test above.)"""
+    exe = os.path.join(BIN, "reference_fmt_interop")
+    proc = subprocess.run([exe, "--batch", "12", "--seed", "3", "--oversize-input"], stdout=subprocess.PIPE,
+                          stderr=subprocess.PIPE, text=True, timeout=120)
+    assert proc.returncode == 255 and "exceeds the bound" in proc.stderr, (proc.returncode, proc.stderr)
