@@ -82,6 +82,11 @@ conv3x3_mfma_f4_kernel(
     extern __shared__ v4i lds_dyn[];
     v4i* lds_w = lds_dyn;  // [NQ][NT][64] fragments
     float* lds_thr = reinterpret_cast<float*>(lds_dyn + NQ * NT * 64);  // [NT*32]
+    // RM_RAW with short K (the output-bound shapes): a wave's private [32 images][kRawPitch] int32 staging area, through
+    // which a 32-image tile's sums are transposed so that every store writes whole contiguous channel runs
+    constexpr bool kRawTranspose = RM == RM_RAW && SPT <= 2 && NT == 2 && FULLT;
+    constexpr int kRawPitch = 32 * NT + 4;  // words per image row: the odd multiple of 4 keeps both directions conflict-free
+    int* lds_raw = reinterpret_cast<int*>(lds_thr + NT * 32);
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -453,6 +458,7 @@ conv3x3_mfma_f4_kernel(
                         __builtin_amdgcn_raw_buffer_store_b128(q[g], r_rout, (int)vo, (int)(so + 16u * (unsigned)g), 0);
                     }
                     asm volatile("s_nop 4" ::"v"(q[0]), "v"(q[1]), "v"(q[2]), "v"(q[3]));  // see the residual stores
+                    __builtin_amdgcn_sched_barrier(0);
                 } else {
 #pragma unroll
                     for (int v = 0; v < 16; ++v)
@@ -570,10 +576,57 @@ conv3x3_mfma_f4_kernel(
         }
     };
 
+    // int32 output [N][P][Q][O] (bmma_kernel.cu:247-263): for one image and pixel the wave's 32 NT channels are one
+    // contiguous run, but in the accumulator a lane holds 16 channels of ONE image, so a direct store scatters
+    // 16-byte pieces over 64 different rows per instruction.  The sums of a 32-image tile go through the wave's LDS
+    // area instead (row = image, conflict-free both ways) and leave as 128-bit stores in which 16 consecutive lanes
+    // cover one image's whole run (4 images, i.e. 4 runs of 256 bytes, per instruction).
+    auto epilogue_raw_transposed = [&](unsigned pix) __attribute__((always_inline)) {
+        if constexpr (kRawTranspose) {
+            int* mine = lds_raw + wave * (32 * kRawPitch);
+            const int rl = lane >> 4, cl = lane & 15;  // image within a group of 4, 16-byte column of the run
+            const unsigned so0 = (pix * (unsigned)p.raw_pix_stride + (unsigned)n0) * 4u;  // uniform
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        *reinterpret_cast<v4i*>(mine + j * kRawPitch + nt * 32 + 16 * h + 4 * g) =
+                            v4i{(int)acc[mt][nt][4 * g], (int)acc[mt][nt][4 * g + 1], (int)acc[mt][nt][4 * g + 2],
+                                (int)acc[mt][nt][4 * g + 3]};
+                        __builtin_amdgcn_sched_barrier(0);  // convert and write four at a time (registers)
+                    }
+                // (same wave writes and reads: program order and the wait for LDS are all the synchronisation)
+                const int img0 = (bg * MT + mt) * 32;
+                // four rows at a time: eight would not fit the register file next to the activation buffers
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {
+                    v4i q[4];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k)
+                        q[k] = *reinterpret_cast<const v4i*>(mine + (16 * half + 4 * k + rl) * kRawPitch + 4 * cl);
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const int img = img0 + 16 * half + 4 * k + rl;
+                        const unsigned vo = img < p.B ? ((unsigned)img * (unsigned)p.raw_b_stride + 4u * (unsigned)cl) * 4u : kOutOfRange;
+                        __builtin_amdgcn_raw_buffer_store_b128(q[k], r_rout, (int)vo, (int)so0, 0);
+                    }
+                    asm volatile("s_nop 4" ::"v"(q[0]), "v"(q[1]), "v"(q[2]), "v"(q[3]));  // see the residual stores
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        }
+    };
+
     // (yy, xx): the output pixel, or the window when pooled (sub = pixel of the window, 3 = last)
     auto epilogue = [&](int yy, int xx, int sub, int (*rv)[NW]) __attribute__((always_inline)) {
         const unsigned pix = (unsigned)yy * (unsigned)roww + (unsigned)xx;
         const unsigned bits_pix = pix * (unsigned)p.bits_pix_stride * 4u;  // uniform
+        if constexpr (kRawTranspose) {  // (the host only picks this instantiation for 16-byte aligned outputs)
+            epilogue_raw_transposed(pix);
+            return;
+        }
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
             const int cb = n0 + nt * 32;
@@ -781,7 +834,9 @@ TensorBytes tensor_bytes(const BgemmParams& p) {
 template <int SPT, int RM, int MT, int NT, bool R16, bool POOL, bool FULLT>
 int launch_f(const BgemmParams& p, hipStream_t stream) {
     constexpr int NQ = 9 * SPT;
-    const size_t lds_bytes = (size_t)NQ * NT * 64 * 16 + NT * 32 * sizeof(float);
+    constexpr bool kRawTranspose = RM == RM_RAW && SPT <= 2 && NT == 2 && FULLT;  // as in the kernel
+    const size_t lds_bytes = (size_t)NQ * NT * 64 * 16 + NT * 32 * sizeof(float) +
+                             (kRawTranspose ? (size_t)kWaves * 32 * (32 * NT + 4) * sizeof(int) : 0);
     // Per instantiation and device, set up by the first launch there: the dynamic LDS limit, and how many of its
     // workgroups a CU holds at once (registers and LDS).  Atomics only so that two host threads that both find the
     // entry empty do no harm (both store the same value).
@@ -836,7 +891,10 @@ int launch_f(const BgemmParams& p, hipStream_t stream) {
 template <int SPT, int RM, int MT, int NT, bool R16, bool POOL>
 int launch_t(const BgemmParams& p, hipStream_t stream) {
     const int res_lim = p.res_in != nullptr ? std::min(std::min(p.res_limit, p.res_in_ch), p.N) : 0;
-    if (p.N % (32 * NT) == 0 && res_lim % 32 == 0) return launch_f<SPT, RM, MT, NT, R16, POOL, true>(p, stream);
+    // (with the int32 output, that instantiation also stores whole 128-bit words: the output must be aligned for them)
+    const bool raw_ok = RM != RM_RAW || (p.raw_pix_stride % 4 == 0 && p.raw_b_stride % 4 == 0 &&
+                                         (reinterpret_cast<uintptr_t>(p.out_i32) & 15) == 0);
+    if (p.N % (32 * NT) == 0 && res_lim % 32 == 0 && raw_ok) return launch_f<SPT, RM, MT, NT, R16, POOL, true>(p, stream);
     return launch_f<SPT, RM, MT, NT, R16, POOL, false>(p, stream);
 }
 
@@ -911,7 +969,9 @@ bool conv3x3_mfma_applicable(const BgemmParams& p) {
 void conv3x3_mfma_kernel_name(const BgemmParams& p, char* buf, size_t len) {
     const Pick k = pick(p);
     const int res_lim = p.res_in != nullptr ? std::min(std::min(p.res_limit, p.res_in_ch), p.N) : 0;
-    const bool full = p.N % (32 * k.nt) == 0 && res_lim % 32 == 0;
+    const bool raw_ok = k.rm != RM_RAW || (p.raw_pix_stride % 4 == 0 && p.raw_b_stride % 4 == 0 &&
+                                           (reinterpret_cast<uintptr_t>(p.out_i32) & 15) == 0);
+    const bool full = p.N % (32 * k.nt) == 0 && res_lim % 32 == 0 && raw_ok;
     snprintf(buf, len, "conv3x3_mfma_f4_kernel<%d, %d, %d, %d, %s, %s, %s>", p.cw / 2, k.rm, k.mt, k.nt,
              k.r16 ? "true" : "false", k.pool ? "true" : "false", full ? "true" : "false");
 }
