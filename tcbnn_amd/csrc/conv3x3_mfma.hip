@@ -859,14 +859,17 @@ int launch_f(const BgemmParams& p, hipStream_t stream) {
     const int n_groups = (p.N + 32 * NT - 1) / (32 * NT);
     const int b_groups = (p.B + 32 * MT - 1) / (32 * MT);
     const int quads = ((POOL ? p.OH * p.OW : p.PH * p.PW) + kWaves - 1) / kWaves;  // items of the four waves
-    // Persistent workgroups, all resident at once: two per CU (three for Cin = 256 with one tile per wave), fewer
+    // Persistent workgroups, all resident at once: two per CU (three for residual layers), fewer
     // when registers or LDS hold fewer.  Measured on every layer of ResNet-18 at batch 256: more, shorter-lived
     // workgroups stage the weights more often and lose; and a grid even slightly larger than the resident slots
     // loses more (its last workgroups start, stage and ramp up only when the first ones have finished: the 14 x 14
     // and 7 x 7 layers ran 10-18 % longer with 1.5 rounds than with one round of workgroups that each take two
     // items per wave).  So: as many pixel streams as fit in one round, never more.
     static const int wg_env = getenv("TCBNN_WG_PER_CU") ? atoi(getenv("TCBNN_WG_PER_CU")) : 0;  // tuning switch
-    const int wg_want = wg_env > 0 ? wg_env : (SPT == 4 && NT == 1 && MT == 1 ? 3 : 2);
+    // Residual layers with one image tile per wave are bound by HBM: a third workgroup per CU, where registers and
+    // LDS hold one (`resident`), keeps more requests in flight (stage-1 and stage-2 layers of ResNet-18: -3 to -8 %).
+    constexpr bool kResLayer = RM == RM_PLAIN || RM == RM_POOLED;
+    const int wg_want = wg_env > 0 ? wg_env : (kResLayer && MT == 1 ? 3 : 2);
     const int wg_per_cu = std::max(1, std::min(wg_want, resident));
     const int best = std::max(1, std::min(cus * wg_per_cu / (n_groups * b_groups), quads));
     // channels that receive an injected residual: o < residual_channels, and only those the
