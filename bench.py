@@ -71,7 +71,7 @@ def layer_work(L, spec=(), res_bytes=None):
     """Algorithmic work of one layer launch: binary ops (2 per +-1 multiply-accumulate, border taps
     included), fp32 adds of the first layer, and the HBM bytes the launch has to move once
     (inputs + outputs + weights, packed activations at 1 bit per value, residuals at the width
-    they are stored in: res_bytes[layer name] = 2 or 4 bytes per value of that layer's saved
+    they are stored in: res_bytes[layer name] = 1.5, 2 or 4 bytes per value of that layer's saved
     residual, 4 = the reference's int32 when not given)."""
     res_bytes = res_bytes or {}
     from tcbnn_amd import nets
@@ -300,7 +300,8 @@ def main():
     layer_ms = {k: float(np.median(v)) for k, v in per_layer.items()}
 
     # width each saved residual is stored in (16 bits where its bound proves that exact)
-    res_bytes = {L["name"]: (2 if net.layers[L["name"]].output_residual_gpu.format == _lib.RES_I16 else 4)
+    width = {_lib.RES_I32: 4, _lib.RES_I16: 2, _lib.RES_I12: 1.5}
+    res_bytes = {L["name"]: width[net.layers[L["name"]].output_residual_gpu.format]
                  for L in spec if L.get("save_residual") or (L["kind"] == "pool" and L.get("res_src"))}
     # group launches by device kernel, as a profiler does
     groups = {}
@@ -382,8 +383,11 @@ def main():
                                              "imagenet_vgg": "imagenet_vgg.cu:217-286",
                                              "imagenet_resnet_textbook": "no reference driver"}[args.net], batch),
                    "variant": variant, "layers": len(spec), "launch": "hip graph replay" if args.graph else "eager",
-                   "residual_storage": ("int16 where the bound of |residual| proves it exact (%d of %d tensors), "
-                                        "else int32" % (sum(1 for v in res_bytes.values() if v == 2), len(res_bytes)))
+                   "residual_storage": ("the narrowest width the bound of |residual| proves exact: 12 bits for %d, "
+                                        "16 bits for %d, int32 for %d of %d tensors"
+                                        % (sum(1 for v in res_bytes.values() if v == 1.5),
+                                           sum(1 for v in res_bytes.values() if v == 2),
+                                           sum(1 for v in res_bytes.values() if v == 4), len(res_bytes)))
                    if res_bytes else "none"},
         "binary_tops": round(bops * args.steps / wall / 1e12, 2),
         "binary_ops_per_step": bops, "fp32_first_layer_flops_per_step": flops,

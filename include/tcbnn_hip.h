@@ -72,6 +72,11 @@ extern "C" {
  * this ABI track it from the actual input data).  Producer and consumer must agree. */
 #define TCBNN_RES_I32 0
 #define TCBNN_RES_I16 1
+/* 12 bits per value, for tensors whose bound is <= 2047 (the first layer's and the first stage's of a ResNet on
+ * normalised images: they are the largest tensors of the path).  Groups of 16 channels: the 192-bit string that
+ * holds value e (two's complement) at bits 12e..12e+11 is stored as words w0..w5, laid out per pixel and group as
+ * uint32 [B][4] (w0..w3 of every image) followed by uint32 [B][2] (w4, w5): 24 bytes per image, pixel and group. */
+#define TCBNN_RES_I12 2
 
 /* ------------------------------------------------------------------ misc */
 int tcbnn_abi_version(void);
@@ -104,10 +109,18 @@ size_t tcbnn_residual_bytes(int height, int width, int channels, int batch, int 
  * (R*S*3 terms plus rounding slack), and of a bit convolution that adds its own
  * Cin*R*S to an injected residual bounded by injected_bound (0 if none).  INT32_MAX
  * when unknown (non-finite input_abs_max, overflow).  tcbnn_residual_format_for_bound:
- * TCBNN_RES_I16 when 0 <= bound <= 32767, else TCBNN_RES_I32. */
+ * TCBNN_RES_I16 when 0 <= bound <= 32767, else TCBNN_RES_I32.  tcbnn_residual_format_narrowest also
+ * considers TCBNN_RES_I12: 0 <= bound <= 2047 and an even batch (its 128-bit pieces are then aligned).
+ * tcbnn_inconv_residual_bound_of_input is the first layer's bound from the actual batch (HOST pointer,
+ * float [batch][3][height][width]): the largest sum of |x| over any filter window, plus rounding slack;
+ * far tighter than R*S*3*max|x| on real images, which is what lets the first stage use 12 bits. */
 int tcbnn_inconv_residual_bound(int filter_height, int filter_width, float input_abs_max);
+int tcbnn_inconv_residual_bound_of_input(const float* input_host, int batch, int height, int width,
+                                         int filter_height, int filter_width, int stride_height,
+                                         int stride_width, int padding);
 int tcbnn_conv_residual_bound(int input_channels, int filter_height, int filter_width, int injected_bound);
 int tcbnn_residual_format_for_bound(int bound);
+int tcbnn_residual_format_narrowest(int bound, int batch);
 
 /* ------------------------------------------------- one-time weight packing */
 /* fp32 [K][N] (param.h:58-59) -> packed [NPAD32][KW128].  Replaces

@@ -100,6 +100,8 @@ ABI = {
     "tcbnn_inconv_residual_bound": (c_int, [c_int, c_int, C.c_float]),
     "tcbnn_conv_residual_bound": (c_int, [c_int] * 4),
     "tcbnn_residual_format_for_bound": (c_int, [c_int]),
+    "tcbnn_residual_format_narrowest": (c_int, [c_int, c_int]),
+    "tcbnn_inconv_residual_bound_of_input": (c_int, [c_void_p] + [c_int] * 8),
     "tcbnn_pack_fc_weight": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "tcbnn_pack_conv_filter": (c_int, [c_void_p, c_void_p] + [c_int] * 4 + [c_void_p]),
     "tcbnn_pack_inconv_filter": (c_int, [c_void_p, c_void_p] + [c_int] * 4 + [c_void_p]),
@@ -135,7 +137,7 @@ for _name, (_res, _args) in ABI.items():
 
 VARIANT_AUTO, VARIANT_POPC, VARIANT_MFMA_I8, VARIANT_MFMA_F4 = 0, 1, 2, 3
 VARIANTS = {"auto": 0, "popc": 1, "mfma_i8": 2, "mfma_f4": 3}
-RES_I32, RES_I16 = 0, 1
+RES_I32, RES_I16, RES_I12 = 0, 1, 2
 INT32_MAX = 2 ** 31 - 1
 
 

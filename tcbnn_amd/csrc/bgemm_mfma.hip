@@ -289,7 +289,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(MT == 
                             const size_t ngrp = r16 ? (p.res_in_ch + 7) / 8 : (p.res_in_ch + 3) / 4;
                             const int4* __restrict__ src = reinterpret_cast<const int4*>(rin);
                             auto fetch = [&](size_t sp, int* dst) {
-                                if (r16) {
+                                if (p.res_in_fmt == TCBNN_RES_I12) {  // the lane's 16 channels are one 12-bit group
+                                    residual_load_group16(rin, TCBNN_RES_I12, sp, p.res_in_ch, cbase / 16, p.B, bb, dst);
+                                } else if (r16) {
                                     const size_t g0 = (sp * ngrp + cbase / 8) * p.B + bb;
 #pragma unroll
                                     for (int g = 0; g < 2; ++g) {
@@ -354,7 +356,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(MT == 
                         // a lane's 16 channels are whole 16-byte groups of the residual layouts: 128-bit stores
                         if (rout != nullptr && b_ok && cbase < p.N) {
                             int4* __restrict__ dst = reinterpret_cast<int4*>(rout);
-                            if (p.res_out_fmt == TCBNN_RES_I16) {
+                            if (p.res_out_fmt == TCBNN_RES_I12) {
+                                residual_store_group16(rout, TCBNN_RES_I12, pix, p.N, cbase / 16, p.B, b, resv);
+                            } else if (p.res_out_fmt == TCBNN_RES_I16) {
                                 const size_t g0 = (pix * (size_t)((p.N + 7) / 8) + cbase / 8) * p.B + b;
 #pragma unroll
                                 for (int g = 0; g < 2; ++g)

@@ -282,6 +282,7 @@ __global__ __launch_bounds__(kThreads)
                 }
                 const float* __restrict__ bn = bnp;
                 int32_t* __restrict__ rout = p.res_out;
+                const bool by_group = KM == KM_THRESH_RES && rout != nullptr && p.res_out_fmt == TCBNN_RES_I12;
 #pragma unroll
                 for (int n = 0; n < kNTile; ++n) {
                     const int ch = n0 + n;
@@ -290,7 +291,10 @@ __global__ __launch_bounds__(kThreads)
                         int res = base - 2 * acc[r][n];
                         if constexpr (KM == KM_THRESH_RES) {
                             res += rv[n];
-                            if (rout != nullptr) residual_store(rout, p.res_out_fmt, pix, p.N, ch, p.B, b, res);
+                            if (by_group)
+                                rv[n] = res;  // 12-bit values share words: the tile's two groups are stored whole below
+                            else if (rout != nullptr)
+                                residual_store(rout, p.res_out_fmt, pix, p.N, ch, p.B, b, res);
                         }
                         if constexpr (KM == KM_THRESH_FC)
                             bit = (float)res >= bn[ch] ? 1u : 0u;
@@ -298,6 +302,14 @@ __global__ __launch_bounds__(kThreads)
                             bit = (float)res < bn[ch] ? 0u : 1u;
                     }
                     word = word + word + bit;  // shift the next channel in (MSB first)
+                }
+                if constexpr (KM == KM_THRESH_RES) {
+                    if (by_group) {
+#pragma unroll
+                        for (int g = 0; g < 2; ++g)
+                            if (n0 + 16 * g < p.N)
+                                residual_store_group16(rout, TCBNN_RES_I12, pix, p.N, (n0 >> 4) + g, p.B, b, &rv[16 * g]);
+                    }
                 }
                 outword[r] |= word;
             } else if constexpr (KM == KM_AFFINE) {

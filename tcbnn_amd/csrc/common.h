@@ -46,7 +46,7 @@ int resolve_variant(int requested);
 // residual and output access one contiguous run):
 //   activations  uint32 [H][W][cw][B]
 //   weights      uint32 [npad32][taps*cw]
-//   residuals    int32 [P][Q][ceil(O/4)][B][4] or int16 [P][Q][ceil(O/8)][B][8]
+//   residuals    int32 [P][Q][ceil(O/4)][B][4], int16 [P][Q][ceil(O/8)][B][8] or 12-bit groups of 16 channels
 // ---------------------------------------------------------------------------
 enum EpilogueMode : int {
     EPI_THRESH = 0,  // threshold -> bit, OR over the pool window, packed store
@@ -92,18 +92,61 @@ struct BgemmParams {
     int ws_is_dot;  // workspace holds +-1 dot products (matrix-core engines) instead of popcounts
 };
 
-// One residual value in either storage format.  Both interleave small groups of channels below
-// the batch index, so that a lane (= image) reads or writes 16 contiguous bytes per access:
+// One residual value in any storage format.  All of them interleave small groups of channels below the batch
+// index, so that a lane (= image) reads or writes whole 16- or 8-byte pieces and consecutive lanes are contiguous:
 //   TCBNN_RES_I32: int32 [pix][ceil(ch/4)][B][4]     TCBNN_RES_I16: int16 [pix][ceil(ch/8)][B][8]
+//   TCBNN_RES_I12: groups of 16 channels, 12 bits each = 192 bits = six words w0..w5 per image, value e at bits
+//                  12e..12e+11 of that string (two's complement); stored as [pix][ceil(ch/16)] x { uint32 [B][4]
+//                  (w0..w3), then uint32 [B][2] (w4, w5) }: 24 B bytes per (pixel, group)
+__host__ __device__ constexpr inline size_t residual_group_channels(int fmt) {
+    return fmt == TCBNN_RES_I12 ? 16 : (fmt == TCBNN_RES_I16 ? 8 : 4);
+}
+__host__ __device__ constexpr inline size_t residual_group_bytes(int fmt) { return fmt == TCBNN_RES_I12 ? 24 : 16; }
+__host__ __device__ constexpr inline bool residual_format_known(int fmt) {
+    return fmt == TCBNN_RES_I32 || fmt == TCBNN_RES_I16 || fmt == TCBNN_RES_I12;
+}
+// word k (0..5) of group g of image b at pixel pix of a 12-bit tensor with G groups per pixel
+__device__ __forceinline__ size_t i12_word_index(size_t pix, size_t G, int g, int batch, int b, int k) {
+    const size_t base = (pix * G + (size_t)g) * (size_t)batch * 6;
+    return k < 4 ? base + (size_t)b * 4 + k : base + (size_t)batch * 4 + (size_t)b * 2 + (k - 4);
+}
+// eight 12-bit values <-> three words (a 16-channel group is two such units: w0..w2 and w3..w5)
+__device__ __forceinline__ void i12_unpack8(uint32_t d0, uint32_t d1, uint32_t d2, int* v) {
+    v[0] = ((int)(d0 << 20)) >> 20;
+    v[1] = ((int)(d0 << 8)) >> 20;
+    v[2] = ((int)__builtin_amdgcn_alignbit(d1, d0, 24) << 20) >> 20;
+    v[3] = ((int)(d1 << 16)) >> 20;
+    v[4] = ((int)(d1 << 4)) >> 20;
+    v[5] = ((int)__builtin_amdgcn_alignbit(d2, d1, 28) << 20) >> 20;
+    v[6] = ((int)(d2 << 12)) >> 20;
+    v[7] = (int)d2 >> 20;
+}
+__device__ __forceinline__ void i12_pack8(const int* v, uint32_t& d0, uint32_t& d1, uint32_t& d2) {
+    const uint32_t m = 0xfffu;
+    d0 = ((uint32_t)v[0] & m) | (((uint32_t)v[1] & m) << 12) | ((uint32_t)v[2] << 24);
+    d1 = (((uint32_t)v[2] & m) >> 8) | (((uint32_t)v[3] & m) << 4) | (((uint32_t)v[4] & m) << 16) | ((uint32_t)v[5] << 28);
+    d2 = (((uint32_t)v[5] & m) >> 4) | (((uint32_t)v[6] & m) << 8) | ((uint32_t)v[7] << 20);
+}
 __device__ __forceinline__ size_t residual_index(int fmt, size_t pix, int channels, int c, int batch, int b) {
     if (fmt == TCBNN_RES_I16) return ((pix * (size_t)((channels + 7) / 8) + (c >> 3)) * batch + b) * 8 + (c & 7);
     return ((pix * (size_t)((channels + 3) / 4) + (c >> 2)) * batch + b) * 4 + (c & 3);
 }
 __device__ __forceinline__ int residual_load(const int32_t* __restrict__ base, int fmt, size_t pix, int channels,
                                              int c, int batch, int b) {
+    if (fmt == TCBNN_RES_I12) {
+        const uint32_t* w = reinterpret_cast<const uint32_t*>(base);
+        const size_t G = (size_t)((channels + 15) / 16);
+        const int g = c >> 4, bit = 12 * (c & 15), k = bit >> 5, sh = bit & 31;
+        const uint32_t lo = w[i12_word_index(pix, G, g, batch, b, k)];
+        const uint32_t hi = sh > 20 ? w[i12_word_index(pix, G, g, batch, b, k + 1)] : 0u;  // the value straddles two words
+        const uint64_t both = ((uint64_t)hi << 32) | lo;
+        return ((int)((uint32_t)(both >> sh) << 20)) >> 20;
+    }
     const size_t i = residual_index(fmt, pix, channels, c, batch, b);
     return fmt == TCBNN_RES_I16 ? (int)reinterpret_cast<const int16_t*>(base)[i] : base[i];
 }
+// Stores of single values exist for the 32- and 16-bit formats only (a 12-bit value shares its words with its
+// neighbours); every producer writes whole groups of a 12-bit tensor with residual_store_group16.
 __device__ __forceinline__ void residual_store(int32_t* __restrict__ base, int fmt, size_t pix, int channels, int c,
                                                int batch, int b, int v) {
     const size_t i = residual_index(fmt, pix, channels, c, batch, b);
@@ -111,6 +154,38 @@ __device__ __forceinline__ void residual_store(int32_t* __restrict__ base, int f
         reinterpret_cast<int16_t*>(base)[i] = (int16_t)v;
     else
         base[i] = v;
+}
+// Channels 16g .. 16g+15 of one image and pixel (values of channels >= `channels` are whatever the caller passes;
+// consumers never look at them), in any format.
+__device__ __forceinline__ void residual_store_group16(int32_t* __restrict__ base, int fmt, size_t pix, int channels,
+                                                       int g, int batch, int b, const int* v) {
+    if (fmt == TCBNN_RES_I12) {
+        uint32_t* w = reinterpret_cast<uint32_t*>(base);
+        const size_t G = (size_t)((channels + 15) / 16);
+        uint32_t d[6];
+        i12_pack8(v, d[0], d[1], d[2]);
+        i12_pack8(v + 8, d[3], d[4], d[5]);
+        *reinterpret_cast<uint4*>(w + i12_word_index(pix, G, g, batch, b, 0)) = make_uint4(d[0], d[1], d[2], d[3]);
+        *reinterpret_cast<uint2*>(w + i12_word_index(pix, G, g, batch, b, 4)) = make_uint2(d[4], d[5]);
+        return;
+    }
+#pragma unroll
+    for (int e = 0; e < 16; ++e)
+        if (16 * g + e < channels) residual_store(base, fmt, pix, channels, 16 * g + e, batch, b, v[e]);
+}
+__device__ __forceinline__ void residual_load_group16(const int32_t* __restrict__ base, int fmt, size_t pix, int channels,
+                                                      int g, int batch, int b, int* v) {
+    if (fmt == TCBNN_RES_I12) {
+        const uint32_t* w = reinterpret_cast<const uint32_t*>(base);
+        const size_t G = (size_t)((channels + 15) / 16);
+        const uint4 a = *reinterpret_cast<const uint4*>(w + i12_word_index(pix, G, g, batch, b, 0));
+        const uint2 c2 = *reinterpret_cast<const uint2*>(w + i12_word_index(pix, G, g, batch, b, 4));
+        i12_unpack8(a.x, a.y, a.z, v);
+        i12_unpack8(a.w, c2.x, c2.y, v + 8);
+        return;
+    }
+#pragma unroll
+    for (int e = 0; e < 16; ++e) v[e] = 16 * g + e < channels ? residual_load(base, fmt, pix, channels, 16 * g + e, batch, b) : 0;
 }
 
 int launch_bgemm_popc(const BgemmParams& p, hipStream_t stream);

@@ -57,14 +57,14 @@ constexpr int RM_RAW = 3;     // no threshold: the +-1 dot products are stored a
 constexpr int waves_hint(int spt, int rm, int nt) { return rm == RM_PLAIN && spt == 4 && nt == 1 ? 3 : 2; }
 
 // SPT = k-steps (64 bits) per filter tap = Cin / 64; MT = 32-image tiles per wave (2 for plain
-// layers, 1 for residual layers); NT = 32-channel tiles per wave; R16 = the injected residual is
-// stored as int16 (half the registers hold it while it is in flight); POOL = 2x2 OR-pooling of the
+// layers, 1 for residual layers); NT = 32-channel tiles per wave; RF = TCBNN_RES_* format of the
+// injected residual (the narrower, the fewer registers hold it while it is in flight); POOL = 2x2 OR-pooling of the
 // output bits (kernel.cuh:797-816): a wave multiplies the four pixels of a window one after the
 // other and stores the OR of their words once.  FULLT = every 32-channel tile of the launch exists in full
 // and, with an injected residual, lies entirely below or entirely above the channel limit: the per-channel
 // tests of partial tiles are then not even compiled (they cost scalar registers and set-up instructions in
 // every launch, and the networks' channel counts are multiples of 64).
-template <int SPT, int RM, int MT, int NT, bool R16, bool POOL, bool FULLT>
+template <int SPT, int RM, int MT, int NT, int RF, bool POOL, bool FULLT>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(waves_hint(SPT, RM, NT)))) void
 conv3x3_mfma_f4_kernel(
     const BgemmParams p, const uint32_t* __restrict__ act, const uint32_t* __restrict__ wgt,
@@ -343,15 +343,19 @@ conv3x3_mfma_f4_kernel(
     // that raw form until its epilogue, a pooled one is reduced to 16 ints by finish_residual.
     constexpr int NRV = kRes ? MT * NT : 1;
     constexpr int NTMP = RM == RM_POOLED ? 3 : 1;
-    constexpr int NRAW = R16 ? 8 : 16;                    // words loaded per channel tile
+    constexpr bool R16 = RF == TCBNN_RES_I16, R12 = RF == TCBNN_RES_I12;  // format of the injected tensor
+    constexpr int NRAW = R12 ? 6 : (R16 ? 8 : 16);        // words loaded per channel tile
     constexpr int NW = RM == RM_POOLED ? 16 : NRAW;       // words kept per channel tile
     int tmp[NTMP][NRV][NRAW];  // pooled: the other three pixels of the 2x2 window
-    // A lane's 16 channels are 4 groups of 4 (int32) or 2 groups of 8 (int16): 16 bytes each.
+    // A lane's 16 channels are 4 groups of 4 (int32) or 2 groups of 8 (int16), 16 bytes each, or one 12-bit group
+    // of 24 bytes (a 16-byte piece in the group's first plane, an 8-byte piece in its second).
     unsigned lane_off[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
-        lane_off[mt] = ((unsigned)((R16 ? 2 : 4) * h) * (unsigned)p.B + (unsigned)bload[mt]) * 16u;
-    const unsigned grp_b = (unsigned)p.B * 16u;  // bytes between consecutive channel groups
+        lane_off[mt] = R12 ? (unsigned)h * (unsigned)p.B * 24u + (unsigned)bload[mt] * 16u
+                           : ((unsigned)((R16 ? 2 : 4) * h) * (unsigned)p.B + (unsigned)bload[mt]) * 16u;
+    const unsigned grp_b = (unsigned)p.B * 16u;  // bytes between consecutive channel groups (32- and 16-bit formats)
+    const unsigned g12_b = (unsigned)p.B * 24u;  // bytes of a 12-bit group of 16 channels
 
     auto request_residual = [&](int yy, int xx, int (*rv)[NW]) __attribute__((always_inline)) {
         if constexpr (kRes) {
@@ -371,6 +375,26 @@ conv3x3_mfma_f4_kernel(
                 // a channel tile that receives no residual (uniform) reads zeros through an out-of-range
                 // offset: no branch, no memory traffic
                 const unsigned loff = cb < res_lim ? lane_off[sl / NT] : kOutOfRange;
+                if constexpr (R12) {
+                    // the lane's group: 16 bytes in its first plane, 8 in its second (B * 16 bytes further on, at half
+                    // the per-image pitch); same out-of-range trick for tiles that receive nothing
+                    const unsigned pb = (unsigned)((p.res_in_ch + 15) / 16) * g12_b;  // bytes per source pixel
+                    const unsigned b0 = pix * pb + (unsigned)(cb / 16) * g12_b;       // uniform
+                    const unsigned loff2 = cb < res_lim ? (unsigned)h * g12_b + grp_b + (unsigned)bload[sl / NT] * 8u : kOutOfRange;
+                    auto fetch = [&](unsigned so, int* dst) __attribute__((always_inline)) {
+                        const v4i a = __builtin_amdgcn_raw_buffer_load_b128(r_rin, (int)loff, (int)so, kResLoadAux);
+                        const auto c2 = __builtin_amdgcn_raw_buffer_load_b64(r_rin, (int)loff2, (int)so, kResLoadAux);
+                        dst[0] = a[0], dst[1] = a[1], dst[2] = a[2], dst[3] = a[3], dst[4] = c2[0], dst[5] = c2[1];
+                    };
+                    fetch(b0, rv[sl]);
+                    if constexpr (RM == RM_POOLED) {
+                        const unsigned dd = (unsigned)(2 * p.PW) * pb;
+                        fetch(b0 + pb, tmp[0][sl]);
+                        fetch(b0 + dd, tmp[1][sl]);
+                        fetch(b0 + dd + pb, tmp[2][sl]);
+                    }
+                    continue;
+                }
                 const unsigned base = pix * ch_b + (unsigned)(i16 ? cb / 8 : cb / 4) * grp_b;  // uniform
 #pragma unroll
                 for (int g = 0; g < nld; ++g) {
@@ -398,7 +422,20 @@ conv3x3_mfma_f4_kernel(
         if constexpr (RM == RM_POOLED) {
 #pragma unroll
             for (int nt = 0; nt < MT * NT; ++nt) {  // every (image tile, channel tile) slot
-                if constexpr (R16) {
+                if constexpr (R12) {
+                    int m[16], t[16];
+                    i12_unpack8((uint32_t)rv[nt][0], (uint32_t)rv[nt][1], (uint32_t)rv[nt][2], m);
+                    i12_unpack8((uint32_t)rv[nt][3], (uint32_t)rv[nt][4], (uint32_t)rv[nt][5], m + 8);
+#pragma unroll
+                    for (int k = 0; k < 3; ++k) {
+                        i12_unpack8((uint32_t)tmp[k][nt][0], (uint32_t)tmp[k][nt][1], (uint32_t)tmp[k][nt][2], t);
+                        i12_unpack8((uint32_t)tmp[k][nt][3], (uint32_t)tmp[k][nt][4], (uint32_t)tmp[k][nt][5], t + 8);
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) m[v] = max(m[v], t[v]);
+                    }
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) rv[nt][v] = m[v];
+                } else if constexpr (R16) {
 #pragma unroll
                     for (int k = 7; k >= 0; --k) {  // downwards: slot k is read before 2k, 2k+1 are written
                         const int w = rv[nt][k];
@@ -476,10 +513,18 @@ conv3x3_mfma_f4_kernel(
             uint32_t hw = 0;
             if constexpr (kRes) {
                 int res[16];
+                int un[16];  // a plain 12-bit operand is still packed: six words -> sixteen values
+                if constexpr (RM == RM_PLAIN && R12) {
+                    const int* w = rv[mt * NT + nt];
+                    i12_unpack8((uint32_t)w[0], (uint32_t)w[1], (uint32_t)w[2], un);
+                    i12_unpack8((uint32_t)w[3], (uint32_t)w[4], (uint32_t)w[5], un + 8);
+                }
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     int val;
-                    if constexpr (RM == RM_PLAIN && R16) {
+                    if constexpr (RM == RM_PLAIN && R12) {
+                        val = un[v];
+                    } else if constexpr (RM == RM_PLAIN && R16) {
                         const int w = rv[mt * NT + nt][v >> 1];
                         val = (v & 1) ? (w >> 16) : (int)(short)(w & 0xffff);
                     } else {
@@ -503,7 +548,21 @@ conv3x3_mfma_f4_kernel(
                     // therefore kept alive, by the empty-but-for-wait-states asm below, until well after the
                     // last store has issued.
                     v4i q[4];
-                    if (rout_fmt == TCBNN_RES_I16) {  // groups of 8 channels, two per word
+                    if (rout_fmt == TCBNN_RES_I12) {  // the lane's 16 channels are one group: 16 + 8 bytes
+                        uint32_t d[6];
+                        i12_pack8(res, d[0], d[1], d[2]);
+                        i12_pack8(res + 8, d[3], d[4], d[5]);
+                        const unsigned so = (pix * (unsigned)((p.N + 15) / 16) + (unsigned)((n0 + nt * 32) / 16)) * g12_b;
+                        const bool wr = b_ok && (FAST || cbase < p.N);  // a group that starts past N is not written
+                        const unsigned vo = wr ? (unsigned)h * g12_b + (unsigned)b * 16u : kOutOfRange;
+                        const unsigned vo2 = wr ? (unsigned)h * g12_b + grp_b + (unsigned)b * 8u : kOutOfRange;
+                        q[0] = v4i{(int)d[0], (int)d[1], (int)d[2], (int)d[3]};
+                        typedef int v2i_t __attribute__((ext_vector_type(2)));
+                        const v2i_t q2 = {(int)d[4], (int)d[5]};
+                        __builtin_amdgcn_raw_buffer_store_b128(q[0], r_rout, (int)vo, (int)so, 0);
+                        __builtin_amdgcn_raw_buffer_store_b64(q2, r_rout, (int)vo2, (int)so, 0);
+                        asm volatile("s_nop 4" ::"v"(q[0]), "v"(q2));
+                    } else if (rout_fmt == TCBNN_RES_I16) {  // groups of 8 channels, two per word
                         const unsigned so = (pix * (unsigned)((p.N + 7) / 8) + (unsigned)((n0 + nt * 32) / 8)) * grp_b;
                         const unsigned vo = b_ok ? ((unsigned)(2 * h) * (unsigned)p.B + (unsigned)b) * 16u : kOutOfRange;
 #pragma unroll
@@ -651,6 +710,8 @@ conv3x3_mfma_f4_kernel(
     // buffers: the chunk that will be multiplied NB-1 steps from now is requested before the current
     // one is multiplied (two steps of lookahead for Cin >= 192, where one chunk of MFMAs is shorter
     // than the memory latency and few waves share a SIMD).
+    // (Two tiles of lookahead for the short residual tiles, with a third buffer for words and operand, measured no
+    // faster on ResNet-18's first two stages and cost the Cin = 128 layers their third wave per SIMD.)
     constexpr int NB = kAhead ? 2 : (SPT >= 3 && !(kRes && MT == 2 && SPT >= 6) ? 3 : 2);  // (registers)
     constexpr int LOOK = NB - 1;
     struct Cursor {
@@ -681,17 +742,17 @@ conv3x3_mfma_f4_kernel(
     auto pix_x = [&](const Cursor& c) __attribute__((always_inline)) { return POOL ? 2 * c.x + (c.sub & 1) : c.x; };
     uint32_t buf[NB][TPC * SPT][MT];
     uint32_t msk[NB];
-    int rv[kAhead ? 2 : 1][NRV][NW];
+    int rv[kAhead ? NB : 1][NRV][NW];
     Cursor cc = {pi, y, (xr + y) % roww, 0, 0, xr};  // chunk being multiplied
     Cursor lc = cc;             // chunk being requested (LOOK steps ahead)
 #pragma unroll
     for (int i = 0; i < LOOK; ++i) {
         msk[i] = 0;
-        if (lc.pi < npix) msk[i] = load_chunk(pix_y(lc), pix_x(lc), lc.chunk, buf[i]);
+        if (lc.pi < npix) {
+            msk[i] = load_chunk(pix_y(lc), pix_x(lc), lc.chunk, buf[i]);
+            if constexpr (kAhead) request_residual(lc.y, lc.x, rv[i]);  // (a chunk is a whole tile here)
+        }
         advance(lc);
-    }
-    if constexpr (kAhead) {
-        if (cc.pi < npix) request_residual(cc.y, cc.x, rv[0]);
     }
 
     // The first activation (and residual) requests are on their way as well.
@@ -732,7 +793,7 @@ conv3x3_mfma_f4_kernel(
     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc0[nt][v] = RM == RM_NONE ? lds_thr[nt * 32 + 16 * h + v] : 0.0f;
-    if constexpr (kAhead && RM == RM_POOLED) {
+    if constexpr (kAhead && RM == RM_POOLED) {  // (one tile ahead: the first tile's operand)
         if (cc.pi < npix) finish_residual(rv[0]);
     }
 
@@ -744,25 +805,25 @@ conv3x3_mfma_f4_kernel(
         // this one's MFMAs.
         bool fused = false;
         unsigned nsoff = 0;
-        if (lc.pi < npix) {
+        const bool ahead = lc.pi < npix;  // (uniform) there is a chunk LOOK steps ahead
+        if (ahead) {
             if (SPT <= 2 && msk[I] == kAllTaps && chunk_interior(pix_y(lc), pix_x(lc), lc.chunk, nsoff)) {
                 fused = true;
                 msk[J] = kAllTaps;
             } else {
                 msk[J] = load_chunk(pix_y(lc), pix_x(lc), lc.chunk, buf[J]);
             }
+            // NCH == 1: that chunk is a whole tile, whose residual operand is requested with it
+            if constexpr (kAhead) request_residual(lc.y, lc.x, rv[J]);
         }
         advance(lc);
         int (*rcur)[NW] = rv[kAhead ? I : 0];
-        if constexpr (kAhead) {  // NCH == 1: the next chunk is the next tile
-            Cursor nt = cc;
-            advance(nt);
-            if (nt.pi < npix) request_residual(nt.y, nt.x, rv[1 - I]);
+        if constexpr (kAhead) {
             compute_chunk(cc.chunk, buf[I], msk[I], fused, buf[J], nsoff);
             // a pooled source is reduced as soon as its tile has been multiplied (frees the registers of
             // the window); otherwise the operand is left in flight until its own epilogue
             if constexpr (RM == RM_POOLED) {
-                if (nt.pi < npix) finish_residual(rv[1 - I]);
+                if (ahead) finish_residual(rv[J]);
             }
         } else {
             if constexpr (kRes) {
@@ -815,8 +876,9 @@ struct TensorBytes {
     long long act, rin, rout, bits;
 };
 TensorBytes tensor_bytes(const BgemmParams& p) {
-    auto res_words = [&](long long pixels, int channels, int fmt) {
-        return pixels * (fmt == TCBNN_RES_I16 ? (channels + 7) / 8 : (channels + 3) / 4) * p.B * 4;
+    auto res_words = [&](long long pixels, int channels, int fmt) {  // (32-bit words)
+        const long long per = (long long)residual_group_channels(fmt);
+        return pixels * ((channels + per - 1) / per) * p.B * (long long)(residual_group_bytes(fmt) / 4);
     };
     TensorBytes t;
     t.act = 4LL * p.H * p.W * p.cw * p.B;
@@ -831,7 +893,7 @@ TensorBytes tensor_bytes(const BgemmParams& p) {
     return t;
 }
 
-template <int SPT, int RM, int MT, int NT, bool R16, bool POOL, bool FULLT>
+template <int SPT, int RM, int MT, int NT, int RF, bool POOL, bool FULLT>
 int launch_f(const BgemmParams& p, hipStream_t stream) {
     constexpr int NQ = 9 * SPT;
     constexpr bool kRawTranspose = RM == RM_RAW && SPT <= 2 && NT == 2 && FULLT;  // as in the kernel
@@ -845,7 +907,7 @@ int launch_f(const BgemmParams& p, hipStream_t stream) {
     if (int rc = device_info(&dev, &cus)) return rc;
     int resident = resident_on[dev].load(std::memory_order_acquire);
     if (resident == 0) {
-        const void* fn = reinterpret_cast<const void*>(&conv3x3_mfma_f4_kernel<SPT, RM, MT, NT, R16, POOL, FULLT>);
+        const void* fn = reinterpret_cast<const void*>(&conv3x3_mfma_f4_kernel<SPT, RM, MT, NT, RF, POOL, FULLT>);
         if (int rc = check_hip(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes),
                                "hipFuncSetAttribute(MaxDynamicSharedMemorySize)"))
             return rc;
@@ -881,7 +943,7 @@ int launch_f(const BgemmParams& p, hipStream_t stream) {
     // a wave's stride over the work items, split into rows and columns once here instead of in every wave
     const int roww = POOL ? p.OW : p.PW, dpi = best * kWaves;
     const int dy = dpi / roww, dx = dpi % roww, dxs = (dx + dy) % roww;
-    hipLaunchKernelGGL((conv3x3_mfma_f4_kernel<SPT, RM, MT, NT, R16, POOL, FULLT>),
+    hipLaunchKernelGGL((conv3x3_mfma_f4_kernel<SPT, RM, MT, NT, RF, POOL, FULLT>),
                        dim3((unsigned)n_groups, (unsigned)b_groups, (unsigned)best), dim3(kThreads), lds_bytes,
                        stream, p, p.act, p.wgt, p.bn, p.res_in, RM == RM_RAW ? p.out_i32 : p.res_out, res_lim, p.res_out_fmt,
                        (unsigned)tb.act, (unsigned)tb.rin, (unsigned)tb.rout, (unsigned)tb.bits, n_groups, b_groups, best,
@@ -891,14 +953,14 @@ int launch_f(const BgemmParams& p, hipStream_t stream) {
 }
 
 // Every channel tile of the launch full, and the residual limit on a tile boundary?  (see FULLT at the kernel)
-template <int SPT, int RM, int MT, int NT, bool R16, bool POOL>
+template <int SPT, int RM, int MT, int NT, int RF, bool POOL>
 int launch_t(const BgemmParams& p, hipStream_t stream) {
     const int res_lim = p.res_in != nullptr ? std::min(std::min(p.res_limit, p.res_in_ch), p.N) : 0;
     // (with the int32 output, that instantiation also stores whole 128-bit words: the output must be aligned for them)
     const bool raw_ok = RM != RM_RAW || (p.raw_pix_stride % 4 == 0 && p.raw_b_stride % 4 == 0 &&
                                          (reinterpret_cast<uintptr_t>(p.out_i32) & 15) == 0);
-    if (p.N % (32 * NT) == 0 && res_lim % 32 == 0 && raw_ok) return launch_f<SPT, RM, MT, NT, R16, POOL, true>(p, stream);
-    return launch_f<SPT, RM, MT, NT, R16, POOL, false>(p, stream);
+    if (p.N % (32 * NT) == 0 && res_lim % 32 == 0 && raw_ok) return launch_f<SPT, RM, MT, NT, RF, POOL, true>(p, stream);
+    return launch_f<SPT, RM, MT, NT, RF, POOL, false>(p, stream);
 }
 
 // Which instantiation serves a layer.  Measured on ResNet-18 at batch 256: the HBM-bound residual
@@ -907,7 +969,7 @@ int launch_t(const BgemmParams& p, hipStream_t stream) {
 // tile (each operand fragment feeds two MFMAs) until the weights of 64 channels no longer leave
 // room for a second workgroup (Cin = 512).
 struct Pick {
-    int rm, mt, nt, r16, pool;
+    int rm, mt, nt, r16, pool;  // r16: TCBNN_RES_* format of the injected residual
 };
 constexpr int pick_nt(int spt, int rm) {
     return rm == RM_POOLED ? 1 : (rm == RM_PLAIN ? (spt >= 4 ? 1 : 2) : (spt >= 6 ? 1 : 2));  // RM_RAW as RM_NONE
@@ -921,7 +983,7 @@ Pick pick(const BgemmParams& p) {
                    : p.res_in == nullptr && p.res_out == nullptr
                        ? RM_NONE
                        : (p.res_in != nullptr && p.res_pool ? RM_POOLED : RM_PLAIN);
-    return {rm, pick_mt(p.cw / 2, rm), pick_nt(p.cw / 2, rm), p.res_in != nullptr && p.res_in_fmt == TCBNN_RES_I16,
+    return {rm, pick_mt(p.cw / 2, rm), pick_nt(p.cw / 2, rm), p.res_in != nullptr ? p.res_in_fmt : TCBNN_RES_I32,
             p.pool_h == 2};
 }
 
@@ -930,16 +992,22 @@ int launch_m(const BgemmParams& p, hipStream_t stream) {
     const Pick k = pick(p);
     switch (k.rm) {
         case RM_NONE:
-            return k.pool ? launch_t<SPT, RM_NONE, 2, pick_nt(SPT, RM_NONE), false, true>(p, stream)
-                          : launch_t<SPT, RM_NONE, 2, pick_nt(SPT, RM_NONE), false, false>(p, stream);
+            return k.pool ? launch_t<SPT, RM_NONE, 2, pick_nt(SPT, RM_NONE), TCBNN_RES_I32, true>(p, stream)
+                          : launch_t<SPT, RM_NONE, 2, pick_nt(SPT, RM_NONE), TCBNN_RES_I32, false>(p, stream);
         case RM_RAW:
-            return launch_t<SPT, RM_RAW, 2, pick_nt(SPT, RM_RAW), false, false>(p, stream);
+            return launch_t<SPT, RM_RAW, 2, pick_nt(SPT, RM_RAW), TCBNN_RES_I32, false>(p, stream);
         case RM_PLAIN:
-            return k.r16 ? launch_t<SPT, RM_PLAIN, pick_mt(SPT, RM_PLAIN), pick_nt(SPT, RM_PLAIN), true, false>(p, stream)
-                         : launch_t<SPT, RM_PLAIN, pick_mt(SPT, RM_PLAIN), pick_nt(SPT, RM_PLAIN), false, false>(p, stream);
+            return k.r16 == TCBNN_RES_I12
+                       ? launch_t<SPT, RM_PLAIN, pick_mt(SPT, RM_PLAIN), pick_nt(SPT, RM_PLAIN), TCBNN_RES_I12, false>(p, stream)
+                       : (k.r16 == TCBNN_RES_I16
+                              ? launch_t<SPT, RM_PLAIN, pick_mt(SPT, RM_PLAIN), pick_nt(SPT, RM_PLAIN), TCBNN_RES_I16, false>(p, stream)
+                              : launch_t<SPT, RM_PLAIN, pick_mt(SPT, RM_PLAIN), pick_nt(SPT, RM_PLAIN), TCBNN_RES_I32, false>(p, stream));
         default:
-            return k.r16 ? launch_t<SPT, RM_POOLED, pick_mt(SPT, RM_POOLED), pick_nt(SPT, RM_POOLED), true, false>(p, stream)
-                         : launch_t<SPT, RM_POOLED, pick_mt(SPT, RM_POOLED), pick_nt(SPT, RM_POOLED), false, false>(p, stream);
+            return k.r16 == TCBNN_RES_I12
+                       ? launch_t<SPT, RM_POOLED, pick_mt(SPT, RM_POOLED), pick_nt(SPT, RM_POOLED), TCBNN_RES_I12, false>(p, stream)
+                       : (k.r16 == TCBNN_RES_I16
+                              ? launch_t<SPT, RM_POOLED, pick_mt(SPT, RM_POOLED), pick_nt(SPT, RM_POOLED), TCBNN_RES_I16, false>(p, stream)
+                              : launch_t<SPT, RM_POOLED, pick_mt(SPT, RM_POOLED), pick_nt(SPT, RM_POOLED), TCBNN_RES_I32, false>(p, stream));
     }
 }
 
@@ -975,8 +1043,8 @@ void conv3x3_mfma_kernel_name(const BgemmParams& p, char* buf, size_t len) {
     const bool raw_ok = k.rm != RM_RAW || (p.raw_pix_stride % 4 == 0 && p.raw_b_stride % 4 == 0 &&
                                            (reinterpret_cast<uintptr_t>(p.out_i32) & 15) == 0);
     const bool full = p.N % (32 * k.nt) == 0 && res_lim % 32 == 0 && raw_ok;
-    snprintf(buf, len, "conv3x3_mfma_f4_kernel<%d, %d, %d, %d, %s, %s, %s>", p.cw / 2, k.rm, k.mt, k.nt,
-             k.r16 ? "true" : "false", k.pool ? "true" : "false", full ? "true" : "false");
+    snprintf(buf, len, "conv3x3_mfma_f4_kernel<%d, %d, %d, %d, %d, %s, %s>", p.cw / 2, k.rm, k.mt, k.nt, k.r16,
+             k.pool ? "true" : "false", full ? "true" : "false");
 }
 
 int launch_conv3x3_mfma(const BgemmParams& p, hipStream_t stream) {

@@ -344,7 +344,22 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS &
                     // streaming stores: the tensor (103 MB at batch 256) is far larger than the caches and is
                     // read two launches later
                     v4i_t* __restrict__ dst = reinterpret_cast<v4i_t*>(res);
-                    if (p.res_fmt == TCBNN_RES_I16) {
+                    if (p.res_fmt == TCBNN_RES_I12) {  // two groups of 16 channels: 16 + 8 bytes each
+                        typedef int v2i_t __attribute__((ext_vector_type(2)));
+                        uint32_t* __restrict__ w = reinterpret_cast<uint32_t*>(res);
+                        const size_t G = (size_t)((p.O + 15) / 16);
+#pragma unroll
+                        for (int g = 0; g < 2; ++g)
+                            if (wi * 32 + 16 * g < p.O) {
+                                uint32_t d[6];
+                                i12_pack8(&r32[16 * g], d[0], d[1], d[2]);
+                                i12_pack8(&r32[16 * g + 8], d[3], d[4], d[5]);
+                                __builtin_nontemporal_store(v4i_t{(int)d[0], (int)d[1], (int)d[2], (int)d[3]},
+                                                            reinterpret_cast<v4i_t*>(w + i12_word_index(pix, G, wi * 2 + g, p.B, b, 0)));
+                                __builtin_nontemporal_store(v2i_t{(int)d[4], (int)d[5]},
+                                                            reinterpret_cast<v2i_t*>(w + i12_word_index(pix, G, wi * 2 + g, p.B, b, 4)));
+                            }
+                    } else if (p.res_fmt == TCBNN_RES_I16) {
                         const size_t g0 = (pix * ((p.O + 7) / 8) + wi * 4) * p.B + b;
 #pragma unroll
                         for (int g = 0; g < 4; ++g)
@@ -427,10 +442,13 @@ __global__ __launch_bounds__(kThreads) void inconv_generic_kernel(const InConvPa
                     if (ch < p.O) word |= (acc[n] < p.bn[ch] ? 0u : 1u) << (31 - n);
                 }
                 if (p.res != nullptr) {
+                    int r32[32];
 #pragma unroll
-                    for (int n = 0; n < 32; ++n)
-                        if (g * 32 + n < p.O)
-                            residual_store(p.res, p.res_fmt, (size_t)y * p.PW + x, p.O, g * 32 + n, p.B, b, (int)acc[n]);
+                    for (int n = 0; n < 32; ++n) r32[n] = g * 32 + n < p.O ? (int)acc[n] : 0;
+#pragma unroll
+                    for (int q = 0; q < 2; ++q)  // whole groups of 16 channels (12-bit values share words)
+                        if (g * 32 + 16 * q < p.O)
+                            residual_store_group16(p.res, p.res_fmt, (size_t)y * p.PW + x, p.O, g * 2 + q, p.B, b, &r32[16 * q]);
                 }
             }
         }
@@ -470,8 +488,9 @@ static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name
     p.out = d->output;
     p.res = d->save_residual ? d->output_residual : nullptr;
     p.res_fmt = d->residual_format;
-    TCBNN_REQUIRE(!d->save_residual || p.res_fmt == TCBNN_RES_I32 || p.res_fmt == TCBNN_RES_I16,
-                  "inconv128: unknown residual_format");
+    TCBNN_REQUIRE(!d->save_residual || residual_format_known(p.res_fmt), "inconv128: unknown residual_format");
+    TCBNN_REQUIRE(!d->save_residual || p.res_fmt != TCBNN_RES_I12 || d->batch % 2 == 0,
+                  "inconv128: a 12-bit residual needs an even batch");
     p.H = d->input_height;
     p.W = d->input_width;
     p.B = d->batch;

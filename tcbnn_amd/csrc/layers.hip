@@ -6,8 +6,10 @@
 
 #include <atomic>
 
+#include <algorithm>
 #include <cmath>
 #include <cstdint>
+#include <vector>
 
 #include "common.h"
 
@@ -154,9 +156,10 @@ size_t tcbnn_inconv_filter_words(int r, int s, int in_ch, int out_ch) {
 }
 
 size_t tcbnn_residual_bytes(int height, int width, int channels, int batch, int format) {
-    if (height <= 0 || width <= 0 || channels <= 0 || batch <= 0) return 0;
+    if (height <= 0 || width <= 0 || channels <= 0 || batch <= 0 || !residual_format_known(format)) return 0;
     const size_t pix_b = (size_t)height * width * batch;
-    return pix_b * 16 * (format == TCBNN_RES_I16 ? (channels + 7) / 8 : (channels + 3) / 4);
+    const size_t per = residual_group_channels(format);
+    return pix_b * residual_group_bytes(format) * ((channels + per - 1) / per);
 }
 
 int tcbnn_inconv_residual_bound(int filter_height, int filter_width, float input_abs_max) {
@@ -176,6 +179,55 @@ int tcbnn_conv_residual_bound(int input_channels, int filter_height, int filter_
 
 int tcbnn_residual_format_for_bound(int bound) {
     return bound >= 0 && bound <= 32767 ? TCBNN_RES_I16 : TCBNN_RES_I32;
+}
+
+int tcbnn_residual_format_narrowest(int bound, int batch) {
+    if (bound >= 0 && bound <= 2047 && batch > 0 && batch % 2 == 0) return TCBNN_RES_I12;
+    return tcbnn_residual_format_for_bound(bound);
+}
+
+// The first layer's sum at an output pixel is a signed sum of the inputs under the filter window, so its
+// magnitude is at most the window's sum of |x| (all three channels); fp32 rounding of the 3*R*S additions adds at
+// most 3*R*S*2^-24 of that relative, far inside the 0.1 % + 1 of slack taken here.  Separable running sums: per
+// image, column sums of |x| over the window's rows, then a sliding sum along the row.
+int tcbnn_inconv_residual_bound_of_input(const float* input_host, int batch, int height, int width,
+                                         int filter_height, int filter_width, int stride_height,
+                                         int stride_width, int padding) {
+    if (input_host == nullptr || batch <= 0 || height <= 0 || width <= 0 || filter_height <= 0 ||
+        filter_width <= 0 || stride_height <= 0 || stride_width <= 0)
+        return INT32_MAX;
+    const int pad_h = tcbnn_conv_pad(height, filter_height, stride_height, padding);
+    const int pad_w = tcbnn_conv_pad(width, filter_width, stride_width, padding);
+    const int oh = tcbnn_conv_out(height, filter_height, stride_height, padding, 1);
+    const int ow = tcbnn_conv_out(width, filter_width, stride_width, padding, 1);
+    if (oh <= 0 || ow <= 0) return INT32_MAX;
+    const size_t plane = (size_t)height * width;
+    double worst = 0.0;
+    bool bad = false;
+    std::vector<double> rowsum((size_t)height * width), col(width);
+    for (int b = 0; b < batch && !bad; ++b) {
+        const float* img = input_host + (size_t)b * 3 * plane;
+        for (size_t i = 0; i < plane; ++i) {
+            const double a = std::fabs((double)img[i]) + std::fabs((double)img[plane + i]) + std::fabs((double)img[2 * plane + i]);
+            if (!(a <= 1e30)) bad = true;  // NaN or infinity
+            rowsum[i] = a;
+        }
+        for (int y = 0; y < oh; ++y) {
+            const int y0 = std::max(0, y * stride_height - pad_h), y1 = std::min(height, y * stride_height - pad_h + filter_height);
+            for (int x = 0; x < width; ++x) col[x] = 0.0;
+            for (int yy = y0; yy < y1; ++yy)
+                for (int x = 0; x < width; ++x) col[x] += rowsum[(size_t)yy * width + x];
+            for (int x = 0; x < ow; ++x) {
+                const int x0 = std::max(0, x * stride_width - pad_w), x1 = std::min(width, x * stride_width - pad_w + filter_width);
+                double sum = 0.0;
+                for (int xx = x0; xx < x1; ++xx) sum += col[xx];
+                if (sum > worst) worst = sum;
+            }
+        }
+    }
+    if (bad) return INT32_MAX;
+    const double bound = worst * 1.001 + 1.0;
+    return bound < (double)(INT32_MAX / 2) ? (int)std::ceil(bound) : INT32_MAX;
 }
 
 int tcbnn_fc128_forward(const tcbnn_fc128_desc* d, void* stream) {
@@ -293,14 +345,16 @@ static int conv_problem(const tcbnn_conv128_desc* d, bool launch, BgemmParams* o
         p.res_in_ch = d->input_residual_channels;
         p.res_limit = d->residual_channels;
         p.res_pool = d->residual_pool ? 1 : 0;
-        TCBNN_REQUIRE(d->input_residual_format == TCBNN_RES_I32 || d->input_residual_format == TCBNN_RES_I16,
-                      "conv128: unknown input_residual_format");
+        TCBNN_REQUIRE(residual_format_known(d->input_residual_format), "conv128: unknown input_residual_format");
+        TCBNN_REQUIRE(d->input_residual_format != TCBNN_RES_I12 || d->batch % 2 == 0,
+                      "conv128: a 12-bit residual needs an even batch");
         p.res_in_fmt = d->input_residual_format;
     }
     if (d->save_residual) {
         if (launch) TCBNN_NOTNULL(d->output_residual);
-        TCBNN_REQUIRE(d->output_residual_format == TCBNN_RES_I32 || d->output_residual_format == TCBNN_RES_I16,
-                      "conv128: unknown output_residual_format");
+        TCBNN_REQUIRE(residual_format_known(d->output_residual_format), "conv128: unknown output_residual_format");
+        TCBNN_REQUIRE(d->output_residual_format != TCBNN_RES_I12 || d->batch % 2 == 0,
+                      "conv128: a 12-bit residual needs an even batch");
         p.res_out = launch ? d->output_residual : some;
         p.res_out_fmt = d->output_residual_format;
     }

@@ -229,7 +229,7 @@ __global__ void residual_to_reference_kernel(const int32_t* __restrict__ res,
 // channels past `ch` are stored as 0, which is what the consumers of the padding lanes expect.
 __global__ void residual_from_reference_kernel(const int32_t* __restrict__ ref, int32_t* __restrict__ res,
                                                long long pixels, int batch, int ch, int b8, int c128, int fmt) {
-    const int per = fmt == TCBNN_RES_I16 ? 8 : 4;
+    const int per = (int)residual_group_channels(fmt);
     const int groups = (ch + per - 1) / per;
     const long long idx = (long long)blockIdx.x * kThreads + threadIdx.x;
     if (idx >= pixels * groups * batch) return;
@@ -237,6 +237,13 @@ __global__ void residual_from_reference_kernel(const int32_t* __restrict__ ref, 
     const int g = (int)((idx / batch) % groups);
     const long long pix = idx / ((long long)batch * groups);
     const int32_t* src = ref + ((size_t)pix * b8 + b) * c128 + (size_t)g * per;
+    if (fmt == TCBNN_RES_I12) {  // one thread per group of 16 channels
+        int v16[16];
+#pragma unroll
+        for (int i = 0; i < 16; ++i) v16[i] = g * 16 + i < ch ? src[i] : 0;
+        residual_store_group16(res, fmt, (size_t)pix, ch, g, batch, b, v16);
+        return;
+    }
     int v[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) v[i] = (i < per && g * per + i < ch) ? src[i] : 0;
@@ -429,7 +436,8 @@ int tcbnn_residual_to_reference(const int32_t* res, int32_t* ref, int height, in
     TCBNN_NOTNULL(res);
     TCBNN_NOTNULL(ref);
     TCBNN_REQUIRE(batch > 0 && height > 0 && width > 0 && ch > 0, "residual_to_reference: bad shape");
-    TCBNN_REQUIRE(format == TCBNN_RES_I32 || format == TCBNN_RES_I16, "residual_to_reference: unknown format");
+    TCBNN_REQUIRE(residual_format_known(format), "residual_to_reference: unknown format");
+    TCBNN_REQUIRE(format != TCBNN_RES_I12 || batch % 2 == 0, "residual_to_reference: a 12-bit residual needs an even batch");
     const long long pixels = (long long)height * width;
     const long long total = pixels * pad8(batch) * pad128(ch);
     hipLaunchKernelGGL(residual_to_reference_kernel, dim3(blocks_for(total)), dim3(kThreads), 0,
@@ -443,9 +451,10 @@ int tcbnn_residual_from_reference(const int32_t* ref, int32_t* res, int height, 
     TCBNN_NOTNULL(ref);
     TCBNN_NOTNULL(res);
     TCBNN_REQUIRE(batch > 0 && height > 0 && width > 0 && ch > 0, "residual_from_reference: bad shape");
-    TCBNN_REQUIRE(format == TCBNN_RES_I32 || format == TCBNN_RES_I16, "residual_from_reference: unknown format");
+    TCBNN_REQUIRE(residual_format_known(format), "residual_from_reference: unknown format");
+    TCBNN_REQUIRE(format != TCBNN_RES_I12 || batch % 2 == 0, "residual_from_reference: a 12-bit residual needs an even batch");
     const long long pixels = (long long)height * width;
-    const int per = format == TCBNN_RES_I16 ? 8 : 4;
+    const int per = (int)residual_group_channels(format);
     const long long total = pixels * ((ch + per - 1) / per) * batch;
     hipLaunchKernelGGL(residual_from_reference_kernel, dim3(blocks_for(total)), dim3(kThreads), 0,
                        (hipStream_t)stream, ref, res, pixels, batch, ch, pad8(batch), pad128(ch), format);

@@ -38,7 +38,25 @@ __global__ __launch_bounds__(kThreads) void pool128_kernel(const PoolParams p) {
         p.out[((size_t)opix * p.cw + u) * p.B + b] = acc;
         return;
     }
-    const int g = u - p.cw;  // maximum of the window's 16-byte residual groups
+    const int g = u - p.cw;  // maximum of the window's residual groups
+    if (p.fmt == TCBNN_RES_I12) {  // groups of 16 channels, unpacked to ints and packed again
+        int m[16], v[16];
+        bool none = true;
+        for (int r = 0; r < p.window; ++r)
+            for (int s = 0; s < p.window; ++s) {
+                const int y = y0 + r, x = x0 + s;
+                if (y < 0 || y >= p.H || x < 0 || x >= p.W) continue;
+                residual_load_group16(p.rin, p.fmt, (size_t)y * p.W + x, p.C, g, p.B, b, v);
+#pragma unroll
+                for (int e = 0; e < 16; ++e) m[e] = none ? v[e] : max(m[e], v[e]);
+                none = false;
+            }
+        if (none)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) m[e] = 0;
+        residual_store_group16(p.rout, p.fmt, (size_t)opix, p.C, g, p.B, b, m);
+        return;
+    }
     const int4* __restrict__ src = reinterpret_cast<const int4*>(p.rin);
     int4 m;
     bool first = true;
@@ -89,6 +107,20 @@ __global__ __launch_bounds__(kThreads) void avgpool_fc_kernel(const HeadParams p
     for (int u = tid; u < p.groups * kHeadImages; u += kThreads) {
         const int g = u / kHeadImages, i = u % kHeadImages;  // image fastest: 128-byte runs
         const int bb = min(b0 + i, p.B - 1);
+        if (p.fmt == TCBNN_RES_I12) {  // groups of 16 channels
+            int s16[16], v16[16];
+#pragma unroll
+            for (int e = 0; e < 16; ++e) s16[e] = 0;
+            for (int pix = 0; pix < p.P; ++pix) {
+                residual_load_group16(p.rin, p.fmt, (size_t)pix, p.C, g, p.B, bb, v16);
+#pragma unroll
+                for (int e = 0; e < 16; ++e) s16[e] += v16[e];
+            }
+#pragma unroll
+            for (int e = 0; e < 16; ++e)
+                if (16 * g + e < p.C) mean[16 * g + e][i] = (float)s16[e] / npix;
+            continue;
+        }
         int sum[8] = {0, 0, 0, 0, 0, 0, 0, 0};
         // eight pixels requested at a time (a load per loop pass waits for each one in turn); integer sums, so
         // the order does not matter
@@ -177,9 +209,10 @@ extern "C" int tcbnn_pool128_forward(const tcbnn_pool128_desc* d, void* stream) 
                   "pool128: bad shape");
     TCBNN_REQUIRE((d->input_residual == nullptr) == (d->output_residual == nullptr),
                   "pool128: input_residual and output_residual go together");
-    TCBNN_REQUIRE(d->input_residual == nullptr || d->residual_format == TCBNN_RES_I32 ||
-                      d->residual_format == TCBNN_RES_I16,
+    TCBNN_REQUIRE(d->input_residual == nullptr || residual_format_known(d->residual_format),
                   "pool128: unknown residual_format");
+    TCBNN_REQUIRE(d->input_residual == nullptr || d->residual_format != TCBNN_RES_I12 || d->batch % 2 == 0,
+                  "pool128: a 12-bit residual needs an even batch");
     PoolParams p;
     p.in = d->input;
     p.out = d->output;
@@ -194,7 +227,7 @@ extern "C" int tcbnn_pool128_forward(const tcbnn_pool128_desc* d, void* stream) 
     TCBNN_REQUIRE(p.OH > 0 && p.OW > 0, "pool128: empty output");
     p.cw = step32(p.C);
     p.fmt = d->residual_format;
-    p.groups = p.rin == nullptr ? 0 : (p.fmt == TCBNN_RES_I16 ? (p.C + 7) / 8 : (p.C + 3) / 4);
+    p.groups = p.rin == nullptr ? 0 : (int)((p.C + residual_group_channels(p.fmt) - 1) / residual_group_channels(p.fmt));
     p.window = d->window;
     p.stride = d->stride;
     p.pad = d->padding;
@@ -215,8 +248,9 @@ extern "C" int tcbnn_avgpool_fc_forward(const tcbnn_avgpool_fc_desc* d, void* st
     TCBNN_REQUIRE(d->input_height > 0 && d->input_width > 0 && d->channels > 0 && d->batch > 0 && d->out_features > 0,
                   "avgpool_fc: bad shape");
     TCBNN_REQUIRE(d->channels <= kHeadMaxC, "avgpool_fc: at most 512 channels");
-    TCBNN_REQUIRE(d->residual_format == TCBNN_RES_I32 || d->residual_format == TCBNN_RES_I16,
-                  "avgpool_fc: unknown residual_format");
+    TCBNN_REQUIRE(residual_format_known(d->residual_format), "avgpool_fc: unknown residual_format");
+    TCBNN_REQUIRE(d->residual_format != TCBNN_RES_I12 || d->batch % 2 == 0,
+                  "avgpool_fc: a 12-bit residual needs an even batch");
     HeadParams p;
     p.rin = d->input_residual;
     p.w = d->weight;
@@ -227,7 +261,7 @@ extern "C" int tcbnn_avgpool_fc_forward(const tcbnn_avgpool_fc_desc* d, void* st
     p.B = d->batch;
     p.N = d->out_features;
     p.fmt = d->residual_format;
-    p.per_group = p.fmt == TCBNN_RES_I16 ? 8 : 4;
+    p.per_group = (int)residual_group_channels(p.fmt);
     p.groups = (p.C + p.per_group - 1) / p.per_group;
     const dim3 grid((unsigned)((p.B + kHeadImages - 1) / kHeadImages), (unsigned)((p.N + kHeadOutputs - 1) / kHeadOutputs));
     hipLaunchKernelGGL(avgpool_fc_kernel, grid, dim3(kThreads), 0, (hipStream_t)stream, p);

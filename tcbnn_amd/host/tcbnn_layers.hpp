@@ -138,8 +138,9 @@ inline std::map<const void*, ResidualInfo>& residual_registry() {
     static std::map<const void*, ResidualInfo> reg;
     return reg;
 }
-inline ResidualInfo make_residual_info(int channels, int bound) {
-    ResidualInfo info = {channels, bound, tcbnn_residual_format_for_bound(bound)};
+// (the narrowest format that is exact for the bound: 12 bits up to 2047 for even batches, 16 bits up to 32767)
+inline ResidualInfo make_residual_info(int channels, int bound, int batch) {
+    ResidualInfo info = {channels, bound, tcbnn_residual_format_narrowest(bound, batch)};
     return info;
 }
 
@@ -461,9 +462,14 @@ class InConv128LayerParam {  // param.h:701-870
           padding(_padding), bn(NULL), bn_gpu(NULL), batch(_batch), stride_height(_stride_height),
           stride_width(_stride_width), pool_width(_pool_width), pool_height(_pool_height),
           save_residual(_save_residual), output_residual_gpu(NULL), gpu(this) {
-        residual_info = tcbnn_host::make_residual_info(_output_channels, INT32_MAX);
+        residual_info = tcbnn_host::make_residual_info(_output_channels, INT32_MAX, _batch);
         strncpy(this->name, name, 8);
         TCBNN_CONV_GEOMETRY();
+    }
+    // upper bound of |first-layer sum| for a batch: the largest sum of |x| under any filter window
+    int residual_bound_of(const float* batch_input) {
+        return tcbnn_inconv_residual_bound_of_input(batch_input, batch, input_height, input_width, filter_height,
+                                                    filter_width, stride_height, stride_width, padding ? 1 : 0);
     }
     int input_size() { return input_channels * input_height * input_width * batch; }
     int input_bytes() { return input_size() * sizeof(float); }
@@ -484,14 +490,8 @@ class InConv128LayerParam {  // param.h:701-870
     InConv128LayerParam* initialize(float* input, tcbnn_host::ConfigSource config_file) {
         CHECK_NULL_POINTER(input);
         this->input = input;
-        // |first-layer sum| <= R*S*3*max|x|: decides whether the saved residual fits 16 bits
-        float input_abs_max = 0.0f;
-        for (int i = 0; i < input_size(); ++i) {
-            const float a = input[i] < 0 ? -input[i] : input[i];
-            if (!(a <= input_abs_max)) input_abs_max = a;  // also catches NaN
-        }
-        residual_info = tcbnn_host::make_residual_info(
-            output_channels, tcbnn_inconv_residual_bound(filter_height, filter_width, input_abs_max));
+        // |first-layer sum| <= the window's sum of |x|: decides whether the saved residual fits 12 or 16 bits
+        residual_info = tcbnn_host::make_residual_info(output_channels, residual_bound_of(input), batch);
         SAFE_ALOC_GPU(input_gpu, input_bytes());
         HIP_SAFE_CALL(hipMemcpy(input_gpu, input, input_bytes(), hipMemcpyHostToDevice));
         SAFE_ALOC_HOST(filter, filter_bytes());
@@ -519,17 +519,12 @@ class InConv128LayerParam {  // param.h:701-870
     // A new batch for the same layer objects (the reference's objects are single-shot, this engine's are not):
     // uploads `input` into input_gpu.  The format of the saved residual, and of every residual downstream of it,
     // was chosen at initialize() from the largest |value| of the first batch; a batch that exceeds the bound the
-    // format was proven for would wrap in 16 bits, so it is refused (print + exit, like every error here).
+    // format was proven for would wrap in its 12 or 16 bits, so it is refused (print + exit, like every error here).
     void set_input(float* input) {
         CHECK_NULL_POINTER(input);
         CHECK_NULL_POINTER(input_gpu);
         if (save_residual) {
-            float input_abs_max = 0.0f;
-            for (int i = 0; i < input_size(); ++i) {
-                const float a = input[i] < 0 ? -input[i] : input[i];
-                if (!(a <= input_abs_max)) input_abs_max = a;  // also catches NaN
-            }
-            if (tcbnn_inconv_residual_bound(filter_height, filter_width, input_abs_max) > residual_info.bound) {
+            if (residual_bound_of(input) > residual_info.bound) {
                 fprintf(stderr, "Error: set_input: |input| exceeds the bound the residual formats were chosen for "
                                 "(initialize the layers with the batch of largest magnitude).\n");
                 exit(-1);
@@ -652,7 +647,7 @@ class Conv128LayerParam {  // param.h:872-1065
           save_residual(_save_residual), output_residual_gpu(NULL), inject_residual(_inject_residual),
           input_residual_gpu(NULL), residual_channels(_residual_channels), residual_pool(_residual_pool),
           gpu(this), variant(TCBNN_VARIANT_AUTO), input_residual_channels(0) {
-        residual_info = input_residual_info = tcbnn_host::make_residual_info(_output_channels, INT32_MAX);
+        residual_info = input_residual_info = tcbnn_host::make_residual_info(_output_channels, INT32_MAX, _batch);
         strncpy(this->name, name, 8);
         TCBNN_CONV_GEOMETRY();
     }
@@ -718,7 +713,7 @@ class Conv128LayerParam {  // param.h:872-1065
             residual_info = tcbnn_host::make_residual_info(
                 output_channels, injected < INT32_MAX / 4 ? tcbnn_conv_residual_bound(input_channels, filter_height,
                                                                                       filter_width, injected)
-                                                          : INT32_MAX);
+                                                          : INT32_MAX, batch);
             SAFE_ALOC_GPU(output_residual_gpu, residual_bytes());
             tcbnn_host::residual_registry()[output_residual_gpu] = residual_info;
         }

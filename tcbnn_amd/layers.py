@@ -82,8 +82,9 @@ def _stream_handle(stream):
 
 def _residual_buffer(channels, height, width, batch, bound, force_format=None):
     """Device buffer of a saved residual.  `bound` is an upper bound of |value| (INT32_MAX when
-    unknown); the 16-bit format is chosen when the bound allows it (or as `force_format` says)."""
-    fmt = lib.tcbnn_residual_format_for_bound(bound) if force_format is None else force_format
+    unknown); the narrowest format the bound allows is chosen: 12 bits up to 2047 (even batches), 16 bits up to
+    32767, else int32 (or as `force_format` says)."""
+    fmt = lib.tcbnn_residual_format_narrowest(bound, batch) if force_format is None else force_format
     buf = DeviceBuffer(lib.tcbnn_residual_bytes(height, width, channels, batch, fmt))
     buf.channels, buf.height, buf.width, buf.batch = channels, height, width, batch
     buf.bound, buf.format = bound, fmt
@@ -413,6 +414,22 @@ class _ConvGeometry(_ReferenceLayoutIO):
     def download_residual(self):
         """Saved residual as int32 [P][Q][B][O] (host transpose of the engine's layouts)."""
         P, Q, O, B = self.buf_height, self.buf_width, self.output_channels, self.batch
+        if self.output_residual_gpu.format == _lib.RES_I12:
+            # groups of 16 channels; per pixel and group the words w0..w3 of every image, then w4, w5 of every image;
+            # value e sits at bits 12e..12e+11 of the 192-bit string w0..w5 (two's complement)
+            G = (O + 15) // 16
+            raw = self.output_residual_gpu.to_numpy(np.uint32, (P, Q, G, 6 * B)).astype(np.uint64)
+            words = np.concatenate([raw[..., :4 * B].reshape(P, Q, G, B, 4), raw[..., 4 * B:].reshape(P, Q, G, B, 2)],
+                                   axis=-1)
+            vals = np.empty((P, Q, G, B, 16), np.int64)
+            for e in range(16):
+                k, sh = (12 * e) >> 5, (12 * e) & 31
+                v = words[..., k] >> np.uint64(sh)
+                if sh > 20:
+                    v = v | (words[..., k + 1] << np.uint64(32 - sh))
+                v = (v & np.uint64(0xfff)).astype(np.int64)
+                vals[..., e] = (v ^ 0x800) - 0x800
+            return np.ascontiguousarray(vals.transpose(0, 1, 3, 2, 4).reshape(P, Q, B, G * 16)[..., :O].astype(np.int32))
         # engine layouts: int32 [P][Q][ceil(O/4)][B][4] or int16 [P][Q][ceil(O/8)][B][8]
         grp, dt = (8, np.int16) if self.output_residual_gpu.format == _lib.RES_I16 else (4, np.int32)
         ng = (O + grp - 1) // grp
@@ -508,16 +525,21 @@ class InConv128LayerParam(_ConvGeometry):
         self.output_gpu = DeviceBuffer(4 * lib.tcbnn_conv_act_words(
             self.output_height, self.output_width, self.batch, self.output_channels))
         if self.save_residual:
-            bound = lib.tcbnn_inconv_residual_bound(self.filter_height, self.filter_width, self.input_abs_max)
+            bound = self._residual_bound(x)
             self.output_residual_gpu = _residual_buffer(self.output_channels, self.buf_height, self.buf_width,
                                                         self.batch, bound, self.residual_format)
         return self
 
+    def _residual_bound(self, x):
+        """Upper bound of |first-layer sum| for this batch: the largest sum of |x| under any filter window."""
+        return lib.tcbnn_inconv_residual_bound_of_input(
+            x.ctypes.data, self.batch, self.input_height, self.input_width, self.filter_height, self.filter_width,
+            self.stride_height, self.stride_width, int(self.padding))
+
     def set_input(self, input):
         x = np.ascontiguousarray(input, dtype=np.float32)
-        amax = float(np.max(np.abs(x))) if x.size else 0.0
-        if self.save_residual and lib.tcbnn_inconv_residual_bound(
-                self.filter_height, self.filter_width, amax) > self.output_residual_gpu.bound:
+        assert x.size == self.input_size(), (x.size, self.input_size())
+        if self.save_residual and self._residual_bound(x) > self.output_residual_gpu.bound:
             raise _lib.TcbnnError("input magnitude exceeds the bound the residual format was chosen for")
         self.input_gpu.upload(x)
 

@@ -170,14 +170,36 @@ def _residual_source(res_in, fmt):
     """Device copy of a residual [Hr][Wr][B][C] in the engine layout of format `fmt`, tagged the way the
     layer classes tag the tensors they produce (channel count, format, bound of |value|)."""
     hr, wr, b, c = res_in.shape
-    grp, dt = (8, np.int16) if fmt == 1 else (4, np.int32)  # [Hr][Wr][ceil(C/grp)][B][grp]
-    ng = (c + grp - 1) // grp
-    pad = np.zeros((hr, wr, b, ng * grp), dt)
-    pad[..., :c] = res_in
-    host = np.ascontiguousarray(pad.reshape(hr, wr, b, ng, grp).transpose(0, 1, 3, 2, 4))
+    if fmt == 2:  # 12 bits: groups of 16 channels, per pixel and group w0..w3 of every image, then w4, w5
+        host = _pack_i12(res_in)
+    else:
+        grp, dt = (8, np.int16) if fmt == 1 else (4, np.int32)  # [Hr][Wr][ceil(C/grp)][B][grp]
+        ng = (c + grp - 1) // grp
+        pad = np.zeros((hr, wr, b, ng * grp), dt)
+        pad[..., :c] = res_in
+        host = np.ascontiguousarray(pad.reshape(hr, wr, b, ng, grp).transpose(0, 1, 3, 2, 4))
     rbuf = gpuops.dev(host)
     rbuf.channels, rbuf.format, rbuf.bound = c, fmt, int(np.abs(res_in).max())
     return rbuf
+
+
+def _pack_i12(res):
+    """int32 [Hr][Wr][B][C] -> the engine's 12-bit layout, written from its definition: value e of a group of 16
+    channels at bits 12e..12e+11 (two's complement) of the 192-bit string w0..w5; per pixel and group the words
+    w0..w3 of every image, then w4, w5 of every image."""
+    hr, wr, b, c = res.shape
+    assert np.abs(res).max() <= 2047 and b % 2 == 0
+    g = (c + 15) // 16
+    v = np.zeros((hr, wr, b, g * 16), np.int64)
+    v[..., :c] = res
+    v = (v & 0xfff).reshape(hr, wr, b, g, 16)
+    big = np.zeros((hr, wr, b, g), object)
+    for e in range(16):
+        big = big + (v[..., e].astype(object) << (12 * e))
+    words = np.stack([((big >> (32 * k)) & 0xffffffff).astype(np.uint64) for k in range(6)], axis=-1).astype(np.uint32)
+    words = words.transpose(0, 1, 3, 2, 4)  # [Hr][Wr][G][B][6]
+    return np.ascontiguousarray(np.concatenate([words[..., :4].reshape(hr, wr, g, 4 * b),
+                                                words[..., 4:].reshape(hr, wr, g, 2 * b)], axis=-1))
 
 
 def _run_conv_layer(gpu, variant, x, f, bn, stride=1, pool=1, ahead_fc=False, save_residual=False,
@@ -262,6 +284,19 @@ def test_conv128_residual_modes(gpu, variant, cin, cout, in_fmt, out_fmt):
     _residual_modes(gpu, variant, cin, cout, in_fmt, out_fmt, 72)
 
 
+# the 12-bit format (|value| <= 2047: short filters, small injected values), against itself and the other two
+@pytest.mark.parametrize("variant", VARIANTS)
+@pytest.mark.parametrize("in_fmt,out_fmt", [(2, 2), (2, 1), (1, 2), (0, 2), (2, 0)])
+@pytest.mark.parametrize("cin,cout", [(64, 96), (128, 64), (64, 35), (128, 160)])
+def test_conv128_residual_modes_12_bit(gpu, variant, cin, cout, in_fmt, out_fmt):
+    _residual_modes(gpu, variant, cin, cout, in_fmt, out_fmt, 72, amp=800)
+
+
+@pytest.mark.parametrize("b", [2, 34, 66])
+def test_conv128_residual_modes_12_bit_small_batch(gpu, b):
+    _residual_modes(gpu, "mfma_f4", 64, 64, 2, 2, b, amp=800)
+
+
 @pytest.mark.parametrize("b", [1, 5, 33])
 @pytest.mark.parametrize("cin,cout", [(64, 64), (256, 96), (512, 64)])
 def test_conv128_residual_modes_small_batch(gpu, b, cin, cout):
@@ -269,7 +304,7 @@ def test_conv128_residual_modes_small_batch(gpu, b, cin, cout):
     _residual_modes(gpu, "mfma_f4", cin, cout, 1, 1, b)
 
 
-def _residual_modes(gpu, variant, cin, cout, in_fmt, out_fmt, b):
+def _residual_modes(gpu, variant, cin, cout, in_fmt, out_fmt, b, amp=3000):
     r = rng(41 + cin + cout + b)
     h = 6
     x = rm.pm1(r, (b, h, h, cin))
@@ -287,7 +322,7 @@ def _residual_modes(gpu, variant, cin, cout, in_fmt, out_fmt, b):
 
     # source narrower than the consumer and a limit that cuts through a channel tile
     src_ch, lim = (cout * 2) // 3, (cout * 5) // 6
-    src = r.integers(-3000, 3000, size=(h, h, b, src_ch)).astype(np.int32)
+    src = r.integers(-amp, amp, size=(h, h, b, src_ch)).astype(np.int32)
     layer = _run_conv_layer(gpu, variant, x, f, bn, save_residual=True, inject_residual=True,
                             residual_channels=lim, res_in=src, in_fmt=in_fmt, out_fmt=out_fmt)
     want, wres = orc.conv128(inp, filt, bn, cin, cout, 3, 3, save_residual=True, inject_residual=True,
@@ -297,7 +332,7 @@ def _residual_modes(gpu, variant, cin, cout, in_fmt, out_fmt, b):
     layer.release()
 
     # 2x2 max of a source twice the size; source wider than the limit
-    src2 = r.integers(-3000, 3000, size=(2 * h, 2 * h, b, cout)).astype(np.int32)
+    src2 = r.integers(-amp, amp, size=(2 * h, 2 * h, b, cout)).astype(np.int32)
     layer = _run_conv_layer(gpu, variant, x, f, bn, save_residual=True, inject_residual=True,
                             residual_channels=cout // 2, residual_pool=True, res_in=src2, in_fmt=in_fmt,
                             out_fmt=out_fmt)
@@ -321,6 +356,9 @@ def test_residual_format_follows_the_bound(gpu):
     layer's bound comes from the actual input, every bit convolution adds Cin*R*S."""
     lib = gpu.lib
     assert lib.tcbnn_residual_format_for_bound(32767) == 1 and lib.tcbnn_residual_format_for_bound(32768) == 0
+    assert lib.tcbnn_residual_format_narrowest(2047, 8) == 2 and lib.tcbnn_residual_format_narrowest(2048, 8) == 1
+    assert lib.tcbnn_residual_format_narrowest(2047, 7) == 1 and lib.tcbnn_residual_format_narrowest(40000, 8) == 0
+    assert lib.tcbnn_residual_bytes(3, 5, 17, 12, 2) == 3 * 5 * 2 * 12 * 24  # 17 channels: 2 groups of 16, 24 bytes
     assert lib.tcbnn_inconv_residual_bound(7, 7, float("inf")) == 2 ** 31 - 1
     assert lib.tcbnn_inconv_residual_bound(7, 7, float("nan")) == 2 ** 31 - 1
     assert 147 * 5 <= lib.tcbnn_inconv_residual_bound(7, 7, 5.0) <= 147 * 5 + 3
@@ -331,18 +369,24 @@ def test_residual_format_follows_the_bound(gpu):
     b, h, cout = 4, 16, 64
     f = rm.pm1(r, (7, 7, 3, cout))
     bn = r.normal(0, 12, cout).astype(np.float32)
-    for scale, fmt in ((1.0, 1), (400.0, 0)):  # 147 * 400 * |x| overflows 16 bits: int32 is kept
+    # the bound is the largest window sum of |x| (147 terms of mean 0.8 here): 12 bits; x 20: 16 bits; x 400: int32
+    for scale, fmt in ((1.0, 2), (20.0, 1), (400.0, 0)):
         x = (r.standard_normal((b, 3, h, h)) * scale).astype(np.float32)
         want, wres = orc.inconv128(x, f, bn, 4, True, 1, True)
         layer = gpu.InConv128LayerParam("Conv1", h, h, 7, 7, 3, cout, b, 4, 4, True, 1, 1, True)
         layer.initialize(x, gpu.ArrayWeights([f, bn]))
         assert layer.output_residual_gpu.format == fmt
         assert np.abs(wres).max() <= layer.output_residual_gpu.bound
+        # the bound is the window sum of |x|, within its slack, and never below what any filter can reach
+        xa = np.abs(x).sum(axis=1)
+        win = max(xa[i, max(0, 4 * y - 3):4 * y + 4, max(0, 4 * q - 3):4 * q + 4].sum()
+                  for i in range(b) for y in range(4) for q in range(4))
+        assert win <= layer.output_residual_gpu.bound <= win * 1.002 + 2
         layer.forward()
         gpuops.sync()
         np.testing.assert_array_equal(layer.download_packed(), want)
         np.testing.assert_array_equal(layer.download_residual(), wres)
-        if fmt == 1:
+        if fmt != 0:
             with pytest.raises(gpu.TcbnnError):
                 layer.set_input(x * 1000)
         layer.release()
@@ -519,15 +563,18 @@ def test_inconv128_presigned_input_is_exact_integer_conv(gpu):
 
 
 # --------------------------------------------------------------------------- whole networks
-@pytest.mark.parametrize("fmt", [0, 1])
+@pytest.mark.parametrize("fmt", [0, 1, 2])
 @pytest.mark.parametrize("h,b,c", [(5, 9, 64), (3, 70, 35), (2, 8, 130)])
 def test_residual_from_reference(gpu, h, b, c, fmt):
     """Reference layout int32 [P][Q][PAD8(B)][PAD128(C)] -> engine layouts: against a host transpose, and back
     through the existing converter (whose oracle twin is pinned on the CPU)."""
     from tcbnn_amd import _lib
     from tcbnn_amd.device import DeviceBuffer
+    if fmt == 2 and b % 2:
+        b += 1  # the 12-bit layout wants an even batch
     r = rng(h * 100 + b + c + fmt)
-    res = r.integers(-30000, 30000, size=(h, h, b, c)).astype(np.int32)
+    amp = 2047 if fmt == 2 else 30000
+    res = r.integers(-amp, amp + 1, size=(h, h, b, c)).astype(np.int32)
     ref_host = orc.residual_to_reference(res)
     ref_host[:, :, b:, :] = 0x5A5A5A5A  # padding images / channels of a foreign buffer hold anything
     ref_host[:, :, :, c:] = 0x5A5A5A5A
@@ -537,9 +584,14 @@ def test_residual_from_reference(gpu, h, b, c, fmt):
     gpuops.check(_lib.lib.tcbnn_residual_from_reference(ref.ptr, own.ptr, h, h, b, c, fmt, None))
     gpuops.sync()
     want = _residual_source(res, fmt)  # the engine layout by host transpose, channels past c zero
-    grp, dt = (8, np.int16) if fmt == 1 else (4, np.int32)
-    shape = (h, h, (c + grp - 1) // grp, b, grp)
-    np.testing.assert_array_equal(own.to_numpy(dt, shape), want.to_numpy(dt, shape))
+    if fmt == 2:  # (channels past c in the last group are zero on both sides)
+        G = (c + 15) // 16
+        words = lambda buf: buf.to_numpy(np.uint32, (h, h, G, 6 * b))
+        np.testing.assert_array_equal(words(own), words(want))
+    else:
+        grp, dt = (8, np.int16) if fmt == 1 else (4, np.int32)
+        shape = (h, h, (c + grp - 1) // grp, b, grp)
+        np.testing.assert_array_equal(own.to_numpy(dt, shape), want.to_numpy(dt, shape))
     back = DeviceBuffer(ref_host.nbytes)
     gpuops.check(_lib.lib.tcbnn_residual_to_reference(own.ptr, back.ptr, h, h, b, c, fmt, None))
     gpuops.sync()
@@ -692,18 +744,19 @@ def test_cifar10_vgg_batch256_presigned_input(gpu):
     net.release()
 
 
-@pytest.mark.parametrize("residual_format", [None, 0], ids=["narrowest", "int32"])
+@pytest.mark.parametrize("residual_format", [None, 0, 1], ids=["narrowest", "int32", "int16"])
 @pytest.mark.parametrize("variant", VARIANTS)
 def test_imagenet_resnet18(gpu, variant, residual_format):
-    """Residuals in the narrowest exact format (16 bits all the way for N(0,1) input: the test checks that
-    this is what was chosen) and, as the reference stores them, in int32: same bits either way."""
+    """Residuals in the narrowest exact format (for N(0,1) input: 12 bits for the first layer's and the first
+    stage's tensors, whose bounds stay below 2048, and 16 bits from the second stage on: the test checks that this
+    is what was chosen), all in 16 bits, and, as the reference stores them, in int32: same bits every way."""
     from tcbnn_amd import nets
     spec = nets.imagenet_resnet_spec(batch=8)
     if residual_format is None:
         net = gpu.Network(spec, gpu.synthetic_weights(spec, 3), gpu.synthetic_input(spec, 3))
         fmts = {L["name"]: net.layers[L["name"]].output_residual_gpu.format for L in spec if L.get("save_residual")}
         net.release()
-        assert fmts and all(f == 1 for f in fmts.values()), fmts
+        assert fmts and all(f == (2 if name in ("Conv1", "L1B1C2", "L1B2C2") else 1) for name, f in fmts.items()), fmts
     _compare_network(gpu, spec, 3, variant, residual_format)
 
 
@@ -738,15 +791,18 @@ def test_imagenet_resnet18_textbook_wiring(gpu, variant):
     _compare_network(gpu, nets.imagenet_resnet_textbook_spec(batch=8), 14, variant)
 
 
-@pytest.mark.parametrize("fmt", [0, 1])
+@pytest.mark.parametrize("fmt", [0, 1, 2])
 @pytest.mark.parametrize("b,h,c,window,stride,pad", [(8, 12, 64, 3, 2, 1), (70, 7, 40, 3, 2, 1), (5, 9, 100, 2, 2, 0),
                                                      (3, 5, 33, 3, 1, 1)])
 def test_pool128(gpu, b, h, c, window, stride, pad, fmt):
-    """Overlapping OR / max pooling: bits and residual against the oracle, both residual formats, odd shapes."""
+    """Overlapping OR / max pooling: bits and residual against the oracle, every residual format, odd shapes."""
     from tcbnn_amd import layers
+    if fmt == 2 and b % 2:
+        b += 1  # the 12-bit layout wants an even batch
     r = rng(b + h + c)
     x = rm.pm1(r, (b, h, h, c))
-    res = r.integers(-30000, 30000, size=(h, h, b, c)).astype(np.int32)
+    amp = 2047 if fmt == 2 else 30000
+    res = r.integers(-amp, amp + 1, size=(h, h, b, c)).astype(np.int32)
     inp = orc.pack_conv_input_nhwc(x)
     want_bits, want_res = orc.pool128(inp, c, window, stride, pad, res)
     layer = layers.Pool128LayerParam("p", h, h, c, b, window, stride, pad, pool_residual=True)
@@ -758,12 +814,15 @@ def test_pool128(gpu, b, h, c, window, stride, pad, fmt):
     layer.release()
 
 
-@pytest.mark.parametrize("fmt", [0, 1])
+@pytest.mark.parametrize("fmt", [0, 1, 2])
 @pytest.mark.parametrize("b,h,c,n", [(8, 7, 512, 1000), (70, 3, 100, 37), (33, 1, 64, 10)])
 def test_avgpool_fc(gpu, b, h, c, n, fmt):
     from tcbnn_amd import layers
+    if fmt == 2 and b % 2:
+        b += 1  # the 12-bit layout wants an even batch
     r = rng(b + h + c + n)
-    res = r.integers(-20000, 20000, size=(h, h, b, c)).astype(np.int32)
+    amp = 2047 if fmt == 2 else 20000
+    res = r.integers(-amp, amp + 1, size=(h, h, b, c)).astype(np.int32)
     w = r.standard_normal((c, n)).astype(np.float32)
     bias = r.standard_normal(n).astype(np.float32)
     want = orc.avgpool_fc(res, w, bias)
