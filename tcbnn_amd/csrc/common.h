@@ -121,11 +121,18 @@ __device__ __forceinline__ void i12_unpack8(uint32_t d0, uint32_t d1, uint32_t d
     v[6] = ((int)(d2 << 12)) >> 20;
     v[7] = (int)d2 >> 20;
 }
+// (only the low 12 bits of each v[] are looked at; 12 instructions: shift-or, and-or, bit-field extract, byte permute)
 __device__ __forceinline__ void i12_pack8(const int* v, uint32_t& d0, uint32_t& d1, uint32_t& d2) {
     const uint32_t m = 0xfffu;
-    d0 = ((uint32_t)v[0] & m) | (((uint32_t)v[1] & m) << 12) | ((uint32_t)v[2] << 24);
-    d1 = (((uint32_t)v[2] & m) >> 8) | (((uint32_t)v[3] & m) << 4) | (((uint32_t)v[4] & m) << 16) | ((uint32_t)v[5] << 28);
-    d2 = (((uint32_t)v[5] & m) >> 4) | (((uint32_t)v[6] & m) << 8) | ((uint32_t)v[7] << 20);
+    const uint32_t u0 = (uint32_t)v[0], u1 = (uint32_t)v[1], u2 = (uint32_t)v[2], u3 = (uint32_t)v[3], u4 = (uint32_t)v[4],
+                   u5 = (uint32_t)v[5], u6 = (uint32_t)v[6], u7 = (uint32_t)v[7];
+    const uint32_t a = (u1 << 12) | (u0 & m);                    // v0, v1 in bits 0-23 (above: leftovers of v1)
+    d0 = __builtin_amdgcn_perm(u2, a, 0x04020100u);              // ... and the low byte of v2 on top
+    const uint32_t lo = (u3 << 4) | __builtin_amdgcn_ubfe(u2, 8, 4);   // bits 0-15: high nibble of v2, v3
+    const uint32_t hi = (u5 << 12) | (u4 & m);                         // bits 0-15: v4, low nibble of v5
+    d1 = __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+    const uint32_t f = (u7 << 12) | (u6 & m);                    // v6, v7 in bits 0-23
+    d2 = (f << 8) | __builtin_amdgcn_ubfe(u5, 4, 8);             // high byte of v5 below them
 }
 __device__ __forceinline__ size_t residual_index(int fmt, size_t pix, int channels, int c, int batch, int b) {
     if (fmt == TCBNN_RES_I16) return ((pix * (size_t)((channels + 7) / 8) + (c >> 3)) * batch + b) * 8 + (c & 7);

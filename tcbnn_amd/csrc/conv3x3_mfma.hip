@@ -344,8 +344,19 @@ conv3x3_mfma_f4_kernel(
     constexpr int NRV = kRes ? MT * NT : 1;
     constexpr int NTMP = RM == RM_POOLED ? 3 : 1;
     constexpr bool R16 = RF == TCBNN_RES_I16, R12 = RF == TCBNN_RES_I12;  // format of the injected tensor
+    // Narrow injected residual on full tiles: the sum, the residual and the threshold meet as floats that carry
+    // small integers on top of 1.5 * 2^23 (kMagicBits), where the float's bit pattern IS 0x4B400000 + integer:
+    //   the accumulators start from 1.5 * 2^23, so the finished one is such a float (exact: every partial sum is an
+    //   integer below 2^24), and adding the residual is ONE integer add on its bit pattern (no conversions),
+    //   its low 16 (or 12) bits are the two's complement value to store (no conversion, no subtraction),
+    //   minus (1.5 * 2^23 + ceil(threshold)) has the sign the output bit needs.
+    // The layers this serves are bound by instruction issue (the matrix pipeline and the VALU of a SIMD do not
+    // overlap): 4.5 to 6.5 VALU instructions per value instead of 9.
+    constexpr bool kMagic = kRes && FULLT && (R16 || R12);
+    constexpr uint32_t kMagicBits = 0x4B400000u;  // 12582912.0f
     constexpr int NRAW = R12 ? 6 : (R16 ? 8 : 16);        // words loaded per channel tile
-    constexpr int NW = RM == RM_POOLED ? 16 : NRAW;       // words kept per channel tile
+    constexpr bool kPackedMax = RM == RM_POOLED && R16 && kMagic;  // 2x2 maximum taken on the packed 16-bit pairs
+    constexpr int NW = RM == RM_POOLED && !kPackedMax ? 16 : NRAW;  // words kept per channel tile
     int tmp[NTMP][NRV][NRAW];  // pooled: the other three pixels of the 2x2 window
     // A lane's 16 channels are 4 groups of 4 (int32) or 2 groups of 8 (int16), 16 bytes each, or one 12-bit group
     // of 24 bytes (a 16-byte piece in the group's first plane, an 8-byte piece in its second).
@@ -435,6 +446,15 @@ conv3x3_mfma_f4_kernel(
                     }
 #pragma unroll
                     for (int v = 0; v < 16; ++v) rv[nt][v] = m[v];
+                } else if constexpr (kPackedMax) {
+                    typedef short s2_t __attribute__((ext_vector_type(2)));
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) {
+                        s2_t m = __builtin_bit_cast(s2_t, rv[nt][k]);
+#pragma unroll
+                        for (int t = 0; t < 3; ++t) m = __builtin_elementwise_max(m, __builtin_bit_cast(s2_t, tmp[t][nt][k]));
+                        rv[nt][k] = __builtin_bit_cast(int, m);
+                    }
                 } else if constexpr (R16) {
 #pragma unroll
                     for (int k = 7; k >= 0; --k) {  // downwards: slot k is read before 2k, 2k+1 are written
@@ -511,7 +531,78 @@ conv3x3_mfma_f4_kernel(
             const int b = bimg[mt];
             const bool b_ok = b < p.B;
             uint32_t hw = 0;
-            if constexpr (kRes) {
+            if constexpr (kMagic && FAST) {
+                // The accumulators started from 1.5 * 2^23 (acc0), so their bit patterns are 0x4B400000 + sum: the
+                // residual is added to the PATTERN with an integer add, and the result is again such a float.
+                uint32_t tb[16];
+                const int* w = rv[mt * NT + nt];
+                if constexpr (R12 && RM == RM_PLAIN) {  // still packed: six words
+                    int un[16];
+                    i12_unpack8((uint32_t)w[0], (uint32_t)w[1], (uint32_t)w[2], un);
+                    i12_unpack8((uint32_t)w[3], (uint32_t)w[4], (uint32_t)w[5], un + 8);
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) tb[v] = __float_as_uint(acc[mt][nt][v]) + (uint32_t)un[v];
+                } else if constexpr (R12 || !kPackedMax && RM == RM_POOLED) {  // sixteen ints (2x2 maximum taken)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) tb[v] = __float_as_uint(acc[mt][nt][v]) + (uint32_t)w[v];
+                } else {  // eight words of two int16 (plain, or the packed 2x2 maximum)
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) {
+                        tb[2 * k] = __float_as_uint(acc[mt][nt][2 * k]) + (uint32_t)(int)(short)(w[k] & 0xffff);
+                        tb[2 * k + 1] = __float_as_uint(acc[mt][nt][2 * k + 1]) + (uint32_t)(w[k] >> 16);
+                    }
+                }
+                float t[16];  // 1.5 * 2^23 + (sum + residual)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) t[v] = __uint_as_float(tb[v]);
+                if (rout != nullptr) {
+                    // the value to store is in the low bits of t's bit pattern (see the 128-bit store note below)
+                    v4i q[4];
+                    if (rout_fmt == TCBNN_RES_I12) {
+                        int tb[16];
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) tb[v] = (int)__float_as_uint(t[v]);
+                        uint32_t d[6];
+                        i12_pack8(tb, d[0], d[1], d[2]);
+                        i12_pack8(tb + 8, d[3], d[4], d[5]);
+                        const unsigned so = (pix * (unsigned)((p.N + 15) / 16) + (unsigned)((n0 + nt * 32) / 16)) * g12_b;
+                        const unsigned vo = b_ok ? (unsigned)h * g12_b + (unsigned)b * 16u : kOutOfRange;
+                        const unsigned vo2 = b_ok ? (unsigned)h * g12_b + grp_b + (unsigned)b * 8u : kOutOfRange;
+                        q[0] = v4i{(int)d[0], (int)d[1], (int)d[2], (int)d[3]};
+                        typedef int v2i_t __attribute__((ext_vector_type(2)));
+                        const v2i_t q2 = {(int)d[4], (int)d[5]};
+                        __builtin_amdgcn_raw_buffer_store_b128(q[0], r_rout, (int)vo, (int)so, 0);
+                        __builtin_amdgcn_raw_buffer_store_b64(q2, r_rout, (int)vo2, (int)so, 0);
+                        asm volatile("s_nop 4" ::"v"(q[0]), "v"(q2));
+                    } else if (rout_fmt == TCBNN_RES_I16) {
+                        const unsigned so = (pix * (unsigned)((p.N + 7) / 8) + (unsigned)((n0 + nt * 32) / 8)) * grp_b;
+                        const unsigned vo = b_ok ? ((unsigned)(2 * h) * (unsigned)p.B + (unsigned)b) * 16u : kOutOfRange;
+#pragma unroll
+                        for (int g = 0; g < 2; ++g) {
+#pragma unroll
+                            for (int k = 0; k < 4; ++k)  // the low halves of two bit patterns: one byte permute
+                                q[g][k] = (int)__builtin_amdgcn_perm(__float_as_uint(t[8 * g + 2 * k + 1]),
+                                                                     __float_as_uint(t[8 * g + 2 * k]), 0x05040100u);
+                            __builtin_amdgcn_raw_buffer_store_b128(q[g], r_rout, (int)vo, (int)(so + (unsigned)g * grp_b), 0);
+                        }
+                        asm volatile("s_nop 4" ::"v"(q[0]), "v"(q[1]));
+                    } else {
+                        const unsigned so = (pix * (unsigned)((p.N + 3) / 4) + (unsigned)((n0 + nt * 32) / 4)) * grp_b;
+                        const unsigned vo = b_ok ? ((unsigned)(4 * h) * (unsigned)p.B + (unsigned)b) * 16u : kOutOfRange;
+#pragma unroll
+                        for (int g = 0; g < 4; ++g) {
+#pragma unroll
+                            for (int k = 0; k < 4; ++k) q[g][k] = (int)(__float_as_uint(t[4 * g + k]) - kMagicBits);
+                            __builtin_amdgcn_raw_buffer_store_b128(q[g], r_rout, (int)vo, (int)(so + (unsigned)g * grp_b), 0);
+                        }
+                        asm volatile("s_nop 4" ::"v"(q[0]), "v"(q[1]), "v"(q[2]), "v"(q[3]));
+                    }
+                }
+                // bit = !(sum + residual < threshold): the inverted sign of t - (1.5 * 2^23 + ceil(threshold))
+#pragma unroll
+                for (int v = 0; v < 16; ++v) hw = __builtin_amdgcn_alignbit(hw, __float_as_uint(t[v] - thr[v]), 31);
+                hw = ~hw & 0xffffu;
+            } else if constexpr (kRes) {
                 int res[16];
                 int un[16];  // a plain 12-bit operand is still packed: six words -> sixteen values
                 if constexpr (RM == RM_PLAIN && R12) {
@@ -786,13 +877,16 @@ conv3x3_mfma_f4_kernel(
         float t = thr_stage;
         t = t != t ? -__builtin_huge_valf() : t;
         if constexpr (RM == RM_NONE) t = 0.0f - fminf(fmaxf(ceilf(t), -8192.0f), 8192.0f);
+        // (narrow residuals: |sum + residual| < 2^16 + 4608, so thresholds beyond +-2^21 decide like +-2^21)
+        if constexpr (kMagic) t = __uint_as_float(kMagicBits) + fminf(fmaxf(ceilf(t), -2097152.0f), 2097152.0f);
         lds_thr[tid] = t;
     }
     __syncthreads();
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) acc0[nt][v] = RM == RM_NONE ? lds_thr[nt * 32 + 16 * h + v] : 0.0f;
+        for (int v = 0; v < 16; ++v)
+            acc0[nt][v] = RM == RM_NONE ? lds_thr[nt * 32 + 16 * h + v] : (kMagic ? __uint_as_float(kMagicBits) : 0.0f);
     if constexpr (kAhead && RM == RM_POOLED) {  // (one tile ahead: the first tile's operand)
         if (cc.pi < npix) finish_residual(rv[0]);
     }
