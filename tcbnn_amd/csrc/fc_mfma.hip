@@ -11,6 +11,7 @@
 //   wave 0    = epilogue: threshold + pack (FC) or scale + bias (output layer).
 // No split-K workspace in HBM, no clearing or finishing launch.
 #include <algorithm>
+#include <type_traits>
 
 #include "common.h"
 #include "mfma_util.h"
@@ -23,11 +24,13 @@ using namespace mfma;
 constexpr int kMaxWaves = 16;
 constexpr int FC_THRESH = 0, FC_AFFINE = 1;
 
-template <int MODE>
+// PRE > 0: the wave's K slice is at most PRE groups and is requested whole before the first multiply.
+template <int MODE, int PRE>
 __global__ __launch_bounds__(64 * kMaxWaves) void fc_mfma_f4_kernel(
     const BgemmParams p, const uint32_t* __restrict__ act, const uint32_t* __restrict__ wgt,
     const float* __restrict__ bnp, const float* __restrict__ bias, int n_tiles, int groups_per_wave) {
     __shared__ int red[16 * 64];
+    __shared__ float par[64];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -78,35 +81,57 @@ __global__ __launch_bounds__(64 * kMaxWaves) void fc_mfma_f4_kernel(
         }
     };
 
-    // two groups (8 k-steps) per stage, double-buffered in registers
-    v4i a0[2], a1[2];
-    uint32_t w0[2][4], w1[2][4];
-    auto load_stage = [&](int g, v4i (&a)[2], uint32_t (&bw)[2][4]) {
+    // Epilogue parameters (thresholds, or scales and biases) of the tile's 32 neurons: one per lane, requested here,
+    // ahead of the K loop, so that their round trip hides behind the operands'.  Neurons past N read the last valid
+    // entry and are discarded.  Wave 0 passes them through LDS into the epilogue's layout (16 neurons per lane).
+    const float my_thr = bnp[min(n0 + j, p.N - 1)];
+    const float my_bias = MODE == FC_AFFINE ? bias[min(n0 + j, p.N - 1)] : 0.0f;
+
+    if constexpr (PRE > 0) {
+        // short slice: every operand word of the wave is requested before the first multiply (one round trip)
+        v4i a[PRE];
+        uint32_t bw[PRE][4];
 #pragma unroll
-        for (int u = 0; u < 2; ++u)
-            if (g + u < g_end) load_group(g + u, a[u], bw[u]);
-    };
-    auto compute_stage = [&](int g, v4i (&a)[2], uint32_t (&bw)[2][4]) {
+        for (int u = 0; u < PRE; ++u)
+            if (g_begin + u < g_end) load_group(g_begin + u, a[u], bw[u]);
 #pragma unroll
-        for (int u = 0; u < 2; ++u)
-            if (g + u < g_end) compute_group(g + u, a[u], bw[u]);
-    };
-    int g = g_begin;
-    if (g < g_end) load_stage(g, a0, w0);
-    while (g < g_end) {
-        if (g + 2 < g_end) load_stage(g + 2, a1, w1);
-        compute_stage(g, a0, w0);
-        g += 2;
-        if (g >= g_end) break;
-        if (g + 2 < g_end) load_stage(g + 2, a0, w0);
-        compute_stage(g, a1, w1);
-        g += 2;
+        for (int u = 0; u < PRE; ++u)
+            if (g_begin + u < g_end) compute_group(g_begin + u, a[u], bw[u]);
+    } else {
+        // two groups (8 k-steps) per stage, double-buffered in registers
+        v4i a0[2], a1[2];
+        uint32_t w0[2][4], w1[2][4];
+        auto load_stage = [&](int g, v4i (&a)[2], uint32_t (&bw)[2][4]) {
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+                if (g + u < g_end) load_group(g + u, a[u], bw[u]);
+        };
+        auto compute_stage = [&](int g, v4i (&a)[2], uint32_t (&bw)[2][4]) {
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+                if (g + u < g_end) compute_group(g + u, a[u], bw[u]);
+        };
+        int g = g_begin;
+        if (g < g_end) load_stage(g, a0, w0);
+        while (g < g_end) {
+            if (g + 2 < g_end) load_stage(g + 2, a1, w1);
+            compute_stage(g, a0, w0);
+            g += 2;
+            if (g >= g_end) break;
+            if (g + 2 < g_end) load_stage(g + 2, a0, w0);
+            compute_stage(g, a1, w1);
+            g += 2;
+        }
     }
 
     // ---- sum the K slices of the waves (exact integers) in LDS
     int dot[16];
 #pragma unroll
     for (int v = 0; v < 16; ++v) dot[v] = (int)acc[v];
+    if (wave == 0) {
+        par[j] = my_thr;
+        if constexpr (MODE == FC_AFFINE) par[32 + j] = my_bias;
+    }
     if (kwaves > 1) {
         if (wave == 0) {
 #pragma unroll
@@ -121,17 +146,17 @@ __global__ __launch_bounds__(64 * kMaxWaves) void fc_mfma_f4_kernel(
         if (wave != 0) return;
 #pragma unroll
         for (int v = 0; v < 16; ++v) dot[v] = red[v * 64 + lane];
+    } else {
+        __syncthreads();
     }
 
-    // ---- epilogue (wave 0): the lane holds neurons cbase + v of image b.  Its 16 thresholds (or scales and
-    // biases) are requested together, without bounds tests around the loads (neurons past N read the last valid
-    // entry and are discarded): a load under each test would be a chain of memory round trips.
+    // ---- epilogue (wave 0): the lane holds neurons cbase + v of image b
     const int cbase = n0 + 16 * h;
     float thr[16], bia[MODE == FC_AFFINE ? 16 : 1];
 #pragma unroll
     for (int v = 0; v < 16; ++v) {
-        thr[v] = bnp[min(cbase + v, p.N - 1)];
-        if constexpr (MODE == FC_AFFINE) bia[v] = bias[min(cbase + v, p.N - 1)];
+        thr[v] = par[16 * h + v];
+        if constexpr (MODE == FC_AFFINE) bia[v] = par[32 + 16 * h + v];
     }
     if constexpr (MODE == FC_THRESH) {
         uint32_t hw = 0;
@@ -170,25 +195,47 @@ bool fc_mfma_applicable(const BgemmParams& p) {
     return tiles <= 16384;
 }
 
-void fc_mfma_kernel_name(const BgemmParams& p, char* buf, size_t len) {
-    snprintf(buf, len, "fc_mfma_f4_kernel<%d>", p.mode == EPI_AFFINE ? FC_AFFINE : FC_THRESH);
-}
-
-int launch_fc_mfma(const BgemmParams& p, hipStream_t stream) {
-    const int n_tiles = (p.N + 31) / 32, b_tiles = (p.B + 31) / 32;
+namespace {
+// Split of K over the waves of a workgroup: waves per tile, 8-word groups per wave, and how many groups the
+// kernel requests ahead of its first multiply (0: a streaming loop).
+struct FcPlan {
+    int n_tiles, b_tiles, kwaves, gpw, pre;
+};
+FcPlan fc_plan(const BgemmParams& p) {
+    FcPlan f;
+    f.n_tiles = (p.N + 31) / 32;
+    f.b_tiles = (p.B + 31) / 32;
     const int groups = (p.cw + 7) / 8;
     // waves per tile: at least 4 groups (16 k-steps) each, no more than fill the machine a few times
     int kwaves = std::max(1, std::min(kMaxWaves, groups / 4));
-    while (kwaves > 1 && (long long)n_tiles * b_tiles * kwaves > 8192) --kwaves;
-    const int gpw = (groups + kwaves - 1) / kwaves;
-    kwaves = (groups + gpw - 1) / gpw;
+    while (kwaves > 1 && (long long)f.n_tiles * f.b_tiles * kwaves > 8192) --kwaves;
+    f.gpw = (groups + kwaves - 1) / kwaves;
+    f.kwaves = (groups + f.gpw - 1) / f.gpw;
+    f.pre = f.gpw <= 2 ? 2 : (f.gpw <= 7 ? 7 : 0);
+    return f;
+}
+}  // namespace
+
+void fc_mfma_kernel_name(const BgemmParams& p, char* buf, size_t len) {
+    snprintf(buf, len, "fc_mfma_f4_kernel<%d, %d>", p.mode == EPI_AFFINE ? FC_AFFINE : FC_THRESH, fc_plan(p).pre);
+}
+
+int launch_fc_mfma(const BgemmParams& p, hipStream_t stream) {
+    const FcPlan f = fc_plan(p);
+    const int n_tiles = f.n_tiles, b_tiles = f.b_tiles, kwaves = f.kwaves, gpw = f.gpw;
     const dim3 grid((unsigned)(n_tiles * b_tiles)), block(64 * kwaves);
-    if (p.mode == EPI_AFFINE)
-        hipLaunchKernelGGL(fc_mfma_f4_kernel<FC_AFFINE>, grid, block, 0, stream, p, p.act, p.wgt, p.bn_scale, p.bn_bias,
-                           n_tiles, gpw);
-    else
-        hipLaunchKernelGGL(fc_mfma_f4_kernel<FC_THRESH>, grid, block, 0, stream, p, p.act, p.wgt, p.bn, p.bn, n_tiles,
-                           gpw);
+    auto launch = [&](auto mode, auto pre) {
+        constexpr int MODE = decltype(mode)::value, PRE = decltype(pre)::value;
+        hipLaunchKernelGGL((fc_mfma_f4_kernel<MODE, PRE>), grid, block, 0, stream, p, p.act, p.wgt,
+                           MODE == FC_AFFINE ? p.bn_scale : p.bn, MODE == FC_AFFINE ? p.bn_bias : p.bn, n_tiles, gpw);
+    };
+    auto by_slice = [&](auto mode) {
+        if (f.pre == 2) launch(mode, std::integral_constant<int, 2>{});
+        else if (f.pre == 7) launch(mode, std::integral_constant<int, 7>{});
+        else launch(mode, std::integral_constant<int, 0>{});
+    };
+    if (p.mode == EPI_AFFINE) by_slice(std::integral_constant<int, FC_AFFINE>{});
+    else by_slice(std::integral_constant<int, FC_THRESH>{});
     TCBNN_LAUNCH_CHECK("fc_mfma_f4_kernel");
     return TCBNN_OK;
 }
