@@ -52,9 +52,9 @@ constexpr int RM_PLAIN = 1;   // residual injected from a source of the same siz
 constexpr int RM_POOLED = 2;  // residual injected as the 2x2 max of a source twice the size
 constexpr int RM_RAW = 3;     // no threshold: the +-1 dot products are stored as int32 (tcbnn_bconv)
 
-// Waves per SIMD the register allocator is asked to make room for: the residual layers are
-// bound by HBM and want more memory requests in flight, the plain layers want registers.
-constexpr int waves_hint(int spt, int rm, int nt) { return rm == RM_PLAIN && spt == 4 && nt == 1 ? 3 : 2; }
+// Waves per SIMD the register allocator is asked to make room for (256 registers per lane: the plain layers
+// use them for two image tiles and two channel tiles, the residual layers for operands in flight).
+constexpr int kWavesPerSimd = 2;
 
 // SPT = k-steps (64 bits) per filter tap = Cin / 64; MT = 32-image tiles per wave (2 for plain
 // layers, 1 for residual layers); NT = 32-channel tiles per wave; RF = TCBNN_RES_* format of the
@@ -65,7 +65,7 @@ constexpr int waves_hint(int spt, int rm, int nt) { return rm == RM_PLAIN && spt
 // tests of partial tiles are then not even compiled (they cost scalar registers and set-up instructions in
 // every launch, and the networks' channel counts are multiples of 64).
 template <int SPT, int RM, int MT, int NT, int RF, bool POOL, bool FULLT>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(waves_hint(SPT, RM, NT)))) void
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(kWavesPerSimd))) void
 conv3x3_mfma_f4_kernel(
     const BgemmParams p, const uint32_t* __restrict__ act, const uint32_t* __restrict__ wgt,
     const float* __restrict__ bnp, const int32_t* __restrict__ rin, int32_t* __restrict__ rout, int res_lim,
@@ -1057,16 +1057,17 @@ int launch_t(const BgemmParams& p, hipStream_t stream) {
     return launch_f<SPT, RM, MT, NT, RF, POOL, false>(p, stream);
 }
 
-// Which instantiation serves a layer.  Measured on ResNet-18 at batch 256: the HBM-bound residual
-// layers run best with one image tile per wave and, from Cin = 256 on, one channel tile (more
-// workgroups fit a CU's LDS, so more residual requests are in flight); plain layers want the 2 x 2
-// tile (each operand fragment feeds two MFMAs) until the weights of 64 channels no longer leave
-// room for a second workgroup (Cin = 512).
+// Which instantiation serves a layer.  Measured on ResNet-18 at batch 256: two channel tiles per wave (each
+// expanded activation fragment feeds two MFMAs) wherever the weights of 64 channels leave room for a second
+// workgroup in a CU's LDS (up to Cin = 256; one workgroup of eight waves with two channel tiles was 20-45 %
+// slower on the Cin = 512 layers: one long tile per wave, nothing to overlap it with); layers that inject the
+// 2 x 2 maximum of a larger tensor run best with one (four times the residual operands per tile: more
+// workgroups keep more requests in flight).
 struct Pick {
     int rm, mt, nt, r16, pool;  // r16: TCBNN_RES_* format of the injected residual
 };
 constexpr int pick_nt(int spt, int rm) {
-    return rm == RM_POOLED ? 1 : (rm == RM_PLAIN ? (spt >= 4 ? 1 : 2) : (spt >= 6 ? 1 : 2));  // RM_RAW as RM_NONE
+    return rm == RM_POOLED ? 1 : (spt >= 6 ? 1 : 2);
 }
 // image tiles per wave: two wherever the layer is bound by issue slots rather than by HBM
 constexpr int pick_mt(int spt, int rm) {
