@@ -309,6 +309,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS &
         }
 
         if (work && b < p.B && wi < p.ow) {
+            // The stores' addresses are worked out here, after the tap loops: formed ahead of them (the compiler hoists
+            // what does not depend on the loops) they were live across the whole kernel and were spilled.
+            int b = b0 + lane;
+            asm volatile("" : "+v"(b));
 #pragma unroll
             for (int px = 0; px < 2; ++px) {
                 if (px == 1 && !xb_ok) continue;
