@@ -52,6 +52,15 @@ constexpr int RM_PLAIN = 1;   // residual injected from a source of the same siz
 constexpr int RM_POOLED = 2;  // residual injected as the 2x2 max of a source twice the size
 constexpr int RM_RAW = 3;     // no threshold: the +-1 dot products are stored as int32 (tcbnn_bconv)
 
+// RM_RAW: a wave's sums are transposed through a private LDS area of [32 images][32 NT + 4] words, so that every store
+// writes whole contiguous channel runs, wherever that area leaves room for two workgroups in a CU's 160 KB of LDS
+// next to the staged weights (9 SPT NT KB).  (The pitch, an odd multiple of 4 words, keeps both directions free of
+// bank conflicts.)
+constexpr int raw_pitch(int nt) { return 32 * nt + 4; }
+constexpr bool raw_transposed(int spt, int rm, int nt, bool fullt) {
+    return rm == RM_RAW && fullt && 9 * spt * nt * 1024 + kWaves * 32 * raw_pitch(nt) * 4 <= 80 * 1024;
+}
+
 // Waves per SIMD the register allocator is asked to make room for (256 registers per lane: the plain layers
 // use them for two image tiles and two channel tiles, the residual layers for operands in flight).
 constexpr int kWavesPerSimd = 2;
@@ -84,8 +93,8 @@ conv3x3_mfma_f4_kernel(
     float* lds_thr = reinterpret_cast<float*>(lds_dyn + NQ * NT * 64);  // [NT*32]
     // RM_RAW with short K (the output-bound shapes): a wave's private [32 images][kRawPitch] int32 staging area, through
     // which a 32-image tile's sums are transposed so that every store writes whole contiguous channel runs
-    constexpr bool kRawTranspose = RM == RM_RAW && SPT <= 2 && NT == 2 && FULLT;
-    constexpr int kRawPitch = 32 * NT + 4;  // words per image row: the odd multiple of 4 keeps both directions conflict-free
+    constexpr bool kRawTranspose = raw_transposed(SPT, RM, NT, FULLT);
+    constexpr int kRawPitch = raw_pitch(NT);
     int* lds_raw = reinterpret_cast<int*>(lds_thr + NT * 32);
 
     const int tid = threadIdx.x;
@@ -729,12 +738,13 @@ conv3x3_mfma_f4_kernel(
     // int32 output [N][P][Q][O] (bmma_kernel.cu:247-263): for one image and pixel the wave's 32 NT channels are one
     // contiguous run, but in the accumulator a lane holds 16 channels of ONE image, so a direct store scatters
     // 16-byte pieces over 64 different rows per instruction.  The sums of a 32-image tile go through the wave's LDS
-    // area instead (row = image, conflict-free both ways) and leave as 128-bit stores in which 16 consecutive lanes
-    // cover one image's whole run (4 images, i.e. 4 runs of 256 bytes, per instruction).
+    // area instead (row = image, conflict-free both ways) and leave as 128-bit stores in which 8 NT consecutive lanes
+    // cover one image's whole run (4 runs of 256 bytes or 8 runs of 128 bytes per instruction).
     auto epilogue_raw_transposed = [&](unsigned pix) __attribute__((always_inline)) {
         if constexpr (kRawTranspose) {
             int* mine = lds_raw + wave * (32 * kRawPitch);
-            const int rl = lane >> 4, cl = lane & 15;  // image within a group of 4, 16-byte column of the run
+            constexpr int kCols = 8 * NT, kRows = 64 / kCols;  // 16-byte columns of a run; images per store instruction
+            const int rl = lane / kCols, cl = lane % kCols;
             const unsigned so0 = (pix * (unsigned)p.raw_pix_stride + (unsigned)n0) * 4u;  // uniform
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
@@ -749,16 +759,16 @@ conv3x3_mfma_f4_kernel(
                     }
                 // (same wave writes and reads: program order and the wait for LDS are all the synchronisation)
                 const int img0 = (bg * MT + mt) * 32;
-                // four rows at a time: eight would not fit the register file next to the activation buffers
+                // four store instructions at a time: eight would not fit the register file next to the activation buffers
 #pragma unroll
-                for (int half = 0; half < 2; ++half) {
+                for (int part = 0; part < 32 / (4 * kRows); ++part) {
                     v4i q[4];
 #pragma unroll
                     for (int k = 0; k < 4; ++k)
-                        q[k] = *reinterpret_cast<const v4i*>(mine + (16 * half + 4 * k + rl) * kRawPitch + 4 * cl);
+                        q[k] = *reinterpret_cast<const v4i*>(mine + ((4 * part + k) * kRows + rl) * kRawPitch + 4 * cl);
 #pragma unroll
                     for (int k = 0; k < 4; ++k) {
-                        const int img = img0 + 16 * half + 4 * k + rl;
+                        const int img = img0 + (4 * part + k) * kRows + rl;
                         const unsigned vo = img < p.B ? ((unsigned)img * (unsigned)p.raw_b_stride + 4u * (unsigned)cl) * 4u : kOutOfRange;
                         __builtin_amdgcn_raw_buffer_store_b128(q[k], r_rout, (int)vo, (int)so0, 0);
                     }
@@ -990,9 +1000,9 @@ TensorBytes tensor_bytes(const BgemmParams& p) {
 template <int SPT, int RM, int MT, int NT, int RF, bool POOL, bool FULLT>
 int launch_f(const BgemmParams& p, hipStream_t stream) {
     constexpr int NQ = 9 * SPT;
-    constexpr bool kRawTranspose = RM == RM_RAW && SPT <= 2 && NT == 2 && FULLT;  // as in the kernel
+    constexpr bool kRawTranspose = raw_transposed(SPT, RM, NT, FULLT);
     const size_t lds_bytes = (size_t)NQ * NT * 64 * 16 + NT * 32 * sizeof(float) +
-                             (kRawTranspose ? (size_t)kWaves * 32 * (32 * NT + 4) * sizeof(int) : 0);
+                             (kRawTranspose ? (size_t)kWaves * 32 * raw_pitch(NT) * sizeof(int) : 0);
     // Per instantiation and device, set up by the first launch there: the dynamic LDS limit, and how many of its
     // workgroups a CU holds at once (registers and LDS).  Atomics only so that two host threads that both find the
     // entry empty do no harm (both store the same value).
@@ -1067,7 +1077,7 @@ struct Pick {
     int rm, mt, nt, r16, pool;  // r16: TCBNN_RES_* format of the injected residual
 };
 constexpr int pick_nt(int spt, int rm) {
-    return rm == RM_POOLED ? 1 : (spt >= 6 ? 1 : 2);
+    return rm == RM_POOLED ? 1 : (rm == RM_RAW ? (spt >= 3 ? 1 : 2) : (spt >= 6 ? 1 : 2));
 }
 // image tiles per wave: two wherever the layer is bound by issue slots rather than by HBM
 constexpr int pick_mt(int spt, int rm) {
