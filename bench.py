@@ -231,6 +231,14 @@ def main():
     ap.add_argument("--layers", action="store_true", help="also print a per-layer table to stderr")
     ap.add_argument("--graph", action="store_true",
                     help="time the steps as replays of one captured HIP graph instead of eager launches")
+    ap.add_argument("--preheat-ms", type=float, default=100.0,
+                    help="untimed forward passes for this long before the --warmup steps: a freshly started process "
+                         "finds the GPU in a low clock state, and the step time keeps falling for the first 30-40 "
+                         "passes (about 20 ms); 0 = none")
+    ap.add_argument("--in-flight", type=int, default=2,
+                    help="after the timed steps, also time the same number of steps with this many independent "
+                         "batches in flight (one network copy and one stream each); reported as a separate "
+                         "object, never as `value`; 1 = skip")
     ap.add_argument("--sweep", action="store_true",
                     help="instead of a network: the stand-alone bit-GEMM and 3x3 bit-convolution shapes "
                          "(int32 outputs), every engine; one JSON line with a row per case")
@@ -265,6 +273,15 @@ def main():
     bops, flops = nets.binary_ops(spec)
 
     # ------------------------------------------------------------------ timed region
+    # Untimed: bring the GPU to its steady clock state first (measured on this device, fresh process, batch 256: the
+    # first pass after start-up takes 0.546 ms, the 40th and every later one 0.473 ms), then the W warm-up steps.
+    preheat_steps = 0
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < args.preheat_ms:
+        for _ in range(8):
+            net.forward(stream)
+        stream.synchronize()
+        preheat_steps += 8
     for _ in range(args.warmup):
         net.forward(stream)
     stream.synchronize()
@@ -284,6 +301,36 @@ def main():
     wall = time.perf_counter() - t0
     ms_per_step = wall / args.steps * 1e3
     images_per_s = batch * args.steps / wall
+
+    # ------------------------------------------------------------------ several batches in flight (a serving
+    # pipeline: batch n + 1 starts while batch n is still in its later layers, so the ragged end of one launch and
+    # the gap before the next are filled with the other batch's workgroups).  Same K steps = K forward passes of one
+    # batch each, dealt round-robin to N network copies (own activations, residuals and input; same weights) on N
+    # streams of the same priority.  Latency of one batch grows; reported beside `value`, never as `value`.
+    in_flight = None
+    if args.in_flight > 1 and not args.graph:
+        others = [tcbnn_amd.Network(spec, weights, tcbnn_amd.synthetic_input(spec, seed=i + 1))
+                  for i in range(args.in_flight - 1)]
+        copies = [net] + others
+        streams = [stream] + [Stream() for _ in others]
+        for k in range(max(args.warmup, args.in_flight)):
+            copies[k % len(copies)].forward(streams[k % len(copies)])
+        _lib.device_synchronize()
+        steps_n = max(args.steps, 100)  # (filling and draining the pipeline is one batch latency: keep it small)
+        t0 = time.perf_counter()
+        for k in range(steps_n):
+            copies[k % len(copies)].forward(streams[k % len(copies)])
+        for st in streams:
+            st.synchronize()
+        _lib.device_synchronize()
+        wall_n = time.perf_counter() - t0
+        in_flight = {"batches_in_flight": args.in_flight, "steps": steps_n,
+                     "value": round(batch * steps_n / wall_n, 1), "unit": "images/s",
+                     "ms_per_step": round(wall_n / steps_n * 1e3, 4),
+                     "note": "K forward passes of one batch each, round-robin over %d network copies on %d streams; "
+                             "throughput of a pipeline, not the latency of a batch" % (len(copies), len(streams))}
+        for o in others:
+            o.release()
 
     # ------------------------------------------------------------------ per-launch timing (HIP events
     # on the launch stream), outside the timed region
@@ -367,7 +414,10 @@ def main():
         "metric": "images/sec ResNet-18 BNN 224x224 batch 256 on 1 MI355X" if args.net == "imagenet_resnet"
         else "images/sec %s batch %d on 1 MI355X" % (args.net, batch),
         "value": round(images_per_s, 1), "unit": "images/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+        "warmup": args.warmup, "preheat": {"ms": args.preheat_ms, "steps": preheat_steps,
+                                           "what": "untimed forward passes before the warm-up steps, until the GPU's "
+                                                   "clocks have settled"},
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": round(images_per_s / PAPER_IMAGES_PER_S, 2) if args.net == "imagenet_resnet" and batch == 256
         else None,
@@ -393,6 +443,7 @@ def main():
         "binary_ops_per_step": bops, "fp32_first_layer_flops_per_step": flops,
         "roofline": roofline,
         "cpu_baseline": cpu,
+        "batches_in_flight": in_flight,
         "bit_layers_binary_tops": bit_layers_tops,
         "roofline_all_kernels": roofline_all,
     }
