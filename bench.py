@@ -162,12 +162,13 @@ def sweep(args, np, _lib):
         stream.synchronize()
         ts = []
         e0, e1 = Event(), Event()
-        for _ in range(reps):
+        for _ in range(3):  # `reps` back-to-back launches between two events (includes the gap between two launches)
             e0.record(stream)
-            launch()
+            for _r in range(reps):
+                launch()
             e1.record(stream)
             stream.synchronize()
-            ts.append(e0.elapsed_ms(e1))
+            ts.append(e0.elapsed_ms(e1) / reps)
         return float(np.median(ts))
 
     rows = []
@@ -333,17 +334,24 @@ def main():
             o.release()
 
     # ------------------------------------------------------------------ per-launch timing (HIP events
-    # on the launch stream), outside the timed region
+    # on the launch stream), outside the timed region.  A layer's duration = R back-to-back launches of it between
+    # two events, divided by R: it includes the gap between two launches of a stream, as the layer's share of a step
+    # does, but not the two event records, which cost about 5 us per launch when every launch of a pass is bracketed
+    # (the sum of such per-layer figures was 0.09 ms above the step they were taken from).  Layers are idempotent:
+    # every output word is rewritten by each launch.  One pass over the layers first, so that each layer finds its
+    # inputs as the forward leaves them.
+    R = 10
     per_layer = {L["name"]: [] for L in spec}
-    evs = [Event() for _ in range(len(spec) + 1)]
-    for _ in range(max(3, min(args.steps, 10))):
-        evs[0].record(stream)
-        for i, layer in enumerate(net.order):
-            layer.forward(stream)
-            evs[i + 1].record(stream)
-        stream.synchronize()
-        for i, L in enumerate(spec):
-            per_layer[L["name"]].append(evs[i].elapsed_ms(evs[i + 1]))
+    e0, e1 = Event(), Event()
+    net.forward(stream)
+    for _ in range(3):
+        for L, layer in zip(spec, net.order):
+            e0.record(stream)
+            for _r in range(R):
+                layer.forward(stream)
+            e1.record(stream)
+            stream.synchronize()
+            per_layer[L["name"]].append(e0.elapsed_ms(e1) / R)
     layer_ms = {k: float(np.median(v)) for k, v in per_layer.items()}
 
     # width each saved residual is stored in (16 bits where its bound proves that exact)
