@@ -80,3 +80,57 @@ def test_network_specs_match_reference_wiring():
     assert abs(bops / 1e9 - 47.68) < 0.05
     bops, _ = nets.binary_ops(nets.cifar10_vgg_spec(256))
     assert abs(bops / 1e9 - 314.1) < 0.5
+
+
+def test_residual_formats_sizes_and_choice():
+    """Host-only helpers of the residual storage formats: bytes per tensor, and the narrowest format a bound allows
+    (12 bits need an even batch: the format's 128-bit accesses are aligned only then)."""
+    from tcbnn_amd import _lib
+    L = _lib.lib
+    h, w, c, b = 5, 7, 64, 6
+    assert L.tcbnn_residual_bytes(h, w, c, b, _lib.RES_I32) == h * w * c * b * 4
+    assert L.tcbnn_residual_bytes(h, w, c, b, _lib.RES_I16) == h * w * c * b * 2
+    assert L.tcbnn_residual_bytes(h, w, c, b, _lib.RES_I12) == h * w * c * b * 3 // 2
+    # channels are stored in whole groups: 4 (int32), 8 (int16) or 16 (12 bits)
+    assert L.tcbnn_residual_bytes(1, 1, 17, 2, _lib.RES_I32) == 20 * 2 * 4
+    assert L.tcbnn_residual_bytes(1, 1, 17, 2, _lib.RES_I16) == 24 * 2 * 2
+    assert L.tcbnn_residual_bytes(1, 1, 17, 2, _lib.RES_I12) == 32 * 2 * 3 // 2
+    for bound, batch, want in ((0, 2, _lib.RES_I12), (2047, 256, _lib.RES_I12), (2048, 256, _lib.RES_I16),
+                               (2047, 255, _lib.RES_I16), (32767, 8, _lib.RES_I16), (32768, 8, _lib.RES_I32),
+                               (-1, 8, _lib.RES_I32), (2 ** 31 - 1, 8, _lib.RES_I32)):
+        assert L.tcbnn_residual_format_narrowest(bound, batch) == want, (bound, batch)
+    assert L.tcbnn_residual_format_for_bound(2047) == _lib.RES_I16  # (never 12 bits: it does not know the batch)
+    assert L.tcbnn_conv_residual_bound(64, 3, 3, 155) == 155 + 576
+    assert L.tcbnn_conv_residual_bound(64, 3, 3, 0) == 576
+
+
+def test_first_layer_bound_of_input_is_the_largest_window_sum():
+    """tcbnn_inconv_residual_bound_of_input against a brute-force window walk in numpy: no first-layer sum can
+    exceed the largest sum of |x| over one filter window (all three channels), and the returned bound lies between
+    that sum and that sum * 1.001 + 2."""
+    import ctypes as C
+
+    import numpy as np
+    from tcbnn_amd import _lib
+    L = _lib.lib
+    rng = np.random.default_rng(11)
+    for (b, h, w, r, s, sh, sw, padding) in ((2, 9, 11, 3, 3, 1, 1, 1), (3, 16, 13, 7, 7, 4, 4, 1), (1, 12, 12, 5, 3, 2, 1, 0),
+                                             (2, 23, 19, 11, 11, 4, 4, 1), (1, 7, 7, 7, 7, 1, 1, 1)):
+        x = (rng.standard_normal((b, 3, h, w)) * rng.uniform(0.1, 30)).astype(np.float32)
+        pad_h, pad_w = L.tcbnn_conv_pad(h, r, sh, padding), L.tcbnn_conv_pad(w, s, sw, padding)
+        oh, ow = L.tcbnn_conv_out(h, r, sh, padding, 1), L.tcbnn_conv_out(w, s, sw, padding, 1)
+        a = np.abs(x.astype(np.float64)).sum(axis=1)
+        worst = 0.0
+        for y in range(oh):
+            for xx in range(ow):
+                y0, x0 = y * sh - pad_h, xx * sw - pad_w
+                win = a[:, max(0, y0):min(h, y0 + r), max(0, x0):min(w, x0 + s)]
+                worst = max(worst, float(win.sum(axis=(1, 2)).max()))
+        got = L.tcbnn_inconv_residual_bound_of_input(x.ctypes.data_as(C.c_void_p), b, h, w, r, s, sh, sw, padding)
+        assert worst <= got <= worst * 1.001 + 2, (got, worst)
+        # and it is a bound: the largest |sum| any +-1 filter can reach is that window's sum of |x|
+        assert got >= np.floor(worst)
+    bad = np.ones((1, 3, 8, 8), np.float32)
+    bad[0, 1, 3, 3] = np.nan
+    assert L.tcbnn_inconv_residual_bound_of_input(bad.ctypes.data_as(C.c_void_p), 1, 8, 8, 3, 3, 1, 1, 1) == 2 ** 31 - 1
+    assert L.tcbnn_inconv_residual_bound_of_input(None, 1, 8, 8, 3, 3, 1, 1, 1) == 2 ** 31 - 1
