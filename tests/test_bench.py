@@ -40,3 +40,10 @@ def test_one_json_line_with_the_contract_keys(gpu):
     for key in ("value", "unit", "cores", "kind", "sample"):
         assert key in c, key
     assert c["kind"] in ("port", "reference") and c["cores"] >= 1
+    # the untimed clock-settling passes are reported, and the several-batches-in-flight figure stays out of `value`
+    assert d["preheat"]["steps"] >= 8 and d["preheat"]["ms"] > 0
+    f = d["batches_in_flight"]
+    assert f["batches_in_flight"] == 2 and f["unit"] == "images/s" and f["steps"] >= 100
+    assert abs(f["value"] - 256 / (f["ms_per_step"] * 1e-3)) <= 0.01 * f["value"]
+    assert r["traffic"] is None or r["traffic"] > 0
+    assert r["traffic_stale"] == (r["traffic"] is None)
