@@ -146,7 +146,9 @@ def test_bconv_sweep_shapes_batch256(gpu, h, c):
                                                    # 3x3 shapes of the persistent kernel's int32 epilogue: partial
                                                    # channel tile, partial image tile, stride 2, one-pixel frame
                                                    (70, 9, 64, 48, 3, 2), (33, 7, 192, 100, 3, 1), (8, 1, 128, 64, 3, 1),
-                                                   (40, 2, 384, 32, 3, 1), (9, 6, 64, 33, 3, 1)])
+                                                   (40, 2, 384, 32, 3, 1), (9, 6, 64, 33, 3, 1),
+                                                   # whole channel tiles at Cin = 192 / 256 (one channel tile per wave through LDS)
+                                                   (64, 4, 192, 64, 3, 1), (48, 3, 256, 96, 3, 1)])
 def test_bconv_odd_shapes(gpu, variant, b, h, cin, cout, R, stride):
     r = rng(b + h + cin)
     x = rm.pm1(r, (b, h, h, cin))
