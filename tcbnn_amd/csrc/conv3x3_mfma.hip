@@ -40,12 +40,10 @@ using namespace mfma;
 // Cache policy of the residual loads: non-temporal (the operand is read exactly once; measured 2 % on the
 // ResNet-18 step, while non-temporal stores cost time: the next layer finds less of its input in the caches).
 constexpr int kResLoadAux = 2;
-constexpr int kWaves = 4;
-// Residual layers run two image tiles per wave from this Cin / 64 on (Cin = 512: the layer is bound by
-// issue slots, not by HBM; measured slower for Cin = 256 and for pooled sources).
-constexpr int kResMt2From = 8;
-constexpr int kThreads = 64 * kWaves;
-
+// Waves per workgroup: four, sharing the staged weights of their channel group; eight where the FP4 fragments of
+// two channel tiles (18 KB per tile and 64 input channels) leave room for only one workgroup in a CU's 160 KB of
+// LDS: the CU then still runs two waves per SIMD, and each expanded activation fragment still feeds two MFMAs.
+constexpr int waves_of(int spt, int nt) { return 9 * spt * nt * 1024 > 80 * 1024 ? 8 : 4; }
 // Residual mode of an instantiation.
 constexpr int RM_NONE = 0;    // threshold only
 constexpr int RM_PLAIN = 1;   // residual injected from a source of the same size and / or saved
@@ -58,7 +56,7 @@ constexpr int RM_RAW = 3;     // no threshold: the +-1 dot products are stored a
 // bank conflicts.)
 constexpr int raw_pitch(int nt) { return 32 * nt + 4; }
 constexpr bool raw_transposed(int spt, int rm, int nt, bool fullt) {
-    return rm == RM_RAW && fullt && 9 * spt * nt * 1024 + kWaves * 32 * raw_pitch(nt) * 4 <= 80 * 1024;
+    return rm == RM_RAW && fullt && 9 * spt * nt * 1024 + 4 * 32 * raw_pitch(nt) * 4 <= 80 * 1024;
 }
 
 // Waves per SIMD the register allocator is asked to make room for (256 registers per lane: the plain layers
@@ -74,7 +72,7 @@ constexpr int kWavesPerSimd = 2;
 // tests of partial tiles are then not even compiled (they cost scalar registers and set-up instructions in
 // every launch, and the networks' channel counts are multiples of 64).
 template <int SPT, int RM, int MT, int NT, int RF, bool POOL, bool FULLT>
-__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(kWavesPerSimd))) void
+__global__ __launch_bounds__(64 * waves_of(SPT, NT)) __attribute__((amdgpu_waves_per_eu(kWavesPerSimd))) void
 conv3x3_mfma_f4_kernel(
     const BgemmParams p, const uint32_t* __restrict__ act, const uint32_t* __restrict__ wgt,
     const float* __restrict__ bnp, const int32_t* __restrict__ rin, int32_t* __restrict__ rout, int res_lim,
@@ -85,6 +83,7 @@ conv3x3_mfma_f4_kernel(
     constexpr int TPC = SPT >= 3 ? 3 : 9;  // taps per prefetch chunk (a filter row, or all of it)
     constexpr int NCH = 9 / TPC;           // chunks per tile
     constexpr int NQ = 9 * SPT;            // k-steps per tile
+    constexpr int kWaves = waves_of(SPT, NT);
     // A tile of one chunk is shorter than the memory latency: its residual operand is then
     // requested a whole tile ahead (double-buffered); otherwise with the tile's first chunk.
     constexpr bool kAhead = kRes && NCH == 1;
@@ -1000,6 +999,7 @@ TensorBytes tensor_bytes(const BgemmParams& p) {
 template <int SPT, int RM, int MT, int NT, int RF, bool POOL, bool FULLT>
 int launch_f(const BgemmParams& p, hipStream_t stream) {
     constexpr int NQ = 9 * SPT;
+    constexpr int kWaves = waves_of(SPT, NT), kThreads = 64 * kWaves;
     constexpr bool kRawTranspose = raw_transposed(SPT, RM, NT, FULLT);
     const size_t lds_bytes = (size_t)NQ * NT * 64 * 16 + NT * 32 * sizeof(float) +
                              (kRawTranspose ? (size_t)kWaves * 32 * raw_pitch(NT) * sizeof(int) : 0);
@@ -1024,7 +1024,7 @@ int launch_f(const BgemmParams& p, hipStream_t stream) {
     }
     const int n_groups = (p.N + 32 * NT - 1) / (32 * NT);
     const int b_groups = (p.B + 32 * MT - 1) / (32 * MT);
-    const int quads = ((POOL ? p.OH * p.OW : p.PH * p.PW) + kWaves - 1) / kWaves;  // items of the four waves
+    const int quads = ((POOL ? p.OH * p.OW : p.PH * p.PW) + kWaves - 1) / kWaves;  // items per wave of a pixel stream
     // Persistent workgroups, all resident at once: two per CU (three for residual layers), fewer
     // when registers or LDS hold fewer.  Measured on every layer of ResNet-18 at batch 256: more, shorter-lived
     // workgroups stage the weights more often and lose; and a grid even slightly larger than the resident slots
@@ -1067,21 +1067,22 @@ int launch_t(const BgemmParams& p, hipStream_t stream) {
     return launch_f<SPT, RM, MT, NT, RF, POOL, false>(p, stream);
 }
 
-// Which instantiation serves a layer.  Measured on ResNet-18 at batch 256: two channel tiles per wave (each
-// expanded activation fragment feeds two MFMAs) wherever the weights of 64 channels leave room for a second
-// workgroup in a CU's LDS (up to Cin = 256; one workgroup of eight waves with two channel tiles was 20-45 %
-// slower on the Cin = 512 layers: one long tile per wave, nothing to overlap it with); layers that inject the
-// 2 x 2 maximum of a larger tensor run best with one (four times the residual operands per tile: more
-// workgroups keep more requests in flight).
+// Which instantiation serves a layer.  Measured on ResNet-18 and VGG-16 at batch 256: two channel tiles per wave
+// (each expanded activation fragment feeds two MFMAs) everywhere except on layers that inject the 2 x 2 maximum of a
+// larger tensor (four times the residual operands per tile: more, smaller workgroups keep more requests in flight)
+// and on the int32-output kernel from Cin = 192 on (its LDS staging area); from Cin = 384 on the weights of two
+// channel tiles leave room for one workgroup per CU only, which then has eight waves (waves_of).  Two image tiles
+// per wave (each weight fragment read from LDS feeds two MFMAs) on the plain and int32-output layers up to
+// Cin = 256; one on residual layers (their operands fill the registers) and from Cin = 384 on (the activation ring
+// of two image tiles no longer fits next to two channel tiles' accumulators).
 struct Pick {
     int rm, mt, nt, r16, pool;  // r16: TCBNN_RES_* format of the injected residual
 };
 constexpr int pick_nt(int spt, int rm) {
-    return rm == RM_POOLED ? 1 : (rm == RM_RAW ? (spt >= 3 ? 1 : 2) : (spt >= 6 ? 1 : 2));
+    return rm == RM_POOLED ? 1 : (rm == RM_RAW ? (spt >= 3 && spt < 8 ? 1 : 2) : 2);
 }
-// image tiles per wave: two wherever the layer is bound by issue slots rather than by HBM
 constexpr int pick_mt(int spt, int rm) {
-    return rm == RM_NONE || rm == RM_RAW ? 2 : (rm == RM_PLAIN && spt >= kResMt2From ? 2 : 1);
+    return rm == RM_RAW ? (spt >= 8 ? 1 : 2) : (rm == RM_NONE ? (spt >= 6 ? 1 : 2) : 1);
 }
 Pick pick(const BgemmParams& p) {
     const int rm = p.mode == EPI_RAW ? RM_RAW
@@ -1097,10 +1098,10 @@ int launch_m(const BgemmParams& p, hipStream_t stream) {
     const Pick k = pick(p);
     switch (k.rm) {
         case RM_NONE:
-            return k.pool ? launch_t<SPT, RM_NONE, 2, pick_nt(SPT, RM_NONE), TCBNN_RES_I32, true>(p, stream)
-                          : launch_t<SPT, RM_NONE, 2, pick_nt(SPT, RM_NONE), TCBNN_RES_I32, false>(p, stream);
+            return k.pool ? launch_t<SPT, RM_NONE, pick_mt(SPT, RM_NONE), pick_nt(SPT, RM_NONE), TCBNN_RES_I32, true>(p, stream)
+                          : launch_t<SPT, RM_NONE, pick_mt(SPT, RM_NONE), pick_nt(SPT, RM_NONE), TCBNN_RES_I32, false>(p, stream);
         case RM_RAW:
-            return launch_t<SPT, RM_RAW, 2, pick_nt(SPT, RM_RAW), TCBNN_RES_I32, false>(p, stream);
+            return launch_t<SPT, RM_RAW, pick_mt(SPT, RM_RAW), pick_nt(SPT, RM_RAW), TCBNN_RES_I32, false>(p, stream);
         case RM_PLAIN:
             return k.r16 == TCBNN_RES_I12
                        ? launch_t<SPT, RM_PLAIN, pick_mt(SPT, RM_PLAIN), pick_nt(SPT, RM_PLAIN), TCBNN_RES_I12, false>(p, stream)
