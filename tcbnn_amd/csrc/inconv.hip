@@ -138,7 +138,7 @@ template <int NST, bool ROWS, bool POOLED>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS && NST <= 16 ? 4 : 3))) void inconv_tiled_kernel(
     const InConvParams p, const float* __restrict__ in, const uint4* __restrict__ masks,
     const float* __restrict__ bn, uint32_t* __restrict__ out, int32_t* __restrict__ res, int b_tiles,
-    int x_groups, int y_phases, int div_magic, int rpw) {
+    int x_groups, int y_phases, int div_magic, int rpw, int row_il, int rows_total) {
     __shared__ float tile[3 * kMaxCols * kLB];
 
     const int tid = threadIdx.x;
@@ -156,6 +156,16 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS &
         bt = slot % b_tiles;
         xg = (slot / b_tiles) * xg_per + j % xg_per;
         y = j / xg_per;
+        // Rows are dealt 0, k, 2k, ... then 1, k + 1, ... (k = row_il, chosen by the host): consecutive output rows
+        // share R - stride input rows, and the workgroup of row r + 1 needs a shared row stride/R of a workgroup's
+        // lifetime BEFORE the workgroup of row r does.  Dealt in natural order the two start almost together and the
+        // row has left the XCD's L2 by the time it is needed again; dealt k rows apart the later start of row r + 1
+        // makes the two requests meet (fetched bytes of ResNet-18's first layer at batch 256: 286 -> 214 MB).
+        if (row_il > 1) {
+            const int G = (rows_total + row_il - 1) / row_il;
+            y = (y % G) * row_il + y / G;
+            if (y >= rows_total) return;  // whole workgroup: grid padding
+        }
         if (xg >= x_groups) return;  // whole workgroup: grid padding
     } else {
         bt = blockIdx.x % b_tiles;
@@ -552,8 +562,22 @@ static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name
         // XCD-aware order when the image tiles divide the 8 XCD slots (see the kernel)
         static const bool plain_order = getenv("TCBNN_INCONV_ORDER") != nullptr;  // tuning switch
         const int y_phases = (!plain_order && 8 % b_tiles == 0) ? 8 / b_tiles : 0;
+        // Row interleave of the XCD-aware order (see the kernel): an XCD starts its resident workgroups (4 per CU
+        // x 32 CUs) once per workgroup lifetime, xg_per of them per output row, and the start of row r + 1 should
+        // lag that of row r by stride/R of a lifetime: k = stride/R x 128 / xg_per rows, taken at 0.7 of that (measured
+        // on the 7x7 stride-4 layer: 214-217 MB fetched for k = 7..10, 222 for 5, 241 for 14, 286 without).
+        static const int il_env = getenv("TCBNN_INCONV_ROWIL") ? atoi(getenv("TCBNN_INCONV_ROWIL")) : -1;  // tuning switch
+        int row_il = 0;
+        if (y_phases > 0 && !pooled) {
+            const int xg_per = (x_groups + y_phases - 1) / y_phases;
+            row_il = (int)(0.7 * p.stride_h * 128.0 / ((double)p.R * xg_per) + 0.5);
+            if (il_env >= 0) row_il = il_env;
+            row_il = std::min(row_il, rows_out / 2);
+            if (il_env < 0 && row_il < 4) row_il = 0;  // (little to gain where rows already start close to the right lag)
+        }
+        const int rows_grid = row_il > 1 ? (rows_out + row_il - 1) / row_il * row_il : rows_out;
         const long long blocks = y_phases > 0
-                                     ? 8LL * ((x_groups + y_phases - 1) / y_phases) * rows_out
+                                     ? 8LL * ((x_groups + y_phases - 1) / y_phases) * rows_grid
                                      : (long long)b_tiles * x_groups * rows_out;
         TCBNN_REQUIRE(blocks <= 0x7fffffffLL, "inconv128: grid too large");
         // staging scheme (see the kernel): whole segments per wave, a multiple of 3 of them when 3 fit its 64
@@ -561,7 +585,7 @@ static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name
         const int rpw = 64 / ncols >= 3 ? (64 / ncols) / 3 * 3 : 2;
         auto launch = [&](auto kernel) {
             hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(kThreads), 0, (hipStream_t)stream, p, p.in,
-                               p.masks, p.bn, p.out, p.res, b_tiles, x_groups, y_phases, div_magic, rpw);
+                               p.masks, p.bn, p.out, p.res, b_tiles, x_groups, y_phases, div_magic, rpw, row_il, rows_out);
         };
         auto launch_nst = [&](auto nst_tag, auto rows_tag) {
             constexpr int NST = decltype(nst_tag)::value;
