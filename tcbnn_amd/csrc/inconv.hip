@@ -321,8 +321,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS &
         if (work && b < p.B && wi < p.ow) {
             // The stores' addresses are worked out here, after the tap loops: formed ahead of them (the compiler hoists
             // what does not depend on the loops) they were live across the whole kernel and were spilled.
-            int b = b0 + lane;
-            asm volatile("" : "+v"(b));
+            // (the lane index comes from the hardware's lane count here, not from a register kept since the start)
+            const int b = b0 + (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
 #pragma unroll
             for (int px = 0; px < 2; ++px) {
                 if (px == 1 && !xb_ok) continue;
