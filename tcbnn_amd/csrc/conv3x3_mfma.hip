@@ -1067,19 +1067,20 @@ int launch_t(const BgemmParams& p, hipStream_t stream) {
     return launch_f<SPT, RM, MT, NT, RF, POOL, false>(p, stream);
 }
 
-// Which instantiation serves a layer.  Measured on ResNet-18 and VGG-16 at batch 256: two channel tiles per wave
-// (each expanded activation fragment feeds two MFMAs) everywhere except on layers that inject the 2 x 2 maximum of a
-// larger tensor (four times the residual operands per tile: more, smaller workgroups keep more requests in flight)
-// and on the int32-output kernel from Cin = 192 on (its LDS staging area); from Cin = 384 on the weights of two
-// channel tiles leave room for one workgroup per CU only, which then has eight waves (waves_of).  Two image tiles
-// per wave (each weight fragment read from LDS feeds two MFMAs) on the plain and int32-output layers up to
-// Cin = 256; one on residual layers (their operands fill the registers) and from Cin = 384 on (the activation ring
-// of two image tiles no longer fits next to two channel tiles' accumulators).
+// Which instantiation serves a layer.  Measured on ResNet-18 and VGG-16 at batch 256 (10 launches back to back):
+// two channel tiles per wave (each expanded activation fragment feeds two MFMAs) everywhere except on layers of
+// Cin >= 384 that inject the 2 x 2 maximum of a larger tensor (the eight-wave workgroup below was 8 % slower
+// there: four times the residual operands per tile) and on the int32-output kernel for Cin = 192..384 (its LDS
+// staging area); from Cin = 384 on the weights of two channel tiles leave room for one workgroup per CU only, which
+// then has eight waves (waves_of).  Two image tiles per wave (each weight fragment read from LDS feeds two MFMAs)
+// on the plain and int32-output layers up to Cin = 256; one on residual layers (their operands fill the registers)
+// and from Cin = 384 on (the activation ring of two image tiles no longer fits next to two channel tiles'
+// accumulators).
 struct Pick {
     int rm, mt, nt, r16, pool;  // r16: TCBNN_RES_* format of the injected residual
 };
 constexpr int pick_nt(int spt, int rm) {
-    return rm == RM_POOLED ? 1 : (rm == RM_RAW ? (spt >= 3 && spt < 8 ? 1 : 2) : 2);
+    return rm == RM_POOLED ? (spt >= 6 ? 1 : 2) : (rm == RM_RAW ? (spt >= 3 && spt < 8 ? 1 : 2) : 2);
 }
 constexpr int pick_mt(int spt, int rm) {
     return rm == RM_RAW ? (spt >= 8 ? 1 : 2) : (rm == RM_NONE ? (spt >= 6 ? 1 : 2) : 1);
@@ -1089,8 +1090,10 @@ Pick pick(const BgemmParams& p) {
                    : p.res_in == nullptr && p.res_out == nullptr
                        ? RM_NONE
                        : (p.res_in != nullptr && p.res_pool ? RM_POOLED : RM_PLAIN);
-    return {rm, pick_mt(p.cw / 2, rm), pick_nt(p.cw / 2, rm), p.res_in != nullptr ? p.res_in_fmt : TCBNN_RES_I32,
-            p.pool_h == 2};
+    const int fmt = p.res_in != nullptr ? p.res_in_fmt : TCBNN_RES_I32;
+    // (a pooled int32 source keeps one channel tile per wave: four times sixteen words per tile and lane spilled)
+    const int nt = rm == RM_POOLED && fmt == TCBNN_RES_I32 ? 1 : pick_nt(p.cw / 2, rm);
+    return {rm, pick_mt(p.cw / 2, rm), nt, fmt, p.pool_h == 2};
 }
 
 template <int SPT>
@@ -1113,7 +1116,7 @@ int launch_m(const BgemmParams& p, hipStream_t stream) {
                        ? launch_t<SPT, RM_POOLED, pick_mt(SPT, RM_POOLED), pick_nt(SPT, RM_POOLED), TCBNN_RES_I12, false>(p, stream)
                        : (k.r16 == TCBNN_RES_I16
                               ? launch_t<SPT, RM_POOLED, pick_mt(SPT, RM_POOLED), pick_nt(SPT, RM_POOLED), TCBNN_RES_I16, false>(p, stream)
-                              : launch_t<SPT, RM_POOLED, pick_mt(SPT, RM_POOLED), pick_nt(SPT, RM_POOLED), TCBNN_RES_I32, false>(p, stream));
+                              : launch_t<SPT, RM_POOLED, pick_mt(SPT, RM_POOLED), 1, TCBNN_RES_I32, false>(p, stream));
     }
 }
 
