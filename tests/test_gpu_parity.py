@@ -872,6 +872,38 @@ def test_forward_captured_in_a_hip_graph(gpu):
     net.release()
 
 
+def test_two_networks_in_flight_on_two_streams(gpu):
+    """Two copies of the network (own activations, residuals and inputs, same weights) run at the same time on two
+    streams, batches dealt alternately: the persistent kernels of one copy share the GPU with those of the
+    other.  Each copy's logits after several interleaved passes must equal its own solo result bit for bit."""
+    from tcbnn_amd import nets
+    from tcbnn_amd.device import Stream
+    spec = nets.imagenet_resnet_spec(batch=64, image=96, output_size=200)
+    weights = gpu.synthetic_weights(spec, 31)
+    xs = [gpu.synthetic_input(spec, 31), gpu.synthetic_input(spec, 32)]
+    copies = [gpu.Network(spec, weights, x) for x in xs]
+    streams = [Stream(), Stream()]
+    solo = []
+    for net, st in zip(copies, streams):
+        net.forward(st)
+        st.synchronize()
+        solo.append(net.logits().copy())
+    assert not np.array_equal(solo[0], solo[1])
+    for net in copies:
+        net.layers["Fout"].output_gpu.fill(0)
+    gpuops.sync()
+    for k in range(10):  # no synchronisation inside: the two forwards overlap on the device
+        copies[k % 2].forward(streams[k % 2])
+    for st in streams:
+        st.synchronize()
+    for net, want in zip(copies, solo):
+        np.testing.assert_array_equal(net.logits(), want)
+    want0 = orc_nets.run(spec, weights, xs[0])["Fout"]["out"]
+    np.testing.assert_allclose(solo[0], want0, rtol=1e-5, atol=0)
+    for net in copies:
+        net.release()
+
+
 def test_imagenet_resnet18_batch256_every_image(gpu):
     """Full configured size on the default engine, every one of the 256 images and every layer against the
     oracle (packed activations and residuals bit for bit, logits to 1e-5 relative), three forward passes:
