@@ -42,6 +42,8 @@ def test_one_json_line_with_the_contract_keys(gpu):
     assert c["kind"] in ("port", "reference") and c["cores"] >= 1
     # the untimed clock-settling passes are reported, and the several-batches-in-flight figure stays out of `value`
     assert d["preheat"]["steps"] >= 8 and d["preheat"]["ms"] > 0
+    a = d["as_launched"]
+    assert a["unit"] == "images/s" and abs(a["value"] - 256 / (a["ms_per_step"] * 1e-3)) <= 0.01 * a["value"]
     f = d["batches_in_flight"]
     assert f["batches_in_flight"] == 2 and f["unit"] == "images/s" and f["steps"] >= 100
     assert abs(f["value"] - 256 / (f["ms_per_step"] * 1e-3)) <= 0.01 * f["value"]
