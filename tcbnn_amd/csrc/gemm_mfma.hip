@@ -171,6 +171,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) v
     atomicAdd(&colc[snt * 32 + row_to_channel(j)], csum);
     __syncthreads();
 
+    // int32 output, all 64 columns of the group exist and every row's run of them is 16-byte aligned (uniform): the
+    // sums leave through LDS, a row at a time (below)
+    const bool raw_rows = EPI == EPI_RAW && n0 + 32 * kNT <= p.N && p.raw_b_stride % 4 == 0 &&
+                          (reinterpret_cast<uintptr_t>(p.out_i32) & 15) == 0;
+
     // ---- epilogue: the lane holds columns cbase + v of image bimg[mt]
 #pragma unroll
     for (int nt = 0; nt < kNT; ++nt) {
@@ -214,6 +219,8 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) v
                             p.out_f32[(size_t)b * p.N + cbase + v] =
                                 __fadd_rn(__fmul_rn((float)((int)acc[mt][nt][v] - off[v]), thr[v]), bia[v]);
                 }
+            } else if (raw_rows) {
+                // (int32 output of whole, aligned column groups: written further down, a row at a time)
             } else {
                 if (b_ok) {
                     int32_t* dst = p.out_i32 + (size_t)b * p.raw_b_stride + cbase;
@@ -230,6 +237,49 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(2))) v
 #pragma unroll
                         for (int v = 0; v < 16; ++v)
                             if (cbase + v < p.N) dst[v] = (int)acc[mt][nt][v] - off[v];
+                    }
+                }
+            }
+        }
+    }
+
+    // int32 output [rows][N] (BMMAS_new, tensorcore_kernel.cu:355): in the accumulator a lane holds 16 columns of ONE
+    // row, so a direct store scatters 16-byte pieces over 64 different rows per instruction (the product writes
+    // 4 M N bytes: a quarter of the 8192^3 launch was this).  The sums of a 32-row tile go through a per-wave LDS
+    // area instead (row = image, pitch 68 words: conflict-free both ways; the weight buffers are free by now) and
+    // leave as 128-bit stores in which 16 consecutive lanes cover one row's whole run of 64 columns (4 runs of
+    // 256 bytes per instruction).
+    if constexpr (EPI == EPI_RAW) {
+        if (raw_rows) {
+            constexpr int kPitch = 32 * kNT + 4;
+            // (behind the column constants, which stay where they are)
+            int* mine = reinterpret_cast<int*>(&lds_w[0][0]) + kNT * 32 + wave * (32 * kPitch);
+            const int rl = lane >> 4, cl = lane & 15;
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+#pragma unroll
+                for (int nt = 0; nt < kNT; ++nt) {
+                    int off[16];
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) off[v] = corr + colc[nt * 32 + 16 * h + v];
+#pragma unroll
+                    for (int g = 0; g < 4; ++g)
+                        *reinterpret_cast<v4i*>(mine + j * kPitch + nt * 32 + 16 * h + 4 * g) =
+                            v4i{(int)acc[mt][nt][4 * g] - off[4 * g], (int)acc[mt][nt][4 * g + 1] - off[4 * g + 1],
+                                (int)acc[mt][nt][4 * g + 2] - off[4 * g + 2], (int)acc[mt][nt][4 * g + 3] - off[4 * g + 3]};
+                }
+                // (same wave writes and reads: program order and the wait for LDS are all the synchronisation)
+                const int row0 = b0 + mt * 32;
+#pragma unroll
+                for (int part = 0; part < 2; ++part) {
+                    v4i q[4];
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) q[k] = *reinterpret_cast<const v4i*>(mine + (16 * part + 4 * k + rl) * kPitch + 4 * cl);
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const int row = row0 + 16 * part + 4 * k + rl;
+                        if (row < p.B)
+                            *reinterpret_cast<v4i*>(p.out_i32 + (size_t)row * p.raw_b_stride + n0 + 4 * cl) = q[k];
                     }
                 }
             }
