@@ -210,8 +210,10 @@ int tcbnn_out128_forward(const tcbnn_out128_desc* d, void* stream);
  * raster order; bit = !((float)acc < bn[o]); OR-pool; residual = (int)acc.
  * save_residual requires pool 1x1 (the reference index by*output_width+bx,
  * kernel.cuh:666, is only meaningful then). */
+#define TCBNN_INCONV_INPUT_NCHW 0   /* float [batch][3][H][W], the reference's device layout (kernel.cuh:620-625) */
+#define TCBNN_INCONV_INPUT_PACKED 1 /* float [Hp][Wp][batch][3], zero-padded: see tcbnn_inconv_pack_input */
 typedef struct tcbnn_inconv128_desc {
-    const float* input;        /* [batch][3][input_height][input_width] */
+    const float* input;        /* device, in the layout `input_layout` names */
     const uint32_t* filter;    /* tcbnn_pack_inconv_filter output */
     const float* bn;           /* [output_channels] */
     uint32_t* output;          /* [OH][OW][CW(output_channels)][B] */
@@ -224,8 +226,20 @@ typedef struct tcbnn_inconv128_desc {
     int pool_height, pool_width;
     int save_residual;         /* bool */
     int residual_format;       /* TCBNN_RES_* of output_residual */
+    int input_layout;          /* TCBNN_INCONV_INPUT_*; PACKED needs pool 1x1 */
 } tcbnn_inconv128_desc;
 int tcbnn_inconv128_forward(const tcbnn_inconv128_desc* d, void* stream);
+/* The engine's own layout of the first layer's input: batch innermost like every other tensor, and zero-padded, so
+ * that a lane (= image) reads the three channels of an input pixel as 12 contiguous bytes, a wavefront 768, and no
+ * tap needs a test for the frame: float [Hp][Wp][batch][3] with Hp = (P - 1) * stride_height + filter_height,
+ * Wp = (Q - 1) * stride_width + filter_width (P x Q = tcbnn_conv_out of the two dimensions, pool 1) and the frame's
+ * pixel (0, 0) at (tcbnn_conv_pad(height...), tcbnn_conv_pad(width...)).  The reference reads [batch][3][H][W]
+ * directly (kernel.cuh:620-625) and has no such step; here it belongs to the upload of an input
+ * (InConv128LayerParam::initialize / set_input), not to the forward pass.  Both pointers are device pointers. */
+size_t tcbnn_inconv_packed_input_floats(int batch, int height, int width, int filter_height, int filter_width,
+                                        int stride_height, int stride_width, int padding);
+int tcbnn_inconv_pack_input(const float* input, float* packed, int batch, int height, int width, int filter_height,
+                            int filter_width, int stride_height, int stride_width, int padding, void* stream);
 
 /* Conv128LayerFMT (kernel.cuh:676-827), fields of Conv128LayerParam (param.h:1028-1064).
  *   res = Cin*R*S - exclude*Cin - 2*popc                      (kernel.cuh:766-768)

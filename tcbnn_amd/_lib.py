@@ -51,7 +51,8 @@ class InConv128Desc(C.Structure):
                 ("input_channels", c_int), ("filter_height", c_int), ("filter_width", c_int),
                 ("output_channels", c_int), ("batch", c_int), ("stride_height", c_int),
                 ("stride_width", c_int), ("padding", c_int), ("pool_height", c_int),
-                ("pool_width", c_int), ("save_residual", c_int), ("residual_format", c_int)]
+                ("pool_width", c_int), ("save_residual", c_int), ("residual_format", c_int),
+                ("input_layout", c_int)]
 
 
 class Conv128Desc(C.Structure):
@@ -113,6 +114,8 @@ ABI = {
     "tcbnn_fc128_forward_static_scratch": (c_int, [C.POINTER(Fc128Desc), c_void_p]),
     "tcbnn_out128_forward": (c_int, [C.POINTER(Out128Desc), c_void_p]),
     "tcbnn_inconv128_forward": (c_int, [C.POINTER(InConv128Desc), c_void_p]),
+    "tcbnn_inconv_packed_input_floats": (c_size_t, [c_int] * 8),
+    "tcbnn_inconv_pack_input": (c_int, [c_void_p, c_void_p] + [c_int] * 8 + [c_void_p]),
     "tcbnn_conv128_forward": (c_int, [C.POINTER(Conv128Desc), c_void_p]),
     "tcbnn_conv128_kernel_name": (c_int, [C.POINTER(Conv128Desc), C.c_char_p, c_size_t]),
     "tcbnn_fc128_kernel_name": (c_int, [C.POINTER(Fc128Desc), C.c_char_p, c_size_t]),
@@ -138,6 +141,7 @@ for _name, (_res, _args) in ABI.items():
 VARIANT_AUTO, VARIANT_POPC, VARIANT_MFMA_I8, VARIANT_MFMA_F4 = 0, 1, 2, 3
 VARIANTS = {"auto": 0, "popc": 1, "mfma_i8": 2, "mfma_f4": 3}
 RES_I32, RES_I16, RES_I12 = 0, 1, 2
+INCONV_INPUT_NCHW, INCONV_INPUT_PACKED = 0, 1
 INT32_MAX = 2 ** 31 - 1
 
 

@@ -17,6 +17,7 @@
 //     wave-uniform scalar loads, and the packed words / int32 residuals are written as
 //     contiguous 256-byte runs of the batch-innermost output layouts.
 //   inconv_generic_kernel (any pooling): one lane per pooled output pixel.
+#include <algorithm>
 #include <stdlib.h>
 #include <string.h>
 
@@ -410,6 +411,203 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS &
     }
 }
 
+// First layer on an input that is already batch-innermost and zero-padded: float [Hp][Wp][B][3] with
+// Hp = (PH - 1) stride_h + R, Wp = (PW - 1) stride_w + S and the frame at (pad_h, pad_w) (tcbnn_inconv_pack_input
+// writes it).  A lane's three channels of one input pixel are 12 contiguous bytes and a wave's 64 images 768, so a
+// tap is ONE 96-bit buffer load per pixel, straight into registers: no staging through LDS, no barrier, no
+// transposition, and no test for the frame (the border holds zeros, which add +-0 like the reference's skipped tap).
+// Waves are independent; the four of a workgroup (two pixel pairs x two channel halves) only share cache lines.
+// Same arithmetic, same order, same sign-combination and register-index scheme as inconv_tiled_kernel.
+constexpr int kDirectAhead = 3;  // taps requested ahead of their use
+__global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) void inconv_direct_kernel(
+    const InConvParams p, const float* __restrict__ in, const uint4* __restrict__ masks,
+    const float* __restrict__ bn, uint32_t* __restrict__ out, int32_t* __restrict__ res, int b_tiles,
+    int x_groups, int y_phases, int row_il, int Wp, unsigned in_bytes) {
+    const int rows_total = p.PH;
+    typedef float v3f __attribute__((ext_vector_type(3)));
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    int bt, xg, y;
+    if (y_phases > 0) {  // XCD-aware order with row interleave, as in inconv_tiled_kernel
+        const int slot = blockIdx.x & 7, j = blockIdx.x >> 3;
+        const int xg_per = (x_groups + y_phases - 1) / y_phases;
+        bt = slot % b_tiles;
+        xg = (slot / b_tiles) * xg_per + j % xg_per;
+        y = j / xg_per;
+        if (row_il > 1) {
+            const int G = (rows_total + row_il - 1) / row_il;
+            y = (y % G) * row_il + y / G;
+            if (y >= rows_total) return;
+        }
+        if (xg >= x_groups) return;
+    } else {
+        bt = blockIdx.x % b_tiles;
+        xg = (blockIdx.x / b_tiles) % x_groups;
+        y = blockIdx.x / (b_tiles * x_groups);
+    }
+    const int pp = wave & 1, chh = wave >> 1;
+    const int xa = xg * kXT + 2 * pp;
+    const bool xa_ok = xa < p.PW, xb_ok = xa + 1 < p.PW;  // uniform
+    if (!xa_ok) return;  // (no barrier in this kernel)
+    const int b0 = bt * 64;
+    const int b = b0 + lane;
+    const int n_groups = (p.O + 63) / 64;
+    const uint32_t* __restrict__ pats =
+        reinterpret_cast<const uint32_t*>(masks) + (size_t)p.R * p.S * p.opad * 4;
+    constexpr unsigned kOutOfRange = 0x80000000u;
+    __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(in), 0, (int)in_bytes, 0x00020000);
+    const unsigned voff = b < p.B ? (unsigned)b * 12u : kOutOfRange;
+    const unsigned col_b = (unsigned)p.B * 12u;               // bytes per padded input column
+    const unsigned row_b = (unsigned)Wp * col_b;              // ... per padded input row
+    // from the wave's first pixel to its second (an odd width's last wave has none: it reads its first pixel twice)
+    const unsigned pix_b = xb_ok ? (unsigned)p.stride_w * col_b : 0u;
+    const int taps = p.R * p.S;
+
+    for (int g = 0; g < n_groups; ++g) {
+        const int wi = g * 2 + chh;
+        if (wi * 32 >= p.opad) continue;  // uniform
+        float acca[32], accb[32];
+#pragma unroll
+        for (int n = 0; n < 32; ++n) acca[n] = accb[n] = 0.0f;
+        // cursor of the requests: tap (rr, rs) at byte offset roff
+        const unsigned base = (unsigned)(y * p.stride_h) * row_b + (unsigned)(xa * p.stride_w) * col_b;
+        unsigned roff = base;
+        int rs = 0, rt = 0;
+        v3f qa[kDirectAhead], qb[kDirectAhead];
+        // (the cursor stops on the last tap: the requests issued past it ask for that tap again and are not used, so
+        // nothing outside the packed input is ever addressed)
+        auto request = [&](int slot) {
+            qa[slot] = __builtin_bit_cast(v3f, __builtin_amdgcn_raw_buffer_load_b96(rsrc, (int)voff, (int)roff, 0));
+            qb[slot] = __builtin_bit_cast(v3f, __builtin_amdgcn_raw_buffer_load_b96(rsrc, (int)voff, (int)(roff + pix_b), 0));
+            if (++rt < taps) {
+                roff += col_b;
+                if (++rs == p.S) {
+                    rs = 0;
+                    roff += row_b - (unsigned)p.S * col_b;
+                }
+            }
+        };
+#pragma unroll
+        for (int d = 0; d < kDirectAhead; ++d) request(d);
+        for (int t0 = 0; t0 < taps; t0 += kDirectAhead) {
+#pragma unroll
+            for (int d = 0; d < kDirectAhead; ++d) {
+                const int t = t0 + d;
+                if (t < taps) {  // uniform
+                    const u16v* pw = reinterpret_cast<const u16v*>(pats + (size_t)t * p.opad + wi * 32);
+                    const u16v i0 = pw[0], i1 = pw[1];
+                    const v8f ca = sign_combos(qa[d][0], qa[d][1], qa[d][2]);
+                    const v8f cb = sign_combos(qb[d][0], qb[d][1], qb[d][2]);
+                    request(d);
+                    add_indexed8x2(&acca[0], &accb[0], ca, cb, i0[0], i0[1], i0[2], i0[3], i0[4], i0[5], i0[6], i0[7]);
+                    add_indexed8x2(&acca[8], &accb[8], ca, cb, i0[8], i0[9], i0[10], i0[11], i0[12], i0[13], i0[14], i0[15]);
+                    add_indexed8x2(&acca[16], &accb[16], ca, cb, i1[0], i1[1], i1[2], i1[3], i1[4], i1[5], i1[6], i1[7]);
+                    add_indexed8x2(&acca[24], &accb[24], ca, cb, i1[8], i1[9], i1[10], i1[11], i1[12], i1[13], i1[14], i1[15]);
+                }
+            }
+        }
+        if (b < p.B && wi < p.ow) {
+#pragma unroll
+            for (int px = 0; px < 2; ++px) {
+                if (px == 1 && !xb_ok) continue;
+                const float* acc = px == 0 ? acca : accb;
+                const size_t pix = (size_t)y * p.PW + xa + px;
+                uint32_t word = 0;
+                if (wi * 32 + 32 <= p.O) {  // uniform: full channel tile
+#pragma unroll
+                    for (int n = 0; n < 32; ++n) {
+                        const float t = bn[wi * 32 + n];
+                        word = __builtin_amdgcn_alignbit(word, __float_as_uint(acc[n] - (t != t ? -__builtin_huge_valf() : t)), 31);
+                    }
+                    word = ~word;
+                } else {
+#pragma unroll
+                    for (int n = 0; n < 32; ++n) {
+                        const int ch = wi * 32 + n;
+                        if (ch < p.O) word |= (acc[n] < bn[ch] ? 0u : 1u) << (31 - n);
+                    }
+                }
+                out[(pix * p.ow + wi) * p.B + b] = word;
+                if (res != nullptr) {
+                    int r32[32];
+#pragma unroll
+                    for (int n = 0; n < 32; ++n) r32[n] = wi * 32 + n < p.O ? (int)acc[n] : 0;
+                    v4i_t* __restrict__ dst = reinterpret_cast<v4i_t*>(res);
+                    if (p.res_fmt == TCBNN_RES_I12) {
+                        typedef int v2i_t __attribute__((ext_vector_type(2)));
+                        uint32_t* __restrict__ w = reinterpret_cast<uint32_t*>(res);
+                        const size_t G = (size_t)((p.O + 15) / 16);
+#pragma unroll
+                        for (int gg = 0; gg < 2; ++gg)
+                            if (wi * 32 + 16 * gg < p.O) {
+                                uint32_t d[6];
+                                i12_pack8(&r32[16 * gg], d[0], d[1], d[2]);
+                                i12_pack8(&r32[16 * gg + 8], d[3], d[4], d[5]);
+                                __builtin_nontemporal_store(v4i_t{(int)d[0], (int)d[1], (int)d[2], (int)d[3]},
+                                                            reinterpret_cast<v4i_t*>(w + i12_word_index(pix, G, wi * 2 + gg, p.B, b, 0)));
+                                __builtin_nontemporal_store(v2i_t{(int)d[4], (int)d[5]},
+                                                            reinterpret_cast<v2i_t*>(w + i12_word_index(pix, G, wi * 2 + gg, p.B, b, 4)));
+                            }
+                    } else if (p.res_fmt == TCBNN_RES_I16) {
+                        const size_t g0 = (pix * ((p.O + 7) / 8) + wi * 4) * p.B + b;
+#pragma unroll
+                        for (int gg = 0; gg < 4; ++gg)
+                            if (wi * 32 + 8 * gg < p.O)
+                                __builtin_nontemporal_store(
+                                    v4i_t{(r32[8 * gg] & 0xffff) | (r32[8 * gg + 1] << 16),
+                                          (r32[8 * gg + 2] & 0xffff) | (r32[8 * gg + 3] << 16),
+                                          (r32[8 * gg + 4] & 0xffff) | (r32[8 * gg + 5] << 16),
+                                          (r32[8 * gg + 6] & 0xffff) | (r32[8 * gg + 7] << 16)},
+                                    dst + g0 + (size_t)gg * p.B);
+                    } else {
+                        const size_t g0 = (pix * ((p.O + 3) / 4) + wi * 8) * p.B + b;
+#pragma unroll
+                        for (int gg = 0; gg < 8; ++gg)
+                            if (wi * 32 + 4 * gg < p.O)
+                                __builtin_nontemporal_store(
+                                    v4i_t{r32[4 * gg], r32[4 * gg + 1], r32[4 * gg + 2], r32[4 * gg + 3]},
+                                    dst + g0 + (size_t)gg * p.B);
+                    }
+                }
+            }
+        }
+    }
+}
+
+// fp32 [B][3][H][W] -> zero-padded, batch-innermost [Hp][Wp][B][3] (the frame at (pad_h, pad_w)).  One workgroup
+// per (padded row, 64 images, 64 columns): the strip's 3 x 64 segments are read along the image row (lanes = columns) and
+// written with lanes = (image, channel), through LDS.
+__global__ __launch_bounds__(256) void inconv_pack_input_kernel(const float* __restrict__ in, float* __restrict__ out,
+                                                                int B, int H, int W, int Hp, int Wp, int pad_h,
+                                                                int pad_w) {
+    __shared__ float tile[64 * 3][65];  // [image * 3 + channel][column of a 64-column strip]
+    const int yp = blockIdx.x, b0 = blockIdx.y * 64;
+    const int y = yp - pad_h;
+    const size_t plane = (size_t)H * W;
+    {
+        const int x0 = blockIdx.z * 64;
+        const int cols = min(64, Wp - x0);
+        const int c = threadIdx.x & 63, x = x0 + c - pad_w;  // lanes run along the row
+        const bool in_frame = c < cols && y >= 0 && y < H && x >= 0 && x < W;
+        for (int s0 = threadIdx.x >> 6; s0 < 192; s0 += 4 * 12) {  // 12 segments (= image * 3 + channel) in flight
+            float v[12];
+#pragma unroll
+            for (int k = 0; k < 12; ++k) {
+                const int seg = s0 + 4 * k, b = b0 + seg / 3;
+                v[k] = in_frame && b < B ? in[((size_t)b * 3 + seg % 3) * plane + (size_t)y * W + x] : 0.0f;
+            }
+#pragma unroll
+            for (int k = 0; k < 12; ++k) tile[s0 + 4 * k][c] = v[k];
+        }
+        __syncthreads();
+        for (int e = threadIdx.x; e < cols * 192; e += 256) {
+            const int c = e / 192, seg = e % 192;  // lanes run along (image, channel)
+            if (b0 + seg / 3 < B) out[((size_t)yp * Wp + x0 + c) * B * 3 + (size_t)b0 * 3 + seg] = tile[seg][c];
+        }
+    }
+}
+
 __global__ __launch_bounds__(kThreads) void inconv_generic_kernel(const InConvParams p) {
     const long long m = (long long)blockIdx.x * kThreads + threadIdx.x;
     const long long total = (long long)p.B * p.OH * p.OW;
@@ -533,6 +731,39 @@ static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name
     static const bool force_linear = getenv("TCBNN_INCONV_STAGING") != nullptr &&
                                      strcmp(getenv("TCBNN_INCONV_STAGING"), "linear") == 0;
     const bool row_staging = !force_linear && 64LL * 3 * p.H * p.W * 4 < (1LL << 31);
+    if (d->input_layout == TCBNN_INCONV_INPUT_PACKED) {
+        // zero-padded, batch-innermost input (tcbnn_inconv_pack_input): the direct kernel, un-pooled layers only
+        TCBNN_REQUIRE(!pooled, "inconv128: a packed input is for un-pooled first layers (pool 1x1)");
+        const long long Hp = (long long)(p.PH - 1) * p.stride_h + p.R, Wp = (long long)(p.PW - 1) * p.stride_w + p.S;
+        const long long in_bytes = Hp * Wp * p.B * 12;
+        TCBNN_REQUIRE(in_bytes < (1LL << 31), "inconv128: packed input of 2 GiB or more");
+        if (name_buf != nullptr) {
+            snprintf(name_buf, name_len, "inconv_direct_kernel");
+            return TCBNN_OK;
+        }
+        const int b_tiles = (p.B + 63) / 64;
+        const int x_groups = (p.PW + kXT - 1) / kXT;
+        static const bool plain_order = getenv("TCBNN_INCONV_ORDER") != nullptr;  // tuning switch
+        const int y_phases = (!plain_order && 8 % b_tiles == 0) ? 8 / b_tiles : 0;
+        static const int il_env = getenv("TCBNN_INCONV_ROWIL") ? atoi(getenv("TCBNN_INCONV_ROWIL")) : -1;  // tuning switch
+        int row_il = 0;  // row interleave, as for the staged kernel below
+        if (y_phases > 0) {
+            const int xg_per = (x_groups + y_phases - 1) / y_phases;
+            row_il = (int)(0.7 * p.stride_h * 128.0 / ((double)p.R * xg_per) + 0.5);
+            if (il_env >= 0) row_il = il_env;
+            row_il = std::min(row_il, p.PH / 2);
+            if (il_env < 0 && row_il < 4) row_il = 0;
+        }
+        const int rows_grid = row_il > 1 ? (p.PH + row_il - 1) / row_il * row_il : p.PH;
+        const long long blocks = y_phases > 0 ? 8LL * ((x_groups + y_phases - 1) / y_phases) * rows_grid
+                                              : (long long)b_tiles * x_groups * p.PH;
+        TCBNN_REQUIRE(blocks <= 0x7fffffffLL, "inconv128: grid too large");
+        hipLaunchKernelGGL(inconv_direct_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, (hipStream_t)stream, p, p.in,
+                           p.masks, p.bn, p.out, p.res, b_tiles, x_groups, y_phases, row_il, (int)Wp, (unsigned)in_bytes);
+        TCBNN_LAUNCH_CHECK("inconv_direct_kernel");
+        return TCBNN_OK;
+    }
+    TCBNN_REQUIRE(d->input_layout == TCBNN_INCONV_INPUT_NCHW, "inconv128: unknown input_layout");
     if (name_buf != nullptr) {  // report the kernel instead of launching it
         if (!tiled) {
             snprintf(name_buf, name_len, "inconv_generic_kernel");
@@ -621,6 +852,39 @@ static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name
     hipLaunchKernelGGL(inconv_generic_kernel, dim3((unsigned)blocks), dim3(kThreads), 0,
                        (hipStream_t)stream, p);
     TCBNN_LAUNCH_CHECK("inconv_generic_kernel");
+    return TCBNN_OK;
+}
+
+extern "C" size_t tcbnn_inconv_packed_input_floats(int batch, int height, int width, int filter_height,
+                                                   int filter_width, int stride_height, int stride_width, int padding) {
+    if (batch <= 0 || height <= 0 || width <= 0 || filter_height <= 0 || filter_width <= 0 || stride_height <= 0 ||
+        stride_width <= 0)
+        return 0;
+    const long long ph = tcbnn_conv_out(height, filter_height, stride_height, padding, 1);
+    const long long pw = tcbnn_conv_out(width, filter_width, stride_width, padding, 1);
+    if (ph <= 0 || pw <= 0) return 0;
+    return (size_t)(((ph - 1) * stride_height + filter_height) * ((pw - 1) * stride_width + filter_width)) *
+           (size_t)batch * 3;
+}
+
+extern "C" int tcbnn_inconv_pack_input(const float* input, float* packed, int batch, int height, int width,
+                                       int filter_height, int filter_width, int stride_height, int stride_width,
+                                       int padding, void* stream) {
+    TCBNN_NOTNULL(input);
+    TCBNN_NOTNULL(packed);
+    TCBNN_REQUIRE(tcbnn_inconv_packed_input_floats(batch, height, width, filter_height, filter_width, stride_height,
+                                                   stride_width, padding) > 0,
+                  "inconv_pack_input: bad shape");
+    const int ph = tcbnn_conv_out(height, filter_height, stride_height, padding, 1);
+    const int pw = tcbnn_conv_out(width, filter_width, stride_width, padding, 1);
+    const int Hp = (ph - 1) * stride_height + filter_height, Wp = (pw - 1) * stride_width + filter_width;
+    const int pad_h = tcbnn_conv_pad(height, filter_height, stride_height, padding);
+    const int pad_w = tcbnn_conv_pad(width, filter_width, stride_width, padding);
+    const int b_tiles = (batch + 63) / 64;
+    TCBNN_REQUIRE(b_tiles <= 65535 && (Wp + 63) / 64 <= 65535, "inconv_pack_input: batch or width too large");
+    hipLaunchKernelGGL(inconv_pack_input_kernel, dim3((unsigned)Hp, (unsigned)b_tiles, (unsigned)((Wp + 63) / 64)), dim3(256), 0,
+                       (hipStream_t)stream, input, packed, batch, height, width, Hp, Wp, pad_h, pad_w);
+    TCBNN_LAUNCH_CHECK("inconv_pack_input_kernel");
     return TCBNN_OK;
 }
 

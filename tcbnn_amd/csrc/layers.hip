@@ -117,7 +117,7 @@ using namespace tcbnn;
 
 extern "C" {
 
-int tcbnn_abi_version(void) { return 4; }
+int tcbnn_abi_version(void) { return 5; }
 const char* tcbnn_last_error(void) { return g_err; }
 
 int tcbnn_set_default_variant(int variant) {

@@ -120,6 +120,7 @@ int main(int argc, char** argv) {
         const float* cursor = syn.values.data();
         tcbnn_host::ConfigSource cfg(&cursor, syn.values.data() + syn.values.size());
         InConv128LayerParam stem("Conv1", image, image, 3, 3, 3, ch, batch, 1, 1, true, 1, 1, true);
+        stem.use_packed_input();  // (set_input() must also renew the packed copy; `fresh` below reads the plain one)
         stem.initialize(images.data(), cfg);
         std::vector<float> half(images);
         for (float& v : half) v *= 0.5f;

@@ -473,6 +473,27 @@ class InConv128LayerParam {  // param.h:701-870
     }
     int input_size() { return input_channels * input_height * input_width * batch; }
     int input_bytes() { return input_size() * sizeof(float); }
+    // On request (before initialize), the un-pooled first layer reads a zero-padded, batch-innermost copy of the
+    // input (tcbnn_inconv_pack_input) with a kernel that needs no staging; initialize / set_input then make that
+    // copy after the upload: one more pass over the input there, a shorter forward pass.  Without the request,
+    // and for pooled layers, the layer reads input_gpu ([batch][3][H][W], kernel.cuh:620-625) itself.
+    InConv128LayerParam* use_packed_input(bool on = true) {
+        packed_input = on;
+        return this;
+    }
+    size_t input_packed_bytes() {
+        if (!packed_input || pool_height != 1 || pool_width != 1) return 0;
+        const size_t n = tcbnn_inconv_packed_input_floats(batch, input_height, input_width, filter_height,
+                                                          filter_width, stride_height, stride_width, padding ? 1 : 0);
+        return n > 0 && n * sizeof(float) < ((size_t)1 << 31) ? n * sizeof(float) : 0;
+    }
+    void pack_input() {  // input_gpu -> input_packed_gpu
+        if (input_packed_gpu == NULL) return;
+        TCBNN_SAFE_CALL(tcbnn_inconv_pack_input(input_gpu, input_packed_gpu, batch, input_height, input_width,
+                                                filter_height, filter_width, stride_height, stride_width,
+                                                padding ? 1 : 0, 0));
+        HIP_SAFE_CALL(hipDeviceSynchronize());
+    }
     int filter_size() { return output_channels * input_channels * filter_height * filter_width; }
     int filter_bytes() { return filter_size() * sizeof(float); }
     int output_size() { return output_channels * output_height * output_width * batch; }
@@ -494,6 +515,10 @@ class InConv128LayerParam {  // param.h:701-870
         residual_info = tcbnn_host::make_residual_info(output_channels, residual_bound_of(input), batch);
         SAFE_ALOC_GPU(input_gpu, input_bytes());
         HIP_SAFE_CALL(hipMemcpy(input_gpu, input, input_bytes(), hipMemcpyHostToDevice));
+        if (input_packed_bytes() > 0) {
+            SAFE_ALOC_GPU(input_packed_gpu, input_packed_bytes());
+            pack_input();
+        }
         SAFE_ALOC_HOST(filter, filter_bytes());
         config_file.read(this->filter, filter_size());
         SAFE_ALOC_GPU(filter_gpu,
@@ -532,14 +557,18 @@ class InConv128LayerParam {  // param.h:701-870
         }
         this->input = input;
         HIP_SAFE_CALL(hipMemcpy(input_gpu, input, input_bytes(), hipMemcpyHostToDevice));
+        pack_input();
     }
     uin32* get_output_gpu() { return this->output_gpu; }
     int* get_output_residual_gpu() { return this->output_residual_gpu; }
     void forward(hipStream_t stream = 0) {
-        tcbnn_inconv128_desc d = {input_gpu,      filter_gpu,     bn_gpu,        output_gpu,   output_residual_gpu,
+        const bool packed = input_packed_gpu != NULL;
+        tcbnn_inconv128_desc d = {packed ? input_packed_gpu : input_gpu, filter_gpu, bn_gpu, output_gpu,
+                                  output_residual_gpu,
                                   input_height,   input_width,    input_channels, filter_height, filter_width,
                                   output_channels, batch,         stride_height, stride_width, padding ? 1 : 0,
-                                  pool_height,    pool_width,     save_residual ? 1 : 0, residual_info.format};
+                                  pool_height,    pool_width,     save_residual ? 1 : 0, residual_info.format,
+                                  packed ? TCBNN_INCONV_INPUT_PACKED : TCBNN_INCONV_INPUT_NCHW};
         TCBNN_SAFE_CALL(tcbnn_inconv128_forward(&d, stream));
     }
     // Output and saved residual in the reference's own device layouts (kernel.cuh:650-668), converted on `stream`
@@ -586,6 +615,7 @@ class InConv128LayerParam {  // param.h:701-870
         SAFE_FREE_HOST(bn);
         SAFE_FREE_HOST(output);
         SAFE_FREE_GPU(input_gpu);
+        SAFE_FREE_GPU(input_packed_gpu);
         SAFE_FREE_GPU(output_gpu);
         SAFE_FREE_GPU(filter_gpu);
         SAFE_FREE_GPU(bn_gpu);
@@ -629,6 +659,8 @@ class InConv128LayerParam {  // param.h:701-870
     int buf_height, buf_width;  // conv output size before pooling
     uin32* output_fmt_gpu = NULL;        // reference-layout copies of the output and the saved residual
     int* output_residual_ref_gpu = NULL;
+    bool packed_input = false;           // use_packed_input()
+    float* input_packed_gpu = NULL;      // [Hp][Wp][batch][3] copy of input_gpu (un-pooled layers, on request)
 };
 
 // ======================================================================================

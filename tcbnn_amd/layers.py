@@ -489,9 +489,14 @@ class InConv128LayerParam(_ConvGeometry):
 
     def __init__(self, name, input_height, input_width, filter_height, filter_width, input_channels,
                  output_channels, batch, stride_height=1, stride_width=1, padding=True, pool_height=1,
-                 pool_width=1, save_residual=False, residual_format=None):
+                 pool_width=1, save_residual=False, residual_format=None, input_layout=None):
         self.name = name
         self.residual_format = residual_format  # None: narrowest exact format; or _lib.RES_I32 / RES_I16
+        # None / _lib.INCONV_INPUT_NCHW: the layer reads the uploaded [batch][3][H][W] array (the reference's device
+        # layout, kernel.cuh:620-625).  _lib.INCONV_INPUT_PACKED: initialize / set_input also make a zero-padded,
+        # batch-innermost copy on the device and the (un-pooled) layer reads that with a kernel that needs no
+        # staging; the upload then costs one more pass over the input, the forward pass less.
+        self.input_layout = input_layout
         self.input_height, self.input_width = input_height, input_width
         self.filter_height, self.filter_width = filter_height, filter_width
         self.input_channels, self.output_channels, self.batch = input_channels, output_channels, batch
@@ -500,10 +505,29 @@ class InConv128LayerParam(_ConvGeometry):
         self.save_residual = save_residual
         self.filter = self.bn = None
         self.input_gpu = self.filter_gpu = self.bn_gpu = self.output_gpu = self.output_residual_gpu = None
+        self.input_packed_gpu = None
         self._derive()
 
     def input_size(self):
         return self.input_channels * self.input_height * self.input_width * self.batch
+
+    def _packed_floats(self):
+        """Size of the zero-padded, batch-innermost copy of the input that the un-pooled first layer reads
+        (tcbnn_inconv_pack_input), or 0 where the layer reads the uploaded [batch][3][H][W] array itself."""
+        if self.pool_height != 1 or self.pool_width != 1 or self.input_layout != _lib.INCONV_INPUT_PACKED:
+            return 0
+        n = lib.tcbnn_inconv_packed_input_floats(
+            self.batch, self.input_height, self.input_width, self.filter_height, self.filter_width,
+            self.stride_height, self.stride_width, int(self.padding))
+        return n if 0 < 4 * n < (1 << 31) else 0
+
+    def _pack_input(self):
+        if self.input_packed_gpu is None:
+            return
+        check(lib.tcbnn_inconv_pack_input(
+            self.input_gpu.ptr, self.input_packed_gpu.ptr, self.batch, self.input_height, self.input_width,
+            self.filter_height, self.filter_width, self.stride_height, self.stride_width, int(self.padding), None))
+        _lib.device_synchronize()
 
     def initialize(self, input, config_file):
         if input is None:
@@ -511,6 +535,9 @@ class InConv128LayerParam(_ConvGeometry):
         x = np.ascontiguousarray(input, dtype=np.float32)
         assert x.size == self.input_size(), (x.size, self.input_size())
         self.input_gpu = DeviceBuffer.from_numpy(x)
+        if self._packed_floats():
+            self.input_packed_gpu = DeviceBuffer(4 * self._packed_floats())
+            self._pack_input()
         self.input_abs_max = float(np.max(np.abs(x))) if x.size else 0.0
         self.filter = np.array(config_file.launch_array(self.filter_size()), dtype=np.float32)
         self.filter_gpu = DeviceBuffer(4 * lib.tcbnn_inconv_filter_words(
@@ -542,15 +569,18 @@ class InConv128LayerParam(_ConvGeometry):
         if self.save_residual and self._residual_bound(x) > self.output_residual_gpu.bound:
             raise _lib.TcbnnError("input magnitude exceeds the bound the residual format was chosen for")
         self.input_gpu.upload(x)
+        self._pack_input()
 
     def _desc(self):
+        packed = self.input_packed_gpu is not None
         return _lib.InConv128Desc(
-            self.input_gpu.ptr, self.filter_gpu.ptr, self.bn_gpu.ptr, self.output_gpu.ptr,
+            (self.input_packed_gpu if packed else self.input_gpu).ptr, self.filter_gpu.ptr, self.bn_gpu.ptr, self.output_gpu.ptr,
             self.output_residual_gpu.ptr if self.output_residual_gpu is not None else None,
             self.input_height, self.input_width, self.input_channels, self.filter_height, self.filter_width,
             self.output_channels, self.batch, self.stride_height, self.stride_width, int(self.padding),
             self.pool_height, self.pool_width, int(self.save_residual),
-            self.output_residual_gpu.format if self.output_residual_gpu is not None else 0)
+            self.output_residual_gpu.format if self.output_residual_gpu is not None else 0,
+            _lib.INCONV_INPUT_PACKED if packed else _lib.INCONV_INPUT_NCHW)
 
     def forward(self, stream=None):
         d = self._desc()
@@ -564,10 +594,12 @@ class InConv128LayerParam(_ConvGeometry):
 
     def release(self):
         self._release_ref_bufs()
-        for b in (self.input_gpu, self.filter_gpu, self.bn_gpu, self.output_gpu, self.output_residual_gpu):
+        for b in (self.input_gpu, self.input_packed_gpu, self.filter_gpu, self.bn_gpu, self.output_gpu,
+                  self.output_residual_gpu):
             if b is not None:
                 b.free()
         self.input_gpu = self.filter_gpu = self.bn_gpu = self.output_gpu = self.output_residual_gpu = None
+        self.input_packed_gpu = None
 
 
 class Conv128LayerParam(_ConvGeometry):

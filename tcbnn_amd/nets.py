@@ -258,9 +258,10 @@ def synthetic_input(spec, seed=0):
 class Network:
     """Layer objects of one network, wired as in the reference drivers."""
 
-    def __init__(self, spec, weights, input, variant=_lib.VARIANT_AUTO, residual_format=None):
+    def __init__(self, spec, weights, input, variant=_lib.VARIANT_AUTO, residual_format=None, input_layout=None):
         """residual_format: None = every saved residual in the narrowest format that is exact for its
-        bound; _lib.RES_I32 keeps them all as int32 (the reference's type)."""
+        bound; _lib.RES_I32 keeps them all as int32 (the reference's type).  input_layout:
+        _lib.INCONV_INPUT_PACKED = the first convolution reads a packed copy of the input that the upload makes."""
         self.spec = spec
         self.layers = {}
         self.order = []
@@ -272,7 +273,7 @@ class Network:
             elif k == "inconv":
                 layer = InConv128LayerParam(L["name"], L["h"], L["w"], L["r"], L["s"], L["cin"], L["cout"],
                                             L["batch"], L["stride"], L["stride"], L["padding"], L["pool"],
-                                            L["pool"], L["save_residual"], residual_format).initialize(input, src)
+                                            L["pool"], L["save_residual"], residual_format, input_layout).initialize(input, src)
             elif k == "conv":
                 layer = Conv128LayerParam(L["name"], L["h"], L["w"], L["r"], L["s"], L["cin"], L["cout"],
                                           L["batch"], L["stride"], L["stride"], L["padding"], L["pool"],

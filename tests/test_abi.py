@@ -23,7 +23,7 @@ def test_library_exports_every_declared_symbol():
     for s in syms:
         assert hasattr(_lib.lib, s), "libtcbnn_hip.so does not export %s" % s
     assert sorted(_lib.ABI) == syms, "Python binding table and header disagree"
-    assert _lib.lib.tcbnn_abi_version() == 4
+    assert _lib.lib.tcbnn_abi_version() == 5
 
 
 def test_geometry_entry_points_match_reference_formulas():

@@ -49,3 +49,8 @@ def test_one_json_line_with_the_contract_keys(gpu):
     assert abs(f["value"] - 256 / (f["ms_per_step"] * 1e-3)) <= 0.01 * f["value"]
     assert r["traffic"] is None or r["traffic"] > 0
     assert r["traffic_stale"] == (r["traffic"] is None)
+    # the packed first-layer input is a request: its figures stay beside `value`, with the cost of the extra pass
+    u = d["packed_input"]
+    assert "direct" in u["kernel"] and "direct" not in r["kernel"]
+    assert u["pack_ms"] > 0 and u["value_with_pack_in_every_step"] < u["value"]
+    assert abs(u["value_with_pack_in_every_step"] - 256e3 / (u["ms_per_step"] + u["pack_ms"])) <= 0.01 * u["value"]

@@ -459,14 +459,74 @@ def test_inconv128_layer(gpu, b, h, R, stride, cout, pool, save):
     bn = r.normal(0, np.sqrt(3 * R * R), cout).astype(np.float32)
     bn[:4] = [0.0, -0.0, 1e-30, -1e-30]  # decide pixels whose window has no tap in the frame (sum 0)
     want, wres = orc.inconv128(x, f, bn, stride, True, pool, save)
-    layer = gpu.InConv128LayerParam("Conv1", h, h, R, R, 3, cout, b, stride, stride, True, pool, pool, save)
+    # the kernel that stages [batch][3][H][W] through LDS and, for un-pooled layers, the one that reads a packed
+    # copy of the input: two paths of the same entry point (a pooled layer ignores the request for a packed copy)
+    for layout in ([None, gpu._lib.INCONV_INPUT_PACKED] if pool == 1 else [gpu._lib.INCONV_INPUT_PACKED]):
+        layer = gpu.InConv128LayerParam("Conv1", h, h, R, R, 3, cout, b, stride, stride, True, pool, pool, save,
+                                        input_layout=layout)
+        layer.initialize(x, gpu.ArrayWeights([f, bn]))
+        assert ("direct" in layer.kernel_name()) == (pool == 1 and layout is not None), layer.kernel_name()
+        layer.forward()
+        gpuops.sync()
+        np.testing.assert_array_equal(layer.download_packed(), want)
+        np.testing.assert_array_equal(layer.download_output(), orc.conv_to_fmt(want, cout))
+        if save:
+            np.testing.assert_array_equal(layer.download_residual(), wres)
+        layer.release()
+
+
+@pytest.mark.parametrize("b,h,w,R,S,sh,sw,padding", [(5, 20, 20, 7, 7, 4, 4, 1), (70, 9, 13, 3, 5, 1, 2, 1),
+                                                     (64, 70, 66, 3, 3, 1, 1, 1), (3, 16, 16, 3, 3, 1, 1, 0),
+                                                     (130, 11, 8, 11, 3, 4, 1, 1)])
+def test_inconv_pack_input(gpu, b, h, w, R, S, sh, sw, padding):
+    """The packed copy of a first-layer input: [Hp][Wp][batch][3], the frame at the padding offsets, zeros around."""
+    lib = gpu._lib.lib
+    x = rng(b + h + w).standard_normal((b, 3, h, w)).astype(np.float32)
+    P, Q = lib.tcbnn_conv_out(h, R, sh, padding, 1), lib.tcbnn_conv_out(w, S, sw, padding, 1)
+    Hp, Wp = (P - 1) * sh + R, (Q - 1) * sw + S
+    ph, pw = lib.tcbnn_conv_pad(h, R, sh, padding), lib.tcbnn_conv_pad(w, S, sw, padding)
+    n = lib.tcbnn_inconv_packed_input_floats(b, h, w, R, S, sh, sw, padding)
+    assert n == Hp * Wp * b * 3
+    want = np.zeros((max(Hp, ph + h), max(Wp, pw + w), b, 3), np.float32)
+    want[ph:ph + h, pw:pw + w] = np.transpose(x, (2, 3, 0, 1))
+    want = want[:Hp, :Wp]  # (without padding the last rows / columns that no window reaches are cut)
+    src = gpuops.DeviceBuffer.from_numpy(x)
+    dst = gpuops.DeviceBuffer(4 * n)
+    dst.fill(0xff)
+    gpu._lib.check(lib.tcbnn_inconv_pack_input(src.ptr, dst.ptr, b, h, w, R, S, sh, sw, padding, None))
+    gpuops.sync()
+    got = dst.to_numpy(np.float32, (Hp, Wp, b, 3))
+    np.testing.assert_array_equal(got.view(np.uint32), want.view(np.uint32))
+    src.free()
+    dst.free()
+
+
+def test_inconv128_packed_input_rules(gpu):
+    """A packed input is refused for a pooled layer and for an unknown layout value; set_input repacks."""
+    r = rng(77)
+    b, h, cout = 6, 18, 64
+    x = r.standard_normal((b, 3, h, h)).astype(np.float32)
+    f = rm.pm1(r, (3, 3, 3, cout))
+    bn = r.normal(0, 5, cout).astype(np.float32)
+    plain = gpu.InConv128LayerParam("Conv1", h, h, 3, 3, 3, cout, b, 1, 1, True, 1, 1, True)
+    assert plain.input_layout is None and plain._packed_floats() == 0  # the packed copy is a request, never a default
+    layer = gpu.InConv128LayerParam("Conv1", h, h, 3, 3, 3, cout, b, 1, 1, True, 1, 1, True,
+                                    input_layout=gpu._lib.INCONV_INPUT_PACKED)
     layer.initialize(x, gpu.ArrayWeights([f, bn]))
+    d = layer._desc()
+    assert d.input_layout == gpu._lib.INCONV_INPUT_PACKED
+    d.pool_height = d.pool_width = 2
+    assert gpu._lib.lib.tcbnn_inconv128_forward(d, None) != 0
+    d = layer._desc()
+    d.input_layout = 7
+    assert gpu._lib.lib.tcbnn_inconv128_forward(d, None) != 0
+    x2 = (0.5 * r.standard_normal((b, 3, h, h))).astype(np.float32)
+    want, wres = orc.inconv128(x2, f, bn, 1, True, 1, True)
+    layer.set_input(x2)
     layer.forward()
     gpuops.sync()
     np.testing.assert_array_equal(layer.download_packed(), want)
-    np.testing.assert_array_equal(layer.download_output(), orc.conv_to_fmt(want, cout))
-    if save:
-        np.testing.assert_array_equal(layer.download_residual(), wres)
+    np.testing.assert_array_equal(layer.download_residual(), wres)
     layer.release()
 
 
