@@ -355,7 +355,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS &
                     // 16 bytes per (channel group, image): 4 int32 or 8 int16; channels past O are 0
                     int r32[32];
 #pragma unroll
-                    for (int n = 0; n < 32; ++n) r32[n] = wi * 32 + n < p.O ? (int)acc[n] : 0;
+                    for (int n = 0; n < 32; ++n) r32[n] = (int)acc[n];
+                    if (wi * 32 + 32 > p.O) {  // uniform: channels past O are stored as 0
+#pragma unroll
+                        for (int n = 0; n < 32; ++n) r32[n] = wi * 32 + n < p.O ? r32[n] : 0;
+                    }
                     // streaming stores: the tensor (103 MB at batch 256) is far larger than the caches and is
                     // read two launches later
                     v4i_t* __restrict__ dst = reinterpret_cast<v4i_t*>(res);
@@ -517,8 +521,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
                 if (wi * 32 + 32 <= p.O) {  // uniform: full channel tile
 #pragma unroll
                     for (int n = 0; n < 32; ++n) {
-                        const float t = bn[wi * 32 + n];
-                        word = __builtin_amdgcn_alignbit(word, __float_as_uint(acc[n] - (t != t ? -__builtin_huge_valf() : t)), 31);
+                        // (the NaN test on the threshold's bits: wave-uniform, so it stays on the scalar unit)
+                        const uint32_t tb = __float_as_uint(bn[wi * 32 + n]);
+                        const float t = __uint_as_float((tb & 0x7fffffffu) > 0x7f800000u ? 0xff800000u : tb);
+                        word = __builtin_amdgcn_alignbit(word, __float_as_uint(acc[n] - t), 31);
                     }
                     word = ~word;
                 } else {
@@ -532,7 +538,11 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
                 if (res != nullptr) {
                     int r32[32];
 #pragma unroll
-                    for (int n = 0; n < 32; ++n) r32[n] = wi * 32 + n < p.O ? (int)acc[n] : 0;
+                    for (int n = 0; n < 32; ++n) r32[n] = (int)acc[n];
+                    if (wi * 32 + 32 > p.O) {  // uniform: channels past O are stored as 0
+#pragma unroll
+                        for (int n = 0; n < 32; ++n) r32[n] = wi * 32 + n < p.O ? r32[n] : 0;
+                    }
                     v4i_t* __restrict__ dst = reinterpret_cast<v4i_t*>(res);
                     if (p.res_fmt == TCBNN_RES_I12) {
                         typedef int v2i_t __attribute__((ext_vector_type(2)));

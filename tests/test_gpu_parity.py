@@ -575,20 +575,21 @@ def test_inconv128_special_thresholds(gpu):
     f = rm.pm1(r, (7, 7, 3, cout))
     _, res = orc.inconv128(x, f, np.zeros(cout, np.float32), 4, True, 1, True)
     bn = r.normal(0, 8, cout).astype(np.float32)
-    bn[0:4] = np.nan
-    bn[4:6] = np.inf
+    bn[0:4] = np.array([0x7fc00000, 0xffc00000, 0x7fa00000, 0xff800001], np.uint32).view(np.float32)  # quiet,
+    bn[4:6] = np.inf                                                     # negative, signalling, smallest payload
     bn[6:8] = -np.inf
     bn[8:40] = res[1, 2, 3, 8:40]
     want, wres = orc.inconv128(x, f, bn, 4, True, 1, True)
-    layer = gpu.InConv128LayerParam("Conv1", h, h, 7, 7, 3, cout, b, 4, 4, True, 1, 1, True)
-    layer.initialize(x, gpu.ArrayWeights([f, bn]))
-    layer.forward()
-    gpuops.sync()
-    np.testing.assert_array_equal(layer.download_packed(), want)
-    np.testing.assert_array_equal(layer.download_residual(), wres)
     bits = orc.unpack_bits(want, cout)
     assert (bits[..., 0:4] == 1).all() and (bits[..., 4:6] == -1).all() and (bits[..., 6:8] == 1).all()
-    layer.release()
+    for layout in (None, gpu._lib.INCONV_INPUT_PACKED):  # the two kernels test a threshold for NaN in different ways
+        layer = gpu.InConv128LayerParam("Conv1", h, h, 7, 7, 3, cout, b, 4, 4, True, 1, 1, True, input_layout=layout)
+        layer.initialize(x, gpu.ArrayWeights([f, bn]))
+        layer.forward()
+        gpuops.sync()
+        np.testing.assert_array_equal(layer.download_packed(), want)
+        np.testing.assert_array_equal(layer.download_residual(), wres)
+        layer.release()
 
 
 def test_inconv128_small_batch_is_repeatable(gpu):
