@@ -135,7 +135,9 @@ typedef int v4i_t __attribute__((ext_vector_type(4)));
 // POOLED: blockIdx selects a row of the POOLED output; the workgroup runs the pool_h convolution rows
 // of it one after the other and ORs their words (kernel.cuh:646-664); with pool_w = 2 the two columns of
 // a wave are one window.  pool_w is 1 or 2 (the host checks), no residual is saved.
-template <int NST, bool ROWS, bool POOLED>
+// ALLIN (ROWS, un-pooled): the host found every staging pass of every lane inside the 192 segments and the batch a
+// multiple of 64, so no pass is tested (and none of those tests' invariants is computed or kept).
+template <int NST, bool ROWS, bool POOLED, bool ALLIN>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS && NST <= 16 ? 4 : 3))) void inconv_tiled_kernel(
     const InConvParams p, const float* __restrict__ in, const uint4* __restrict__ masks,
     const float* __restrict__ bn, uint32_t* __restrict__ out, int32_t* __restrict__ res, int b_tiles,
@@ -232,14 +234,14 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS &
         const int lds1 = (scol * 3 + (seg0 + rp) % 3) * kLB + (seg0 + rp) / 3;
         const int lds2 = (scol * 3 + (seg0 + 2 * rp) % 3) * kLB + (seg0 + 2 * rp) / 3;
         // every pass of every lane inside the 192 segments and the batch (wave-uniform)?
-        const bool all_in = NST * rp == 3 * 64 && b0 + 64 <= p.B;
+        constexpr bool all_in = ALLIN;
         __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
             const_cast<float*>(in + (size_t)b0 * 3 * plane), 0, (int)tile_bytes, 0x00020000);
         auto fetch_row = [&](int r) {
             if constexpr (ROWS) {
                 const unsigned row_bytes = (unsigned)(ay0 + r) * (unsigned)p.W * 4u;       // uniform
                 const unsigned pass_bytes = (unsigned)rp * (unsigned)plane * 4u;           // uniform
-                if (all_in) {
+                if constexpr (all_in) {
 #pragma unroll
                     for (int k = 0; k < NST; ++k)
                         stg[k] = __builtin_bit_cast(
@@ -335,8 +337,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS &
                     // counts as -inf: the bit is 1 either way)
 #pragma unroll
                     for (int n = 0; n < 32; ++n) {
-                        const float t = bn[wi * 32 + n];
-                        word = __builtin_amdgcn_alignbit(word, __float_as_uint(acc[n] - (t != t ? -__builtin_huge_valf() : t)), 31);
+                        // (the NaN test on the threshold's bits: wave-uniform, so it stays on the scalar unit)
+                        const uint32_t tb = __float_as_uint(bn[wi * 32 + n]);
+                        const float t = __uint_as_float((tb & 0x7fffffffu) > 0x7f800000u ? 0xff800000u : tb);
+                        word = __builtin_amdgcn_alignbit(word, __float_as_uint(acc[n] - t), 31);
                     }
                     word = ~word;
                 } else {
@@ -783,10 +787,11 @@ static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name
         const int rpw = 64 / ncols >= 3 ? (64 / ncols) / 3 * 3 : 2;
         if (row_staging) {
             const int passes = (3 * 64 + 4 * rpw - 1) / (4 * rpw);
-            snprintf(name_buf, name_len, "inconv_tiled_kernel<%d, true, %s>",
-                     passes <= 4 ? 4 : (passes <= 8 ? 8 : (passes <= 16 ? 16 : 24)), pooled ? "true" : "false");
+            const int nst = passes <= 4 ? 4 : (passes <= 8 ? 8 : (passes <= 16 ? 16 : 24));
+            snprintf(name_buf, name_len, "inconv_tiled_kernel<%d, true, %s, %s>", nst, pooled ? "true" : "false",
+                     !pooled && nst * 4 * rpw == 3 * 64 && p.B % 64 == 0 ? "true" : "false");
         } else {
-            snprintf(name_buf, name_len, "inconv_tiled_kernel<%d, false, %s>",
+            snprintf(name_buf, name_len, "inconv_tiled_kernel<%d, false, %s, false>",
                      (3 * 64 * ncols + kThreads - 1) / kThreads <= 15 ? 15 : 24, pooled ? "true" : "false");
         }
         return TCBNN_OK;
@@ -831,10 +836,14 @@ static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name
         auto launch_nst = [&](auto nst_tag, auto rows_tag) {
             constexpr int NST = decltype(nst_tag)::value;
             constexpr bool ROWS = decltype(rows_tag)::value;
-            if (pooled)
-                launch(inconv_tiled_kernel<NST, ROWS, true>);
-            else
-                launch(inconv_tiled_kernel<NST, ROWS, false>);
+            if (pooled) {
+                launch(inconv_tiled_kernel<NST, ROWS, true, false>);
+            } else {
+                if constexpr (ROWS) {
+                    if (NST * 4 * rpw == 3 * 64 && p.B % 64 == 0) return launch(inconv_tiled_kernel<NST, true, false, true>);
+                }
+                launch(inconv_tiled_kernel<NST, ROWS, false, false>);
+            }
         };
         if (row_staging) {
             const int passes = (3 * 64 + 4 * rpw - 1) / (4 * rpw);
