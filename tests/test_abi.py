@@ -48,6 +48,12 @@ def test_size_helpers():
     assert L.tcbnn_conv_filter_words(3, 3, 96, 64) == 64 * 9 * 3       # sign bits only
     assert L.tcbnn_conv_filter_words(5, 5, 64, 40) == 64 * 25 * 2
     assert L.tcbnn_inconv_filter_words(7, 7, 3, 64) == 49 * 64 * 5
+    # packed first-layer input: (P - 1) stride + R rows and columns of [batch][3]
+    assert L.tcbnn_inconv_packed_input_floats(256, 224, 224, 7, 7, 4, 4, 1) == 227 * 227 * 256 * 3
+    assert L.tcbnn_inconv_packed_input_floats(5, 32, 30, 3, 5, 1, 2, 1) == 34 * 33 * 5 * 3
+    assert L.tcbnn_inconv_packed_input_floats(5, 16, 16, 3, 3, 2, 2, 0) == 15 * 15 * 5 * 3  # the last row is unused
+    assert L.tcbnn_inconv_packed_input_floats(0, 16, 16, 3, 3, 1, 1, 1) == 0
+    assert L.tcbnn_inconv_packed_input_floats(4, 2, 16, 3, 3, 1, 1, 0) == 0   # no output row
 
 
 def test_errors_are_codes_not_exits():
@@ -59,6 +65,8 @@ def test_errors_are_codes_not_exits():
     assert L.tcbnn_fc128_forward(d, None) == -1
     assert L.tcbnn_bmm(1, 1, 1, 8, 8, 100, 1, None) == -1  # K not a multiple of 32
     assert L.tcbnn_set_default_variant(99) == -1
+    assert L.tcbnn_inconv_pack_input(None, None, 4, 8, 8, 3, 3, 1, 1, 1, None) == -2
+    assert L.tcbnn_inconv_pack_input(1, 1, 0, 8, 8, 3, 3, 1, 1, 1, None) == -1  # batch 0; never launches
     with pytest.raises(_lib.TcbnnError):
         _lib.check(-1)
 
