@@ -135,7 +135,7 @@ typedef int v4i_t __attribute__((ext_vector_type(4)));
 // POOLED: blockIdx selects a row of the POOLED output; the workgroup runs the pool_h convolution rows
 // of it one after the other and ORs their words (kernel.cuh:646-664); with pool_w = 2 the two columns of
 // a wave are one window.  pool_w is 1 or 2 (the host checks), no residual is saved.
-// ALLIN (ROWS, un-pooled): the host found every staging pass of every lane inside the 192 segments and the batch a
+// ALLIN (ROWS): the host found every staging pass of every lane inside the 192 segments and the batch a
 // multiple of 64, so no pass is tested (and none of those tests' invariants is computed or kept).
 template <int NST, bool ROWS, bool POOLED, bool ALLIN>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS && NST <= 16 ? 4 : 3))) void inconv_tiled_kernel(
@@ -789,7 +789,7 @@ static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name
             const int passes = (3 * 64 + 4 * rpw - 1) / (4 * rpw);
             const int nst = passes <= 4 ? 4 : (passes <= 8 ? 8 : (passes <= 16 ? 16 : 24));
             snprintf(name_buf, name_len, "inconv_tiled_kernel<%d, true, %s, %s>", nst, pooled ? "true" : "false",
-                     !pooled && nst * 4 * rpw == 3 * 64 && p.B % 64 == 0 ? "true" : "false");
+                     nst * 4 * rpw == 3 * 64 && p.B % 64 == 0 ? "true" : "false");
         } else {
             snprintf(name_buf, name_len, "inconv_tiled_kernel<%d, false, %s, false>",
                      (3 * 64 * ncols + kThreads - 1) / kThreads <= 15 ? 15 : 24, pooled ? "true" : "false");
@@ -836,14 +836,16 @@ static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name
         auto launch_nst = [&](auto nst_tag, auto rows_tag) {
             constexpr int NST = decltype(nst_tag)::value;
             constexpr bool ROWS = decltype(rows_tag)::value;
-            if (pooled) {
-                launch(inconv_tiled_kernel<NST, ROWS, true, false>);
-            } else {
-                if constexpr (ROWS) {
-                    if (NST * 4 * rpw == 3 * 64 && p.B % 64 == 0) return launch(inconv_tiled_kernel<NST, true, false, true>);
+            if constexpr (ROWS) {
+                if (NST * 4 * rpw == 3 * 64 && p.B % 64 == 0) {
+                    if (pooled) return launch(inconv_tiled_kernel<NST, true, true, true>);
+                    return launch(inconv_tiled_kernel<NST, true, false, true>);
                 }
-                launch(inconv_tiled_kernel<NST, ROWS, false, false>);
             }
+            if (pooled)
+                launch(inconv_tiled_kernel<NST, ROWS, true, false>);
+            else
+                launch(inconv_tiled_kernel<NST, ROWS, false, false>);
         };
         if (row_staging) {
             const int passes = (3 * 64 + 4 * rpw - 1) / (4 * rpw);
