@@ -687,6 +687,18 @@ __global__ __launch_bounds__(kThreads) void inconv_generic_kernel(const InConvPa
 
 using namespace tcbnn;
 
+// Row-wise staging: segments (image, channel) a wave takes per pass, ncols lanes each.  Whole segments only; a
+// multiple of 3 where 3 fit the 64 lanes (the channel of a lane's segment is then the same in every pass), and among
+// those the largest that divides 48, so that the workgroup's passes cover the 192 segments exactly and no pass needs a
+// test (rpw = 9 for 6-column segments used more lanes per pass but left a ragged sixth pass); else 2.
+static int inconv_segments_per_wave(int ncols) {
+    const int fit = 64 / ncols;
+    if (fit < 3) return 2;
+    for (int r : {48, 24, 12, 6})
+        if (r <= fit) return r;
+    return 3;
+}
+
 static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name_buf, size_t name_len) {
     TCBNN_NOTNULL(d);
     if (name_buf == nullptr) {
@@ -784,7 +796,7 @@ static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name
             return TCBNN_OK;
         }
         const int ncols = (kXT - 1) * p.stride_w + p.S;
-        const int rpw = 64 / ncols >= 3 ? (64 / ncols) / 3 * 3 : 2;
+        const int rpw = inconv_segments_per_wave(ncols);
         if (row_staging) {
             const int passes = (3 * 64 + 4 * rpw - 1) / (4 * rpw);
             const int nst = passes <= 4 ? 4 : (passes <= 8 ? 8 : (passes <= 16 ? 16 : 24));
@@ -826,9 +838,8 @@ static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name
                                      ? 8LL * ((x_groups + y_phases - 1) / y_phases) * rows_grid
                                      : (long long)b_tiles * x_groups * rows_out;
         TCBNN_REQUIRE(blocks <= 0x7fffffffLL, "inconv128: grid too large");
-        // staging scheme (see the kernel): whole segments per wave, a multiple of 3 of them when 3 fit its 64
-        // lanes, else 2 (ncols <= kMaxCols = 32)
-        const int rpw = 64 / ncols >= 3 ? (64 / ncols) / 3 * 3 : 2;
+        // staging scheme (see the kernel and inconv_segments_per_wave; ncols <= kMaxCols = 32)
+        const int rpw = inconv_segments_per_wave(ncols);
         auto launch = [&](auto kernel) {
             hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(kThreads), 0, (hipStream_t)stream, p, p.in,
                                p.masks, p.bn, p.out, p.res, b_tiles, x_groups, y_phases, div_magic, rpw, row_il, rows_out);
