@@ -442,6 +442,9 @@ def test_conv128_rejects_residual_with_pooling(gpu):
                                                          (70, 24, 11, 4, 64, 1, True), (66, 20, 7, 4, 40, 1, True),
                                                          (9, 17, 3, 2, 33, 1, True), (64, 16, 7, 4, 64, 1, True),
                                                          (128, 10, 3, 1, 64, 1, True),
+                                                         # three image tiles: not a divisor of the 8 XCD slots, so
+                                                         # the plain workgroup order of both un-pooled kernels
+                                                         (130, 12, 3, 1, 32, 1, True), (192, 9, 5, 2, 64, 1, False),
                                                          # pooled first layers (alexnet.cu:143-144): tiled kernel
                                                          # with 2x2 windows, odd row / column counts, a 3x3 pool
                                                          # (generic kernel)
