@@ -504,6 +504,43 @@ def test_inconv_pack_input(gpu, b, h, w, R, S, sh, sw, padding):
     dst.free()
 
 
+def test_inconv128_random_shapes(gpu):
+    """Seeded random first layers (non-square frames and filters, strides 1-4, pools 1-3, with and without padding,
+    ragged batches and channel counts, thresholds 0 / -0 / NaN / inf) on every kernel the entry point chooses from,
+    both input layouts where the layer is un-pooled."""
+    r = rng(2024)
+    kernels = set()
+    for it in range(70):
+        R, S = int(r.choice([1, 2, 3, 5, 7, 11])), int(r.choice([1, 2, 3, 5, 7, 11]))
+        stride, pool = int(r.choice([1, 1, 2, 3, 4])), int(r.choice([1, 1, 1, 2, 3]))
+        padding = bool(r.integers(0, 4) > 0)
+        h, w = int(r.integers(max(R, 2), 41)), int(r.integers(max(S, 2), 41))
+        b = int(r.choice([1, 2, 7, 33, 64, 65, 128, 130, 192]))
+        cout = int(r.choice([8, 32, 33, 40, 64, 96, 100, 128]))
+        save = bool(r.integers(0, 2)) and pool == 1
+        x = (r.standard_normal((b, 3, h, w)) * r.choice([0.1, 1.0, 3.0])).astype(np.float32)
+        f = rm.pm1(r, (R, S, 3, cout))
+        bn = r.normal(0, np.sqrt(3 * R * S), cout).astype(np.float32)
+        bn[:4] = [0.0, -0.0, np.nan, np.inf]
+        want, wres = orc.inconv128(x, f, bn, stride, padding, pool, save)
+        if want.size == 0:
+            continue
+        for layout in ([None, gpu._lib.INCONV_INPUT_PACKED] if pool == 1 else [None]):
+            case = dict(b=b, h=h, w=w, R=R, S=S, stride=stride, pool=pool, padding=padding, cout=cout, save=save,
+                        layout=layout)
+            layer = gpu.InConv128LayerParam("Conv1", h, w, R, S, 3, cout, b, stride, stride, padding, pool, pool,
+                                            save, input_layout=layout)
+            layer.initialize(x, gpu.ArrayWeights([f, bn]))
+            kernels.add(layer.kernel_name())
+            layer.forward()
+            gpuops.sync()
+            np.testing.assert_array_equal(layer.download_packed(), want, err_msg=str(case))
+            if save:
+                np.testing.assert_array_equal(layer.download_residual(), wres, err_msg=str(case))
+            layer.release()
+    assert {"inconv_direct_kernel", "inconv_generic_kernel"} <= kernels and len(kernels) >= 8, kernels
+
+
 def test_inconv128_packed_input_rules(gpu):
     """A packed input is refused for a pooled layer and for an unknown layout value; set_input repacks."""
     r = rng(77)
