@@ -355,6 +355,62 @@ def _residual_modes(gpu, variant, cin, cout, in_fmt, out_fmt, b, amp=3000):
     layer.release()
 
 
+def test_conv128_random_shapes(gpu):
+    """Seeded random bit-convolution layers: non-square frames of 1-14 pixels, 3x3 mostly (also 1x1 / 3x5 / 5x5 ...),
+    strides, pools, FC-ready outputs, every residual mode with random storage formats, channel limits that cut through
+    tiles and sources narrower or wider than the consumer, all three engines."""
+    r = rng(777)
+    kernels = set()
+    for it in range(90):
+        R, S = (3, 3) if r.integers(0, 5) else (int(r.choice([1, 3, 5])), int(r.choice([1, 3, 5])))
+        stride, pool = int(r.choice([1, 1, 2])), int(r.choice([1, 1, 1, 2, 2, 3]))
+        h, w = int(r.integers(1, 15)), int(r.integers(1, 15))
+        b = int(r.choice([1, 3, 8, 32, 33, 40, 64, 70, 128, 130]))
+        cin = int(r.choice([32, 64, 64, 96, 128, 128, 160, 192, 256, 384, 512]))
+        cout = int(r.choice([32, 35, 40, 64, 64, 96, 128, 160, 256]))
+        if b * h * w * cin > 3e6:
+            b = max(1, int(3e6 // (h * w * cin)))
+        ahead_fc = bool(r.integers(0, 4) == 0)
+        variant = str(r.choice(["mfma_f4"] * 4 + ["popc", "mfma_i8"]))
+        # 0 none, 1 save, 2 inject + save, 3 inject the 2x2 maximum + save, 4 inject only
+        mode = int(r.integers(0, 5)) if pool == 1 and not ahead_fc else 0
+        save, inject, rpool = mode in (1, 2, 3), mode in (2, 3, 4), mode == 3
+        in_fmt, out_fmt = int(r.integers(0, 3)), int(r.integers(0, 3))
+        amp = 800 if 2 in (in_fmt, out_fmt) else 3000
+        if 2 in (in_fmt, out_fmt) and b % 2:
+            b += 1  # the 12-bit format pairs images
+        if out_fmt == 2 and cin * R * S + amp > 2047:
+            out_fmt = 1
+        x, f = rm.pm1(r, (b, h, w, cin)), rm.pm1(r, (R, S, cin, cout))
+        bn = r.normal(0, np.sqrt(cin * R * S) * 0.5, cout).astype(np.float32)
+        bn[:4] = [0.0, -0.0, 0.5, np.nan]
+        inp, filt = orc.pack_conv_input_nhwc(x), orc.pack_conv_filter(f)
+        ph, pw = gpu.lib.tcbnn_conv_out(h, R, stride, 1, 1), gpu.lib.tcbnn_conv_out(w, S, stride, 1, 1)
+        lim = int(r.choice([cout, cout // 2, (cout * 5) // 6, max(1, cout - 1)])) if inject else 0
+        src = None
+        if inject:
+            src_ch = int(r.choice([cout, max(1, (cout * 2) // 3), cout + 16]))
+            src = r.integers(-amp, amp, size=((2 * ph, 2 * pw) if rpool else (ph, pw)) + (b, src_ch)).astype(np.int32)
+        case = dict(it=it, b=b, h=h, w=w, cin=cin, cout=cout, R=R, S=S, stride=stride, pool=pool, ahead_fc=ahead_fc,
+                    variant=variant, mode=mode, in_fmt=in_fmt, out_fmt=out_fmt, lim=lim)
+        want, wres = orc.conv128(inp, filt, bn, cin, cout, R, S, stride, True, pool, ahead_fc, save, inject, lim,
+                                 rpool, src)
+        layer = gpu.Conv128LayerParam("C", h, w, R, S, cin, cout, b, stride, stride, True, pool, pool, ahead_fc,
+                                      save, inject, lim, rpool, variant=_variant(gpu, variant),
+                                      residual_format=out_fmt if save else None)
+        layer.initialize(gpu.ArrayWeights([f, bn]), gpuops.pack_conv_input(x),
+                         _residual_source(src, in_fmt) if inject else None)
+        layer.output_gpu.fill(0xCD)
+        kernels.add(layer.kernel_name())
+        layer.forward()
+        gpuops.sync()
+        np.testing.assert_array_equal(layer.download_packed(), want, err_msg=str(case))
+        if save:
+            np.testing.assert_array_equal(layer.download_residual(), wres, err_msg=str(case))
+        layer.release()
+    assert sum(k.startswith("conv3x3_mfma_f4_kernel") for k in kernels) >= 15, kernels
+
+
 def test_residual_format_follows_the_bound(gpu):
     """The layer classes store a residual in 16 bits only when |value| <= 32767 is certain: the first
     layer's bound comes from the actual input, every bit convolution adds Cin*R*S."""
