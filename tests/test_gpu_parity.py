@@ -162,6 +162,58 @@ def test_bconv_odd_shapes(gpu, variant, b, h, cin, cout, R, stride):
     np.testing.assert_array_equal(got, want)
 
 
+def test_fc_out_bmm_bconv_random_shapes(gpu):
+    """Seeded random FC / output layers and stand-alone bit-GEMMs / bit-convolutions on all three engines: ragged
+    batches, K from one word to 25088, N from 8 to 1024, exact ties on FC thresholds, with and without split-K."""
+    r = rng(4242)
+    for it in range(60):
+        variant = str(r.choice(["mfma_f4"] * 4 + ["popc", "mfma_i8"]))
+        V = _variant(gpu, variant)
+        kind = it % 4
+        if kind == 0:
+            b = int(r.choice([1, 3, 8, 13, 64, 100, 130, 256, 1000, 4100]))
+            k = int(r.choice([32, 96, 128, 300, 512, 784, 1000, 1024, 2048, 4096, 25088]))
+            n = int(r.choice([8, 32, 40, 64, 100, 160, 512, 1000, 1024]))
+            b = min(b, max(1, int(1e7 // k)))
+            case = ("fc", b, k, n, variant)
+            x, w = r.standard_normal((b, k)).astype(np.float32), rm.pm1(r, (k, n))
+            bn = r.normal(0, np.sqrt(k), n).astype(np.float32)
+            wl = orc.pack_fc_weight(w)
+            _, acc = orc.fc128(orc.in128(x), wl, bn, k, n, want_acc=True)
+            bn[: min(n, 8)] = (k - 2 * acc)[0, : min(n, 8)]
+            want = orc.fc128(orc.in128(x), wl, bn, k, n)
+            inp, wbuf = gpuops.in128(x), gpuops.pack_fc_weight(w)
+            np.testing.assert_array_equal(gpuops.fc128(inp, wbuf, bn, b, k, n, V), want, err_msg=str(case))
+            np.testing.assert_array_equal(gpuops.fc128(inp, wbuf, bn, b, k, n, V, workspace=False), want,
+                                          err_msg=str(case))
+        elif kind == 1:
+            b, k = int(r.choice([1, 8, 70, 256, 1000, 4100])), int(r.choice([32, 300, 512, 1000, 1024, 1536, 4096]))
+            n = int(r.choice([10, 33, 72, 100, 1000]))
+            case = ("out", b, k, n, variant)
+            x, w = r.standard_normal((b, k)).astype(np.float32), rm.pm1(r, (k, n))
+            scale, bias = r.normal(1, 0.1, n).astype(np.float32), r.normal(0, 1, n).astype(np.float32)
+            want = orc.out128(orc.in128(x), orc.pack_fc_weight(w), scale, bias, k, n)
+            got = gpuops.out128(gpuops.in128(x), gpuops.pack_fc_weight(w), scale, bias, b, k, n, V)
+            np.testing.assert_array_equal(got, want, err_msg=str(case))
+        elif kind == 2:
+            m, n = int(r.choice([8, 77, 100, 300, 1024, 4100, 5000])), 32 * int(r.integers(1, 40))
+            k = 32 * int(r.choice([1, 2, 3, 6, 16, 33, 48, 64]))
+            a = r.integers(0, 2 ** 32, size=(m, k // 32), dtype=np.uint64).astype(np.uint32)
+            bb = r.integers(0, 2 ** 32, size=(n, k // 32), dtype=np.uint64).astype(np.uint32)
+            np.testing.assert_array_equal(gpuops.bmm(a, bb, m, n, k, V), orc.bmm(a, bb, k),
+                                          err_msg=str(("bmm", m, n, k, variant)))
+        else:
+            b, h = int(r.choice([3, 8, 33, 64, 70, 130])), int(r.integers(1, 13))
+            cin, cout = int(r.choice([32, 64, 96, 128, 160, 192, 256, 384])), int(r.choice([8, 16, 24, 33, 40, 48, 64, 100]))
+            R, stride = int(r.choice([1, 3, 3, 3, 5])), int(r.choice([1, 1, 2]))
+            x, f = rm.pm1(r, (b, h, h, cin)), rm.pm1(r, (R, R, cin, cout))
+            pad, buf, _ = orc.conv_geometry(h, R, stride)
+            want = orc.bconv(orc.pack_conv_input_nhwc(x), orc.pack_conv_filter(f), cin, cout, R, R, stride, pad, buf, buf)
+            got = gpuops.bconv(gpuops.pack_conv_input(x), gpuops.pack_conv_filter(f), b, h, h, cin, cout, R, R, stride,
+                               pad, buf, buf, V)
+            np.testing.assert_array_equal(got, want, err_msg=str(("bconv", b, h, cin, cout, R, stride, variant)))
+
+
 # --------------------------------------------------------------------------- Conv128 layer
 class _PackedSource:
     """Stands in for the previous layer: a device buffer holding packed activations."""
