@@ -221,8 +221,8 @@ def cpu_model():
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--net", default="imagenet_resnet", choices=["imagenet_resnet", "cifar10_vgg", "mnist_mlp", "alexnet", "cifar10_resnet", "imagenet_vgg",
                                                                  "imagenet_resnet_textbook"])
     ap.add_argument("--batch", type=int, default=None)
