@@ -31,6 +31,7 @@ struct Options {
     std::string labels;     // raw uint32 labels (read_dataset writes them): scores the logits against them
     std::string variant;    // popc | mfma_i8 | mfma_f4
     bool oversize_input = false;  // reference_fmt_interop: end by giving the first layer a batch beyond its bound
+    bool packed_input = false;    // the first convolution reads a packed copy of the input that the upload makes
 };
 
 inline Options parse(int argc, char** argv, const char* usage) {
@@ -56,6 +57,7 @@ inline Options parse(int argc, char** argv, const char* usage) {
         else if (a == "--labels") o.labels = next();
         else if (a == "--variant") o.variant = next();
         else if (a == "--oversize-input") o.oversize_input = true;
+        else if (a == "--packed-input") o.packed_input = true;
         else {
             fprintf(stderr, "unknown argument %s\n%s\n", a.c_str(), usage);
             exit(1);

@@ -8,7 +8,8 @@
 int main(int argc, char** argv) {
     driver::Options o = driver::parse(argc, argv,
         "imagenet_resnet [--batch N] [--image 224] [--classes 1000] [--seed S] [--reps R] "
-        "[--weights resnet_imagenet.csv] [--input x.f32] [--out logits.f32] [--labels y.u32] [--variant popc|mfma_i8|mfma_f4]");
+        "[--weights resnet_imagenet.csv] [--input x.f32] [--out logits.f32] [--labels y.u32] [--variant popc|mfma_i8|mfma_f4] "
+        "[--packed-input]");
     HIP_SAFE_CALL(hipSetDevice(0));
     const unsigned batch = o.batch ? o.batch : 256;
     const unsigned output_size = o.classes ? o.classes : 1000;
@@ -45,6 +46,7 @@ int main(int argc, char** argv) {
     //Layer-0
     InConv128LayerParam* bconv1 = new InConv128LayerParam("Conv1", image_height, image_width,
             7, 7, 3, 64, batch, 4, 4, true, 1, 1, true);  // save residual
+    if (o.packed_input) bconv1->use_packed_input();
     bconv1->initialize(images.data(), cfg());
     //Layer-1
     Conv128LayerParam* l1b1c1 = new Conv128LayerParam("L1B1C1", bconv1->output_height, bconv1->output_width, 3, 3, 64, 64, batch);

@@ -69,6 +69,13 @@ def test_imagenet_resnet_driver(gpu, tmp_path):
     _run_driver(tmp_path, "imagenet_resnet", spec, ["--image", "64", "--classes", "100"], 7, "mfma_f4")
 
 
+def test_imagenet_resnet_driver_packed_input(gpu, tmp_path):
+    """The C++ classes with the packed first-layer input (the upload packs, the first layer reads without staging)."""
+    from tcbnn_amd import nets
+    spec = nets.imagenet_resnet_spec(batch=70, image=64, output_size=100)
+    _run_driver(tmp_path, "imagenet_resnet", spec, ["--image", "64", "--classes", "100", "--packed-input"], 9, "mfma_f4")
+
+
 def test_alexnet_driver(gpu, tmp_path):
     from tcbnn_amd import nets
     spec = nets.alexnet_spec(batch=8, image=96, output_size=100)
