@@ -699,6 +699,37 @@ static int inconv_segments_per_wave(int ncols) {
     return 3;
 }
 
+// How the workgroups of the tiled and the direct kernel are dealt (see inconv_tiled_kernel): grid size and order.
+struct InConvOrder {
+    int b_tiles, x_groups, y_phases, row_il;
+    long long blocks;
+};
+static InConvOrder inconv_order(const InConvParams& p, bool pooled, int rows_out) {
+    InConvOrder o;
+    o.b_tiles = (p.B + 63) / 64;
+    o.x_groups = ((pooled ? p.pool_w * p.OW : p.PW) + kXT - 1) / kXT;
+    // XCD-aware order when the image tiles divide the 8 XCD slots
+    static const bool plain_order = getenv("TCBNN_INCONV_ORDER") != nullptr;  // tuning switch
+    o.y_phases = (!plain_order && 8 % o.b_tiles == 0) ? 8 / o.b_tiles : 0;
+    // Row interleave of the XCD-aware order: an XCD starts its resident workgroups (4 per CU x 32 CUs) once per
+    // workgroup lifetime, xg_per of them per output row, and the start of row r + 1 should lag that of row r by
+    // stride/R of a lifetime: k = stride/R x 128 / xg_per rows, taken at 0.7 of that (measured on the 7x7 stride-4
+    // layer: 214-217 MB fetched for k = 7..10, 222 for 5, 241 for 14, 286 without).
+    static const int il_env = getenv("TCBNN_INCONV_ROWIL") ? atoi(getenv("TCBNN_INCONV_ROWIL")) : -1;  // tuning switch
+    o.row_il = 0;
+    if (o.y_phases > 0 && !pooled) {
+        const int xg_per = (o.x_groups + o.y_phases - 1) / o.y_phases;
+        o.row_il = (int)(0.7 * p.stride_h * 128.0 / ((double)p.R * xg_per) + 0.5);
+        if (il_env >= 0) o.row_il = il_env;
+        o.row_il = std::min(o.row_il, rows_out / 2);
+        if (il_env < 0 && o.row_il < 4) o.row_il = 0;  // (little to gain where rows already start close to the right lag)
+    }
+    const int rows_grid = o.row_il > 1 ? (rows_out + o.row_il - 1) / o.row_il * o.row_il : rows_out;
+    o.blocks = o.y_phases > 0 ? 8LL * ((o.x_groups + o.y_phases - 1) / o.y_phases) * rows_grid
+                              : (long long)o.b_tiles * o.x_groups * rows_out;
+    return o;
+}
+
 static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name_buf, size_t name_len) {
     TCBNN_NOTNULL(d);
     if (name_buf == nullptr) {
@@ -767,25 +798,11 @@ static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name
             snprintf(name_buf, name_len, "inconv_direct_kernel");
             return TCBNN_OK;
         }
-        const int b_tiles = (p.B + 63) / 64;
-        const int x_groups = (p.PW + kXT - 1) / kXT;
-        static const bool plain_order = getenv("TCBNN_INCONV_ORDER") != nullptr;  // tuning switch
-        const int y_phases = (!plain_order && 8 % b_tiles == 0) ? 8 / b_tiles : 0;
-        static const int il_env = getenv("TCBNN_INCONV_ROWIL") ? atoi(getenv("TCBNN_INCONV_ROWIL")) : -1;  // tuning switch
-        int row_il = 0;  // row interleave, as for the staged kernel below
-        if (y_phases > 0) {
-            const int xg_per = (x_groups + y_phases - 1) / y_phases;
-            row_il = (int)(0.7 * p.stride_h * 128.0 / ((double)p.R * xg_per) + 0.5);
-            if (il_env >= 0) row_il = il_env;
-            row_il = std::min(row_il, p.PH / 2);
-            if (il_env < 0 && row_il < 4) row_il = 0;
-        }
-        const int rows_grid = row_il > 1 ? (p.PH + row_il - 1) / row_il * row_il : p.PH;
-        const long long blocks = y_phases > 0 ? 8LL * ((x_groups + y_phases - 1) / y_phases) * rows_grid
-                                              : (long long)b_tiles * x_groups * p.PH;
-        TCBNN_REQUIRE(blocks <= 0x7fffffffLL, "inconv128: grid too large");
-        hipLaunchKernelGGL(inconv_direct_kernel, dim3((unsigned)blocks), dim3(kThreads), 0, (hipStream_t)stream, p, p.in,
-                           p.masks, p.bn, p.out, p.res, b_tiles, x_groups, y_phases, row_il, (int)Wp, (unsigned)in_bytes);
+        const InConvOrder o = inconv_order(p, false, p.PH);
+        TCBNN_REQUIRE(o.blocks <= 0x7fffffffLL, "inconv128: grid too large");
+        hipLaunchKernelGGL(inconv_direct_kernel, dim3((unsigned)o.blocks), dim3(kThreads), 0, (hipStream_t)stream, p,
+                           p.in, p.masks, p.bn, p.out, p.res, o.b_tiles, o.x_groups, o.y_phases, o.row_il, (int)Wp,
+                           (unsigned)in_bytes);
         TCBNN_LAUNCH_CHECK("inconv_direct_kernel");
         return TCBNN_OK;
     }
@@ -809,40 +826,20 @@ static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name
         return TCBNN_OK;
     }
     if (tiled) {
-        const int b_tiles = (p.B + 63) / 64;
-        const int x_groups = ((pooled ? p.pool_w * p.OW : p.PW) + kXT - 1) / kXT;
         // e / ncols == (e * magic) >> 16 for every e the staging loop uses
         const int ncols = (kXT - 1) * p.stride_w + p.S;
         const int div_magic = 65536 / ncols + 1;
         for (int e = 0; e < 3 * 64 * ncols; ++e)
             TCBNN_REQUIRE((int)(((unsigned)e * (unsigned)div_magic) >> 16) == e / ncols,
                           "inconv128: internal error (division constant)");
-        // XCD-aware order when the image tiles divide the 8 XCD slots (see the kernel)
-        static const bool plain_order = getenv("TCBNN_INCONV_ORDER") != nullptr;  // tuning switch
-        const int y_phases = (!plain_order && 8 % b_tiles == 0) ? 8 / b_tiles : 0;
-        // Row interleave of the XCD-aware order (see the kernel): an XCD starts its resident workgroups (4 per CU
-        // x 32 CUs) once per workgroup lifetime, xg_per of them per output row, and the start of row r + 1 should
-        // lag that of row r by stride/R of a lifetime: k = stride/R x 128 / xg_per rows, taken at 0.7 of that (measured
-        // on the 7x7 stride-4 layer: 214-217 MB fetched for k = 7..10, 222 for 5, 241 for 14, 286 without).
-        static const int il_env = getenv("TCBNN_INCONV_ROWIL") ? atoi(getenv("TCBNN_INCONV_ROWIL")) : -1;  // tuning switch
-        int row_il = 0;
-        if (y_phases > 0 && !pooled) {
-            const int xg_per = (x_groups + y_phases - 1) / y_phases;
-            row_il = (int)(0.7 * p.stride_h * 128.0 / ((double)p.R * xg_per) + 0.5);
-            if (il_env >= 0) row_il = il_env;
-            row_il = std::min(row_il, rows_out / 2);
-            if (il_env < 0 && row_il < 4) row_il = 0;  // (little to gain where rows already start close to the right lag)
-        }
-        const int rows_grid = row_il > 1 ? (rows_out + row_il - 1) / row_il * row_il : rows_out;
-        const long long blocks = y_phases > 0
-                                     ? 8LL * ((x_groups + y_phases - 1) / y_phases) * rows_grid
-                                     : (long long)b_tiles * x_groups * rows_out;
-        TCBNN_REQUIRE(blocks <= 0x7fffffffLL, "inconv128: grid too large");
+        const InConvOrder o = inconv_order(p, pooled, rows_out);
+        TCBNN_REQUIRE(o.blocks <= 0x7fffffffLL, "inconv128: grid too large");
         // staging scheme (see the kernel and inconv_segments_per_wave; ncols <= kMaxCols = 32)
         const int rpw = inconv_segments_per_wave(ncols);
         auto launch = [&](auto kernel) {
-            hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(kThreads), 0, (hipStream_t)stream, p, p.in,
-                               p.masks, p.bn, p.out, p.res, b_tiles, x_groups, y_phases, div_magic, rpw, row_il, rows_out);
+            hipLaunchKernelGGL(kernel, dim3((unsigned)o.blocks), dim3(kThreads), 0, (hipStream_t)stream, p, p.in,
+                               p.masks, p.bn, p.out, p.res, o.b_tiles, o.x_groups, o.y_phases, div_magic, rpw, o.row_il,
+                               rows_out);
         };
         auto launch_nst = [&](auto nst_tag, auto rows_tag) {
             constexpr int NST = decltype(nst_tag)::value;
