@@ -45,7 +45,7 @@ def kernel_source_digest():
     h = hashlib.sha256()
     src = os.path.join(ROOT, "tcbnn_amd", "csrc")
     for name in sorted(os.listdir(src)):
-        if name.endswith((".hip", ".h")) and name != "hbm_copy_probe.hip":
+        if name.endswith((".hip", ".h")):
             h.update(name.encode())
             with open(os.path.join(src, name), "rb") as f:
                 h.update(f.read())
@@ -67,12 +67,14 @@ def load_measured_traffic():
 MEASURED_TRAFFIC_BYTES, TRAFFIC_STALE, TRAFFIC_NOTE = {}, True, "not loaded"
 
 
-def layer_work(L, spec=(), res_bytes=None):
+def layer_work(L, spec=(), res_bytes=None, pooled=()):
     """Algorithmic work of one layer launch: binary ops (2 per +-1 multiply-accumulate, border taps
     included), fp32 adds of the first layer, and the HBM bytes the launch has to move once
     (inputs + outputs + weights, packed activations at 1 bit per value, residuals at the width
     they are stored in: res_bytes[layer name] = 1.5, 2 or 4 bytes per value of that layer's saved
-    residual, 4 = the reference's int32 when not given)."""
+    residual, 4 = the reference's int32 when not given; `pooled` = names of the layers whose saved residual
+    is stored as its maximum over 2x2 windows of pixels, a quarter of the tensor, because only pooling
+    consumers read it)."""
     res_bytes = res_bytes or {}
     from tcbnn_amd import nets
     bops, flops = nets.binary_ops([L])
@@ -99,12 +101,13 @@ def layer_work(L, spec=(), res_bytes=None):
         else:
             byts = B * L["h"] * L["w"] * L["cin"] / 8 + out_bits + L["r"] * L["s"] * L["cin"] * L["cout"] / 8
             if L["save_residual"]:
-                byts += B * oh * ow * L["cout"] * res_bytes.get(L["name"], 4)
+                byts += B * oh * ow * L["cout"] * res_bytes.get(L["name"], 4) / (4 if L["name"] in pooled else 1)
             if L["inject_residual"]:
                 # channels actually injected: those the source layer saved, capped by residual_channels
                 src_ch = [S.get("cout", S.get("channels")) for S in spec if S["name"] == L.get("res_src")]
                 ch = min([L["residual_channels"], L["cout"]] + src_ch)
-                byts += B * oh * ow * (4 if L["residual_pool"] else 1) * ch * res_bytes.get(L.get("res_src"), 4)
+                src_pixels = 4 if L["residual_pool"] and L.get("res_src") not in pooled else 1
+                byts += B * oh * ow * src_pixels * ch * res_bytes.get(L.get("res_src"), 4)
     return dict(bops=bops, flops=flops, bytes=float(byts))
 
 
@@ -141,6 +144,9 @@ def roofline_of(name, g, variant):
         adds = g["flops"] / 6.0
         rec["valu_fp32"] = {"adds_per_launch": round(adds / g["launches"]), "achieved": round(adds / secs / 1e12, 2),
                             "peak": round(157.3 / 4, 1), "unit": "Tadd/s", "frac": round(adds / secs / 1e12 / (157.3 / 4), 4)}
+        # `bound` stays the roof the kernel's algorithmic bytes and operations put it under; what the hardware
+        # counters show it waiting for is the issue rate of its dependent fp32 additions
+        rec["binding"] = "valu (dependent fp32 adds in the reference's summation order); see valu_fp32"
     return rec
 
 
@@ -424,12 +430,14 @@ def main():
     width = {_lib.RES_I32: 4, _lib.RES_I16: 2, _lib.RES_I12: 1.5}
     res_bytes = {L["name"]: width[net.layers[L["name"]].output_residual_gpu.format]
                  for L in spec if L.get("save_residual") or (L["kind"] == "pool" and L.get("res_src"))}
+    # saved residuals stored as their 2x2 maximum (every reader pools): what the buffers hold after the forward
+    pooled = {name for name in res_bytes if net.layers[name].output_residual_gpu.pooled}
     # group launches by device kernel, as a profiler does
     groups = {}
     for L, layer in zip(spec, net.order):
         name = layer.kernel_name() if hasattr(layer, "kernel_name") else \
             {"in": "in128_kernel"}[L["kind"]]
-        w = layer_work(L, spec, res_bytes)
+        w = layer_work(L, spec, res_bytes, pooled)
         g = groups.setdefault(name, dict(bops=0.0, flops=0.0, bytes=0.0, ms=0.0, launches=0))
         g["bops"] += w["bops"]
         g["flops"] += w["flops"]
@@ -445,14 +453,53 @@ def main():
     roofline = roofline_of(by_time[0][0], by_time[0][1], variant)
     roofline_all = [roofline_of(n, g, variant) for n, g in by_time]
     bit = [g for n, g in groups.items() if g["bops"] > 0]
-    bit_layers_tops = round(sum(g["bops"] for g in bit) / (sum(g["ms"] for g in bit) * 1e-3) / 1e12, 2)
+    bit_ops, bit_ms = sum(g["bops"] for g in bit), sum(g["ms"] for g in bit)
+    bit_layers_tops = round(bit_ops / (bit_ms * 1e-3) / 1e12, 2)
+    # every bit-matmul / bit-convolution launch of the step together against the engine's compute peak
+    peak_name, peak_tops = COMPUTE_PEAKS_TOPS[variant]
+    roofline_bit_layers = {
+        "bound": peak_name, "achieved": bit_layers_tops, "peak": round(peak_tops, 1),
+        "unit": "TFLOP/s" if variant == "mfma_f4" else "TOP/s", "frac": round(bit_layers_tops / peak_tops, 4),
+        "binary_ops_per_step": bit_ops, "ms_per_step": round(bit_ms, 4), "launches_per_step": sum(g["launches"] for g in bit),
+        "hbm_gbs": round(sum(g["bytes"] for g in bit) / (bit_ms * 1e-3) / 1e9, 1),
+        "what": "all bit layers of the step (binary ops: 2 per +-1 multiply-accumulate, border taps included) over the "
+                "sum of their launch durations (10 launches back to back between two events, the gap between launches "
+                "included)"}
+
+    # ------------------------------------------------------------------ shader clock while the step runs: the
+    # published peaks are quoted at the nominal clock; one wavefront on a second stream counts shader cycles against
+    # the device's constant-rate wall clock while forward passes run (outside the timed region)
+    shader_clock = None
+    try:
+        from tcbnn_amd.device import DeviceBuffer
+        counts = DeviceBuffer(16)
+        side = Stream()
+        khz = C.c_int(0)
+        for _ in range(20):
+            net.forward(stream)
+        probe_us = int(max(2.0, min(50.0, 10 * ms_per_step)) * 1000)
+        _lib.check(_lib.lib.tcbnn_shader_clock_probe(counts.ptr, probe_us, C.byref(khz), side.handle))
+        t0 = time.perf_counter()
+        while (time.perf_counter() - t0) * 1e6 < probe_us * 1.5:
+            for _ in range(4):
+                net.forward(stream)
+            stream.synchronize()
+        side.synchronize()
+        cyc, ticks = (int(v) for v in counts.to_numpy(np.uint64, (2,)))
+        shader_clock = {"mhz": round(cyc / ticks * khz.value / 1000.0, 1), "nominal_mhz": 2400,
+                        "what": "shader cycles counted by one wavefront over %d us of the device's %d kHz wall clock "
+                                "while forward passes of this network run; the peaks above are quoted at the nominal "
+                                "clock" % (probe_us, khz.value)}
+        counts.free()
+    except Exception as e:  # (a measurement aid: the line is valid without it)
+        shader_clock = {"mhz": None, "error": str(e)}
 
     if args.layers:
         sys.stderr.write("%-8s %-34s %10s %10s %9s\n" % ("layer", "kernel", "ms", "TOP/s", "GB/s"))
         for L, layer in zip(spec, net.order):
             ops = nets.binary_ops([L])[0]
             kn = layer.kernel_name() if hasattr(layer, "kernel_name") else L["kind"]
-            byts = layer_work(L, spec, res_bytes)["bytes"]
+            byts = layer_work(L, spec, res_bytes, pooled)["bytes"]
             ms = layer_ms[L["name"]]
             sys.stderr.write("%-8s %-34s %10.4f %10.1f %9.0f\n" % (L["name"], kn, ms, ops / (ms * 1e-3) / 1e12,
                                                                    byts / (ms * 1e-3) / 1e9))
@@ -512,6 +559,8 @@ def main():
                                         % (sum(1 for v in res_bytes.values() if v == 1.5),
                                            sum(1 for v in res_bytes.values() if v == 2),
                                            sum(1 for v in res_bytes.values() if v == 4), len(res_bytes)))
+                   + ("; %d of them stored as their maximum over 2x2 windows of pixels (every reader takes that "
+                      "maximum, kernel.cuh:775-782)" % len(pooled) if pooled else "")
                    if res_bytes else "none"},
         "binary_tops": round(bops * args.steps / wall / 1e12, 2),
         "binary_ops_per_step": bops, "fp32_first_layer_flops_per_step": flops,
@@ -521,6 +570,8 @@ def main():
         "packed_input": packed_input,
         "batches_in_flight": in_flight,
         "bit_layers_binary_tops": bit_layers_tops,
+        "roofline_bit_layers": roofline_bit_layers,
+        "shader_clock": shader_clock,
         "roofline_all_kernels": roofline_all,
     }
     net.release()

@@ -31,9 +31,12 @@
  *                                                 FC: KWTOT = KW128; conv: KWTOT = R*S*CW,
  *                                                 K index = (r*S+s)*32*CW + c; rows >= N are 0
  *   residual tensors : TCBNN_RES_I32: int32 [P][Q][ceil(O/4)][B][4]; TCBNN_RES_I16: int16
- *                      [P][Q][ceil(O/8)][B][8] for tensors whose values provably fit 16 bits
- *                      (see "residual formats" below).  Either way an image's group of 4 / 8
- *                      consecutive channels is 16 contiguous bytes and consecutive images follow
+ *                      [P][Q][ceil(O/8)][B][8] for tensors whose values provably fit 16 bits;
+ *                      TCBNN_RES_I12: per pixel and group of 16 channels uint32 [B][4] then
+ *                      uint32 [B][2] (12 bits per value, 24 bytes per image) for tensors whose
+ *                      values provably fit 12 bits (see "residual formats" below).  In every
+ *                      format an image's group of 4 / 8 / 16 consecutive channels is one or two
+ *                      contiguous pieces of 16 (or 16 + 8) bytes and consecutive images follow
  *                      each other; channels are padded to the group, not to 128
  *   fp32 stem input  : float  [B][3][H][W]        (kernel.cuh:620-625)
  * The reference's own tile-contiguous "FMT" layouts ([.../8][.../128][8][4],
@@ -251,7 +254,13 @@ int tcbnn_inconv_pack_input(const float* input, float* packed, int batch, int he
  * Channels o >= input_residual_channels of the source read as 0 (the reference
  * gets the same effect from its zero-filled 128-channel padding, param.h:979-980).
  * save_residual / inject_residual require pool 1x1, residual_pool requires the
- * source to be exactly twice the output size (as the reference indexing assumes). */
+ * source to be exactly twice the output size (as the reference indexing assumes).
+ * output_residual_pool = 2 (no counterpart in the reference): Rout holds, per 2x2 window of output
+ * pixels, the element-wise maximum of `res`: a P/2 x Q/2 x O tensor, i.e. exactly what a consumer
+ * with residual_pool computes from the full tensor before it adds it (kernel.cuh:775-782), so that
+ * consumer then injects it with residual_pool = 0.  A quarter of the bytes are written and read;
+ * meant for a tensor whose every consumer pools.  Available where
+ * tcbnn_conv128_pooled_save_supported says so (TCBNN_EUNSUPPORTED otherwise). */
 typedef struct tcbnn_conv128_desc {
     const uint32_t* input;         /* [H][W][CW(input_channels)][B] */
     const uint32_t* filter;        /* tcbnn_pack_conv_filter output */
@@ -272,8 +281,14 @@ typedef struct tcbnn_conv128_desc {
     int variant;
     int input_residual_format;     /* TCBNN_RES_* of input_residual */
     int output_residual_format;    /* TCBNN_RES_* of output_residual */
+    int output_residual_pool;      /* 0: P x Q x O tensor; 2: its 2x2 maximum, P/2 x Q/2 x O */
 } tcbnn_conv128_desc;
 int tcbnn_conv128_forward(const tcbnn_conv128_desc* d, void* stream);
+/* 1 if the layer `d` describes can be run with output_residual_pool = 2 (whatever d->output_residual_pool says; no
+ * pointer is dereferenced): the FP4 engine's 3x3 kernel on an un-pooled layer with even P and Q, output channels a
+ * multiple of 64, a 12- or 16-bit injected residual whose channel limit is a multiple of 32, and a 12- or 16-bit
+ * output format.  0 otherwise.  No counterpart in the reference. */
+int tcbnn_conv128_pooled_save_supported(const tcbnn_conv128_desc* d);
 
 /* Name of the device kernel (as a profiler lists it, template arguments included) that
  * the corresponding *_forward call would launch for this descriptor; no
@@ -284,6 +299,12 @@ int tcbnn_conv128_kernel_name(const tcbnn_conv128_desc* d, char* buf, size_t len
 int tcbnn_fc128_kernel_name(const tcbnn_fc128_desc* d, char* buf, size_t len);
 int tcbnn_out128_kernel_name(const tcbnn_out128_desc* d, char* buf, size_t len);
 int tcbnn_inconv128_kernel_name(const tcbnn_inconv128_desc* d, char* buf, size_t len);
+
+/* Measurement aid (no counterpart in the reference): one wavefront counts shader clock cycles over `microseconds` of
+ * the device's constant-rate wall clock, on `stream`, while whatever else is queued on other streams runs beside it.
+ * After the stream has been synchronised, counts[0] = shader cycles, counts[1] = wall-clock ticks (DEVICE pointer to
+ * two 64-bit words); *wall_clock_khz = ticks per millisecond.  Shader MHz = counts[0] / counts[1] * khz / 1000. */
+int tcbnn_shader_clock_probe(unsigned long long* counts, int microseconds, int* wall_clock_khz, void* stream);
 
 /* ------------------------------------------------ layers of the textbook ResNet wiring */
 /* The reference wires ResNet-18 without a pooling layer after the first convolution, without

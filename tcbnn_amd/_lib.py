@@ -65,7 +65,8 @@ class Conv128Desc(C.Structure):
                 ("ahead_fc", c_int), ("save_residual", c_int), ("inject_residual", c_int),
                 ("residual_channels", c_int), ("residual_pool", c_int),
                 ("input_residual_channels", c_int), ("variant", c_int),
-                ("input_residual_format", c_int), ("output_residual_format", c_int)]
+                ("input_residual_format", c_int), ("output_residual_format", c_int),
+                ("output_residual_pool", c_int)]
 
 
 class Pool128Desc(C.Structure):
@@ -117,10 +118,12 @@ ABI = {
     "tcbnn_inconv_packed_input_floats": (c_size_t, [c_int] * 8),
     "tcbnn_inconv_pack_input": (c_int, [c_void_p, c_void_p] + [c_int] * 8 + [c_void_p]),
     "tcbnn_conv128_forward": (c_int, [C.POINTER(Conv128Desc), c_void_p]),
+    "tcbnn_conv128_pooled_save_supported": (c_int, [C.POINTER(Conv128Desc)]),
     "tcbnn_conv128_kernel_name": (c_int, [C.POINTER(Conv128Desc), C.c_char_p, c_size_t]),
     "tcbnn_fc128_kernel_name": (c_int, [C.POINTER(Fc128Desc), C.c_char_p, c_size_t]),
     "tcbnn_out128_kernel_name": (c_int, [C.POINTER(Out128Desc), C.c_char_p, c_size_t]),
     "tcbnn_inconv128_kernel_name": (c_int, [C.POINTER(InConv128Desc), C.c_char_p, c_size_t]),
+    "tcbnn_shader_clock_probe": (c_int, [c_void_p, c_int, C.POINTER(c_int), c_void_p]),
     "tcbnn_bmm": (c_int, [c_void_p] * 3 + [c_int] * 4 + [c_void_p]),
     "tcbnn_bconv": (c_int, [c_void_p] * 3 + [c_int] * 14 + [c_void_p]),
     "tcbnn_unpack_fc_output": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),

@@ -85,6 +85,7 @@ struct BgemmParams {
     int res_pool;           // 2x2 max over a source twice the output size
     int32_t* res_out;       // [PH][PW][N][B]
     int res_in_fmt, res_out_fmt;  // TCBNN_RES_* of res_in / res_out
+    int res_out_pool;             // res_out holds the maximum over 2x2 windows of output pixels: [PH/2][PW/2][N][B]
     // split-K (FC-shaped problems only): partial popcounts are atomically added into
     // workspace[n*B + b] and a finishing kernel applies the epilogue
     int32_t* workspace;

@@ -65,13 +65,17 @@ constexpr int kWavesPerSimd = 2;
 
 // SPT = k-steps (64 bits) per filter tap = Cin / 64; MT = 32-image tiles per wave (2 for plain
 // layers, 1 for residual layers); NT = 32-channel tiles per wave; RF = TCBNN_RES_* format of the
-// injected residual (the narrower, the fewer registers hold it while it is in flight); POOL = 2x2 OR-pooling of the
-// output bits (kernel.cuh:797-816): a wave multiplies the four pixels of a window one after the
-// other and stores the OR of their words once.  FULLT = every 32-channel tile of the launch exists in full
+// injected residual (the narrower, the fewer registers hold it while it is in flight); WIN = what a wave does with
+// the 2x2 windows of output pixels: WIN_NONE nothing (its work items are single pixels); WIN_ORPOOL = 2x2 OR-pooling
+// of the output bits (kernel.cuh:797-816): a wave multiplies the four pixels of a window one after the other and
+// stores the OR of their words once; WIN_MAXSAVE = the output bits are stored per pixel, but the saved residual is
+// the element-wise maximum over the window, stored once per window: exactly what a consumer with residual_pool
+// would compute from the full tensor (kernel.cuh:775-782), at a quarter of the bytes written and read.  FULLT = every 32-channel tile of the launch exists in full
 // and, with an injected residual, lies entirely below or entirely above the channel limit: the per-channel
 // tests of partial tiles are then not even compiled (they cost scalar registers and set-up instructions in
 // every launch, and the networks' channel counts are multiples of 64).
-template <int SPT, int RM, int MT, int NT, int RF, bool POOL, bool FULLT>
+constexpr int WIN_NONE = 0, WIN_ORPOOL = 1, WIN_MAXSAVE = 2;
+template <int SPT, int RM, int MT, int NT, int RF, int WIN, bool FULLT>
 __global__ __launch_bounds__(64 * waves_of(SPT, NT)) __attribute__((amdgpu_waves_per_eu(kWavesPerSimd))) void
 conv3x3_mfma_f4_kernel(
     const BgemmParams p, const uint32_t* __restrict__ act, const uint32_t* __restrict__ wgt,
@@ -79,7 +83,10 @@ conv3x3_mfma_f4_kernel(
     int rout_fmt, unsigned act_bytes, unsigned rin_bytes, unsigned rout_bytes, unsigned bits_bytes,
     int n_groups, int b_groups, int pix_streams, int dy, int dx, int dxs) {
     constexpr bool kRes = RM == RM_PLAIN || RM == RM_POOLED;  // a residual is injected and / or saved
+    constexpr bool POOL = WIN == WIN_ORPOOL, PSAVE = WIN == WIN_MAXSAVE, kWin = WIN != WIN_NONE;
     static_assert(RM == RM_NONE || !POOL, "residuals are defined for un-pooled layers only");
+    static_assert(!PSAVE || (RM == RM_PLAIN && FULLT && (RF == TCBNN_RES_I16 || RF == TCBNN_RES_I12)),
+                  "the window maximum is taken on 16-bit pairs in the epilogue of full tiles with a narrow injected residual");
     constexpr int TPC = SPT >= 3 ? 3 : 9;  // taps per prefetch chunk (a filter row, or all of it)
     constexpr int NCH = 9 / TPC;           // chunks per tile
     constexpr int NQ = 9 * SPT;            // k-steps per tile
@@ -153,8 +160,8 @@ conv3x3_mfma_f4_kernel(
     v16f acc0[NT];
 
     // a wave's work items: output pixels, or 2x2 windows of them (row width `roww`)
-    const int roww = POOL ? p.OW : p.PW;
-    const int npix = POOL ? p.OH * p.OW : p.PH * p.PW;
+    const int roww = kWin ? p.PW / 2 : p.PW;
+    const int npix = kWin ? (p.PH / 2) * (p.PW / 2) : p.PH * p.PW;
     int pi = stream * kWaves + wave;
     const int dpi = pix_streams * kWaves;
     // Item pi stands for row pi / roww and column (pi % roww + row) % roww.  The skew by the row keeps
@@ -489,6 +496,7 @@ conv3x3_mfma_f4_kernel(
     // One channel tile of the epilogue.  FAST (wave-uniform choice): all 32 channels exist and, with a
     // residual, all of them receive it, so no per-channel condition is evaluated at all.
     uint32_t poolw[MT][NT];  // POOL: OR of the window's words so far
+    uint32_t winmax[PSAVE ? MT * NT : 1][8];  // PSAVE: maximum of the window's sums so far, as pairs of int16
     auto epilogue_tile = [&](auto fast_tag, int nt, unsigned pix, unsigned bits_pix, int (*rv)[NW],
                              int sub) __attribute__((always_inline)) {
         constexpr bool FAST = decltype(fast_tag)::value;
@@ -563,7 +571,48 @@ conv3x3_mfma_f4_kernel(
                 float t[16];  // 1.5 * 2^23 + (sum + residual)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) t[v] = __uint_as_float(tb[v]);
-                if (rout != nullptr) {
+                if constexpr (PSAVE) {
+                    // Only the window's maximum is saved.  The low 16 bits of a bit pattern are the sum as int16 (the
+                    // host admits this instantiation only for 12- and 16-bit outputs): two sums per word, packed maximum.
+                    typedef short s2_t __attribute__((ext_vector_type(2)));
+                    uint32_t* wm = winmax[mt * NT + nt];
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) {
+                        const uint32_t pr = __builtin_amdgcn_perm(__float_as_uint(t[2 * k + 1]), __float_as_uint(t[2 * k]), 0x05040100u);
+                        wm[k] = sub == 0 ? pr
+                                         : __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(s2_t, wm[k]),
+                                                                                                  __builtin_bit_cast(s2_t, pr)));
+                    }
+                    if (sub == 3) {  // (uniform) `pix` is the window's index in the pooled tensor
+                        v4i q[2];
+                        if (rout_fmt == TCBNN_RES_I12) {
+                            int un[16];
+#pragma unroll
+                            for (int k = 0; k < 8; ++k) un[2 * k] = (int)wm[k], un[2 * k + 1] = (int)(wm[k] >> 16);
+                            uint32_t d[6];
+                            i12_pack8(un, d[0], d[1], d[2]);
+                            i12_pack8(un + 8, d[3], d[4], d[5]);
+                            const unsigned so = (pix * (unsigned)((p.N + 15) / 16) + (unsigned)((n0 + nt * 32) / 16)) * g12_b;
+                            const unsigned vo = b_ok ? (unsigned)h * g12_b + (unsigned)b * 16u : kOutOfRange;
+                            const unsigned vo2 = b_ok ? (unsigned)h * g12_b + grp_b + (unsigned)b * 8u : kOutOfRange;
+                            q[0] = v4i{(int)d[0], (int)d[1], (int)d[2], (int)d[3]};
+                            typedef int v2i_t __attribute__((ext_vector_type(2)));
+                            const v2i_t q2 = {(int)d[4], (int)d[5]};
+                            __builtin_amdgcn_raw_buffer_store_b128(q[0], r_rout, (int)vo, (int)so, 0);
+                            __builtin_amdgcn_raw_buffer_store_b64(q2, r_rout, (int)vo2, (int)so, 0);
+                            asm volatile("s_nop 4" ::"v"(q[0]), "v"(q2));  // see the 128-bit store note below
+                        } else {  // TCBNN_RES_I16
+                            const unsigned so = (pix * (unsigned)((p.N + 7) / 8) + (unsigned)((n0 + nt * 32) / 8)) * grp_b;
+                            const unsigned vo = b_ok ? ((unsigned)(2 * h) * (unsigned)p.B + (unsigned)b) * 16u : kOutOfRange;
+#pragma unroll
+                            for (int g = 0; g < 2; ++g) {
+                                q[g] = v4i{(int)wm[4 * g], (int)wm[4 * g + 1], (int)wm[4 * g + 2], (int)wm[4 * g + 3]};
+                                __builtin_amdgcn_raw_buffer_store_b128(q[g], r_rout, (int)vo, (int)(so + (unsigned)g * grp_b), 0);
+                            }
+                            asm volatile("s_nop 4" ::"v"(q[0]), "v"(q[1]));
+                        }
+                    }
+                } else if (rout != nullptr) {
                     // the value to store is in the low bits of t's bit pattern (see the 128-bit store note below)
                     v4i q[4];
                     if (rout_fmt == TCBNN_RES_I12) {
@@ -779,9 +828,11 @@ conv3x3_mfma_f4_kernel(
     };
 
     // (yy, xx): the output pixel, or the window when pooled (sub = pixel of the window, 3 = last)
+    // PSAVE: the bits belong to the window's pixel `sub`, the saved residual to the window
     auto epilogue = [&](int yy, int xx, int sub, int (*rv)[NW]) __attribute__((always_inline)) {
         const unsigned pix = (unsigned)yy * (unsigned)roww + (unsigned)xx;
-        const unsigned bits_pix = pix * (unsigned)p.bits_pix_stride * 4u;  // uniform
+        const unsigned bpix = PSAVE ? (unsigned)(2 * yy + (sub >> 1)) * (unsigned)p.PW + (unsigned)(2 * xx + (sub & 1)) : pix;
+        const unsigned bits_pix = bpix * (unsigned)p.bits_pix_stride * 4u;  // uniform
         if constexpr (kRawTranspose) {  // (the host only picks this instantiation for 16-byte aligned outputs)
             epilogue_raw_transposed(pix);
             return;
@@ -821,7 +872,7 @@ conv3x3_mfma_f4_kernel(
     auto advance = [&](Cursor& c) __attribute__((always_inline)) {
         if (++c.chunk == NCH) {
             c.chunk = 0;
-            if constexpr (POOL) {
+            if constexpr (kWin) {
                 if (++c.sub < 4) return;
                 c.sub = 0;
             }
@@ -838,8 +889,8 @@ conv3x3_mfma_f4_kernel(
         }
     };
     // output pixel a cursor stands on
-    auto pix_y = [&](const Cursor& c) __attribute__((always_inline)) { return POOL ? 2 * c.y + (c.sub >> 1) : c.y; };
-    auto pix_x = [&](const Cursor& c) __attribute__((always_inline)) { return POOL ? 2 * c.x + (c.sub & 1) : c.x; };
+    auto pix_y = [&](const Cursor& c) __attribute__((always_inline)) { return kWin ? 2 * c.y + (c.sub >> 1) : c.y; };
+    auto pix_x = [&](const Cursor& c) __attribute__((always_inline)) { return kWin ? 2 * c.x + (c.sub & 1) : c.x; };
     uint32_t buf[NB][TPC * SPT][MT];
     uint32_t msk[NB];
     int rv[kAhead ? NB : 1][NRV][NW];
@@ -850,7 +901,7 @@ conv3x3_mfma_f4_kernel(
         msk[i] = 0;
         if (lc.pi < npix) {
             msk[i] = load_chunk(pix_y(lc), pix_x(lc), lc.chunk, buf[i]);
-            if constexpr (kAhead) request_residual(lc.y, lc.x, rv[i]);  // (a chunk is a whole tile here)
+            if constexpr (kAhead) request_residual(pix_y(lc), pix_x(lc), rv[i]);  // (a chunk is a whole tile here)
         }
         advance(lc);
     }
@@ -917,7 +968,7 @@ conv3x3_mfma_f4_kernel(
                 msk[J] = load_chunk(pix_y(lc), pix_x(lc), lc.chunk, buf[J]);
             }
             // NCH == 1: that chunk is a whole tile, whose residual operand is requested with it
-            if constexpr (kAhead) request_residual(lc.y, lc.x, rv[J]);
+            if constexpr (kAhead) request_residual(pix_y(lc), pix_x(lc), rv[J]);
         }
         advance(lc);
         int (*rcur)[NW] = rv[kAhead ? I : 0];
@@ -930,7 +981,7 @@ conv3x3_mfma_f4_kernel(
             }
         } else {
             if constexpr (kRes) {
-                if (cc.chunk == 0) request_residual(cc.y, cc.x, rcur);
+                if (cc.chunk == 0) request_residual(pix_y(cc), pix_x(cc), rcur);
             }
             compute_chunk(cc.chunk, buf[I], msk[I], fused, buf[J], nsoff);
         }
@@ -986,7 +1037,7 @@ TensorBytes tensor_bytes(const BgemmParams& p) {
     TensorBytes t;
     t.act = 4LL * p.H * p.W * p.cw * p.B;
     t.rin = p.res_in != nullptr ? 4 * res_words((long long)p.PH * p.PW * (p.res_pool ? 4 : 1), p.res_in_ch, p.res_in_fmt) : 0;
-    t.rout = p.res_out != nullptr ? 4 * res_words((long long)p.PH * p.PW, p.N, p.res_out_fmt) : 0;
+    t.rout = p.res_out != nullptr ? 4 * res_words((long long)p.PH * p.PW / (p.res_out_pool ? 4 : 1), p.N, p.res_out_fmt) : 0;
     t.bits = 4LL * p.OH * p.OW * p.bits_pix_stride;
     if (p.mode == EPI_RAW) {  // the int32 output takes the place of the saved residual
         const long long last = ((long long)p.PH * p.PW - 1) * p.raw_pix_stride + (long long)(p.B - 1) * p.raw_b_stride + p.N;
@@ -996,7 +1047,7 @@ TensorBytes tensor_bytes(const BgemmParams& p) {
     return t;
 }
 
-template <int SPT, int RM, int MT, int NT, int RF, bool POOL, bool FULLT>
+template <int SPT, int RM, int MT, int NT, int RF, int WIN, bool FULLT>
 int launch_f(const BgemmParams& p, hipStream_t stream) {
     constexpr int NQ = 9 * SPT;
     constexpr int kWaves = waves_of(SPT, NT), kThreads = 64 * kWaves;
@@ -1011,7 +1062,7 @@ int launch_f(const BgemmParams& p, hipStream_t stream) {
     if (int rc = device_info(&dev, &cus)) return rc;
     int resident = resident_on[dev].load(std::memory_order_acquire);
     if (resident == 0) {
-        const void* fn = reinterpret_cast<const void*>(&conv3x3_mfma_f4_kernel<SPT, RM, MT, NT, RF, POOL, FULLT>);
+        const void* fn = reinterpret_cast<const void*>(&conv3x3_mfma_f4_kernel<SPT, RM, MT, NT, RF, WIN, FULLT>);
         if (int rc = check_hip(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes),
                                "hipFuncSetAttribute(MaxDynamicSharedMemorySize)"))
             return rc;
@@ -1024,7 +1075,8 @@ int launch_f(const BgemmParams& p, hipStream_t stream) {
     }
     const int n_groups = (p.N + 32 * NT - 1) / (32 * NT);
     const int b_groups = (p.B + 32 * MT - 1) / (32 * MT);
-    const int quads = ((POOL ? p.OH * p.OW : p.PH * p.PW) + kWaves - 1) / kWaves;  // items per wave of a pixel stream
+    const int items = WIN != WIN_NONE ? (p.PH / 2) * (p.PW / 2) : p.PH * p.PW;  // pixels, or 2x2 windows of them
+    const int quads = (items + kWaves - 1) / kWaves;  // items per wave of a pixel stream
     // Persistent workgroups, all resident at once: two per CU (three for residual layers), fewer
     // when registers or LDS hold fewer.  Measured on every layer of ResNet-18 at batch 256: more, shorter-lived
     // workgroups stage the weights more often and lose; and a grid even slightly larger than the resident slots
@@ -1045,9 +1097,9 @@ int launch_f(const BgemmParams& p, hipStream_t stream) {
     const TensorBytes tb = tensor_bytes(p);
     if (blocks > 0x7fffffffLL || b_groups > 65535 || best > 65535) return fail(TCBNN_EINVAL, "conv3x3: grid too large");
     // a wave's stride over the work items, split into rows and columns once here instead of in every wave
-    const int roww = POOL ? p.OW : p.PW, dpi = best * kWaves;
+    const int roww = WIN != WIN_NONE ? p.PW / 2 : p.PW, dpi = best * kWaves;
     const int dy = dpi / roww, dx = dpi % roww, dxs = (dx + dy) % roww;
-    hipLaunchKernelGGL((conv3x3_mfma_f4_kernel<SPT, RM, MT, NT, RF, POOL, FULLT>),
+    hipLaunchKernelGGL((conv3x3_mfma_f4_kernel<SPT, RM, MT, NT, RF, WIN, FULLT>),
                        dim3((unsigned)n_groups, (unsigned)b_groups, (unsigned)best), dim3(kThreads), lds_bytes,
                        stream, p, p.act, p.wgt, p.bn, p.res_in, RM == RM_RAW ? p.out_i32 : p.res_out, res_lim, p.res_out_fmt,
                        (unsigned)tb.act, (unsigned)tb.rin, (unsigned)tb.rout, (unsigned)tb.bits, n_groups, b_groups, best,
@@ -1057,14 +1109,17 @@ int launch_f(const BgemmParams& p, hipStream_t stream) {
 }
 
 // Every channel tile of the launch full, and the residual limit on a tile boundary?  (see FULLT at the kernel)
-template <int SPT, int RM, int MT, int NT, int RF, bool POOL>
+template <int SPT, int RM, int MT, int NT, int RF, int WIN>
 int launch_t(const BgemmParams& p, hipStream_t stream) {
     const int res_lim = p.res_in != nullptr ? std::min(std::min(p.res_limit, p.res_in_ch), p.N) : 0;
     // (with the int32 output, that instantiation also stores whole 128-bit words: the output must be aligned for them)
     const bool raw_ok = RM != RM_RAW || (p.raw_pix_stride % 4 == 0 && p.raw_b_stride % 4 == 0 &&
                                          (reinterpret_cast<uintptr_t>(p.out_i32) & 15) == 0);
-    if (p.N % (32 * NT) == 0 && res_lim % 32 == 0 && raw_ok) return launch_f<SPT, RM, MT, NT, RF, POOL, true>(p, stream);
-    return launch_f<SPT, RM, MT, NT, RF, POOL, false>(p, stream);
+    if (p.N % (32 * NT) == 0 && res_lim % 32 == 0 && raw_ok) return launch_f<SPT, RM, MT, NT, RF, WIN, true>(p, stream);
+    if constexpr (WIN == WIN_MAXSAVE)  // (conv3x3_mfma_applicable admits the window maximum on full tiles only)
+        return fail(TCBNN_EUNSUPPORTED, "conv3x3: pooled residual save needs full channel tiles");
+    else
+        return launch_f<SPT, RM, MT, NT, RF, WIN, false>(p, stream);
 }
 
 // Which instantiation serves a layer.  Measured on ResNet-18 and VGG-16 at batch 256 (10 launches back to back):
@@ -1077,7 +1132,7 @@ int launch_t(const BgemmParams& p, hipStream_t stream) {
 // and from Cin = 384 on (the activation ring of two image tiles no longer fits next to two channel tiles'
 // accumulators).
 struct Pick {
-    int rm, mt, nt, r16, pool;  // r16: TCBNN_RES_* format of the injected residual
+    int rm, mt, nt, r16, win;  // r16: TCBNN_RES_* format of the injected residual; win: WIN_*
 };
 constexpr int pick_nt(int spt, int rm) {
     return rm == RM_POOLED ? (spt >= 6 ? 1 : 2) : (rm == RM_RAW ? (spt >= 3 && spt < 8 ? 1 : 2) : 2);
@@ -1093,7 +1148,7 @@ Pick pick(const BgemmParams& p) {
     const int fmt = p.res_in != nullptr ? p.res_in_fmt : TCBNN_RES_I32;
     // (a pooled int32 source keeps one channel tile per wave: four times sixteen words per tile and lane spilled)
     const int nt = rm == RM_POOLED && fmt == TCBNN_RES_I32 ? 1 : pick_nt(p.cw / 2, rm);
-    return {rm, pick_mt(p.cw / 2, rm), nt, fmt, p.pool_h == 2};
+    return {rm, pick_mt(p.cw / 2, rm), nt, fmt, p.pool_h == 2 ? WIN_ORPOOL : (p.res_out_pool ? WIN_MAXSAVE : WIN_NONE)};
 }
 
 template <int SPT>
@@ -1101,22 +1156,27 @@ int launch_m(const BgemmParams& p, hipStream_t stream) {
     const Pick k = pick(p);
     switch (k.rm) {
         case RM_NONE:
-            return k.pool ? launch_t<SPT, RM_NONE, pick_mt(SPT, RM_NONE), pick_nt(SPT, RM_NONE), TCBNN_RES_I32, true>(p, stream)
-                          : launch_t<SPT, RM_NONE, pick_mt(SPT, RM_NONE), pick_nt(SPT, RM_NONE), TCBNN_RES_I32, false>(p, stream);
+            return k.win == WIN_ORPOOL
+                       ? launch_t<SPT, RM_NONE, pick_mt(SPT, RM_NONE), pick_nt(SPT, RM_NONE), TCBNN_RES_I32, WIN_ORPOOL>(p, stream)
+                       : launch_t<SPT, RM_NONE, pick_mt(SPT, RM_NONE), pick_nt(SPT, RM_NONE), TCBNN_RES_I32, WIN_NONE>(p, stream);
         case RM_RAW:
-            return launch_t<SPT, RM_RAW, pick_mt(SPT, RM_RAW), pick_nt(SPT, RM_RAW), TCBNN_RES_I32, false>(p, stream);
+            return launch_t<SPT, RM_RAW, pick_mt(SPT, RM_RAW), pick_nt(SPT, RM_RAW), TCBNN_RES_I32, WIN_NONE>(p, stream);
         case RM_PLAIN:
+            if (k.win == WIN_MAXSAVE)  // (a narrow injected residual: conv3x3_mfma_applicable)
+                return k.r16 == TCBNN_RES_I12
+                           ? launch_t<SPT, RM_PLAIN, pick_mt(SPT, RM_PLAIN), pick_nt(SPT, RM_PLAIN), TCBNN_RES_I12, WIN_MAXSAVE>(p, stream)
+                           : launch_t<SPT, RM_PLAIN, pick_mt(SPT, RM_PLAIN), pick_nt(SPT, RM_PLAIN), TCBNN_RES_I16, WIN_MAXSAVE>(p, stream);
             return k.r16 == TCBNN_RES_I12
-                       ? launch_t<SPT, RM_PLAIN, pick_mt(SPT, RM_PLAIN), pick_nt(SPT, RM_PLAIN), TCBNN_RES_I12, false>(p, stream)
+                       ? launch_t<SPT, RM_PLAIN, pick_mt(SPT, RM_PLAIN), pick_nt(SPT, RM_PLAIN), TCBNN_RES_I12, WIN_NONE>(p, stream)
                        : (k.r16 == TCBNN_RES_I16
-                              ? launch_t<SPT, RM_PLAIN, pick_mt(SPT, RM_PLAIN), pick_nt(SPT, RM_PLAIN), TCBNN_RES_I16, false>(p, stream)
-                              : launch_t<SPT, RM_PLAIN, pick_mt(SPT, RM_PLAIN), pick_nt(SPT, RM_PLAIN), TCBNN_RES_I32, false>(p, stream));
+                              ? launch_t<SPT, RM_PLAIN, pick_mt(SPT, RM_PLAIN), pick_nt(SPT, RM_PLAIN), TCBNN_RES_I16, WIN_NONE>(p, stream)
+                              : launch_t<SPT, RM_PLAIN, pick_mt(SPT, RM_PLAIN), pick_nt(SPT, RM_PLAIN), TCBNN_RES_I32, WIN_NONE>(p, stream));
         default:
             return k.r16 == TCBNN_RES_I12
-                       ? launch_t<SPT, RM_POOLED, pick_mt(SPT, RM_POOLED), pick_nt(SPT, RM_POOLED), TCBNN_RES_I12, false>(p, stream)
+                       ? launch_t<SPT, RM_POOLED, pick_mt(SPT, RM_POOLED), pick_nt(SPT, RM_POOLED), TCBNN_RES_I12, WIN_NONE>(p, stream)
                        : (k.r16 == TCBNN_RES_I16
-                              ? launch_t<SPT, RM_POOLED, pick_mt(SPT, RM_POOLED), pick_nt(SPT, RM_POOLED), TCBNN_RES_I16, false>(p, stream)
-                              : launch_t<SPT, RM_POOLED, pick_mt(SPT, RM_POOLED), 1, TCBNN_RES_I32, false>(p, stream));
+                              ? launch_t<SPT, RM_POOLED, pick_mt(SPT, RM_POOLED), pick_nt(SPT, RM_POOLED), TCBNN_RES_I16, WIN_NONE>(p, stream)
+                              : launch_t<SPT, RM_POOLED, pick_mt(SPT, RM_POOLED), 1, TCBNN_RES_I32, WIN_NONE>(p, stream));
     }
 }
 
@@ -1141,7 +1201,16 @@ bool conv3x3_mfma_applicable(const BgemmParams& p) {
     const bool mode_ok = (p.mode == EPI_THRESH && p.nan_bit == 1) ||
                          (p.mode == EPI_RAW && p.pool_h == 1 && p.pool_w == 1 && p.res_in == nullptr &&
                           p.res_out == nullptr && p.raw_pix_stride >= 0 && p.raw_b_stride >= 0);
-    return p.R == 3 && p.S == 3 && pool_ok && centre_ok && mode_ok &&
+    // the saved residual as the maximum over 2x2 windows: whole windows, every channel tile full and entirely below or
+    // above the injection limit, and sums that the epilogue handles as 16-bit pairs (a narrow injected residual, a
+    // 12- or 16-bit output)
+    const int res_lim = p.res_in != nullptr ? std::min(std::min(p.res_limit, p.res_in_ch), p.N) : 0;
+    const bool psave_ok = !p.res_out_pool ||
+                          (p.res_out != nullptr && p.res_in != nullptr && !p.res_pool && p.pool_h == 1 && p.pool_w == 1 &&
+                           p.PH % 2 == 0 && p.PW % 2 == 0 && p.mode == EPI_THRESH && p.N % 64 == 0 && res_lim % 32 == 0 &&
+                           (p.res_in_fmt == TCBNN_RES_I12 || p.res_in_fmt == TCBNN_RES_I16) &&
+                           (p.res_out_fmt == TCBNN_RES_I12 || p.res_out_fmt == TCBNN_RES_I16));
+    return p.R == 3 && p.S == 3 && pool_ok && centre_ok && mode_ok && psave_ok &&
            p.ksplit <= 1 && filter_has_fragments(3, 3, 32 * p.cw) && p.k_tap == 32 * p.cw &&
            (long long)p.PH * p.PW < (1 << 24) && within_2gib(p);
 }
@@ -1152,8 +1221,8 @@ void conv3x3_mfma_kernel_name(const BgemmParams& p, char* buf, size_t len) {
     const bool raw_ok = k.rm != RM_RAW || (p.raw_pix_stride % 4 == 0 && p.raw_b_stride % 4 == 0 &&
                                            (reinterpret_cast<uintptr_t>(p.out_i32) & 15) == 0);
     const bool full = p.N % (32 * k.nt) == 0 && res_lim % 32 == 0 && raw_ok;
-    snprintf(buf, len, "conv3x3_mfma_f4_kernel<%d, %d, %d, %d, %d, %s, %s>", p.cw / 2, k.rm, k.mt, k.nt, k.r16,
-             k.pool ? "true" : "false", full ? "true" : "false");
+    snprintf(buf, len, "conv3x3_mfma_f4_kernel<%d, %d, %d, %d, %d, %d, %s>", p.cw / 2, k.rm, k.mt, k.nt, k.r16, k.win,
+             full ? "true" : "false");
 }
 
 int launch_conv3x3_mfma(const BgemmParams& p, hipStream_t stream) {

@@ -117,7 +117,7 @@ using namespace tcbnn;
 
 extern "C" {
 
-int tcbnn_abi_version(void) { return 5; }
+int tcbnn_abi_version(void) { return 6; }
 const char* tcbnn_last_error(void) { return g_err; }
 
 int tcbnn_set_default_variant(int variant) {
@@ -358,13 +358,35 @@ static int conv_problem(const tcbnn_conv128_desc* d, bool launch, BgemmParams* o
         p.res_out = launch ? d->output_residual : some;
         p.res_out_fmt = d->output_residual_format;
     }
+    if (d->output_residual_pool != 0) {
+        TCBNN_REQUIRE(d->output_residual_pool == 2, "conv128: output_residual_pool is 0 or 2");
+        TCBNN_REQUIRE(d->save_residual, "conv128: output_residual_pool without save_residual");
+        p.res_out_pool = 1;
+    }
     return TCBNN_OK;
+}
+
+// The saved residual as the maximum over 2x2 windows exists in the persistent 3x3 matrix-core kernel only.
+static bool pooled_save_served(const BgemmParams& p, int variant) {
+    return resolve_variant(variant) == TCBNN_VARIANT_MFMA_F4 && conv3x3_mfma_applicable(p);
 }
 
 int tcbnn_conv128_forward(const tcbnn_conv128_desc* d, void* stream) {
     BgemmParams p;
     if (int rc = conv_problem(d, true, &p)) return rc;
+    if (p.res_out_pool && !pooled_save_served(p, d->variant))
+        return fail(TCBNN_EUNSUPPORTED, "conv128: output_residual_pool is not available for this layer "
+                                        "(tcbnn_conv128_pooled_save_supported tells)");
     return run_bgemm(p, d->variant, (hipStream_t)stream);
+}
+
+int tcbnn_conv128_pooled_save_supported(const tcbnn_conv128_desc* d) {
+    if (d == nullptr || !d->save_residual) return 0;
+    tcbnn_conv128_desc own = *d;
+    own.output_residual_pool = 2;
+    BgemmParams p;
+    if (conv_problem(&own, false, &p) != TCBNN_OK) return 0;
+    return pooled_save_served(p, d->variant) ? 1 : 0;
 }
 
 static int kernel_name(const BgemmParams& p, int variant, char* buf, size_t len) {

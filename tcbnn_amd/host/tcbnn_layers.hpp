@@ -131,8 +131,19 @@ class ConfigSource {
 //   bound:    upper bound of |value| (first layer: from the actual input; each bit convolution
 //             adds Cin*R*S), INT32_MAX when unknown;
 //   format:   TCBNN_RES_I16 when the bound proves that 16 bits hold every value, else int32.
+// The registry's copy also records who reads the tensor, which decides whether its producer may store only the
+// maximum over 2x2 windows of pixels (a quarter of the bytes written and read; tcbnn_conv128_desc's
+// output_residual_pool): how often get_output_residual_gpu() handed the pointer out, how many Conv128 consumers
+// registered with residual_pool, how many other consumers of this library, whether the full tensor was ever asked
+// for, and what the buffer holds since the producer's last forward().  The maximum alone is stored when every
+// hand-out went to a pooling consumer (so that nobody else can be reading the tensor), nobody asked for the full
+// tensor, and the producer's kernel can do it (will_pool).
 struct ResidualInfo {
     int channels, bound, format;
+    int handed_out, pool_consumers, other_consumers;
+    bool observed, pooled, written;
+    bool (*will_pool)(void*);  // the producer's decision for its next forward(); NULL: never
+    void* producer;
 };
 inline std::map<const void*, ResidualInfo>& residual_registry() {
     static std::map<const void*, ResidualInfo> reg;
@@ -140,8 +151,29 @@ inline std::map<const void*, ResidualInfo>& residual_registry() {
 }
 // (the narrowest format that is exact for the bound: 12 bits up to 2047 for even batches, 16 bits up to 32767)
 inline ResidualInfo make_residual_info(int channels, int bound, int batch) {
-    ResidualInfo info = {channels, bound, tcbnn_residual_format_narrowest(bound, batch)};
+    ResidualInfo info = {channels, bound, tcbnn_residual_format_narrowest(bound, batch), 0, 0, 0, false, false, false, NULL,
+                         NULL};
     return info;
+}
+inline ResidualInfo* find_residual(const void* gpu) {
+    std::map<const void*, ResidualInfo>::iterator it = residual_registry().find(gpu);
+    return it != residual_registry().end() ? &it->second : NULL;
+}
+// a layer of this library starts (sign = +1) or stops (-1) reading the saved residual at `gpu`
+inline void register_residual_consumer(const void* gpu, bool pools, int sign) {
+    ResidualInfo* u = find_residual(gpu);
+    if (u != NULL) (pools ? u->pool_consumers : u->other_consumers) += sign;
+}
+inline int* hand_out_residual(int* gpu) {
+    ResidualInfo* u = find_residual(gpu);
+    if (u != NULL) u->handed_out += 1;
+    return gpu;
+}
+// does the buffer hold (after its producer's forward) the maximum over 2x2 windows instead of the full tensor?
+inline bool residual_holds_window_maximum(const void* gpu) {
+    const ResidualInfo* u = find_residual(gpu);
+    if (u == NULL) return false;
+    return u->written ? u->pooled : (u->will_pool != NULL && u->will_pool(u->producer));
 }
 
 }  // namespace tcbnn_host
@@ -698,12 +730,17 @@ class Conv128LayerParam {  // param.h:872-1065
 
     void set_input_gpu(uin32* input_gpu) { this->input_gpu = input_gpu; }
     void set_input_residual_gpu(int* input_residual_gpu) {
+        if (inject_residual) {
+            tcbnn_host::register_residual_consumer(this->input_residual_gpu, residual_pool, -1);
+            tcbnn_host::register_residual_consumer(input_residual_gpu, residual_pool, +1);
+        }
         this->input_residual_gpu = input_residual_gpu;
         std::map<const void*, tcbnn_host::ResidualInfo>& reg = tcbnn_host::residual_registry();
         std::map<const void*, tcbnn_host::ResidualInfo>::iterator it = reg.find(input_residual_gpu);
         // a residual that no layer of this library produced: int32 with the consumer's channel
         // limit and no known bound
-        const tcbnn_host::ResidualInfo foreign = {residual_channels, INT32_MAX, TCBNN_RES_I32};
+        tcbnn_host::ResidualInfo foreign = tcbnn_host::make_residual_info(residual_channels, INT32_MAX, batch);
+        foreign.format = TCBNN_RES_I32;
         input_residual_info = it != reg.end() ? it->second : foreign;
         input_residual_channels = input_residual_info.channels;
         if (output_residual_gpu != NULL &&
@@ -747,14 +784,36 @@ class Conv128LayerParam {  // param.h:872-1065
                                                                                       filter_width, injected)
                                                           : INT32_MAX, batch);
             SAFE_ALOC_GPU(output_residual_gpu, residual_bytes());
+            residual_info.will_pool = &Conv128LayerParam::will_pool_thunk;
+            residual_info.producer = this;
             tcbnn_host::residual_registry()[output_residual_gpu] = residual_info;
         }
         CHECK_NULL_POINTER(input_gpu);
         return this;
     }
     uin32* get_output_gpu() { return this->output_gpu; }
-    int* get_output_residual_gpu() { return this->output_residual_gpu; }
+    // (every hand-out is counted: see ResidualInfo)
+    int* get_output_residual_gpu() { return tcbnn_host::hand_out_residual(this->output_residual_gpu); }
+    // Store only the 2x2 maximum of the saved residual in the next forward()?  (see ResidualInfo)
+    bool pooled_save_now() {
+        const tcbnn_host::ResidualInfo* u = tcbnn_host::find_residual(output_residual_gpu);
+        if (u == NULL || u->observed || u->other_consumers != 0 || u->pool_consumers == 0 ||
+            u->handed_out != u->pool_consumers)
+            return false;
+        const tcbnn_conv128_desc d = describe(false);
+        return tcbnn_conv128_pooled_save_supported(&d) == 1;
+    }
+    static bool will_pool_thunk(void* self) { return static_cast<Conv128LayerParam*>(self)->pooled_save_now(); }
     void forward(hipStream_t stream = 0) {
+        const tcbnn_conv128_desc d = describe(true);
+        TCBNN_SAFE_CALL(tcbnn_conv128_forward(&d, stream));
+        tcbnn_host::ResidualInfo* u = tcbnn_host::find_residual(output_residual_gpu);
+        if (u != NULL) {
+            u->pooled = d.output_residual_pool == 2;
+            u->written = true;
+        }
+    }
+    tcbnn_conv128_desc describe(bool decide_pool) {
         tcbnn_conv128_desc d;
         memset(&d, 0, sizeof(d));
         d.input = input_gpu;
@@ -779,12 +838,14 @@ class Conv128LayerParam {  // param.h:872-1065
         d.save_residual = save_residual ? 1 : 0;
         d.inject_residual = inject_residual ? 1 : 0;
         d.residual_channels = residual_channels;
-        d.residual_pool = residual_pool ? 1 : 0;
+        // (a source that already holds the 2x2 maximum is injected as it is)
+        d.residual_pool = residual_pool && !(inject_residual && tcbnn_host::residual_holds_window_maximum(input_residual_gpu)) ? 1 : 0;
         d.input_residual_channels = input_residual_channels;
         d.variant = variant;
         d.input_residual_format = input_residual_info.format;
         d.output_residual_format = residual_info.format;
-        TCBNN_SAFE_CALL(tcbnn_conv128_forward(&d, stream));
+        d.output_residual_pool = decide_pool && pooled_save_now() ? 2 : 0;
+        return d;
     }
     // Reference-layout neighbours.  Input bits [H][W][PAD8(B)/8][STEP128(C)][8][4] (read at kernel.cuh:741-749) and
     // an injected residual int32 [Hr][Wr][PAD8(B)][PAD128(residual_channels)] (kernel.cuh:770-791; Hr x Wr is the
@@ -822,8 +883,15 @@ class Conv128LayerParam {  // param.h:872-1065
                                                         batch, output_channels, stream));
         return output_fmt_gpu;
     }
+    // (The full tensor is asked for: from now on it is what forward() saves, and if the buffer holds the 2x2
+    // maximum from the last forward(), the layer is run again first; its inputs are still in place.)
     int* get_output_residual_gpu_reference(hipStream_t stream = 0) {
         CHECK_NULL_POINTER(output_residual_gpu);
+        tcbnn_host::ResidualInfo* u = tcbnn_host::find_residual(output_residual_gpu);
+        if (u != NULL) {
+            u->observed = true;
+            if (u->pooled) forward(stream);
+        }
         if (output_residual_ref_gpu == NULL)
             SAFE_ALOC_GPU(output_residual_ref_gpu,
                           (size_t)buf_height * buf_width * PAD8(batch) * PAD128(output_channels) * sizeof(int));
@@ -867,6 +935,8 @@ class Conv128LayerParam {  // param.h:872-1065
         SAFE_FREE_GPU(output_gpu);
         SAFE_FREE_GPU(filter_gpu);
         SAFE_FREE_GPU(bn_gpu);
+        if (inject_residual) tcbnn_host::register_residual_consumer(input_residual_gpu, residual_pool, -1);
+        input_residual_gpu = NULL;
         if (output_residual_gpu != NULL) tcbnn_host::residual_registry().erase(output_residual_gpu);
         SAFE_FREE_GPU(output_residual_gpu);
         SAFE_FREE_GPU(input_own_gpu);
@@ -937,8 +1007,7 @@ class Pool128LayerParam {
         strncpy(name, _name, 8);
         output_height = buf_height = tcbnn_pool_out(input_height, window, stride, padding);
         output_width = buf_width = tcbnn_pool_out(input_width, window, stride, padding);
-        residual_info.channels = 0;
-        residual_info.bound = 0;
+        residual_info = tcbnn_host::make_residual_info(0, 0, _batch);
         residual_info.format = TCBNN_RES_I32;
     }
     ~Pool128LayerParam() { release(); }
@@ -951,8 +1020,14 @@ class Pool128LayerParam {
             input_residual_gpu = _input_residual_gpu;
             std::map<const void*, tcbnn_host::ResidualInfo>& reg = tcbnn_host::residual_registry();
             std::map<const void*, tcbnn_host::ResidualInfo>::iterator it = reg.find(input_residual_gpu);
-            const tcbnn_host::ResidualInfo foreign = {output_channels, INT32_MAX, TCBNN_RES_I32};
-            residual_info = it != reg.end() ? it->second : foreign;  // a maximum keeps bound and format
+            tcbnn_host::ResidualInfo foreign = tcbnn_host::make_residual_info(output_channels, INT32_MAX, batch);
+            foreign.format = TCBNN_RES_I32;
+            const int keep_bound = it != reg.end() ? it->second.bound : foreign.bound;
+            const int keep_format = it != reg.end() ? it->second.format : foreign.format;
+            tcbnn_host::register_residual_consumer(input_residual_gpu, false, +1);  // (reads the full tensor)
+            residual_info = foreign;  // a maximum keeps bound and format
+            residual_info.bound = keep_bound;
+            residual_info.format = keep_format;
             residual_info.channels = output_channels;
             SAFE_ALOC_GPU(output_residual_gpu, tcbnn_residual_bytes(output_height, output_width, output_channels,
                                                                     batch, residual_info.format));
@@ -1020,6 +1095,7 @@ class AvgPoolFcLayerParam {
         std::map<const void*, tcbnn_host::ResidualInfo>& reg = tcbnn_host::residual_registry();
         std::map<const void*, tcbnn_host::ResidualInfo>::iterator it = reg.find(input_residual_gpu);
         if (it != reg.end()) input_residual_info = it->second;
+        tcbnn_host::register_residual_consumer(input_residual_gpu, false, +1);  // (reads the full tensor)
         SAFE_ALOC_HOST(weight, weight_size() * sizeof(float));
         config_file.read(weight, weight_size());
         SAFE_ALOC_GPU(weight_gpu, weight_size() * sizeof(float));

@@ -88,7 +88,55 @@ def _residual_buffer(channels, height, width, batch, bound, force_format=None):
     buf = DeviceBuffer(lib.tcbnn_residual_bytes(height, width, channels, batch, fmt))
     buf.channels, buf.height, buf.width, buf.batch = channels, height, width, batch
     buf.bound, buf.format = bound, fmt
+    # Who reads the tensor decides whether its producer may store only the maximum over 2x2 windows of pixels
+    # (_SavedResidualUse): how often the pointer was handed out, how many Conv128 consumers registered with
+    # residual_pool, how many other consumers, whether the full tensor was ever asked for, and what the buffer
+    # holds since the producer's last forward().
+    buf.handed_out = buf.pool_consumers = buf.other_consumers = 0
+    buf.observed = buf.pooled = buf.written = False
+    buf.producer = None
     return buf
+
+
+def _register_residual_consumer(buf, pools, sign=1):
+    """A layer of this library starts (sign = +1) or stops (-1) reading the saved residual `buf`."""
+    if buf is not None and hasattr(buf, "pool_consumers"):
+        if pools:
+            buf.pool_consumers += sign
+        else:
+            buf.other_consumers += sign
+
+
+def _residual_holds_window_maximum(buf):
+    """Does `buf` hold (after its producer's forward) the maximum over 2x2 windows instead of the full tensor?"""
+    if buf is None or getattr(buf, "producer", None) is None:
+        return False
+    return buf.pooled if buf.written else buf.producer._pooled_save_now()
+
+
+def _unpack_residual(buf, P, Q, O, B):
+    """A residual tensor of P x Q pixels in the engine layout `buf.format` -> int32 [P][Q][B][O]."""
+    if buf.format == _lib.RES_I12:
+        # groups of 16 channels; per pixel and group the words w0..w3 of every image, then w4, w5 of every image;
+        # value e sits at bits 12e..12e+11 of the 192-bit string w0..w5 (two's complement)
+        G = (O + 15) // 16
+        raw = buf.to_numpy(np.uint32, (P, Q, G, 6 * B)).astype(np.uint64)
+        words = np.concatenate([raw[..., :4 * B].reshape(P, Q, G, B, 4), raw[..., 4 * B:].reshape(P, Q, G, B, 2)],
+                               axis=-1)
+        vals = np.empty((P, Q, G, B, 16), np.int64)
+        for e in range(16):
+            k, sh = (12 * e) >> 5, (12 * e) & 31
+            v = words[..., k] >> np.uint64(sh)
+            if sh > 20:
+                v = v | (words[..., k + 1] << np.uint64(32 - sh))
+            v = (v & np.uint64(0xfff)).astype(np.int64)
+            vals[..., e] = (v ^ 0x800) - 0x800
+        return np.ascontiguousarray(vals.transpose(0, 1, 3, 2, 4).reshape(P, Q, B, G * 16)[..., :O].astype(np.int32))
+    # engine layouts: int32 [P][Q][ceil(O/4)][B][4] or int16 [P][Q][ceil(O/8)][B][8]
+    grp, dt = (8, np.int16) if buf.format == _lib.RES_I16 else (4, np.int32)
+    ng = (O + grp - 1) // grp
+    eng = buf.to_numpy(dt, (P, Q, ng, B, grp))
+    return np.ascontiguousarray(eng.transpose(0, 1, 3, 2, 4).reshape(P, Q, B, ng * grp)[..., :O].astype(np.int32))
 
 
 class _ReferenceLayoutIO:
@@ -147,6 +195,7 @@ class _ReferenceLayoutIO:
         src = self.output_residual_gpu
         if src is None:
             raise _lib.TcbnnError("Error: NULL pointer (output_residual_gpu)")
+        self._want_full_residual(stream)
         ref = self._ref_buf("res_out", 4 * self.buf_height * self.buf_width * PAD8(self.batch)
                             * PAD128(self.output_channels))
         check(lib.tcbnn_residual_to_reference(src.ptr, ref.ptr, self.buf_height, self.buf_width, self.batch,
@@ -409,35 +458,43 @@ class _ConvGeometry(_ReferenceLayoutIO):
         return self.output_gpu
 
     def get_output_residual_gpu(self):
+        """The saved residual, for a consumer's initialize().  (Every hand-out is counted: as long as each one
+        is matched by a Conv128 consumer that registers with residual_pool, nobody else can be reading the
+        tensor, and the producer may store its 2x2 maximum alone.)"""
+        if self.output_residual_gpu is not None:
+            self.output_residual_gpu.handed_out += 1
         return self.output_residual_gpu
+
+    def _pooled_save_now(self):
+        return False  # (only Conv128 layers can store the window maximum)
+
+    def _want_full_residual(self, stream=None):
+        """The full P x Q tensor is asked for: from now on it is what forward() saves, and if the buffer holds
+        the 2x2 maximum from the last forward(), the layer is run again (its inputs are still in place)."""
+        buf = self.output_residual_gpu
+        buf.observed = True
+        if buf.pooled:
+            self.forward(stream)
 
     def download_residual(self):
         """Saved residual as int32 [P][Q][B][O] (host transpose of the engine's layouts)."""
-        P, Q, O, B = self.buf_height, self.buf_width, self.output_channels, self.batch
-        if self.output_residual_gpu.format == _lib.RES_I12:
-            # groups of 16 channels; per pixel and group the words w0..w3 of every image, then w4, w5 of every image;
-            # value e sits at bits 12e..12e+11 of the 192-bit string w0..w5 (two's complement)
-            G = (O + 15) // 16
-            raw = self.output_residual_gpu.to_numpy(np.uint32, (P, Q, G, 6 * B)).astype(np.uint64)
-            words = np.concatenate([raw[..., :4 * B].reshape(P, Q, G, B, 4), raw[..., 4 * B:].reshape(P, Q, G, B, 2)],
-                                   axis=-1)
-            vals = np.empty((P, Q, G, B, 16), np.int64)
-            for e in range(16):
-                k, sh = (12 * e) >> 5, (12 * e) & 31
-                v = words[..., k] >> np.uint64(sh)
-                if sh > 20:
-                    v = v | (words[..., k + 1] << np.uint64(32 - sh))
-                v = (v & np.uint64(0xfff)).astype(np.int64)
-                vals[..., e] = (v ^ 0x800) - 0x800
-            return np.ascontiguousarray(vals.transpose(0, 1, 3, 2, 4).reshape(P, Q, B, G * 16)[..., :O].astype(np.int32))
-        # engine layouts: int32 [P][Q][ceil(O/4)][B][4] or int16 [P][Q][ceil(O/8)][B][8]
-        grp, dt = (8, np.int16) if self.output_residual_gpu.format == _lib.RES_I16 else (4, np.int32)
-        ng = (O + grp - 1) // grp
-        eng = self.output_residual_gpu.to_numpy(dt, (P, Q, ng, B, grp))
-        return np.ascontiguousarray(eng.transpose(0, 1, 3, 2, 4).reshape(P, Q, B, ng * grp)[..., :O].astype(np.int32))
+        self._want_full_residual()
+        _lib.device_synchronize()
+        return _unpack_residual(self.output_residual_gpu, self.buf_height, self.buf_width, self.output_channels,
+                                self.batch)
+
+    def download_saved_residual(self):
+        """What the buffer holds since the last forward(), without asking for anything: (int32 [P'][Q'][B][O],
+        pooled) with P' x Q' = P/2 x Q/2 and every value the maximum over a 2x2 window when `pooled`."""
+        buf = self.output_residual_gpu
+        _lib.device_synchronize()
+        k = 2 if buf.pooled else 1
+        return _unpack_residual(buf, self.buf_height // k, self.buf_width // k, self.output_channels, self.batch), \
+            buf.pooled
 
     def download_residual_reference(self):
         """Saved residual in the reference layout int32 [P][Q][PAD8(B)][PAD128(O)]."""
+        self._want_full_residual()
         shape = (self.buf_height, self.buf_width, PAD8(self.batch), PAD128(self.output_channels))
         tmp = DeviceBuffer(4 * int(np.prod(shape)))
         check(lib.tcbnn_residual_to_reference(self.output_residual_gpu.ptr, tmp.ptr, self.buf_height,
@@ -638,6 +695,9 @@ class Conv128LayerParam(_ConvGeometry):
                 lib.tcbnn_conv_residual_bound(self.input_channels, self.filter_height, self.filter_width,
                                               min(input_residual_gpu.bound, _lib.INT32_MAX // 4)) > out.bound:
             raise _lib.TcbnnError("injected residual exceeds the bound the saved residual's format was chosen for")
+        if self.inject_residual:
+            _register_residual_consumer(self.input_residual_gpu, self.residual_pool, -1)
+            _register_residual_consumer(input_residual_gpu, self.residual_pool, +1)
         self.input_residual_gpu = input_residual_gpu
 
     def initialize(self, config_file, prev_layer_gpu, input_residual_gpu=None):
@@ -669,12 +729,27 @@ class Conv128LayerParam(_ConvGeometry):
                                                   injected) if injected < _lib.INT32_MAX else _lib.INT32_MAX
             self.output_residual_gpu = _residual_buffer(self.output_channels, self.buf_height, self.buf_width,
                                                         self.batch, bound, self.residual_format)
+            self.output_residual_gpu.producer = self
         if self.input_gpu is None:
             raise _lib.TcbnnError("Error: NULL pointer (input_gpu)")
         return self
 
-    def _desc(self):
+    def _pooled_save_now(self):
+        """Store only the 2x2 maximum of the saved residual?  Yes when that is all anybody reads: every hand-out of
+        the pointer went to a Conv128 layer that injects it with residual_pool, nobody asked for the full tensor,
+        and the kernel that serves this layer can do it."""
+        out = self.output_residual_gpu
+        if out is None or out.observed or out.other_consumers or not out.pool_consumers or \
+                out.handed_out != out.pool_consumers:
+            return False
+        d = self._desc(decide_pool=False)
+        return bool(lib.tcbnn_conv128_pooled_save_supported(C.byref(d)))
+
+    def _desc(self, decide_pool=True):
         rin = self.input_residual_gpu if self.inject_residual else None
+        # a source that holds the 2x2 maximum already is injected as it is
+        pool_source = self.residual_pool and not _residual_holds_window_maximum(rin)
+        pool_out = 2 if decide_pool and self._pooled_save_now() else 0
         return _lib.Conv128Desc(
             self.input_gpu.ptr, self.filter_gpu.ptr, self.bn_gpu.ptr, self.output_gpu.ptr,
             rin.ptr if rin is not None else None,
@@ -682,14 +757,16 @@ class Conv128LayerParam(_ConvGeometry):
             self.input_height, self.input_width, self.input_channels, self.filter_height, self.filter_width,
             self.output_channels, self.batch, self.stride_height, self.stride_width, int(self.padding),
             self.pool_height, self.pool_width, int(self.ahead_fc), int(self.save_residual),
-            int(self.inject_residual), self.residual_channels, int(self.residual_pool),
+            int(self.inject_residual), self.residual_channels, int(pool_source),
             rin.channels if rin is not None else 0, self.variant,
             rin.format if rin is not None else 0,
-            self.output_residual_gpu.format if self.output_residual_gpu is not None else 0)
+            self.output_residual_gpu.format if self.output_residual_gpu is not None else 0, pool_out)
 
     def forward(self, stream=None):
         d = self._desc()
         check(lib.tcbnn_conv128_forward(C.byref(d), _stream_handle(stream)))
+        if self.output_residual_gpu is not None:
+            self.output_residual_gpu.pooled, self.output_residual_gpu.written = d.output_residual_pool == 2, True
 
     def kernel_name(self):
         buf = C.create_string_buffer(128)
@@ -699,6 +776,9 @@ class Conv128LayerParam(_ConvGeometry):
 
     def release(self):
         self._release_ref_bufs()
+        if self.inject_residual:
+            _register_residual_consumer(self.input_residual_gpu, self.residual_pool, -1)
+            self.input_residual_gpu = None
         for b in (self.filter_gpu, self.bn_gpu, self.output_gpu, self.output_residual_gpu):
             if b is not None:
                 b.free()
@@ -732,6 +812,7 @@ class Pool128LayerParam:
             if input_residual_gpu is None:
                 raise _lib.TcbnnError("Error: NULL pointer (input_residual_gpu)")
             self.input_residual_gpu = input_residual_gpu
+            _register_residual_consumer(input_residual_gpu, False)
             # a maximum never exceeds the bound of its operands: same bound, same format
             self.output_residual_gpu = _residual_buffer(self.output_channels, self.output_height, self.output_width,
                                                         self.batch, input_residual_gpu.bound,
@@ -741,8 +822,10 @@ class Pool128LayerParam:
     def get_output_gpu(self):
         return self.output_gpu
 
-    def get_output_residual_gpu(self):
-        return self.output_residual_gpu
+    get_output_residual_gpu = _ConvGeometry.get_output_residual_gpu
+    _pooled_save_now = _ConvGeometry._pooled_save_now
+    _want_full_residual = _ConvGeometry._want_full_residual
+    download_saved_residual = _ConvGeometry.download_saved_residual
 
     def _desc(self):
         rin, rout = self.input_residual_gpu, self.output_residual_gpu
@@ -784,6 +867,7 @@ class AvgPoolFcLayerParam:
         if input_residual_gpu is None:
             raise _lib.TcbnnError("Error: NULL pointer (input_residual_gpu)")
         self.input_residual_gpu = input_residual_gpu
+        _register_residual_consumer(input_residual_gpu, False)
         self.weight = np.array(config_file.launch_array(self.channels * self.out_features), dtype=np.float32)
         self.bias = np.array(config_file.launch_array(self.out_features), dtype=np.float32)
         self.weight_gpu = DeviceBuffer.from_numpy(self.weight)

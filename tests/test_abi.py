@@ -23,11 +23,11 @@ def test_library_exports_every_declared_symbol():
     for s in syms:
         assert hasattr(_lib.lib, s), "libtcbnn_hip.so does not export %s" % s
     assert sorted(_lib.ABI) == syms, "Python binding table and header disagree"
-    assert _lib.lib.tcbnn_abi_version() == 5
+    assert _lib.lib.tcbnn_abi_version() == 6
     # the build entry point refuses a library of another ABI version: it must expect this one
     import inspect
     import __graft_entry__
-    assert "tcbnn_abi_version() == 5" in inspect.getsource(__graft_entry__.build)
+    assert "tcbnn_abi_version() == 6" in inspect.getsource(__graft_entry__.build)
 
 
 def test_geometry_entry_points_match_reference_formulas():

@@ -407,6 +407,119 @@ def _residual_modes(gpu, variant, cin, cout, in_fmt, out_fmt, b, amp=3000):
     layer.release()
 
 
+def _window_maximum(res):
+    """[P][Q][B][O] -> [P/2][Q/2][B][O]: the maximum over non-overlapping 2x2 windows of pixels (kernel.cuh:775-782)."""
+    p, q, b, o = res.shape
+    return res.reshape(p // 2, 2, q // 2, 2, b, o).max(axis=(1, 3))
+
+
+@pytest.mark.parametrize("variant", VARIANTS)
+@pytest.mark.parametrize("b,h,cin,cout,in_fmt,amp,lim", [
+    (64, 8, 64, 64, 2, 100, 64), (70, 6, 128, 128, 1, 3000, 128), (8, 4, 256, 256, 1, 500, 128),
+    (40, 10, 64, 128, 2, 2000, 64), (8, 4, 512, 512, 1, 20000, 512), (24, 6, 192, 64, 2, 50, 32),
+    (40, 4, 384, 128, 1, 900, 96),
+    # not served: odd frame, int32 output (bound above 32767), output channels not a multiple of 64, int32 source
+    (8, 7, 64, 64, 2, 100, 64), (8, 4, 64, 64, 1, 32700, 64), (8, 4, 64, 96, 2, 100, 96), (8, 4, 128, 64, 0, 100, 64)])
+def test_conv128_saved_residual_as_window_maximum(gpu, variant, b, h, cin, cout, in_fmt, amp, lim):
+    """A saved residual whose only reader injects it with residual_pool is stored as its 2x2 maximum (a quarter of
+    the tensor), which that reader then injects as it is.  Same bits and residuals as the reference's order of
+    operations (save the full tensor, kernel.cuh:818-824; take the maximum when reading, kernel.cuh:775-782); the
+    full tensor is still there when somebody asks for it."""
+    r = rng(b * 7 + h + cin + cout)
+    x = rm.pm1(r, (b, h, h, cin))
+    f = rm.pm1(r, (3, 3, cin, cout))
+    bn = r.normal(0, 20, cout).astype(np.float32)
+    src = r.integers(-amp, amp + 1, size=(h, h, b, cout)).astype(np.int32)
+    h2 = (h + 1) // 2
+    x2 = rm.pm1(r, (b, h2, h2, cout))
+    f2 = rm.pm1(r, (3, 3, cout, cout))
+    bn2 = r.normal(0, 40, cout).astype(np.float32)
+    inp, filt = orc.pack_conv_input_nhwc(x), orc.pack_conv_filter(f)
+    want_p, res_p = orc.conv128(inp, filt, bn, cin, cout, 3, 3, save_residual=True, inject_residual=True,
+                                residual_channels=lim, res_in=src)
+
+    prod = gpu.Conv128LayerParam("P", h, h, 3, 3, cin, cout, b, 1, 1, True, 1, 1, False, True, True, lim, False,
+                                 variant=_variant(gpu, variant))
+    prod.initialize(gpu.ArrayWeights([f, bn]), gpuops.pack_conv_input(x), _residual_source(src, in_fmt))
+    served = variant == "mfma_f4" and h % 2 == 0 and cout % 64 == 0 and in_fmt != 0 and prod.output_residual_gpu.format != 0
+    if h % 2:  # an odd frame has no 2x2 reader at all: the producer alone
+        prod.forward()
+        got, pooled = prod.download_saved_residual()
+        assert not pooled
+        np.testing.assert_array_equal(got, res_p)
+        prod.release()
+        return
+    want_c, res_c = orc.conv128(orc.pack_conv_input_nhwc(x2), orc.pack_conv_filter(f2), bn2, cout, cout, 3, 3,
+                                save_residual=True, inject_residual=True, residual_channels=cout // 2,
+                                residual_pool=True, res_in=res_p)
+    cons = gpu.Conv128LayerParam("C", h2, h2, 3, 3, cout, cout, b, 1, 1, True, 1, 1, False, True, True, cout // 2, True,
+                                 variant=_variant(gpu, variant))
+    cons.initialize(gpu.ArrayWeights([f2, bn2]), gpuops.pack_conv_input(x2), prod.get_output_residual_gpu())
+    assert ("conv3x3_mfma_f4_kernel" in prod.kernel_name() and ", 2, true>" in prod.kernel_name()) == served
+    prod.output_residual_gpu.fill(0xCD)
+    for _ in range(2):
+        prod.forward()
+        cons.forward()
+    got, pooled = prod.download_saved_residual()
+    assert pooled == served
+    np.testing.assert_array_equal(got, _window_maximum(res_p) if pooled else res_p)
+    np.testing.assert_array_equal(prod.download_packed(), want_p)
+    np.testing.assert_array_equal(cons.download_packed(), want_c)
+    np.testing.assert_array_equal(cons.download_saved_residual()[0], res_c)
+    # somebody asks for the full tensor: it is produced, and it is what the layers work with from then on
+    np.testing.assert_array_equal(prod.download_residual(), res_p)
+    np.testing.assert_array_equal(prod.download_residual_reference(), orc.residual_to_reference(res_p))
+    prod.forward()
+    cons.output_gpu.fill(0xCD)
+    cons.forward()
+    assert not prod.download_saved_residual()[1]
+    np.testing.assert_array_equal(cons.download_packed(), want_c)
+    np.testing.assert_array_equal(cons.download_residual(), res_c)
+    cons.release()
+    prod.release()
+
+
+def test_saved_residual_stays_full_for_other_readers(gpu):
+    """The 2x2 maximum alone is stored only while every hand-out of the tensor went to a pooling Conv128 reader."""
+    r = rng(31)
+    b, h, c = 8, 8, 64
+    x, f = rm.pm1(r, (b, h, h, c)), rm.pm1(r, (3, 3, c, c))
+    bn = r.normal(0, 20, c).astype(np.float32)
+    src = r.integers(-50, 51, size=(h, h, b, c)).astype(np.int32)
+    _, res_p = orc.conv128(orc.pack_conv_input_nhwc(x), orc.pack_conv_filter(f), bn, c, c, 3, 3, save_residual=True,
+                           inject_residual=True, residual_channels=c, res_in=src)
+
+    def producer():
+        p = gpu.Conv128LayerParam("P", h, h, 3, 3, c, c, b, 1, 1, True, 1, 1, False, True, True, c, False)
+        return p.initialize(gpu.ArrayWeights([f, bn]), gpuops.pack_conv_input(x), _residual_source(src, 2))
+
+    def reader(p, pool, size):
+        x2, f2 = rm.pm1(r, (b, size, size, c)), rm.pm1(r, (3, 3, c, c))
+        q = gpu.Conv128LayerParam("C", size, size, 3, 3, c, c, b, 1, 1, True, 1, 1, False, False, True, c, pool)
+        return q.initialize(gpu.ArrayWeights([f2, bn]), gpuops.pack_conv_input(x2), p.get_output_residual_gpu())
+
+    # no reader at all; a pooling reader; a pooling and a plain reader; a pooling reader and a pointer nobody registered
+    for readers, extra_handout, want_pooled in (((), 0, False), ((True,), 0, True), ((True, False), 0, False),
+                                                 ((True,), 1, False), ((True, True), 0, True)):
+        p = producer()
+        qs = [reader(p, pool, h // 2 if pool else h) for pool in readers]
+        for _ in range(extra_handout):
+            p.get_output_residual_gpu()
+        p.forward()
+        for q in qs:
+            q.forward()
+        got, pooled = p.download_saved_residual()
+        assert pooled == want_pooled, (readers, extra_handout)
+        np.testing.assert_array_equal(got, _window_maximum(res_p) if pooled else res_p)
+        if want_pooled:  # a reader that goes away takes its registration with it
+            qs[0].release()
+            p.forward()
+            assert not p.download_saved_residual()[1]
+        for q in qs:
+            q.release()
+        p.release()
+
+
 def test_conv128_random_shapes(gpu):
     """Seeded random bit-convolution layers: non-square frames of 1-14 pixels, 3x3 mostly (also 1x1 / 3x5 / 5x5 ...),
     strides, pools, FC-ready outputs, every residual mode with random storage formats, channel limits that cut through
@@ -896,6 +1009,7 @@ def _compare_network(gpu, spec, seed, variant, residual_format=None):
     net = gpu.Network(spec, weights, x, variant=_variant(gpu, variant), residual_format=residual_format)
     net.forward()
     logits = net.logits()
+    pooled_layers = []
     for L in spec:
         layer = net.layers[L["name"]]
         w = want[L["name"]]
@@ -908,10 +1022,21 @@ def _compare_network(gpu, spec, seed, variant, residual_format=None):
             got = layer.download_packed()
             np.testing.assert_array_equal(got, w["out"].reshape(got.shape), err_msg=L["name"])
             if w.get("res") is not None:
-                np.testing.assert_array_equal(layer.download_residual(), w["res"], err_msg=L["name"])
+                # (what the buffer holds: the full tensor, or its 2x2 maximum where only pooling readers exist)
+                got, pooled = layer.download_saved_residual()
+                np.testing.assert_array_equal(got, _window_maximum(w["res"]) if pooled else w["res"], err_msg=L["name"])
+                if pooled:
+                    pooled_layers.append(L["name"])
     # second forward on the same objects: identical logits (no stale-bit accumulation)
     net.forward()
     np.testing.assert_array_equal(net.logits(), logits)
+    # the full tensors on request, and the same logits from the layers working with them
+    for name in pooled_layers:
+        np.testing.assert_array_equal(net.layers[name].download_residual(), want[name]["res"], err_msg=name)
+    if pooled_layers:
+        net.forward()
+        np.testing.assert_array_equal(net.logits(), logits)
+        assert not any(net.layers[name].download_saved_residual()[1] for name in pooled_layers)
     net.release()
     return logits
 
