@@ -138,6 +138,30 @@ int main(int argc, char** argv) {
             fprintf(stderr, "Conv1: set_input() and a fresh initialize() disagree on the same batch\n");
             return 1;
         }
+        // a batch LARGER than the one the layer was initialized with, but within what the chosen residual format
+        // holds: accepted (the recorded bound is raised), and again what a fresh layer gives
+        {
+            std::vector<float> twice(images);
+            for (float& v : twice) v *= 2.0f;
+            stem.set_input(twice.data());
+            stem.forward(stream);
+            int* r1 = stem.get_output_residual_gpu_reference(stream);
+            const size_t rn1 = (size_t)stem.buf_height * stem.buf_width * PAD8(batch) * PAD128(ch);
+            const std::vector<int> got_res = to_host(r1, rn1);
+            const float* cursor3 = syn.values.data();
+            tcbnn_host::ConfigSource cfg3(&cursor3, syn.values.data() + syn.values.size());
+            InConv128LayerParam fresh2("Conv1", image, image, 3, 3, 3, ch, batch, 1, 1, true, 1, 1, true);
+            fresh2.initialize(twice.data(), cfg3);
+            fresh2.forward(stream);
+            if (fresh2.residual_info.format != stem.residual_info.format) {
+                fprintf(stderr, "Conv1: the doubled batch was meant to keep the residual format\n");
+                return 1;
+            }
+            if (got_res != to_host(fresh2.get_output_residual_gpu_reference(stream), rn1)) {
+                fprintf(stderr, "Conv1: set_input() of a larger batch and a fresh initialize() disagree\n");
+                return 1;
+            }
+        }
         if (o.oversize_input) {
             std::vector<float> big(images);
             for (float& v : big) v *= 1000.0f;

@@ -24,6 +24,9 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <math.h>
+
+#include <algorithm>
 #include <map>
 #include <vector>
 
@@ -138,12 +141,20 @@ class ConfigSource {
 // for, and what the buffer holds since the producer's last forward().  The maximum alone is stored when every
 // hand-out went to a pooling consumer (so that nobody else can be reading the tensor), nobody asked for the full
 // tensor, and the producer's kernel can do it (will_pool).
+// A reader whose own saved residual depends on the tensor's bound: that tensor's pointer variable (NULL while it
+// saves nothing) and what the reader adds to the bound (Cin*R*S for a bit convolution, 0 for a pooling layer).
+struct ResidualReader {
+    const void* who;
+    int* const* out_gpu;
+    int add;
+};
 struct ResidualInfo {
     int channels, bound, format;
     int handed_out, pool_consumers, other_consumers;
     bool observed, pooled, written;
     bool (*will_pool)(void*);  // the producer's decision for its next forward(); NULL: never
     void* producer;
+    std::vector<ResidualReader> readers;
 };
 inline std::map<const void*, ResidualInfo>& residual_registry() {
     static std::map<const void*, ResidualInfo> reg;
@@ -151,8 +162,14 @@ inline std::map<const void*, ResidualInfo>& residual_registry() {
 }
 // (the narrowest format that is exact for the bound: 12 bits up to 2047 for even batches, 16 bits up to 32767)
 inline ResidualInfo make_residual_info(int channels, int bound, int batch) {
-    ResidualInfo info = {channels, bound, tcbnn_residual_format_narrowest(bound, batch), 0, 0, 0, false, false, false, NULL,
-                         NULL};
+    ResidualInfo info;
+    info.channels = channels;
+    info.bound = bound;
+    info.format = tcbnn_residual_format_narrowest(bound, batch);
+    info.handed_out = info.pool_consumers = info.other_consumers = 0;
+    info.observed = info.pooled = info.written = false;
+    info.will_pool = NULL;
+    info.producer = NULL;
     return info;
 }
 inline ResidualInfo* find_residual(const void* gpu) {
@@ -160,9 +177,45 @@ inline ResidualInfo* find_residual(const void* gpu) {
     return it != residual_registry().end() ? &it->second : NULL;
 }
 // a layer of this library starts (sign = +1) or stops (-1) reading the saved residual at `gpu`
-inline void register_residual_consumer(const void* gpu, bool pools, int sign) {
+inline void register_residual_consumer(const void* gpu, bool pools, int sign, const void* who = NULL,
+                                       int* const* out_gpu = NULL, int add = 0) {
     ResidualInfo* u = find_residual(gpu);
-    if (u != NULL) (pools ? u->pool_consumers : u->other_consumers) += sign;
+    if (u == NULL) return;
+    (pools ? u->pool_consumers : u->other_consumers) += sign;
+    if (who == NULL) return;
+    if (sign > 0) {
+        const ResidualReader r = {who, out_gpu, add};
+        u->readers.push_back(r);
+    } else {
+        for (size_t i = 0; i < u->readers.size(); ++i)
+            if (u->readers[i].who == who) {
+                u->readers.erase(u->readers.begin() + i);
+                break;
+            }
+    }
+}
+// The largest bound of |value| the saved residual at `gpu` can take with every tensor that depends on it staying in
+// the format it was allocated in: its own format's range, and for every reader that saves a residual of its own,
+// that tensor's limit less what the reader adds.
+inline int residual_bound_limit(const void* gpu) {
+    const ResidualInfo* u = find_residual(gpu);
+    if (u == NULL) return INT32_MAX / 4;
+    int lim = u->format == TCBNN_RES_I12 ? 2047 : (u->format == TCBNN_RES_I16 ? 32767 : INT32_MAX / 4);
+    for (size_t i = 0; i < u->readers.size(); ++i) {
+        const ResidualReader& r = u->readers[i];
+        if (r.out_gpu != NULL && *r.out_gpu != NULL) lim = std::min(lim, residual_bound_limit(*r.out_gpu) - r.add);
+    }
+    return lim;
+}
+// records a larger bound (within residual_bound_limit) for the tensor and for everything that depends on it
+inline void raise_residual_bound(const void* gpu, int bound) {
+    ResidualInfo* u = find_residual(gpu);
+    if (u == NULL || bound <= u->bound) return;
+    u->bound = bound;
+    for (size_t i = 0; i < u->readers.size(); ++i) {
+        const ResidualReader& r = u->readers[i];
+        if (r.out_gpu != NULL && *r.out_gpu != NULL) raise_residual_bound(*r.out_gpu, bound + r.add);
+    }
 }
 inline int* hand_out_residual(int* gpu) {
     ResidualInfo* u = find_residual(gpu);
@@ -575,16 +628,34 @@ class InConv128LayerParam {  // param.h:701-870
     }
     // A new batch for the same layer objects (the reference's objects are single-shot, this engine's are not):
     // uploads `input` into input_gpu.  The format of the saved residual, and of every residual downstream of it,
-    // was chosen at initialize() from the largest |value| of the first batch; a batch that exceeds the bound the
-    // format was proven for would wrap in its 12 or 16 bits, so it is refused (print + exit, like every error here).
+    // was chosen at initialize() from the first batch's bound.  A batch whose sums can be larger is accepted as long
+    // as every one of those tensors still holds its values (the recorded bounds are raised); it is refused (print +
+    // exit, like every error here) only when a format would have to change: its values would wrap in 12 or 16
+    // bits.  The window scan of the batch is skipped when R*S*3*max|x| already fits.
     void set_input(float* input) {
         CHECK_NULL_POINTER(input);
         CHECK_NULL_POINTER(input_gpu);
         if (save_residual) {
-            if (residual_bound_of(input) > residual_info.bound) {
-                fprintf(stderr, "Error: set_input: |input| exceeds the bound the residual formats were chosen for "
-                                "(initialize the layers with the batch of largest magnitude).\n");
-                exit(-1);
+            const tcbnn_host::ResidualInfo* u = tcbnn_host::find_residual(output_residual_gpu);
+            const int recorded = u != NULL ? u->bound : residual_info.bound;
+            float amax = 0.0f;
+            bool finite = true;
+            for (size_t i = 0, n = (size_t)input_size(); i < n; ++i) {
+                const float a = fabsf(input[i]);
+                if (!(a <= 3.0e38f)) finite = false;
+                amax = a > amax ? a : amax;
+            }
+            const int coarse = finite ? tcbnn_inconv_residual_bound(filter_height, filter_width, amax) : INT32_MAX;
+            if (coarse > recorded) {
+                const int limit = tcbnn_host::residual_bound_limit(output_residual_gpu);
+                const int bound = coarse <= limit ? coarse : residual_bound_of(input);
+                if (bound > limit) {
+                    fprintf(stderr, "Error: set_input: window sums of |input| up to %d exceed what the residual formats "
+                                    "chosen at initialize() hold (up to %d): initialize the layers with the batch of "
+                                    "largest magnitude.\n", bound, limit);
+                    exit(-1);
+                }
+                tcbnn_host::raise_residual_bound(output_residual_gpu, bound);
             }
         }
         this->input = input;
@@ -731,8 +802,9 @@ class Conv128LayerParam {  // param.h:872-1065
     void set_input_gpu(uin32* input_gpu) { this->input_gpu = input_gpu; }
     void set_input_residual_gpu(int* input_residual_gpu) {
         if (inject_residual) {
-            tcbnn_host::register_residual_consumer(this->input_residual_gpu, residual_pool, -1);
-            tcbnn_host::register_residual_consumer(input_residual_gpu, residual_pool, +1);
+            tcbnn_host::register_residual_consumer(this->input_residual_gpu, residual_pool, -1, this);
+            tcbnn_host::register_residual_consumer(input_residual_gpu, residual_pool, +1, this, &output_residual_gpu,
+                                                   input_channels * filter_height * filter_width);
         }
         this->input_residual_gpu = input_residual_gpu;
         std::map<const void*, tcbnn_host::ResidualInfo>& reg = tcbnn_host::residual_registry();
@@ -743,10 +815,12 @@ class Conv128LayerParam {  // param.h:872-1065
         foreign.format = TCBNN_RES_I32;
         input_residual_info = it != reg.end() ? it->second : foreign;
         input_residual_channels = input_residual_info.channels;
+        const tcbnn_host::ResidualInfo* own = tcbnn_host::find_residual(output_residual_gpu);
         if (output_residual_gpu != NULL &&
             tcbnn_conv_residual_bound(input_channels, filter_height, filter_width,
                                       input_residual_info.bound < INT32_MAX / 4 ? input_residual_info.bound
-                                                                                : INT32_MAX / 4) > residual_info.bound) {
+                                                                                : INT32_MAX / 4) >
+                (own != NULL ? own->bound : residual_info.bound)) {
             fprintf(stderr, "Error: the injected residual exceeds the bound the saved residual was sized for.\n");
             exit(-1);
         }
@@ -935,7 +1009,7 @@ class Conv128LayerParam {  // param.h:872-1065
         SAFE_FREE_GPU(output_gpu);
         SAFE_FREE_GPU(filter_gpu);
         SAFE_FREE_GPU(bn_gpu);
-        if (inject_residual) tcbnn_host::register_residual_consumer(input_residual_gpu, residual_pool, -1);
+        if (inject_residual) tcbnn_host::register_residual_consumer(input_residual_gpu, residual_pool, -1, this);
         input_residual_gpu = NULL;
         if (output_residual_gpu != NULL) tcbnn_host::residual_registry().erase(output_residual_gpu);
         SAFE_FREE_GPU(output_residual_gpu);
@@ -1024,7 +1098,7 @@ class Pool128LayerParam {
             foreign.format = TCBNN_RES_I32;
             const int keep_bound = it != reg.end() ? it->second.bound : foreign.bound;
             const int keep_format = it != reg.end() ? it->second.format : foreign.format;
-            tcbnn_host::register_residual_consumer(input_residual_gpu, false, +1);  // (reads the full tensor)
+            tcbnn_host::register_residual_consumer(input_residual_gpu, false, +1, this, &output_residual_gpu, 0);
             residual_info = foreign;  // a maximum keeps bound and format
             residual_info.bound = keep_bound;
             residual_info.format = keep_format;
@@ -1055,6 +1129,9 @@ class Pool128LayerParam {
         TCBNN_SAFE_CALL(tcbnn_pool128_forward(&d, stream));
     }
     void release() {
+        if (pool_residual && input_residual_gpu != NULL)
+            tcbnn_host::register_residual_consumer(input_residual_gpu, false, -1, this);
+        input_residual_gpu = NULL;
         if (output_residual_gpu != NULL) tcbnn_host::residual_registry().erase(output_residual_gpu);
         SAFE_FREE_GPU(output_gpu);
         SAFE_FREE_GPU(output_residual_gpu);

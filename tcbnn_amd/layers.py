@@ -95,16 +95,48 @@ def _residual_buffer(channels, height, width, batch, bound, force_format=None):
     buf.handed_out = buf.pool_consumers = buf.other_consumers = 0
     buf.observed = buf.pooled = buf.written = False
     buf.producer = None
+    buf.readers = []  # the layers of this library that read the tensor (their own saved residuals depend on its bound)
     return buf
 
 
-def _register_residual_consumer(buf, pools, sign=1):
+def _register_residual_consumer(buf, pools, sign=1, layer=None):
     """A layer of this library starts (sign = +1) or stops (-1) reading the saved residual `buf`."""
     if buf is not None and hasattr(buf, "pool_consumers"):
         if pools:
             buf.pool_consumers += sign
         else:
             buf.other_consumers += sign
+        if layer is not None:
+            if sign > 0:
+                buf.readers.append(layer)
+            elif layer in buf.readers:
+                buf.readers.remove(layer)
+
+
+_FORMAT_LIMIT = {_lib.RES_I12: 2047, _lib.RES_I16: 32767, _lib.RES_I32: _lib.INT32_MAX // 4}
+
+
+def _residual_bound_limit(buf):
+    """The largest bound of |value| the saved residual `buf` can take with every tensor that depends on it
+    staying in the format it was allocated in: its own format's range, and for every reader that saves a
+    residual of its own, that tensor's limit less what the reader adds (Cin*R*S for a bit convolution)."""
+    lim = _FORMAT_LIMIT[buf.format]
+    for reader in buf.readers:
+        out, add = reader._residual_dependency()
+        if out is not None:
+            lim = min(lim, _residual_bound_limit(out) - add)
+    return lim
+
+
+def _raise_residual_bound(buf, bound):
+    """Record a larger bound for `buf` (within _residual_bound_limit) and for everything that depends on it."""
+    if bound <= buf.bound:
+        return
+    buf.bound = bound
+    for reader in buf.readers:
+        out, add = reader._residual_dependency()
+        if out is not None:
+            _raise_residual_bound(out, bound + add)
 
 
 def _residual_holds_window_maximum(buf):
@@ -468,6 +500,10 @@ class _ConvGeometry(_ReferenceLayoutIO):
     def _pooled_save_now(self):
         return False  # (only Conv128 layers can store the window maximum)
 
+    def _residual_dependency(self):
+        """(saved residual that depends on the injected one, what this layer adds to its bound), or (None, 0)."""
+        return None, 0
+
     def _want_full_residual(self, stream=None):
         """The full P x Q tensor is asked for: from now on it is what forward() saves, and if the buffer holds
         the 2x2 maximum from the last forward(), the layer is run again (its inputs are still in place)."""
@@ -621,10 +657,23 @@ class InConv128LayerParam(_ConvGeometry):
             self.stride_height, self.stride_width, int(self.padding))
 
     def set_input(self, input):
+        """A new batch.  The residual formats downstream were chosen from the first batch's bound; a batch whose
+        sums can be larger is accepted as long as every one of those tensors still holds its values (the recorded
+        bounds are raised), and refused only when a format would have to change.  The window scan of the batch is
+        skipped when R*S*3*max|x| already fits."""
         x = np.ascontiguousarray(input, dtype=np.float32)
         assert x.size == self.input_size(), (x.size, self.input_size())
-        if self.save_residual and self._residual_bound(x) > self.output_residual_gpu.bound:
-            raise _lib.TcbnnError("input magnitude exceeds the bound the residual format was chosen for")
+        if self.save_residual:
+            buf = self.output_residual_gpu
+            coarse = lib.tcbnn_inconv_residual_bound(self.filter_height, self.filter_width,
+                                                     float(np.max(np.abs(x))) if x.size else 0.0)
+            limit = _residual_bound_limit(buf)
+            if coarse > buf.bound:
+                bound = coarse if coarse <= limit else self._residual_bound(x)
+                if bound > limit:
+                    raise _lib.TcbnnError("input magnitude (window sums of |x| up to %d) exceeds what the residual "
+                                          "formats chosen at initialize() hold (up to %d)" % (bound, limit))
+                _raise_residual_bound(buf, bound)
         self.input_gpu.upload(x)
         self._pack_input()
 
@@ -696,8 +745,8 @@ class Conv128LayerParam(_ConvGeometry):
                                               min(input_residual_gpu.bound, _lib.INT32_MAX // 4)) > out.bound:
             raise _lib.TcbnnError("injected residual exceeds the bound the saved residual's format was chosen for")
         if self.inject_residual:
-            _register_residual_consumer(self.input_residual_gpu, self.residual_pool, -1)
-            _register_residual_consumer(input_residual_gpu, self.residual_pool, +1)
+            _register_residual_consumer(self.input_residual_gpu, self.residual_pool, -1, self)
+            _register_residual_consumer(input_residual_gpu, self.residual_pool, +1, self)
         self.input_residual_gpu = input_residual_gpu
 
     def initialize(self, config_file, prev_layer_gpu, input_residual_gpu=None):
@@ -733,6 +782,11 @@ class Conv128LayerParam(_ConvGeometry):
         if self.input_gpu is None:
             raise _lib.TcbnnError("Error: NULL pointer (input_gpu)")
         return self
+
+    def _residual_dependency(self):
+        if self.inject_residual and self.output_residual_gpu is not None:
+            return self.output_residual_gpu, self.input_channels * self.filter_height * self.filter_width
+        return None, 0
 
     def _pooled_save_now(self):
         """Store only the 2x2 maximum of the saved residual?  Yes when that is all anybody reads: every hand-out of
@@ -777,7 +831,7 @@ class Conv128LayerParam(_ConvGeometry):
     def release(self):
         self._release_ref_bufs()
         if self.inject_residual:
-            _register_residual_consumer(self.input_residual_gpu, self.residual_pool, -1)
+            _register_residual_consumer(self.input_residual_gpu, self.residual_pool, -1, self)
             self.input_residual_gpu = None
         for b in (self.filter_gpu, self.bn_gpu, self.output_gpu, self.output_residual_gpu):
             if b is not None:
@@ -812,7 +866,7 @@ class Pool128LayerParam:
             if input_residual_gpu is None:
                 raise _lib.TcbnnError("Error: NULL pointer (input_residual_gpu)")
             self.input_residual_gpu = input_residual_gpu
-            _register_residual_consumer(input_residual_gpu, False)
+            _register_residual_consumer(input_residual_gpu, False, +1, self)
             # a maximum never exceeds the bound of its operands: same bound, same format
             self.output_residual_gpu = _residual_buffer(self.output_channels, self.output_height, self.output_width,
                                                         self.batch, input_residual_gpu.bound,
@@ -824,6 +878,10 @@ class Pool128LayerParam:
 
     get_output_residual_gpu = _ConvGeometry.get_output_residual_gpu
     _pooled_save_now = _ConvGeometry._pooled_save_now
+
+    def _residual_dependency(self):
+        return (self.output_residual_gpu, 0) if self.pool_residual else (None, 0)
+
     _want_full_residual = _ConvGeometry._want_full_residual
     download_saved_residual = _ConvGeometry.download_saved_residual
 
@@ -846,6 +904,9 @@ class Pool128LayerParam:
     _is_fc_ready = _ConvGeometry._is_fc_ready
 
     def release(self):
+        if self.pool_residual:
+            _register_residual_consumer(self.input_residual_gpu, False, -1, self)
+            self.input_residual_gpu = None
         for b in (self.output_gpu, self.output_residual_gpu):
             if b is not None:
                 b.free()

@@ -170,11 +170,11 @@ def test_reference_layout_accessors_of_the_cpp_classes(gpu, tmp_path, variant):
 
 
 def test_first_layer_set_input_refuses_a_batch_beyond_its_residual_bound(gpu):
-    """The C++ first layer picks 16-bit residual storage from the first batch's largest |value|; a later batch
-    that exceeds that bound must end in the reference's error convention (message + exit(-1)), not in wrapped
-    residuals.  (The same binary, without the flag, checks that an admissible second batch gives what a fresh
-    layer gives: the test above.)"""
+    """The C++ first layer picks the residual storage format from the first batch's window sums of |x|; a later
+    batch whose sums no longer fit that format must end in the reference's error convention (message +
+    exit(-1)), not in wrapped residuals.  (The same binary, without the flag, checks that admissible later batches,
+    a smaller one and a larger one that the format still holds, give what a fresh layer gives: the test above.)"""
     exe = os.path.join(BIN, "reference_fmt_interop")
     proc = subprocess.run([exe, "--batch", "12", "--seed", "3", "--oversize-input"], stdout=subprocess.PIPE,
                           stderr=subprocess.PIPE, text=True, timeout=120)
-    assert proc.returncode == 255 and "exceeds the bound" in proc.stderr, (proc.returncode, proc.stderr)
+    assert proc.returncode == 255 and "exceed what the residual formats" in proc.stderr, (proc.returncode, proc.stderr)

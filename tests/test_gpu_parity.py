@@ -1002,6 +1002,24 @@ def test_reference_layout_between_layers(gpu, variant):
         layer.release()
 
 
+def _check_layers(net, spec, want):
+    """Every layer's packed activations and saved residual (as stored: the full tensor, or its 2x2 maximum where
+    only pooling readers exist) against the oracle; the names of the layers that store the maximum."""
+    pooled_layers = []
+    for L in spec:
+        if L["kind"] in ("out", "avgfc"):
+            continue
+        layer, w = net.layers[L["name"]], want[L["name"]]
+        got = layer.download_packed()
+        np.testing.assert_array_equal(got, w["out"].reshape(got.shape), err_msg=L["name"])
+        if w.get("res") is not None:
+            got, pooled = layer.download_saved_residual()
+            np.testing.assert_array_equal(got, _window_maximum(w["res"]) if pooled else w["res"], err_msg=L["name"])
+            if pooled:
+                pooled_layers.append(L["name"])
+    return pooled_layers
+
+
 def _compare_network(gpu, spec, seed, variant, residual_format=None):
     weights = gpu.synthetic_weights(spec, seed)
     x = gpu.synthetic_input(spec, seed)
@@ -1129,6 +1147,74 @@ def test_imagenet_resnet18_textbook_wiring(gpu, variant):
     _compare_network(gpu, nets.imagenet_resnet_textbook_spec(batch=8), 14, variant)
 
 
+@pytest.mark.timeout(900)
+@pytest.mark.parametrize("name,batch,seed", [("alexnet", 256, 21), ("cifar10_resnet", 256, 22),
+                                             ("imagenet_resnet_textbook", 256, 23), ("imagenet_vgg", 64, 24)])
+def test_other_networks_at_their_configured_batch(gpu, name, batch, seed):
+    """alexnet.cu:143-177, cifar10_resnet.cu:189-259 and the textbook-wired ResNet-18 at batch 256, VGG-16
+    (imagenet_vgg.cu:217-286) at batch 64, full image size, default engine: every layer and every image against the
+    oracle.  Launch shapes that only occur at this size (grids sized to the whole machine, the pooling layer at
+    112 x 112 x 64 x 256, the 1x1 stride-2 convolutions of the generic kernel) are only covered here."""
+    from tcbnn_amd import nets
+    spec = nets.SPECS[name](batch=batch)
+    weights = gpu.synthetic_weights(spec, seed)
+    x = gpu.synthetic_input(spec, seed)
+    want = orc_nets.run(spec, weights, x)
+    net = gpu.Network(spec, weights, x)
+    net.forward()
+    last = spec[-1]
+    if last["kind"] == "avgfc":  # fp32 head: 1e-5 of the logits' scale
+        w = want[last["name"]]["out"]
+        np.testing.assert_allclose(net.logits(), w, rtol=1e-5, atol=1e-5 * float(np.abs(w).max()))
+    else:
+        np.testing.assert_allclose(net.logits(), want[last["name"]]["out"], rtol=1e-5, atol=0)
+    _check_layers(net, spec, want)
+    net.release()
+
+
+def test_set_input_accepts_batches_of_the_same_distribution(gpu):
+    """The residual formats are chosen from the first batch's window sums of |x|.  Later batches of the same
+    distribution have slightly larger or smaller sums: they must be accepted (nothing would wrap) and give what
+    the oracle gives; so must a batch scaled up as far as every tensor's format still holds; one step beyond
+    that is refused."""
+    from tcbnn_amd import nets
+    from tcbnn_amd.layers import _residual_bound_limit
+    spec = nets.imagenet_resnet_spec(batch=8, image=64, output_size=100)
+    weights = gpu.synthetic_weights(spec, 40)
+    net = gpu.Network(spec, weights, gpu.synthetic_input(spec, 40))
+    first = net.order[0]
+    bound0 = first.output_residual_gpu.bound
+    fmts = {L["name"]: net.layers[L["name"]].output_residual_gpu.format for L in spec if L.get("save_residual")}
+    larger = 0
+    for seed in range(41, 49):
+        x = gpu.synthetic_input(spec, seed)
+        larger += first._residual_bound(x) > bound0
+        net.set_input(x)
+        net.forward()
+        want = orc_nets.run(spec, weights, x)
+        np.testing.assert_allclose(net.logits(), want["Fout"]["out"], rtol=1e-5, atol=0)
+        _check_layers(net, spec, want)
+    assert larger >= 1  # (some of these batches do exceed the first batch's exact bound)
+    # as large as the formats allow: the limit is set by the 12-bit tensors of the first stage
+    limit = _residual_bound_limit(first.output_residual_gpu)
+    assert limit == 2047 - 2 * 64 * 9
+    x = gpu.synthetic_input(spec, 50)
+    x = (x * (0.98 * limit / first._residual_bound(x))).astype(np.float32)
+    assert bound0 < first._residual_bound(x) <= limit
+    net.set_input(x)
+    net.forward()
+    want = orc_nets.run(spec, weights, x)
+    np.testing.assert_allclose(net.logits(), want["Fout"]["out"], rtol=1e-5, atol=0)
+    _check_layers(net, spec, want)
+    for L in spec:  # nothing was re-allocated, every recorded bound covers what the oracle saw
+        if L.get("save_residual"):
+            buf = net.layers[L["name"]].output_residual_gpu
+            assert buf.format == fmts[L["name"]] and np.abs(want[L["name"]]["res"]).max() <= buf.bound
+    with pytest.raises(gpu.TcbnnError):
+        net.set_input((x * 1.1).astype(np.float32))
+    net.release()
+
+
 @pytest.mark.parametrize("fmt", [0, 1, 2])
 @pytest.mark.parametrize("b,h,c,window,stride,pad", [(8, 12, 64, 3, 2, 1), (70, 7, 40, 3, 2, 1), (5, 9, 100, 2, 2, 0),
                                                      (3, 5, 33, 3, 1, 1)])
@@ -1254,12 +1340,14 @@ def test_imagenet_resnet18_batch256_every_image(gpu):
         net.forward()
         logits = net.logits()
         np.testing.assert_allclose(logits, want["Fout"]["out"], rtol=1e-5, atol=0)
-        for L in spec[:-1]:
-            layer, w = net.layers[L["name"]], want[L["name"]]
-            got = layer.download_packed()
-            np.testing.assert_array_equal(got, w["out"].reshape(got.shape), err_msg=L["name"])
-            if w.get("res") is not None:
-                np.testing.assert_array_equal(layer.download_residual(), w["res"], err_msg=L["name"])
+        pooled = _check_layers(net, spec, want)
+        assert pooled == ["L1B2C2", "L2B2C2", "L3B2C2"]  # (the tensors that only the next stage's entry reads)
+    # the full tensors on request, and the same logits from the layers working with them
+    for name in pooled:
+        np.testing.assert_array_equal(net.layers[name].download_residual(), want[name]["res"], err_msg=name)
+    net.forward()
+    np.testing.assert_array_equal(net.logits(), logits)
+    assert _check_layers(net, spec, want) == []
     net.release()
 
 
@@ -1275,12 +1363,7 @@ def test_imagenet_resnet18_ragged_batch_above_256(gpu):
     net = gpu.Network(spec, weights, x)
     net.forward()
     np.testing.assert_allclose(net.logits(), want["Fout"]["out"], rtol=1e-5, atol=0)
-    for L in spec[:-1]:
-        layer, w = net.layers[L["name"]], want[L["name"]]
-        got = layer.download_packed()
-        np.testing.assert_array_equal(got, w["out"].reshape(got.shape), err_msg=L["name"])
-        if w.get("res") is not None:
-            np.testing.assert_array_equal(layer.download_residual(), w["res"], err_msg=L["name"])
+    assert len(_check_layers(net, spec, want)) == 3
     net.release()
 
 
