@@ -1137,6 +1137,11 @@ struct Pick {
 constexpr int pick_nt(int spt, int rm) {
     return rm == RM_POOLED ? (spt >= 6 ? 1 : 2) : (rm == RM_RAW ? (spt >= 3 && spt < 8 ? 1 : 2) : 2);
 }
+// Channel tiles per wave when the saved residual is the window maximum: a work item is then a whole window (four
+// tiles), and from Cin = 128 on the launches have so few of them per wave that finer tiles balance the waves better
+// (ResNet-18 at batch 256: 26.0 -> 25.0 us at Cin = 128, 23.2 -> 22.0 us at Cin = 256; at Cin = 64, where the tile is
+// bound by its VALU work, 30.5 -> 34.4 us).
+constexpr int pick_nt_maxsave(int spt) { return spt >= 2 && spt <= 4 ? 1 : 2; }
 constexpr int pick_mt(int spt, int rm) {
     return rm == RM_RAW ? (spt >= 8 ? 1 : 2) : (rm == RM_NONE ? (spt >= 6 ? 1 : 2) : 1);
 }
@@ -1147,7 +1152,8 @@ Pick pick(const BgemmParams& p) {
                        : (p.res_in != nullptr && p.res_pool ? RM_POOLED : RM_PLAIN);
     const int fmt = p.res_in != nullptr ? p.res_in_fmt : TCBNN_RES_I32;
     // (a pooled int32 source keeps one channel tile per wave: four times sixteen words per tile and lane spilled)
-    const int nt = rm == RM_POOLED && fmt == TCBNN_RES_I32 ? 1 : pick_nt(p.cw / 2, rm);
+    int nt = rm == RM_POOLED && fmt == TCBNN_RES_I32 ? 1 : pick_nt(p.cw / 2, rm);
+    if (rm == RM_PLAIN && p.res_out_pool) nt = pick_nt_maxsave(p.cw / 2);
     return {rm, pick_mt(p.cw / 2, rm), nt, fmt, p.pool_h == 2 ? WIN_ORPOOL : (p.res_out_pool ? WIN_MAXSAVE : WIN_NONE)};
 }
 
@@ -1164,8 +1170,8 @@ int launch_m(const BgemmParams& p, hipStream_t stream) {
         case RM_PLAIN:
             if (k.win == WIN_MAXSAVE)  // (a narrow injected residual: conv3x3_mfma_applicable)
                 return k.r16 == TCBNN_RES_I12
-                           ? launch_t<SPT, RM_PLAIN, pick_mt(SPT, RM_PLAIN), pick_nt(SPT, RM_PLAIN), TCBNN_RES_I12, WIN_MAXSAVE>(p, stream)
-                           : launch_t<SPT, RM_PLAIN, pick_mt(SPT, RM_PLAIN), pick_nt(SPT, RM_PLAIN), TCBNN_RES_I16, WIN_MAXSAVE>(p, stream);
+                           ? launch_t<SPT, RM_PLAIN, pick_mt(SPT, RM_PLAIN), pick_nt_maxsave(SPT), TCBNN_RES_I12, WIN_MAXSAVE>(p, stream)
+                           : launch_t<SPT, RM_PLAIN, pick_mt(SPT, RM_PLAIN), pick_nt_maxsave(SPT), TCBNN_RES_I16, WIN_MAXSAVE>(p, stream);
             return k.r16 == TCBNN_RES_I12
                        ? launch_t<SPT, RM_PLAIN, pick_mt(SPT, RM_PLAIN), pick_nt(SPT, RM_PLAIN), TCBNN_RES_I12, WIN_NONE>(p, stream)
                        : (k.r16 == TCBNN_RES_I16

@@ -57,6 +57,33 @@ def test_fc128_static_scratch_matches_workspace_entry(gpu, variant):
         assert name.value.decode().endswith(", 4>"), name.value
 
 
+def test_fc128_static_scratch_allocates_nothing(gpu):
+    """The property the entry point exists for: with every operand allocated beforehand, repeated calls leave the
+    device's free memory exactly where it was (hipMemGetInfo), for the split-K shape as well as a small one."""
+    from tcbnn_amd import _lib
+    from tcbnn_amd.device import DeviceBuffer
+    lib, hip = _lib.lib, _lib.hip
+    hip.hipMemGetInfo.argtypes = [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]
+    v = gpu.VARIANTS["popc"]
+    r = np.random.default_rng(18)
+    for b, k, n in [(130, 25088, 64), (8, 128, 128)]:
+        x = r.standard_normal((b, k)).astype(np.float32)
+        inp, wbuf = gpuops.in128(x), gpuops.pack_fc_weight(rm.pm1(r, (k, n)))
+        bnb = gpuops.dev(r.normal(0, np.sqrt(k), n).astype(np.float32))
+        out = DeviceBuffer(4 * lib.tcbnn_fc_act_words(b, n))
+        d = _lib.Fc128Desc(inp.ptr, wbuf.ptr, bnb.ptr, out.ptr, b, k, n, v, None, 0)
+        _lib.check(lib.tcbnn_fc128_forward_static_scratch(C.byref(d), None))  # (first call: resolves the buffer's address)
+        gpuops.sync()
+        free0, free1, total = C.c_size_t(0), C.c_size_t(0), C.c_size_t(0)
+        _lib.hip_check(hip.hipMemGetInfo(C.byref(free0), C.byref(total)), "hipMemGetInfo")
+        for _ in range(5):
+            _lib.check(lib.tcbnn_fc128_forward_static_scratch(C.byref(d), None))
+        gpuops.sync()
+        _lib.hip_check(hip.hipMemGetInfo(C.byref(free1), C.byref(total)), "hipMemGetInfo")
+        assert free1.value == free0.value, (free0.value, free1.value)
+        out.free()
+
+
 def test_fc128_static_scratch_rejects_oversize(gpu):
     from tcbnn_amd import _lib
     d = _lib.Fc128Desc(1, 1, 1, 1, 8192, 1024, 1024, 0, None, 0)  # 8 Mi words: beyond the built-in 1 Mi
