@@ -37,9 +37,19 @@ namespace {
 
 using namespace mfma;
 
-// Cache policy of the residual loads: non-temporal (the operand is read exactly once; measured 2 % on the
-// ResNet-18 step, while non-temporal stores cost time: the next layer finds less of its input in the caches).
-constexpr int kResLoadAux = 2;
+// Cache policy of the residual loads: the default one.  (With the stores below written through, a non-temporal
+// hint on the loads costs 0.6 % of the ResNet-18 step at batch 256: 0.4641 -> 0.4611 ms over three runs each without
+// it; before the stores were written through the hint had gained 2 %.)
+constexpr int kResLoadAux = 0;
+// Cache policy of the residual stores of full tiles with a narrow residual (the ResNet layers): written through
+// (sc0 sc1).  The tensors are far larger than an XCD's L2 and are read one or two launches later, mostly by other
+// XCDs: leaving them dirty in the writer's L2 only defers the write to the end of the launch.  Measured on ResNet-18
+// at batch 256, three runs each: step 0.4640 -> 0.4590 ms (the residual launches 1-6 % shorter, the launches that
+// read the tensors unchanged); non-temporal (nt) and agent scope (sc1) gave half of that.
+constexpr int kResStoreAux = 0x11;
+// ... and of the output words: written through as well (the next launch reads them from every XCD); another 0.5 % of
+// that step (0.4633 -> 0.4610 ms, three runs each; non-temporal stores instead: 0.4693 ms).
+constexpr int kBitsStoreAux = 0x11;
 // Waves per workgroup: four, sharing the staged weights of their channel group; eight where the FP4 fragments of
 // two channel tiles (18 KB per tile and 64 input channels) leave room for only one workgroup in a CU's 160 KB of
 // LDS: the CU then still runs two waves per SIMD, and each expanded activation fragment still feeds two MFMAs.
@@ -598,8 +608,8 @@ conv3x3_mfma_f4_kernel(
                             q[0] = v4i{(int)d[0], (int)d[1], (int)d[2], (int)d[3]};
                             typedef int v2i_t __attribute__((ext_vector_type(2)));
                             const v2i_t q2 = {(int)d[4], (int)d[5]};
-                            __builtin_amdgcn_raw_buffer_store_b128(q[0], r_rout, (int)vo, (int)so, 0);
-                            __builtin_amdgcn_raw_buffer_store_b64(q2, r_rout, (int)vo2, (int)so, 0);
+                            __builtin_amdgcn_raw_buffer_store_b128(q[0], r_rout, (int)vo, (int)so, kResStoreAux);
+                            __builtin_amdgcn_raw_buffer_store_b64(q2, r_rout, (int)vo2, (int)so, kResStoreAux);
                             asm volatile("s_nop 4" ::"v"(q[0]), "v"(q2));  // see the 128-bit store note below
                         } else {  // TCBNN_RES_I16
                             const unsigned so = (pix * (unsigned)((p.N + 7) / 8) + (unsigned)((n0 + nt * 32) / 8)) * grp_b;
@@ -607,7 +617,7 @@ conv3x3_mfma_f4_kernel(
 #pragma unroll
                             for (int g = 0; g < 2; ++g) {
                                 q[g] = v4i{(int)wm[4 * g], (int)wm[4 * g + 1], (int)wm[4 * g + 2], (int)wm[4 * g + 3]};
-                                __builtin_amdgcn_raw_buffer_store_b128(q[g], r_rout, (int)vo, (int)(so + (unsigned)g * grp_b), 0);
+                                __builtin_amdgcn_raw_buffer_store_b128(q[g], r_rout, (int)vo, (int)(so + (unsigned)g * grp_b), kResStoreAux);
                             }
                             asm volatile("s_nop 4" ::"v"(q[0]), "v"(q[1]));
                         }
@@ -628,8 +638,8 @@ conv3x3_mfma_f4_kernel(
                         q[0] = v4i{(int)d[0], (int)d[1], (int)d[2], (int)d[3]};
                         typedef int v2i_t __attribute__((ext_vector_type(2)));
                         const v2i_t q2 = {(int)d[4], (int)d[5]};
-                        __builtin_amdgcn_raw_buffer_store_b128(q[0], r_rout, (int)vo, (int)so, 0);
-                        __builtin_amdgcn_raw_buffer_store_b64(q2, r_rout, (int)vo2, (int)so, 0);
+                        __builtin_amdgcn_raw_buffer_store_b128(q[0], r_rout, (int)vo, (int)so, kResStoreAux);
+                        __builtin_amdgcn_raw_buffer_store_b64(q2, r_rout, (int)vo2, (int)so, kResStoreAux);
                         asm volatile("s_nop 4" ::"v"(q[0]), "v"(q2));
                     } else if (rout_fmt == TCBNN_RES_I16) {
                         const unsigned so = (pix * (unsigned)((p.N + 7) / 8) + (unsigned)((n0 + nt * 32) / 8)) * grp_b;
@@ -640,7 +650,7 @@ conv3x3_mfma_f4_kernel(
                             for (int k = 0; k < 4; ++k)  // the low halves of two bit patterns: one byte permute
                                 q[g][k] = (int)__builtin_amdgcn_perm(__float_as_uint(t[8 * g + 2 * k + 1]),
                                                                      __float_as_uint(t[8 * g + 2 * k]), 0x05040100u);
-                            __builtin_amdgcn_raw_buffer_store_b128(q[g], r_rout, (int)vo, (int)(so + (unsigned)g * grp_b), 0);
+                            __builtin_amdgcn_raw_buffer_store_b128(q[g], r_rout, (int)vo, (int)(so + (unsigned)g * grp_b), kResStoreAux);
                         }
                         asm volatile("s_nop 4" ::"v"(q[0]), "v"(q[1]));
                     } else {
@@ -650,7 +660,7 @@ conv3x3_mfma_f4_kernel(
                         for (int g = 0; g < 4; ++g) {
 #pragma unroll
                             for (int k = 0; k < 4; ++k) q[g][k] = (int)(__float_as_uint(t[4 * g + k]) - kMagicBits);
-                            __builtin_amdgcn_raw_buffer_store_b128(q[g], r_rout, (int)vo, (int)(so + (unsigned)g * grp_b), 0);
+                            __builtin_amdgcn_raw_buffer_store_b128(q[g], r_rout, (int)vo, (int)(so + (unsigned)g * grp_b), kResStoreAux);
                         }
                         asm volatile("s_nop 4" ::"v"(q[0]), "v"(q[1]), "v"(q[2]), "v"(q[3]));
                     }
@@ -779,7 +789,7 @@ conv3x3_mfma_f4_kernel(
             const int w = ng * NT + nt;
             if (w < p.bits_row_words)  // uniform
                 __builtin_amdgcn_raw_buffer_store_b32((int)word, r_bits, (int)voff_bits[mt],
-                                                      (int)(bits_pix + (unsigned)w * row_b), 0);
+                                                      (int)(bits_pix + (unsigned)w * row_b), kBitsStoreAux);
         }
     };
 
