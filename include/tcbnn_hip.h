@@ -121,6 +121,9 @@ int tcbnn_inconv_residual_bound(int filter_height, int filter_width, float input
 int tcbnn_inconv_residual_bound_of_input(const float* input_host, int batch, int height, int width,
                                          int filter_height, int filter_width, int stride_height,
                                          int stride_width, int padding);
+/* max |x| over a HOST array (on a few host threads; +infinity if any value is NaN or infinite): the cheap first test of
+ * a new first-layer batch against the recorded bound, before the window scan above. */
+float tcbnn_host_abs_max(const float* values_host, size_t count);
 int tcbnn_conv_residual_bound(int input_channels, int filter_height, int filter_width, int injected_bound);
 int tcbnn_residual_format_for_bound(int bound);
 int tcbnn_residual_format_narrowest(int bound, int batch);

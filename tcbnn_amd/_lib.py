@@ -100,6 +100,7 @@ ABI = {
     "tcbnn_inconv_filter_words": (c_size_t, [c_int] * 4),
     "tcbnn_residual_bytes": (c_size_t, [c_int] * 5),
     "tcbnn_inconv_residual_bound": (c_int, [c_int, c_int, C.c_float]),
+    "tcbnn_host_abs_max": (C.c_float, [c_void_p, c_size_t]),
     "tcbnn_conv_residual_bound": (c_int, [c_int] * 4),
     "tcbnn_residual_format_for_bound": (c_int, [c_int]),
     "tcbnn_residual_format_narrowest": (c_int, [c_int, c_int]),

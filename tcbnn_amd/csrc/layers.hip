@@ -246,6 +246,31 @@ int tcbnn_inconv_residual_bound_of_input(const float* input_host, int batch, int
     return bound < (double)(INT32_MAX / 2) ? (int)std::ceil(bound) : INT32_MAX;
 }
 
+// max |x| over a host array, on a few host threads (NaN or infinity anywhere: +infinity)
+float tcbnn_host_abs_max(const float* values_host, size_t count) {
+    if (values_host == nullptr || count == 0) return 0.0f;
+    const int n_threads = (int)std::max<size_t>(1, std::min<size_t>(std::min<size_t>(count >> 20, 16), std::thread::hardware_concurrency()));
+    std::vector<float> part(n_threads, 0.0f);
+    auto scan = [&](int t) {
+        const size_t lo = count * t / n_threads, hi = count * (t + 1) / n_threads;
+        float m = 0.0f;
+        bool bad = false;
+        for (size_t i = lo; i < hi; ++i) {
+            const float a = std::fabs(values_host[i]);
+            bad |= !(a <= 3.0e38f);
+            m = a > m ? a : m;
+        }
+        part[t] = bad ? INFINITY : m;
+    };
+    std::vector<std::thread> pool;
+    for (int t = 1; t < n_threads; ++t) pool.emplace_back(scan, t);
+    scan(0);
+    for (std::thread& th : pool) th.join();
+    float m = 0.0f;
+    for (float v : part) m = v > m ? v : m;
+    return m;
+}
+
 int tcbnn_fc128_forward(const tcbnn_fc128_desc* d, void* stream) {
     TCBNN_NOTNULL(d);
     TCBNN_NOTNULL(d->input);

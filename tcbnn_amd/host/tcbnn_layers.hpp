@@ -638,14 +638,8 @@ class InConv128LayerParam {  // param.h:701-870
         if (save_residual) {
             const tcbnn_host::ResidualInfo* u = tcbnn_host::find_residual(output_residual_gpu);
             const int recorded = u != NULL ? u->bound : residual_info.bound;
-            float amax = 0.0f;
-            bool finite = true;
-            for (size_t i = 0, n = (size_t)input_size(); i < n; ++i) {
-                const float a = fabsf(input[i]);
-                if (!(a <= 3.0e38f)) finite = false;
-                amax = a > amax ? a : amax;
-            }
-            const int coarse = finite ? tcbnn_inconv_residual_bound(filter_height, filter_width, amax) : INT32_MAX;
+            const int coarse = tcbnn_inconv_residual_bound(filter_height, filter_width,
+                                                           tcbnn_host_abs_max(input, (size_t)input_size()));
             if (coarse > recorded) {
                 const int limit = tcbnn_host::residual_bound_limit(output_residual_gpu);
                 const int bound = coarse <= limit ? coarse : residual_bound_of(input);

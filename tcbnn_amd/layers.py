@@ -666,7 +666,7 @@ class InConv128LayerParam(_ConvGeometry):
         if self.save_residual:
             buf = self.output_residual_gpu
             coarse = lib.tcbnn_inconv_residual_bound(self.filter_height, self.filter_width,
-                                                     float(np.max(np.abs(x))) if x.size else 0.0)
+                                                     lib.tcbnn_host_abs_max(x.ctypes.data, x.size))
             limit = _residual_bound_limit(buf)
             if coarse > buf.bound:
                 bound = coarse if coarse <= limit else self._residual_bound(x)

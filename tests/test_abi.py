@@ -146,3 +146,26 @@ def test_first_layer_bound_of_input_is_the_largest_window_sum():
     bad[0, 1, 3, 3] = np.nan
     assert L.tcbnn_inconv_residual_bound_of_input(bad.ctypes.data_as(C.c_void_p), 1, 8, 8, 3, 3, 1, 1, 1) == 2 ** 31 - 1
     assert L.tcbnn_inconv_residual_bound_of_input(None, 1, 8, 8, 3, 3, 1, 1, 1) == 2 ** 31 - 1
+
+
+def test_host_abs_max_and_threaded_window_scan_on_a_large_batch():
+    """tcbnn_host_abs_max against numpy (sizes below and above its threading threshold, NaN / infinity), and the
+    window scan on a batch large enough for every host thread to take several images."""
+    import numpy as np
+    from tcbnn_amd import _lib
+    L = _lib.lib
+    rng = np.random.default_rng(12)
+    for n in (1, 1000, (3 << 20) + 17):
+        x = (rng.standard_normal(n) * 7).astype(np.float32)
+        assert L.tcbnn_host_abs_max(x.ctypes.data, n) == float(np.abs(x).max())
+        x[n // 2] = np.inf if n % 2 else np.nan
+        assert L.tcbnn_host_abs_max(x.ctypes.data, n) == float("inf")
+    assert L.tcbnn_host_abs_max(None, 5) == 0.0
+    b, h, w = 70, 20, 24
+    x = rng.standard_normal((b, 3, h, w)).astype(np.float32)
+    x[41] *= 9.0  # the image that sets the bound sits in the middle of the batch
+    a = np.abs(x.astype(np.float64)).sum(axis=1)
+    worst = max(float(a[:, max(0, 4 * y - 3):4 * y + 4, max(0, 4 * q - 3):4 * q + 4].sum(axis=(1, 2)).max())
+                for y in range(5) for q in range(6))
+    got = L.tcbnn_inconv_residual_bound_of_input(x.ctypes.data, b, h, w, 7, 7, 4, 4, 1)
+    assert worst <= got <= worst * 1.001 + 2, (got, worst)
