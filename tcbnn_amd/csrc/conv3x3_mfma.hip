@@ -80,7 +80,10 @@ constexpr int kWavesPerSimd = 2;
 // of the output bits (kernel.cuh:797-816): a wave multiplies the four pixels of a window one after the other and
 // stores the OR of their words once; WIN_MAXSAVE = the output bits are stored per pixel, but the saved residual is
 // the element-wise maximum over the window, stored once per window: exactly what a consumer with residual_pool
-// would compute from the full tensor (kernel.cuh:775-782), at a quarter of the bytes written and read.  FULLT = every 32-channel tile of the launch exists in full
+// would compute from the full tensor (kernel.cuh:775-782), at a quarter of the bytes written and read.  A window is
+// then the work item of a whole WORKGROUP: each of its four waves multiplies one of the window's pixels, the sums
+// meet in LDS, and waves 0 .. NT-1 take the maximum of one channel tile each and store it (work items of one
+// pixel tile instead of four: the layers that save such tensors have only one to four windows per wave).  FULLT = every 32-channel tile of the launch exists in full
 // and, with an injected residual, lies entirely below or entirely above the channel limit: the per-channel
 // tests of partial tiles are then not even compiled (they cost scalar registers and set-up instructions in
 // every launch, and the networks' channel counts are multiples of 64).
@@ -97,6 +100,7 @@ conv3x3_mfma_f4_kernel(
     static_assert(RM == RM_NONE || !POOL, "residuals are defined for un-pooled layers only");
     static_assert(!PSAVE || (RM == RM_PLAIN && FULLT && (RF == TCBNN_RES_I16 || RF == TCBNN_RES_I12)),
                   "the window maximum is taken on 16-bit pairs in the epilogue of full tiles with a narrow injected residual");
+    static_assert(!PSAVE || (MT == 1 && waves_of(SPT, NT) == 4), "one wave per pixel of the window, one image tile each");
     constexpr int TPC = SPT >= 3 ? 3 : 9;  // taps per prefetch chunk (a filter row, or all of it)
     constexpr int NCH = 9 / TPC;           // chunks per tile
     constexpr int NQ = 9 * SPT;            // k-steps per tile
@@ -112,6 +116,8 @@ conv3x3_mfma_f4_kernel(
     constexpr bool kRawTranspose = raw_transposed(SPT, RM, NT, FULLT);
     constexpr int kRawPitch = raw_pitch(NT);
     int* lds_raw = reinterpret_cast<int*>(lds_thr + NT * 32);
+    // WIN_MAXSAVE: where the four waves' sums of a window meet, [wave][NT][2][64 lanes] 128-bit words (pairs of int16)
+    v4i* lds_win = reinterpret_cast<v4i*>(lds_thr + NT * 32);
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -172,8 +178,8 @@ conv3x3_mfma_f4_kernel(
     // a wave's work items: output pixels, or 2x2 windows of them (row width `roww`)
     const int roww = kWin ? p.PW / 2 : p.PW;
     const int npix = kWin ? (p.PH / 2) * (p.PW / 2) : p.PH * p.PW;
-    int pi = stream * kWaves + wave;
-    const int dpi = pix_streams * kWaves;
+    int pi = PSAVE ? stream : stream * kWaves + wave;  // (a window is taken by the whole workgroup)
+    const int dpi = PSAVE ? pix_streams : pix_streams * kWaves;
     // Item pi stands for row pi / roww and column (pi % roww + row) % roww.  The skew by the row keeps
     // a wave from staying in one column when its stride is a multiple of the row width (then the waves
     // that own a border column, whose tiles are slower, would finish long after the others).
@@ -506,7 +512,6 @@ conv3x3_mfma_f4_kernel(
     // One channel tile of the epilogue.  FAST (wave-uniform choice): all 32 channels exist and, with a
     // residual, all of them receive it, so no per-channel condition is evaluated at all.
     uint32_t poolw[MT][NT];  // POOL: OR of the window's words so far
-    uint32_t winmax[PSAVE ? MT * NT : 1][8];  // PSAVE: maximum of the window's sums so far, as pairs of int16
     auto epilogue_tile = [&](auto fast_tag, int nt, unsigned pix, unsigned bits_pix, int (*rv)[NW],
                              int sub) __attribute__((always_inline)) {
         constexpr bool FAST = decltype(fast_tag)::value;
@@ -583,45 +588,15 @@ conv3x3_mfma_f4_kernel(
                 for (int v = 0; v < 16; ++v) t[v] = __uint_as_float(tb[v]);
                 if constexpr (PSAVE) {
                     // Only the window's maximum is saved.  The low 16 bits of a bit pattern are the sum as int16 (the
-                    // host admits this instantiation only for 12- and 16-bit outputs): two sums per word, packed maximum.
-                    typedef short s2_t __attribute__((ext_vector_type(2)));
-                    uint32_t* wm = winmax[mt * NT + nt];
+                    // host admits this instantiation only for 12- and 16-bit outputs): two sums per word, handed to the
+                    // wave that takes this channel tile's maximum (window_maximum below).
+                    uint32_t pr[8];
 #pragma unroll
-                    for (int k = 0; k < 8; ++k) {
-                        const uint32_t pr = __builtin_amdgcn_perm(__float_as_uint(t[2 * k + 1]), __float_as_uint(t[2 * k]), 0x05040100u);
-                        wm[k] = sub == 0 ? pr
-                                         : __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(s2_t, wm[k]),
-                                                                                                  __builtin_bit_cast(s2_t, pr)));
-                    }
-                    if (sub == 3) {  // (uniform) `pix` is the window's index in the pooled tensor
-                        v4i q[2];
-                        if (rout_fmt == TCBNN_RES_I12) {
-                            int un[16];
-#pragma unroll
-                            for (int k = 0; k < 8; ++k) un[2 * k] = (int)wm[k], un[2 * k + 1] = (int)(wm[k] >> 16);
-                            uint32_t d[6];
-                            i12_pack8(un, d[0], d[1], d[2]);
-                            i12_pack8(un + 8, d[3], d[4], d[5]);
-                            const unsigned so = (pix * (unsigned)((p.N + 15) / 16) + (unsigned)((n0 + nt * 32) / 16)) * g12_b;
-                            const unsigned vo = b_ok ? (unsigned)h * g12_b + (unsigned)b * 16u : kOutOfRange;
-                            const unsigned vo2 = b_ok ? (unsigned)h * g12_b + grp_b + (unsigned)b * 8u : kOutOfRange;
-                            q[0] = v4i{(int)d[0], (int)d[1], (int)d[2], (int)d[3]};
-                            typedef int v2i_t __attribute__((ext_vector_type(2)));
-                            const v2i_t q2 = {(int)d[4], (int)d[5]};
-                            __builtin_amdgcn_raw_buffer_store_b128(q[0], r_rout, (int)vo, (int)so, kResStoreAux);
-                            __builtin_amdgcn_raw_buffer_store_b64(q2, r_rout, (int)vo2, (int)so, kResStoreAux);
-                            asm volatile("s_nop 4" ::"v"(q[0]), "v"(q2));  // see the 128-bit store note below
-                        } else {  // TCBNN_RES_I16
-                            const unsigned so = (pix * (unsigned)((p.N + 7) / 8) + (unsigned)((n0 + nt * 32) / 8)) * grp_b;
-                            const unsigned vo = b_ok ? ((unsigned)(2 * h) * (unsigned)p.B + (unsigned)b) * 16u : kOutOfRange;
-#pragma unroll
-                            for (int g = 0; g < 2; ++g) {
-                                q[g] = v4i{(int)wm[4 * g], (int)wm[4 * g + 1], (int)wm[4 * g + 2], (int)wm[4 * g + 3]};
-                                __builtin_amdgcn_raw_buffer_store_b128(q[g], r_rout, (int)vo, (int)(so + (unsigned)g * grp_b), kResStoreAux);
-                            }
-                            asm volatile("s_nop 4" ::"v"(q[0]), "v"(q[1]));
-                        }
-                    }
+                    for (int k = 0; k < 8; ++k)
+                        pr[k] = __builtin_amdgcn_perm(__float_as_uint(t[2 * k + 1]), __float_as_uint(t[2 * k]), 0x05040100u);
+                    v4i* x = lds_win + ((wave * NT + nt) * 2) * 64 + lane;
+                    x[0] = v4i{(int)pr[0], (int)pr[1], (int)pr[2], (int)pr[3]};
+                    x[64] = v4i{(int)pr[4], (int)pr[5], (int)pr[6], (int)pr[7]};
                 } else if (rout != nullptr) {
                     // the value to store is in the low bits of t's bit pattern (see the 128-bit store note below)
                     v4i q[4];
@@ -837,10 +812,64 @@ conv3x3_mfma_f4_kernel(
         }
     };
 
+    // WIN_MAXSAVE, waves 0 .. NT-1 after the workgroup's barrier: the element-wise maximum of the four pixels' sums
+    // of channel tile `nt` (packed 16-bit maxima on the pairs), stored in the tensor's 12- or 16-bit format at
+    // window `pix` of the pooled tensor.  A lane reads what the same lane of each wave wrote: its own image and channels.
+    auto window_maximum = [&](int nt, unsigned pix) __attribute__((always_inline)) {
+        if constexpr (PSAVE) {
+            typedef short s2_t __attribute__((ext_vector_type(2)));
+            uint32_t wm[8];
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                const v4i* x = lds_win + ((w * NT + nt) * 2) * 64 + lane;
+                const v4i lo = x[0], hi = x[64];
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    const uint32_t pr = (uint32_t)(k < 4 ? lo[k] : hi[k - 4]);
+                    wm[k] = w == 0 ? pr
+                                   : __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(s2_t, wm[k]),
+                                                                                            __builtin_bit_cast(s2_t, pr)));
+                }
+            }
+            const int b = bimg[0];
+            const bool b_ok = b < p.B;
+            v4i q[2];
+            if (rout_fmt == TCBNN_RES_I12) {
+                int un[16];
+#pragma unroll
+                for (int k = 0; k < 8; ++k) un[2 * k] = (int)wm[k], un[2 * k + 1] = (int)(wm[k] >> 16);
+                uint32_t d[6];
+                i12_pack8(un, d[0], d[1], d[2]);
+                i12_pack8(un + 8, d[3], d[4], d[5]);
+                const unsigned so = (pix * (unsigned)((p.N + 15) / 16) + (unsigned)((n0 + nt * 32) / 16)) * g12_b;
+                const unsigned vo = b_ok ? (unsigned)h * g12_b + (unsigned)b * 16u : kOutOfRange;
+                const unsigned vo2 = b_ok ? (unsigned)h * g12_b + grp_b + (unsigned)b * 8u : kOutOfRange;
+                q[0] = v4i{(int)d[0], (int)d[1], (int)d[2], (int)d[3]};
+                typedef int v2i_t __attribute__((ext_vector_type(2)));
+                const v2i_t q2 = {(int)d[4], (int)d[5]};
+                __builtin_amdgcn_raw_buffer_store_b128(q[0], r_rout, (int)vo, (int)so, kResStoreAux);
+                __builtin_amdgcn_raw_buffer_store_b64(q2, r_rout, (int)vo2, (int)so, kResStoreAux);
+                asm volatile("s_nop 4" ::"v"(q[0]), "v"(q2));  // see the 128-bit store note in epilogue_tile
+            } else {  // TCBNN_RES_I16
+                const unsigned so = (pix * (unsigned)((p.N + 7) / 8) + (unsigned)((n0 + nt * 32) / 8)) * grp_b;
+                const unsigned vo = b_ok ? ((unsigned)(2 * h) * (unsigned)p.B + (unsigned)b) * 16u : kOutOfRange;
+#pragma unroll
+                for (int g = 0; g < 2; ++g) {
+                    q[g] = v4i{(int)wm[4 * g], (int)wm[4 * g + 1], (int)wm[4 * g + 2], (int)wm[4 * g + 3]};
+                    __builtin_amdgcn_raw_buffer_store_b128(q[g], r_rout, (int)vo, (int)(so + (unsigned)g * grp_b), kResStoreAux);
+                }
+                asm volatile("s_nop 4" ::"v"(q[0]), "v"(q[1]));
+            }
+        }
+    };
+
     // (yy, xx): the output pixel, or the window when pooled (sub = pixel of the window, 3 = last)
-    // PSAVE: the bits belong to the window's pixel `sub`, the saved residual to the window
+    // PSAVE: the bits belong to the window's pixel `sub` (this wave's), the saved residual to the window
     auto epilogue = [&](int yy, int xx, int sub, int (*rv)[NW]) __attribute__((always_inline)) {
         const unsigned pix = (unsigned)yy * (unsigned)roww + (unsigned)xx;
+        // PSAVE: the previous window's maxima have been read (every wave of the workgroup runs the same sequence of
+        // windows, so the barriers match; plain s_barrier: no wait for the global requests in flight)
+        if constexpr (PSAVE) asm volatile("s_barrier" ::: "memory");
         const unsigned bpix = PSAVE ? (unsigned)(2 * yy + (sub >> 1)) * (unsigned)p.PW + (unsigned)(2 * xx + (sub & 1)) : pix;
         const unsigned bits_pix = bpix * (unsigned)p.bits_pix_stride * 4u;  // uniform
         if constexpr (kRawTranspose) {  // (the host only picks this instantiation for 16-byte aligned outputs)
@@ -857,6 +886,10 @@ conv3x3_mfma_f4_kernel(
                 epilogue_tile(std::true_type{}, nt, pix, bits_pix, rv, sub);
             else
                 epilogue_tile(std::false_type{}, nt, pix, bits_pix, rv, sub);
+        }
+        if constexpr (PSAVE) {
+            asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // the four pixels' sums are in LDS
+            if (wave < NT) window_maximum(wave, pix);                       // (uniform per wave)
         }
         if (RM != RM_RAW && ng == n_groups - 1 && (!POOL || sub == 3)) {  // zero the pixel's padding words
 #pragma unroll
@@ -882,7 +915,7 @@ conv3x3_mfma_f4_kernel(
     auto advance = [&](Cursor& c) __attribute__((always_inline)) {
         if (++c.chunk == NCH) {
             c.chunk = 0;
-            if constexpr (kWin) {
+            if constexpr (POOL) {  // (WIN_MAXSAVE: a wave stays on its pixel of the window)
                 if (++c.sub < 4) return;
                 c.sub = 0;
             }
@@ -904,7 +937,7 @@ conv3x3_mfma_f4_kernel(
     uint32_t buf[NB][TPC * SPT][MT];
     uint32_t msk[NB];
     int rv[kAhead ? NB : 1][NRV][NW];
-    Cursor cc = {pi, y, (xr + y) % roww, 0, 0, xr};  // chunk being multiplied
+    Cursor cc = {pi, y, (xr + y) % roww, 0, PSAVE ? wave : 0, xr};  // chunk being multiplied
     Cursor lc = cc;             // chunk being requested (LOOK steps ahead)
 #pragma unroll
     for (int i = 0; i < LOOK; ++i) {
@@ -1062,8 +1095,10 @@ int launch_f(const BgemmParams& p, hipStream_t stream) {
     constexpr int NQ = 9 * SPT;
     constexpr int kWaves = waves_of(SPT, NT), kThreads = 64 * kWaves;
     constexpr bool kRawTranspose = raw_transposed(SPT, RM, NT, FULLT);
+    constexpr bool kWgItems = WIN == WIN_MAXSAVE;  // a work item (window) is taken by a whole workgroup
     const size_t lds_bytes = (size_t)NQ * NT * 64 * 16 + NT * 32 * sizeof(float) +
-                             (kRawTranspose ? (size_t)kWaves * 32 * raw_pitch(NT) * sizeof(int) : 0);
+                             (kRawTranspose ? (size_t)kWaves * 32 * raw_pitch(NT) * sizeof(int) : 0) +
+                             (kWgItems ? (size_t)kWaves * NT * 2 * 64 * 16 : 0);
     // Per instantiation and device, set up by the first launch there: the dynamic LDS limit, and how many of its
     // workgroups a CU holds at once (registers and LDS).  Atomics only so that two host threads that both find the
     // entry empty do no harm (both store the same value).
@@ -1086,7 +1121,7 @@ int launch_f(const BgemmParams& p, hipStream_t stream) {
     const int n_groups = (p.N + 32 * NT - 1) / (32 * NT);
     const int b_groups = (p.B + 32 * MT - 1) / (32 * MT);
     const int items = WIN != WIN_NONE ? (p.PH / 2) * (p.PW / 2) : p.PH * p.PW;  // pixels, or 2x2 windows of them
-    const int quads = (items + kWaves - 1) / kWaves;  // items per wave of a pixel stream
+    const int quads = kWgItems ? items : (items + kWaves - 1) / kWaves;  // items per wave of a pixel stream
     // Persistent workgroups, all resident at once: two per CU (three for residual layers), fewer
     // when registers or LDS hold fewer.  Measured on every layer of ResNet-18 at batch 256: more, shorter-lived
     // workgroups stage the weights more often and lose; and a grid even slightly larger than the resident slots
@@ -1107,7 +1142,7 @@ int launch_f(const BgemmParams& p, hipStream_t stream) {
     const TensorBytes tb = tensor_bytes(p);
     if (blocks > 0x7fffffffLL || b_groups > 65535 || best > 65535) return fail(TCBNN_EINVAL, "conv3x3: grid too large");
     // a wave's stride over the work items, split into rows and columns once here instead of in every wave
-    const int roww = WIN != WIN_NONE ? p.PW / 2 : p.PW, dpi = best * kWaves;
+    const int roww = WIN != WIN_NONE ? p.PW / 2 : p.PW, dpi = kWgItems ? best : best * kWaves;
     const int dy = dpi / roww, dx = dpi % roww, dxs = (dx + dy) % roww;
     hipLaunchKernelGGL((conv3x3_mfma_f4_kernel<SPT, RM, MT, NT, RF, WIN, FULLT>),
                        dim3((unsigned)n_groups, (unsigned)b_groups, (unsigned)best), dim3(kThreads), lds_bytes,
@@ -1147,11 +1182,9 @@ struct Pick {
 constexpr int pick_nt(int spt, int rm) {
     return rm == RM_POOLED ? (spt >= 6 ? 1 : 2) : (rm == RM_RAW ? (spt >= 3 && spt < 8 ? 1 : 2) : 2);
 }
-// Channel tiles per wave when the saved residual is the window maximum: a work item is then a whole window (four
-// tiles), and from Cin = 128 on the launches have so few of them per wave that finer tiles balance the waves better
-// (ResNet-18 at batch 256: 26.0 -> 25.0 us at Cin = 128, 23.2 -> 22.0 us at Cin = 256; at Cin = 64, where the tile is
-// bound by its VALU work, 30.5 -> 34.4 us).
-constexpr int pick_nt_maxsave(int spt) { return spt >= 2 && spt <= 4 ? 1 : 2; }
+// Channel tiles per wave when the saved residual is the window maximum (the four waves of a workgroup then share a
+// window): two where the staged weights leave room for three workgroups per CU, one from Cin = 192 on.
+constexpr int pick_nt_maxsave(int spt) { return spt <= 2 ? 2 : 1; }
 constexpr int pick_mt(int spt, int rm) {
     return rm == RM_RAW ? (spt >= 8 ? 1 : 2) : (rm == RM_NONE ? (spt >= 6 ? 1 : 2) : 1);
 }
