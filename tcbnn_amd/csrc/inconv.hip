@@ -123,6 +123,77 @@ __device__ __forceinline__ void add_indexed8x2(float* a, float* b, v8f ca, v8f c
 typedef uint32_t u16v __attribute__((ext_vector_type(16)));
 typedef int v4i_t __attribute__((ext_vector_type(4)));
 
+// The epilogue both first-layer kernels share, for a lane's 32 consecutive channels (word `wi`) of one image and pixel.
+// Output word: bit n (MSB first) = !(acc[n] < bn[32 wi + n]), i.e. the inverted sign of acc - bn (equal operands give
+// +0; a NaN threshold counts as -inf: the bit is 1 either way).
+__device__ __forceinline__ uint32_t inconv_threshold_word(const float* acc, const float* __restrict__ bn, int wi, int O) {
+    uint32_t word = 0;
+    if (wi * 32 + 32 <= O) {  // uniform: full channel tile
+#pragma unroll
+        for (int n = 0; n < 32; ++n) {
+            // (the NaN test on the threshold's bits: wave-uniform, so it stays on the scalar unit)
+            const uint32_t tb = __float_as_uint(bn[wi * 32 + n]);
+            const float t = __uint_as_float((tb & 0x7fffffffu) > 0x7f800000u ? 0xff800000u : tb);
+            word = __builtin_amdgcn_alignbit(word, __float_as_uint(acc[n] - t), 31);
+        }
+        return ~word;
+    }
+#pragma unroll
+    for (int n = 0; n < 32; ++n) {
+        const int ch = wi * 32 + n;
+        if (ch < O) word |= (acc[n] < bn[ch] ? 0u : 1u) << (31 - n);
+    }
+    return word;
+}
+// Saved residual: (int)acc of the 32 channels in the tensor's format; 16 bytes per (channel group, image) (4 int32 or
+// 8 int16), or 24 per group of 16 channels at 12 bits; channels past O are stored as 0, groups past O not at all.
+// Streaming stores: the tensor (77-103 MB for ResNet-18 at batch 256) is far larger than the caches and is read two
+// launches later.
+__device__ __forceinline__ void inconv_store_residual(const float* acc, int32_t* __restrict__ res, int fmt, size_t pix,
+                                                      int wi, int O, int B, int b) {
+    int r32[32];
+#pragma unroll
+    for (int n = 0; n < 32; ++n) r32[n] = (int)acc[n];
+    if (wi * 32 + 32 > O) {  // uniform
+#pragma unroll
+        for (int n = 0; n < 32; ++n) r32[n] = wi * 32 + n < O ? r32[n] : 0;
+    }
+    v4i_t* __restrict__ dst = reinterpret_cast<v4i_t*>(res);
+    if (fmt == TCBNN_RES_I12) {  // two groups of 16 channels: 16 + 8 bytes each
+        typedef int v2i_t __attribute__((ext_vector_type(2)));
+        uint32_t* __restrict__ w = reinterpret_cast<uint32_t*>(res);
+        const size_t G = (size_t)((O + 15) / 16);
+#pragma unroll
+        for (int g = 0; g < 2; ++g)
+            if (wi * 32 + 16 * g < O) {
+                uint32_t d[6];
+                i12_pack8(&r32[16 * g], d[0], d[1], d[2]);
+                i12_pack8(&r32[16 * g + 8], d[3], d[4], d[5]);
+                __builtin_nontemporal_store(v4i_t{(int)d[0], (int)d[1], (int)d[2], (int)d[3]},
+                                            reinterpret_cast<v4i_t*>(w + i12_word_index(pix, G, wi * 2 + g, B, b, 0)));
+                __builtin_nontemporal_store(v2i_t{(int)d[4], (int)d[5]},
+                                            reinterpret_cast<v2i_t*>(w + i12_word_index(pix, G, wi * 2 + g, B, b, 4)));
+            }
+    } else if (fmt == TCBNN_RES_I16) {
+        const size_t g0 = (pix * ((O + 7) / 8) + wi * 4) * B + b;
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+            if (wi * 32 + 8 * g < O)
+                __builtin_nontemporal_store(v4i_t{(r32[8 * g] & 0xffff) | (r32[8 * g + 1] << 16),
+                                                  (r32[8 * g + 2] & 0xffff) | (r32[8 * g + 3] << 16),
+                                                  (r32[8 * g + 4] & 0xffff) | (r32[8 * g + 5] << 16),
+                                                  (r32[8 * g + 6] & 0xffff) | (r32[8 * g + 7] << 16)},
+                                            dst + g0 + (size_t)g * B);
+    } else {
+        const size_t g0 = (pix * ((O + 3) / 4) + wi * 8) * B + b;
+#pragma unroll
+        for (int g = 0; g < 8; ++g)
+            if (wi * 32 + 4 * g < O)
+                __builtin_nontemporal_store(v4i_t{r32[4 * g], r32[4 * g + 1], r32[4 * g + 2], r32[4 * g + 3]},
+                                            dst + g0 + (size_t)g * B);
+    }
+}
+
 // Staging of one filter row: the 3 x 64 (channel, image) row segments of ncols floats each.
 //   ROWS = true: a wave takes rpw segments at a time (a multiple of 3 for ncols <= 21, else 2), lanes
 //     running along the segment; segments are numbered in memory order (image * 3 + channel),
@@ -331,78 +402,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS &
                 if (px == 1 && !xb_ok) continue;
                 const float* acc = px == 0 ? acca : accb;
                 const size_t pix = (size_t)yc * p.PW + xa + px;
-                uint32_t word = 0;
-                if (wi * 32 + 32 <= p.O) {  // uniform: full channel tile
-                    // bit = !(acc < bn) = inverted sign of acc - bn (equal operands give +0; a NaN threshold
-                    // counts as -inf: the bit is 1 either way)
-#pragma unroll
-                    for (int n = 0; n < 32; ++n) {
-                        // (the NaN test on the threshold's bits: wave-uniform, so it stays on the scalar unit)
-                        const uint32_t tb = __float_as_uint(bn[wi * 32 + n]);
-                        const float t = __uint_as_float((tb & 0x7fffffffu) > 0x7f800000u ? 0xff800000u : tb);
-                        word = __builtin_amdgcn_alignbit(word, __float_as_uint(acc[n] - t), 31);
-                    }
-                    word = ~word;
-                } else {
-#pragma unroll
-                    for (int n = 0; n < 32; ++n) {
-                        const int ch = wi * 32 + n;
-                        if (ch < p.O) word |= (acc[n] < bn[ch] ? 0u : 1u) << (31 - n);
-                    }
-                }
+                const uint32_t word = inconv_threshold_word(acc, bn, wi, p.O);
                 if constexpr (POOLED) {
                     pooled[px] |= word;
                     continue;
                 }
                 out[(pix * p.ow + wi) * p.B + b] = word;
-                if (res != nullptr) {
-                    // 16 bytes per (channel group, image): 4 int32 or 8 int16; channels past O are 0
-                    int r32[32];
-#pragma unroll
-                    for (int n = 0; n < 32; ++n) r32[n] = (int)acc[n];
-                    if (wi * 32 + 32 > p.O) {  // uniform: channels past O are stored as 0
-#pragma unroll
-                        for (int n = 0; n < 32; ++n) r32[n] = wi * 32 + n < p.O ? r32[n] : 0;
-                    }
-                    // streaming stores: the tensor (103 MB at batch 256) is far larger than the caches and is
-                    // read two launches later
-                    v4i_t* __restrict__ dst = reinterpret_cast<v4i_t*>(res);
-                    if (p.res_fmt == TCBNN_RES_I12) {  // two groups of 16 channels: 16 + 8 bytes each
-                        typedef int v2i_t __attribute__((ext_vector_type(2)));
-                        uint32_t* __restrict__ w = reinterpret_cast<uint32_t*>(res);
-                        const size_t G = (size_t)((p.O + 15) / 16);
-#pragma unroll
-                        for (int g = 0; g < 2; ++g)
-                            if (wi * 32 + 16 * g < p.O) {
-                                uint32_t d[6];
-                                i12_pack8(&r32[16 * g], d[0], d[1], d[2]);
-                                i12_pack8(&r32[16 * g + 8], d[3], d[4], d[5]);
-                                __builtin_nontemporal_store(v4i_t{(int)d[0], (int)d[1], (int)d[2], (int)d[3]},
-                                                            reinterpret_cast<v4i_t*>(w + i12_word_index(pix, G, wi * 2 + g, p.B, b, 0)));
-                                __builtin_nontemporal_store(v2i_t{(int)d[4], (int)d[5]},
-                                                            reinterpret_cast<v2i_t*>(w + i12_word_index(pix, G, wi * 2 + g, p.B, b, 4)));
-                            }
-                    } else if (p.res_fmt == TCBNN_RES_I16) {
-                        const size_t g0 = (pix * ((p.O + 7) / 8) + wi * 4) * p.B + b;
-#pragma unroll
-                        for (int g = 0; g < 4; ++g)
-                            if (wi * 32 + 8 * g < p.O)
-                                __builtin_nontemporal_store(
-                                    v4i_t{(r32[8 * g] & 0xffff) | (r32[8 * g + 1] << 16),
-                                          (r32[8 * g + 2] & 0xffff) | (r32[8 * g + 3] << 16),
-                                          (r32[8 * g + 4] & 0xffff) | (r32[8 * g + 5] << 16),
-                                          (r32[8 * g + 6] & 0xffff) | (r32[8 * g + 7] << 16)},
-                                    dst + g0 + (size_t)g * p.B);
-                    } else {
-                        const size_t g0 = (pix * ((p.O + 3) / 4) + wi * 8) * p.B + b;
-#pragma unroll
-                        for (int g = 0; g < 8; ++g)
-                            if (wi * 32 + 4 * g < p.O)
-                                __builtin_nontemporal_store(
-                                    v4i_t{r32[4 * g], r32[4 * g + 1], r32[4 * g + 2], r32[4 * g + 3]},
-                                    dst + g0 + (size_t)g * p.B);
-                    }
-                }
+                if (res != nullptr) inconv_store_residual(acc, res, p.res_fmt, pix, wi, p.O, p.B, b);
             }
         }
       }
@@ -521,69 +527,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
                 if (px == 1 && !xb_ok) continue;
                 const float* acc = px == 0 ? acca : accb;
                 const size_t pix = (size_t)y * p.PW + xa + px;
-                uint32_t word = 0;
-                if (wi * 32 + 32 <= p.O) {  // uniform: full channel tile
-#pragma unroll
-                    for (int n = 0; n < 32; ++n) {
-                        // (the NaN test on the threshold's bits: wave-uniform, so it stays on the scalar unit)
-                        const uint32_t tb = __float_as_uint(bn[wi * 32 + n]);
-                        const float t = __uint_as_float((tb & 0x7fffffffu) > 0x7f800000u ? 0xff800000u : tb);
-                        word = __builtin_amdgcn_alignbit(word, __float_as_uint(acc[n] - t), 31);
-                    }
-                    word = ~word;
-                } else {
-#pragma unroll
-                    for (int n = 0; n < 32; ++n) {
-                        const int ch = wi * 32 + n;
-                        if (ch < p.O) word |= (acc[n] < bn[ch] ? 0u : 1u) << (31 - n);
-                    }
-                }
+                const uint32_t word = inconv_threshold_word(acc, bn, wi, p.O);
                 out[(pix * p.ow + wi) * p.B + b] = word;
-                if (res != nullptr) {
-                    int r32[32];
-#pragma unroll
-                    for (int n = 0; n < 32; ++n) r32[n] = (int)acc[n];
-                    if (wi * 32 + 32 > p.O) {  // uniform: channels past O are stored as 0
-#pragma unroll
-                        for (int n = 0; n < 32; ++n) r32[n] = wi * 32 + n < p.O ? r32[n] : 0;
-                    }
-                    v4i_t* __restrict__ dst = reinterpret_cast<v4i_t*>(res);
-                    if (p.res_fmt == TCBNN_RES_I12) {
-                        typedef int v2i_t __attribute__((ext_vector_type(2)));
-                        uint32_t* __restrict__ w = reinterpret_cast<uint32_t*>(res);
-                        const size_t G = (size_t)((p.O + 15) / 16);
-#pragma unroll
-                        for (int gg = 0; gg < 2; ++gg)
-                            if (wi * 32 + 16 * gg < p.O) {
-                                uint32_t d[6];
-                                i12_pack8(&r32[16 * gg], d[0], d[1], d[2]);
-                                i12_pack8(&r32[16 * gg + 8], d[3], d[4], d[5]);
-                                __builtin_nontemporal_store(v4i_t{(int)d[0], (int)d[1], (int)d[2], (int)d[3]},
-                                                            reinterpret_cast<v4i_t*>(w + i12_word_index(pix, G, wi * 2 + gg, p.B, b, 0)));
-                                __builtin_nontemporal_store(v2i_t{(int)d[4], (int)d[5]},
-                                                            reinterpret_cast<v2i_t*>(w + i12_word_index(pix, G, wi * 2 + gg, p.B, b, 4)));
-                            }
-                    } else if (p.res_fmt == TCBNN_RES_I16) {
-                        const size_t g0 = (pix * ((p.O + 7) / 8) + wi * 4) * p.B + b;
-#pragma unroll
-                        for (int gg = 0; gg < 4; ++gg)
-                            if (wi * 32 + 8 * gg < p.O)
-                                __builtin_nontemporal_store(
-                                    v4i_t{(r32[8 * gg] & 0xffff) | (r32[8 * gg + 1] << 16),
-                                          (r32[8 * gg + 2] & 0xffff) | (r32[8 * gg + 3] << 16),
-                                          (r32[8 * gg + 4] & 0xffff) | (r32[8 * gg + 5] << 16),
-                                          (r32[8 * gg + 6] & 0xffff) | (r32[8 * gg + 7] << 16)},
-                                    dst + g0 + (size_t)gg * p.B);
-                    } else {
-                        const size_t g0 = (pix * ((p.O + 3) / 4) + wi * 8) * p.B + b;
-#pragma unroll
-                        for (int gg = 0; gg < 8; ++gg)
-                            if (wi * 32 + 4 * gg < p.O)
-                                __builtin_nontemporal_store(
-                                    v4i_t{r32[4 * gg], r32[4 * gg + 1], r32[4 * gg + 2], r32[4 * gg + 3]},
-                                    dst + g0 + (size_t)gg * p.B);
-                    }
-                }
+                if (res != nullptr) inconv_store_residual(acc, res, p.res_fmt, pix, wi, p.O, p.B, b);
             }
         }
     }
