@@ -72,6 +72,9 @@ constexpr bool raw_transposed(int spt, int rm, int nt, bool fullt) {
 // Waves per SIMD the register allocator is asked to make room for (256 registers per lane: the plain layers
 // use them for two image tiles and two channel tiles, the residual layers for operands in flight).
 constexpr int kWavesPerSimd = 2;
+// ... except where a fourth wave per SIMD is two registers away (one register spilled): Cin = 64 layers that save
+// the window maximum
+constexpr int waves_per_simd(int spt, int rm, int win) { return spt == 1 && rm == 1 && win == 2 ? 4 : kWavesPerSimd; }
 
 // SPT = k-steps (64 bits) per filter tap = Cin / 64; MT = 32-image tiles per wave (2 for plain
 // layers, 1 for residual layers); NT = 32-channel tiles per wave; RF = TCBNN_RES_* format of the
@@ -89,7 +92,7 @@ constexpr int kWavesPerSimd = 2;
 // every launch, and the networks' channel counts are multiples of 64).
 constexpr int WIN_NONE = 0, WIN_ORPOOL = 1, WIN_MAXSAVE = 2;
 template <int SPT, int RM, int MT, int NT, int RF, int WIN, bool FULLT>
-__global__ __launch_bounds__(64 * waves_of(SPT, NT)) __attribute__((amdgpu_waves_per_eu(kWavesPerSimd))) void
+__global__ __launch_bounds__(64 * waves_of(SPT, NT)) __attribute__((amdgpu_waves_per_eu(waves_per_simd(SPT, RM, WIN)))) void
 conv3x3_mfma_f4_kernel(
     const BgemmParams p, const uint32_t* __restrict__ act, const uint32_t* __restrict__ wgt,
     const float* __restrict__ bnp, const int32_t* __restrict__ rin, int32_t* __restrict__ rout, int res_lim,
@@ -1129,10 +1132,12 @@ int launch_f(const BgemmParams& p, hipStream_t stream) {
     // and 7 x 7 layers ran 10-18 % longer with 1.5 rounds than with one round of workgroups that each take two
     // items per wave).  So: as many pixel streams as fit in one round, never more.
     static const int wg_env = getenv("TCBNN_WG_PER_CU") ? atoi(getenv("TCBNN_WG_PER_CU")) : 0;  // tuning switch
-    // Residual layers with one image tile per wave are bound by HBM: a third workgroup per CU, where registers and
-    // LDS hold one (`resident`), keeps more requests in flight (stage-1 and stage-2 layers of ResNet-18: -3 to -8 %).
+    // Residual layers with one image tile per wave are bound by memory and by their epilogue's latency chains: a third
+    // workgroup per CU, where registers and LDS hold one (`resident`), keeps more requests in flight (stage-1 and
+    // stage-2 layers of ResNet-18: -3 to -8 %); a fourth where the kernel was compiled for it (L1B2C2 at batch 256:
+    // 28.0 -> 26.5 us).
     constexpr bool kResLayer = RM == RM_PLAIN || RM == RM_POOLED;
-    const int wg_want = wg_env > 0 ? wg_env : (kResLayer && MT == 1 ? 3 : 2);
+    const int wg_want = wg_env > 0 ? wg_env : (kResLayer && MT == 1 ? (waves_per_simd(SPT, RM, WIN) == 4 ? 4 : 3) : 2);
     const int wg_per_cu = std::max(1, std::min(wg_want, resident));
     const int best = std::max(1, std::min(cus * wg_per_cu / (n_groups * b_groups), quads));
     // channels that receive an injected residual: o < residual_channels, and only those the
