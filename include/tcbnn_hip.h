@@ -29,7 +29,11 @@
  *                                                 (kernel.cuh:798-808): an FC activation
  *   packed weights   : uint32 [NPAD32][KWTOT]     one row per output neuron/channel,
  *                                                 FC: KWTOT = KW128; conv: KWTOT = R*S*CW,
- *                                                 K index = (r*S+s)*32*CW + c; rows >= N are 0
+ *                                                 K index = (r*S+s)*32*CW + c; rows >= N are 0;
+ *                                                 FC weights and 3x3 filters are followed by the
+ *                                                 same words in the order the matrix-core kernels'
+ *                                                 lanes load them (tcbnn_fc_weight_words,
+ *                                                 tcbnn_conv_filter_words give the total)
  *   residual tensors : TCBNN_RES_I32: int32 [P][Q][ceil(O/4)][B][4]; TCBNN_RES_I16: int16
  *                      [P][Q][ceil(O/8)][B][8] for tensors whose values provably fit 16 bits;
  *                      TCBNN_RES_I12: per pixel and group of 16 channels uint32 [B][4] then
@@ -101,7 +105,7 @@ int tcbnn_conv_out(int in_size, int filter, int stride, int padding, int pool);
 /* Word counts of the engine layouts above. */
 size_t tcbnn_fc_act_words(int batch, int features);                    /* B*KW128          */
 size_t tcbnn_conv_act_words(int height, int width, int batch, int ch); /* H*W*B*CW         */
-size_t tcbnn_fc_weight_words(int in_features, int out_features);       /* NPAD32*KW128     */
+size_t tcbnn_fc_weight_words(int in_features, int out_features);       /* NPAD32*KW128 rows + the lane-order copy, NPAD32*8*ceil(KW128/8) */
 size_t tcbnn_conv_filter_words(int r, int s, int in_ch, int out_ch);   /* NPAD32*R*S*CW, x2 for 3x3 filters with
                                                                            Cin = 64/128/192/256/384/512: they carry a
                                                                            copy in MFMA lane order after the bit rows */
@@ -129,8 +133,9 @@ int tcbnn_residual_format_for_bound(int bound);
 int tcbnn_residual_format_narrowest(int bound, int batch);
 
 /* ------------------------------------------------- one-time weight packing */
-/* fp32 [K][N] (param.h:58-59) -> packed [NPAD32][KW128].  Replaces
- * PackFcWeight128FMT (param.h:44-63). */
+/* fp32 [K][N] (param.h:58-59) -> packed [NPAD32][KW128], followed by the same words in the FP4 FC kernel's lane
+ * order, uint32 [NPAD32/32][ceil(KW128/8)][64][4].  `packed` holds tcbnn_fc_weight_words(...) words; the FC and
+ * output layers take only buffers written by this function.  Replaces PackFcWeight128FMT (param.h:44-63). */
 int tcbnn_pack_fc_weight(const float* weight_kn, uint32_t* packed, int in_features,
                          int out_features, void* stream);
 /* fp32 HWIO [R][S][C][O] (param.h:573-574) -> packed [OPAD32][R*S][CW] (+ the FP4 fragment copy

@@ -212,6 +212,13 @@ inline bool filter_has_fragments(int r, int s, int in_ch) {
     return r == 3 && s == 3 &&
            (in_ch == 64 || in_ch == 128 || in_ch == 192 || in_ch == 256 || in_ch == 384 || in_ch == 512);
 }
+// Packed FC weights carry, after their [NPAD32][KW128] sign-bit rows, the same words in the order the FP4 matrix-core
+// FC kernel's lanes load them: uint32 [NPAD32/32][ceil(KW128/8)][64 lanes][4] (lane (j, h) of K group g holds words
+// 8g + 4h .. 8g + 4h + 3 of neuron 32 tile + row_to_channel(j); words past KW128 are 0), written once by
+// tcbnn_pack_fc_weight: a wave then loads a group with ONE contiguous 1 KB request instead of 16 bytes from each of 64
+// rows.
+__host__ __device__ inline size_t fc_weight_row_words(int npad, int kw) { return (size_t)npad * kw; }
+__host__ __device__ inline size_t fc_weight_lane_words(int npad, int kw) { return (size_t)npad * 8 * ((kw + 7) / 8); }
 // persistent FP4 matrix-core kernel for 3x3 convolutions with Cin = 64 / 128 / 192 / 256 / 384 / 512
 bool conv3x3_mfma_applicable(const BgemmParams& p);
 int launch_conv3x3_mfma(const BgemmParams& p, hipStream_t stream);

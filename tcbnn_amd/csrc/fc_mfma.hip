@@ -43,22 +43,23 @@ __global__ __launch_bounds__(64 * kMaxWaves) void fc_mfma_f4_kernel(
     const int b = b0 + j;
     const int bl = min(b, p.B - 1);
     const int cw = p.cw;  // words per image / per neuron; a multiple of 4
-    // rows >= N of the packed weights exist and are zero (their outputs are discarded)
-    const uint32_t* __restrict__ wrow = wgt + (size_t)(n0 + row_to_channel(j)) * cw;
+    // The weights in lane order (after the [NPAD32][cw] rows): a group is 64 lanes x 4 words, contiguous; rows >= N
+    // and words >= cw hold zeros (their outputs are discarded / they multiply activation words that read as 0).
+    const int groups = (cw + 7) / 8;
+    const v4i* __restrict__ wlane = reinterpret_cast<const v4i*>(wgt + fc_weight_row_words(n_tiles * 32, cw)) +
+                                    (size_t)nt * groups * 64 + lane;
 
     // K order: group g = words 8g .. 8g+7; step 4g+i multiplies words 8g+i (lanes 0-31) and 8g+4+i
     // (lanes 32-63) of both operands.
-    const int groups = (cw + 7) / 8;
     const int g_begin = wave * groups_per_wave, g_end = min(groups, g_begin + groups_per_wave);
 
     auto load_group = [&](int g, v4i& a, uint32_t (&bw)[4]) {
         const int w0 = 8 * g + 4 * h;
-        if (w0 < cw) {  // cw % 4 == 0: the lane's four words exist or none does
-            a = *reinterpret_cast<const v4i*>(wrow + w0);
+        a = wlane[(size_t)g * 64];  // (one contiguous 1 KB request per wave)
+        if (w0 < cw) {  // cw % 4 == 0: the lane's four activation words exist or none does
 #pragma unroll
             for (int i = 0; i < 4; ++i) bw[i] = act[(size_t)(w0 + i) * p.B + bl];
         } else {
-            a = v4i{0, 0, 0, 0};
 #pragma unroll
             for (int i = 0; i < 4; ++i) bw[i] = 0;
         }

@@ -118,7 +118,7 @@ using namespace tcbnn;
 
 extern "C" {
 
-int tcbnn_abi_version(void) { return 6; }
+int tcbnn_abi_version(void) { return 7; }
 const char* tcbnn_last_error(void) { return g_err; }
 
 int tcbnn_set_default_variant(int variant) {
@@ -144,7 +144,9 @@ size_t tcbnn_conv_act_words(int height, int width, int batch, int ch) {
     return (size_t)height * width * batch * step32(ch);
 }
 size_t tcbnn_fc_weight_words(int in_features, int out_features) {
-    return (size_t)pad32(out_features) * kw128(in_features);
+    // sign-bit rows, then the same words in the FP4 FC kernel's lane order
+    return fc_weight_row_words(pad32(out_features), kw128(in_features)) +
+           fc_weight_lane_words(pad32(out_features), kw128(in_features));
 }
 size_t tcbnn_conv_filter_words(int r, int s, int in_ch, int out_ch) {
     const size_t bits = (size_t)pad32(out_ch) * r * s * step32(in_ch);

@@ -111,6 +111,22 @@ __global__ void permute_conv_filter_kernel(const uint32_t* __restrict__ bits, ui
     frag_bits[idx] = bits[(size_t)c * 9 * cw + tap * cw + 2 * t + h];
 }
 
+// Re-orders packed FC weights (rows[neuron][kw], neurons padded to 32, written) into the lane order of the FP4 FC
+// kernel: uint32 [npad/32][groups][64][4]; lane (j, h) of group g holds words 8g + 4h + i (i = 0..3) of neuron
+// 32 tile + row_to_channel(j), zero past kw.
+__global__ void permute_fc_weight_kernel(const uint32_t* __restrict__ rows, uint32_t* __restrict__ lanes, int kw,
+                                         long long total) {
+    const long long idx = (long long)blockIdx.x * kThreads + threadIdx.x;
+    if (idx >= total) return;
+    const int i = (int)(idx & 3), lane = (int)((idx >> 2) & 63);
+    const int groups = (kw + 7) / 8;
+    const int g = (int)((idx >> 8) % groups);
+    const long long tile = (idx >> 8) / groups;
+    const int j = lane & 31, h = lane >> 5;
+    const int w = 8 * g + 4 * h + i;
+    lanes[idx] = w < kw ? rows[(size_t)(tile * 32 + mfma::row_to_channel(j)) * kw + w] : 0u;
+}
+
 // HWIO fp32 [R*S][3][O] -> two tables:
 //   [R*S][opad32][4]  sign masks of the three input channels (0x80000000 where the weight is
 //                     negative) and, in the 4th word, the sign pattern 4*neg0 + 2*neg1 + neg2;
@@ -302,7 +318,12 @@ int tcbnn_pack_fc_weight(const float* weight_kn, uint32_t* packed, int in_featur
                            packed + (size_t)out_features * kw, pad_words);
         TCBNN_LAUNCH_CHECK("clear_words_kernel");
     }
-    return tcbnn_pack_cols(weight_kn, packed, in_features, out_features, kw, stream);
+    if (int rc = tcbnn_pack_cols(weight_kn, packed, in_features, out_features, kw, stream)) return rc;
+    const long long lane_words = (long long)fc_weight_lane_words(npad, kw);
+    hipLaunchKernelGGL(permute_fc_weight_kernel, dim3(blocks_for(lane_words)), dim3(kThreads), 0, (hipStream_t)stream,
+                       packed, packed + fc_weight_row_words(npad, kw), kw, lane_words);
+    TCBNN_LAUNCH_CHECK("permute_fc_weight_kernel");
+    return TCBNN_OK;
 }
 
 int tcbnn_pack_conv_filter(const float* filter_hwio, uint32_t* packed, int r, int s, int in_ch,

@@ -23,11 +23,11 @@ def test_library_exports_every_declared_symbol():
     for s in syms:
         assert hasattr(_lib.lib, s), "libtcbnn_hip.so does not export %s" % s
     assert sorted(_lib.ABI) == syms, "Python binding table and header disagree"
-    assert _lib.lib.tcbnn_abi_version() == 6
+    assert _lib.lib.tcbnn_abi_version() == 7
     # the build entry point refuses a library of another ABI version: it must expect this one
     import inspect
     import __graft_entry__
-    assert "tcbnn_abi_version() == 6" in inspect.getsource(__graft_entry__.build)
+    assert "tcbnn_abi_version() == 7" in inspect.getsource(__graft_entry__.build)
 
 
 def test_geometry_entry_points_match_reference_formulas():
@@ -47,7 +47,7 @@ def test_size_helpers():
     L = _lib.lib
     assert L.tcbnn_fc_act_words(8192, 784) == 8192 * 28
     assert L.tcbnn_conv_act_words(56, 56, 256, 64) == 56 * 56 * 256 * 2
-    assert L.tcbnn_fc_weight_words(784, 10) == 32 * 28
+    assert L.tcbnn_fc_weight_words(784, 10) == 32 * 28 + 32 * 8 * 4  # sign-bit rows + the copy in lane order
     assert L.tcbnn_conv_filter_words(3, 3, 64, 64) == 64 * 9 * 2 * 2   # sign bits + a copy in MFMA lane order
     assert L.tcbnn_conv_filter_words(3, 3, 96, 64) == 64 * 9 * 3       # sign bits only
     assert L.tcbnn_conv_filter_words(5, 5, 64, 40) == 64 * 25 * 2
