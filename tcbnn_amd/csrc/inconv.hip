@@ -118,6 +118,38 @@ __device__ __forceinline__ void add_indexed8x2(float* a, float* b, v8f ca, v8f c
         : "m0");
 }
 
+// Which (image tile, group of four output columns, output row) a workgroup takes; false for the padding of the grid.
+// Workgroups are dealt round-robin to the 8 XCDs (each with its own L2).  When the number of image tiles divides 8
+// (y_phases > 0 = column ranges per image tile), XCD slot = (image tile, range of column groups) and the workgroups
+// of a slot walk along x and then down the rows, so that the input rows shared by consecutive output rows (7-row
+// windows at stride 4 overlap by 3) and by neighbouring column groups are found in that XCD's L2 instead of being
+// fetched from HBM again.
+// Rows are dealt 0, k, 2k, ... then 1, k + 1, ... (k = row_il, chosen by the host): consecutive output rows share
+// R - stride input rows, and the workgroup of row r + 1 needs a shared row stride/R of a workgroup's lifetime BEFORE
+// the workgroup of row r does.  Dealt in natural order the two start almost together and the row has left the XCD's
+// L2 by the time it is needed again; dealt k rows apart the later start of row r + 1 makes the two requests meet
+// (fetched bytes of ResNet-18's first layer at batch 256: 286 -> 214 MB).
+__device__ __forceinline__ bool inconv_workgroup_position(int block, int b_tiles, int x_groups, int y_phases, int row_il,
+                                                          int rows_total, int& bt, int& xg, int& y) {
+    if (y_phases > 0) {
+        const int slot = block & 7, j = block >> 3;
+        const int xg_per = (x_groups + y_phases - 1) / y_phases;
+        bt = slot % b_tiles;
+        xg = (slot / b_tiles) * xg_per + j % xg_per;
+        y = j / xg_per;
+        if (row_il > 1) {
+            const int G = (rows_total + row_il - 1) / row_il;
+            y = (y % G) * row_il + y / G;
+            if (y >= rows_total) return false;
+        }
+        return xg < x_groups;
+    }
+    bt = block % b_tiles;
+    xg = (block / b_tiles) % x_groups;
+    y = block / (b_tiles * x_groups);
+    return true;
+}
+
 // The read-only operands are separate __restrict__ kernel arguments so that the
 // wave-uniform mask / threshold loads become scalar loads (s_load) feeding v_xor directly.
 typedef uint32_t u16v __attribute__((ext_vector_type(16)));
@@ -218,34 +250,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS &
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    // Workgroups are dealt round-robin to the 8 XCDs (each with its own L2).  When the number of
-    // image tiles divides 8, XCD slot = (image tile, range of column groups) and the workgroups of a
-    // slot walk along x and then down the rows, so that the input rows shared by consecutive output
-    // rows (7-row windows at stride 4 overlap by 3) and by neighbouring column groups are found in
-    // that XCD's L2 instead of being fetched from HBM again.
     int bt, xg, y;
-    if (y_phases > 0) {  // y_phases = column ranges per image tile
-        const int slot = blockIdx.x & 7, j = blockIdx.x >> 3;
-        const int xg_per = (x_groups + y_phases - 1) / y_phases;
-        bt = slot % b_tiles;
-        xg = (slot / b_tiles) * xg_per + j % xg_per;
-        y = j / xg_per;
-        // Rows are dealt 0, k, 2k, ... then 1, k + 1, ... (k = row_il, chosen by the host): consecutive output rows
-        // share R - stride input rows, and the workgroup of row r + 1 needs a shared row stride/R of a workgroup's
-        // lifetime BEFORE the workgroup of row r does.  Dealt in natural order the two start almost together and the
-        // row has left the XCD's L2 by the time it is needed again; dealt k rows apart the later start of row r + 1
-        // makes the two requests meet (fetched bytes of ResNet-18's first layer at batch 256: 286 -> 214 MB).
-        if (row_il > 1) {
-            const int G = (rows_total + row_il - 1) / row_il;
-            y = (y % G) * row_il + y / G;
-            if (y >= rows_total) return;  // whole workgroup: grid padding
-        }
-        if (xg >= x_groups) return;  // whole workgroup: grid padding
-    } else {
-        bt = blockIdx.x % b_tiles;
-        xg = (blockIdx.x / b_tiles) % x_groups;
-        y = blockIdx.x / (b_tiles * x_groups);
-    }
+    if (!inconv_workgroup_position((int)blockIdx.x, b_tiles, x_groups, y_phases, row_il, rows_total, bt, xg, y))
+        return;  // whole workgroup: grid padding
     const int x0 = xg * kXT;
     const int pp = wave & 1;    // which pair of the workgroup's four columns
     const int chh = wave >> 1;  // which 32 of the pass's 64 channels
@@ -443,23 +450,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     int bt, xg, y;
-    if (y_phases > 0) {  // XCD-aware order with row interleave, as in inconv_tiled_kernel
-        const int slot = blockIdx.x & 7, j = blockIdx.x >> 3;
-        const int xg_per = (x_groups + y_phases - 1) / y_phases;
-        bt = slot % b_tiles;
-        xg = (slot / b_tiles) * xg_per + j % xg_per;
-        y = j / xg_per;
-        if (row_il > 1) {
-            const int G = (rows_total + row_il - 1) / row_il;
-            y = (y % G) * row_il + y / G;
-            if (y >= rows_total) return;
-        }
-        if (xg >= x_groups) return;
-    } else {
-        bt = blockIdx.x % b_tiles;
-        xg = (blockIdx.x / b_tiles) % x_groups;
-        y = blockIdx.x / (b_tiles * x_groups);
-    }
+    if (!inconv_workgroup_position((int)blockIdx.x, b_tiles, x_groups, y_phases, row_il, rows_total, bt, xg, y)) return;
     const int pp = wave & 1, chh = wave >> 1;
     const int xa = xg * kXT + 2 * pp;
     const bool xa_ok = xa < p.PW, xb_ok = xa + 1 < p.PW;  // uniform
