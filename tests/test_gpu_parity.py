@@ -418,6 +418,8 @@ def _window_maximum(res):
     (64, 8, 64, 64, 2, 100, 64), (70, 6, 128, 128, 1, 3000, 128), (8, 4, 256, 256, 1, 500, 128),
     (40, 10, 64, 128, 2, 2000, 64), (8, 4, 512, 512, 1, 20000, 512), (24, 6, 192, 64, 2, 50, 32),
     (40, 4, 384, 128, 1, 900, 96),
+    # more windows than workgroups (a workgroup walks several windows, the last round ragged)
+    (256, 28, 64, 64, 2, 100, 64), (128, 20, 128, 128, 1, 3000, 128),
     # not served: odd frame, int32 output (bound above 32767), output channels not a multiple of 64, int32 source
     (8, 7, 64, 64, 2, 100, 64), (8, 4, 64, 64, 1, 32700, 64), (8, 4, 64, 96, 2, 100, 96), (8, 4, 128, 64, 0, 100, 64)])
 def test_conv128_saved_residual_as_window_maximum(gpu, variant, b, h, cin, cout, in_fmt, amp, lim):
