@@ -181,7 +181,12 @@ conv3x3_mfma_f4_kernel(
     // a wave's work items: output pixels, or 2x2 windows of them (row width `roww`)
     const int roww = kWin ? p.PW / 2 : p.PW;
     const int npix = kWin ? (p.PH / 2) * (p.PW / 2) : p.PH * p.PW;
-    int pi = PSAVE ? stream : stream * kWaves + wave;  // (a window is taken by the whole workgroup)
+    // First item of the wave (its later ones follow at stride dpi).  The items of the last, incomplete round go to
+    // the waves with the lowest first item.  An eight-wave workgroup has a CU to itself, two waves per SIMD: its
+    // waves 0-3 (one per SIMD) are numbered before the waves 4-7 of ANY workgroup, so that the left-over items fall
+    // one to a SIMD over all CUs instead of two to a SIMD in the first CUs and none in the others.
+    int pi = PSAVE ? stream  // (a window is taken by the whole workgroup)
+                   : (kWaves == 8 ? (wave >> 2) * (pix_streams * 4) + stream * 4 + (wave & 3) : stream * kWaves + wave);
     const int dpi = PSAVE ? pix_streams : pix_streams * kWaves;
     // Item pi stands for row pi / roww and column (pi % roww + row) % roww.  The skew by the row keeps
     // a wave from staying in one column when its stride is a multiple of the row width (then the waves
