@@ -52,8 +52,11 @@ constexpr int kResStoreAux = 0x11;
 constexpr int kBitsStoreAux = 0x11;
 // Waves per workgroup: four, sharing the staged weights of their channel group; eight where the FP4 fragments of
 // two channel tiles (18 KB per tile and 64 input channels) leave room for only one workgroup in a CU's 160 KB of
-// LDS: the CU then still runs two waves per SIMD, and each expanded activation fragment still feeds two MFMAs.
-constexpr int waves_of(int spt, int nt) { return 9 * spt * nt * 1024 > 80 * 1024 ? 8 : 4; }
+// LDS (Cin >= 384), and already at Cin = 256, where two four-wave workgroups would fit: the CU then still runs two
+// waves per SIMD, each expanded activation fragment still feeds two MFMAs, the weights are staged once per CU
+// instead of twice, and which waves share a SIMD is known (waves w and w + 4), which the numbering of the work
+// items uses (ResNet-18 at batch 256: L3B2C1 14.6 -> 13.2 us, L3B1C2 17.1 -> 16.1 us).
+constexpr int waves_of(int spt, int nt) { return 9 * spt * nt * 1024 > (nt == 2 ? 64 : 80) * 1024 ? 8 : 4; }
 // Residual mode of an instantiation.
 constexpr int RM_NONE = 0;    // threshold only
 constexpr int RM_PLAIN = 1;   // residual injected from a source of the same size and / or saved
@@ -1129,7 +1132,10 @@ int launch_f(const BgemmParams& p, hipStream_t stream) {
     const int n_groups = (p.N + 32 * NT - 1) / (32 * NT);
     const int b_groups = (p.B + 32 * MT - 1) / (32 * MT);
     const int items = WIN != WIN_NONE ? (p.PH / 2) * (p.PW / 2) : p.PH * p.PW;  // pixels, or 2x2 windows of them
-    const int quads = kWgItems ? items : (items + kWaves - 1) / kWaves;  // items per wave of a pixel stream
+    // streams worth launching: one per item for workgroup-wide items; else one per kWaves items, or per 4 for
+    // eight-wave workgroups, whose waves 0-3 (one per SIMD) are served first (see the kernel's first item)
+    constexpr int kServedFirst = kWaves == 8 ? 4 : kWaves;
+    const int quads = kWgItems ? items : (items + kServedFirst - 1) / kServedFirst;
     // Persistent workgroups, all resident at once: two per CU (three for residual layers), fewer
     // when registers or LDS hold fewer.  Measured on every layer of ResNet-18 at batch 256: more, shorter-lived
     // workgroups stage the weights more often and lose; and a grid even slightly larger than the resident slots
