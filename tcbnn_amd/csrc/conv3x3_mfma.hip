@@ -1213,7 +1213,17 @@ Pick pick(const BgemmParams& p) {
     // (a pooled int32 source keeps one channel tile per wave: four times sixteen words per tile and lane spilled)
     int nt = rm == RM_POOLED && fmt == TCBNN_RES_I32 ? 1 : pick_nt(p.cw / 2, rm);
     if (rm == RM_PLAIN && p.res_out_pool) nt = pick_nt_maxsave(p.cw / 2);
-    return {rm, pick_mt(p.cw / 2, rm), nt, fmt, p.pool_h == 2 ? WIN_ORPOOL : (p.res_out_pool ? WIN_MAXSAVE : WIN_NONE)};
+    int mt = pick_mt(p.cw / 2, rm);
+    // A plain layer with fewer than four two-image tiles per SIMD takes one image tile per wave: twice the items, so
+    // the last round leaves less of the machine idle, which outweighs the weight fragments then being read from LDS
+    // for every MFMA (ResNet-18 at batch 256: the stride-2 layers L3B1C1 9.9 -> 9.3 us, L4B1C1 10.7 -> 10.0 us; with
+    // more tiles the larger tile wins: L1B1C1 15.4 -> 17.5 us).
+    if (rm == RM_NONE && p.pool_h == 1 && mt == 2) {
+        int dev = 0, cus = 0;
+        const long long tiles = (long long)p.PH * p.PW * ((p.B + 63) / 64) * ((p.N + 32 * nt - 1) / (32 * nt));
+        if (device_info(&dev, &cus) == TCBNN_OK && tiles < 4LL * 4 * cus) mt = 1;
+    }
+    return {rm, mt, nt, fmt, p.pool_h == 2 ? WIN_ORPOOL : (p.res_out_pool ? WIN_MAXSAVE : WIN_NONE)};
 }
 
 template <int SPT>
@@ -1223,7 +1233,8 @@ int launch_m(const BgemmParams& p, hipStream_t stream) {
         case RM_NONE:
             return k.win == WIN_ORPOOL
                        ? launch_t<SPT, RM_NONE, pick_mt(SPT, RM_NONE), pick_nt(SPT, RM_NONE), TCBNN_RES_I32, WIN_ORPOOL>(p, stream)
-                       : launch_t<SPT, RM_NONE, pick_mt(SPT, RM_NONE), pick_nt(SPT, RM_NONE), TCBNN_RES_I32, WIN_NONE>(p, stream);
+                       : (k.mt == 1 ? launch_t<SPT, RM_NONE, 1, pick_nt(SPT, RM_NONE), TCBNN_RES_I32, WIN_NONE>(p, stream)
+                                    : launch_t<SPT, RM_NONE, pick_mt(SPT, RM_NONE), pick_nt(SPT, RM_NONE), TCBNN_RES_I32, WIN_NONE>(p, stream));
         case RM_RAW:
             return launch_t<SPT, RM_RAW, pick_mt(SPT, RM_RAW), pick_nt(SPT, RM_RAW), TCBNN_RES_I32, WIN_NONE>(p, stream);
         case RM_PLAIN:
