@@ -56,7 +56,16 @@ constexpr int kBitsStoreAux = 0x11;
 // waves per SIMD, each expanded activation fragment still feeds two MFMAs, the weights are staged once per CU
 // instead of twice, and which waves share a SIMD is known (waves w and w + 4), which the numbering of the work
 // items uses (ResNet-18 at batch 256: L3B2C1 14.6 -> 13.2 us, L3B1C2 17.1 -> 16.1 us).
-constexpr int waves_of(int spt, int nt) { return 9 * spt * nt * 1024 > (nt == 2 ? 64 : 80) * 1024 ? 8 : 4; }
+constexpr int WIN_NONE = 0, WIN_ORPOOL = 1, WIN_MAXSAVE = 2;  // (see the kernel)
+constexpr int waves_of(int spt, int nt, int win) {
+    return win != WIN_MAXSAVE && 9 * spt * nt * 1024 > (nt == 2 ? 64 : 80) * 1024 ? 8 : 4;  // (WIN_MAXSAVE: a wave per pixel)
+}
+// WIN_MAXSAVE: where the four waves' sums of a window meet in LDS.  All channel tiles at once ([wave][NT][2][64]
+// 128-bit words) where that leaves room for two workgroups per CU next to the staged weights; else one channel tile
+// at a time ([3 other waves][2][64]: the wave that takes the tile's maximum keeps its own sums in registers), at the
+// price of two more barriers per window.
+constexpr bool win_two_phase(int spt, int nt) { return 9 * spt * nt * 1024 + nt * 128 + 4 * nt * 2 * 64 * 16 > 80 * 1024; }
+constexpr int win_area_bytes(int spt, int nt) { return win_two_phase(spt, nt) ? 3 * 2 * 64 * 16 : 4 * nt * 2 * 64 * 16; }
 // Residual mode of an instantiation.
 constexpr int RM_NONE = 0;    // threshold only
 constexpr int RM_PLAIN = 1;   // residual injected from a source of the same size and / or saved
@@ -93,9 +102,8 @@ constexpr int waves_per_simd(int spt, int rm, int win) { return spt == 1 && rm =
 // and, with an injected residual, lies entirely below or entirely above the channel limit: the per-channel
 // tests of partial tiles are then not even compiled (they cost scalar registers and set-up instructions in
 // every launch, and the networks' channel counts are multiples of 64).
-constexpr int WIN_NONE = 0, WIN_ORPOOL = 1, WIN_MAXSAVE = 2;
 template <int SPT, int RM, int MT, int NT, int RF, int WIN, bool FULLT>
-__global__ __launch_bounds__(64 * waves_of(SPT, NT)) __attribute__((amdgpu_waves_per_eu(waves_per_simd(SPT, RM, WIN)))) void
+__global__ __launch_bounds__(64 * waves_of(SPT, NT, WIN)) __attribute__((amdgpu_waves_per_eu(waves_per_simd(SPT, RM, WIN)))) void
 conv3x3_mfma_f4_kernel(
     const BgemmParams p, const uint32_t* __restrict__ act, const uint32_t* __restrict__ wgt,
     const float* __restrict__ bnp, const int32_t* __restrict__ rin, int32_t* __restrict__ rout, int res_lim,
@@ -106,11 +114,12 @@ conv3x3_mfma_f4_kernel(
     static_assert(RM == RM_NONE || !POOL, "residuals are defined for un-pooled layers only");
     static_assert(!PSAVE || (RM == RM_PLAIN && FULLT && (RF == TCBNN_RES_I16 || RF == TCBNN_RES_I12)),
                   "the window maximum is taken on 16-bit pairs in the epilogue of full tiles with a narrow injected residual");
-    static_assert(!PSAVE || (MT == 1 && waves_of(SPT, NT) == 4), "one wave per pixel of the window, one image tile each");
+    static_assert(!PSAVE || (MT == 1 && waves_of(SPT, NT, WIN) == 4), "one wave per pixel of the window, one image tile each");
+    constexpr bool kTwoPhase = PSAVE && win_two_phase(SPT, NT);
     constexpr int TPC = SPT >= 3 ? 3 : 9;  // taps per prefetch chunk (a filter row, or all of it)
     constexpr int NCH = 9 / TPC;           // chunks per tile
     constexpr int NQ = 9 * SPT;            // k-steps per tile
-    constexpr int kWaves = waves_of(SPT, NT);
+    constexpr int kWaves = waves_of(SPT, NT, WIN);
     // A tile of one chunk is shorter than the memory latency: its residual operand is then
     // requested a whole tile ahead (double-buffered); otherwise with the tile's first chunk.
     constexpr bool kAhead = kRes && NCH == 1;
@@ -122,7 +131,7 @@ conv3x3_mfma_f4_kernel(
     constexpr bool kRawTranspose = raw_transposed(SPT, RM, NT, FULLT);
     constexpr int kRawPitch = raw_pitch(NT);
     int* lds_raw = reinterpret_cast<int*>(lds_thr + NT * 32);
-    // WIN_MAXSAVE: where the four waves' sums of a window meet, [wave][NT][2][64 lanes] 128-bit words (pairs of int16)
+    // WIN_MAXSAVE: where the four waves' sums of a window meet (pairs of int16; see win_two_phase)
     v4i* lds_win = reinterpret_cast<v4i*>(lds_thr + NT * 32);
 
     const int tid = threadIdx.x;
@@ -523,6 +532,7 @@ conv3x3_mfma_f4_kernel(
     // One channel tile of the epilogue.  FAST (wave-uniform choice): all 32 channels exist and, with a
     // residual, all of them receive it, so no per-channel condition is evaluated at all.
     uint32_t poolw[MT][NT];  // POOL: OR of the window's words so far
+    uint32_t prw[kTwoPhase ? NT : 1][8];  // WIN_MAXSAVE, one channel tile at a time: this pixel's sums until their turn
     auto epilogue_tile = [&](auto fast_tag, int nt, unsigned pix, unsigned bits_pix, int (*rv)[NW],
                              int sub) __attribute__((always_inline)) {
         constexpr bool FAST = decltype(fast_tag)::value;
@@ -605,9 +615,14 @@ conv3x3_mfma_f4_kernel(
 #pragma unroll
                     for (int k = 0; k < 8; ++k)
                         pr[k] = __builtin_amdgcn_perm(__float_as_uint(t[2 * k + 1]), __float_as_uint(t[2 * k]), 0x05040100u);
-                    v4i* x = lds_win + ((wave * NT + nt) * 2) * 64 + lane;
-                    x[0] = v4i{(int)pr[0], (int)pr[1], (int)pr[2], (int)pr[3]};
-                    x[64] = v4i{(int)pr[4], (int)pr[5], (int)pr[6], (int)pr[7]};
+                    if constexpr (kTwoPhase) {
+#pragma unroll
+                        for (int k = 0; k < 8; ++k) prw[nt][k] = pr[k];
+                    } else {
+                        v4i* x = lds_win + ((wave * NT + nt) * 2) * 64 + lane;
+                        x[0] = v4i{(int)pr[0], (int)pr[1], (int)pr[2], (int)pr[3]};
+                        x[64] = v4i{(int)pr[4], (int)pr[5], (int)pr[6], (int)pr[7]};
+                    }
                 } else if (rout != nullptr) {
                     // the value to store is in the low bits of t's bit pattern (see the 128-bit store note below)
                     v4i q[4];
@@ -830,16 +845,21 @@ conv3x3_mfma_f4_kernel(
         if constexpr (PSAVE) {
             typedef short s2_t __attribute__((ext_vector_type(2)));
             uint32_t wm[8];
+            if constexpr (kTwoPhase) {
 #pragma unroll
-            for (int w = 0; w < 4; ++w) {
-                const v4i* x = lds_win + ((w * NT + nt) * 2) * 64 + lane;
+                for (int k = 0; k < 8; ++k) wm[k] = prw[nt][k];  // (this wave's own pixel)
+            }
+#pragma unroll
+            for (int w = 0; w < (kTwoPhase ? 3 : 4); ++w) {
+                const v4i* x = lds_win + (kTwoPhase ? w * 2 : (w * NT + nt) * 2) * 64 + lane;
                 const v4i lo = x[0], hi = x[64];
 #pragma unroll
                 for (int k = 0; k < 8; ++k) {
                     const uint32_t pr = (uint32_t)(k < 4 ? lo[k] : hi[k - 4]);
-                    wm[k] = w == 0 ? pr
-                                   : __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(s2_t, wm[k]),
-                                                                                            __builtin_bit_cast(s2_t, pr)));
+                    wm[k] = !kTwoPhase && w == 0
+                                ? pr
+                                : __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(s2_t, wm[k]),
+                                                                                         __builtin_bit_cast(s2_t, pr)));
                 }
             }
             const int b = bimg[0];
@@ -898,9 +918,22 @@ conv3x3_mfma_f4_kernel(
             else
                 epilogue_tile(std::false_type{}, nt, pix, bits_pix, rv, sub);
         }
-        if constexpr (PSAVE) {
+        if constexpr (PSAVE && !kTwoPhase) {
             asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // the four pixels' sums are in LDS
             if (wave < NT) window_maximum(wave, pix);                       // (uniform per wave)
+        }
+        if constexpr (kTwoPhase) {  // one channel tile at a time: wave nt takes tile nt's maximum, the others hand in
+#pragma unroll
+            for (int nt = 0; nt < NT; ++nt) {
+                if (nt > 0) asm volatile("s_barrier" ::: "memory");  // the previous tile's sums have been read
+                if (wave != nt) {                                    // (uniform per wave)
+                    v4i* x = lds_win + (((wave - nt - 1) & 3) * 2) * 64 + lane;
+                    x[0] = v4i{(int)prw[nt][0], (int)prw[nt][1], (int)prw[nt][2], (int)prw[nt][3]};
+                    x[64] = v4i{(int)prw[nt][4], (int)prw[nt][5], (int)prw[nt][6], (int)prw[nt][7]};
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+                if (wave == nt) window_maximum(nt, pix);
+            }
         }
         if (RM != RM_RAW && ng == n_groups - 1 && (!POOL || sub == 3)) {  // zero the pixel's padding words
 #pragma unroll
@@ -1104,12 +1137,12 @@ TensorBytes tensor_bytes(const BgemmParams& p) {
 template <int SPT, int RM, int MT, int NT, int RF, int WIN, bool FULLT>
 int launch_f(const BgemmParams& p, hipStream_t stream) {
     constexpr int NQ = 9 * SPT;
-    constexpr int kWaves = waves_of(SPT, NT), kThreads = 64 * kWaves;
+    constexpr int kWaves = waves_of(SPT, NT, WIN), kThreads = 64 * kWaves;
     constexpr bool kRawTranspose = raw_transposed(SPT, RM, NT, FULLT);
     constexpr bool kWgItems = WIN == WIN_MAXSAVE;  // a work item (window) is taken by a whole workgroup
     const size_t lds_bytes = (size_t)NQ * NT * 64 * 16 + NT * 32 * sizeof(float) +
                              (kRawTranspose ? (size_t)kWaves * 32 * raw_pitch(NT) * sizeof(int) : 0) +
-                             (kWgItems ? (size_t)kWaves * NT * 2 * 64 * 16 : 0);
+                             (kWgItems ? (size_t)win_area_bytes(SPT, NT) : 0);
     // Per instantiation and device, set up by the first launch there: the dynamic LDS limit, and how many of its
     // workgroups a CU holds at once (registers and LDS).  Atomics only so that two host threads that both find the
     // entry empty do no harm (both store the same value).
@@ -1199,8 +1232,9 @@ constexpr int pick_nt(int spt, int rm) {
     return rm == RM_POOLED ? (spt >= 6 ? 1 : 2) : (rm == RM_RAW ? (spt >= 3 && spt < 8 ? 1 : 2) : 2);
 }
 // Channel tiles per wave when the saved residual is the window maximum (the four waves of a workgroup then share a
-// window): two where the staged weights leave room for three workgroups per CU, one from Cin = 192 on.
-constexpr int pick_nt_maxsave(int spt) { return spt <= 2 ? 2 : 1; }
+// window): two up to Cin = 128 (three or four workgroups per CU) and at Cin = 256 (two workgroups per CU with the
+// one-tile-at-a-time exchange of win_two_phase: L3B2C2 of ResNet-18 at batch 256 20.8 -> 19.8 us), one otherwise.
+constexpr int pick_nt_maxsave(int spt) { return spt <= 2 || spt == 4 ? 2 : 1; }
 constexpr int pick_mt(int spt, int rm) {
     return rm == RM_RAW ? (spt >= 8 ? 1 : 2) : (rm == RM_NONE ? (spt >= 6 ? 1 : 2) : 1);
 }
