@@ -788,7 +788,7 @@ conv3x3_mfma_f4_kernel(
                 if (sub != 3) continue;  // uniform: the window is not complete yet
             }
             const int w = ng * NT + nt;
-            if (w < p.bits_row_words)  // uniform
+            if (FULLT || w < p.bits_row_words)  // uniform; with full tiles every word of the group exists
                 __builtin_amdgcn_raw_buffer_store_b32((int)word, r_bits, (int)voff_bits[mt],
                                                       (int)(bits_pix + (unsigned)w * row_b), kBitsStoreAux);
         }
