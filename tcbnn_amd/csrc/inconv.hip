@@ -158,9 +158,11 @@ typedef int v4i_t __attribute__((ext_vector_type(4)));
 // The epilogue both first-layer kernels share, for a lane's 32 consecutive channels (word `wi`) of one image and pixel.
 // Output word: bit n (MSB first) = !(acc[n] < bn[32 wi + n]), i.e. the inverted sign of acc - bn (equal operands give
 // +0; a NaN threshold counts as -inf: the bit is 1 either way).
+// FULL: the launch has full channel tiles only (O a multiple of 64): the partial-tile code is not even compiled.
+template <bool FULL>
 __device__ __forceinline__ uint32_t inconv_threshold_word(const float* acc, const float* __restrict__ bn, int wi, int O) {
     uint32_t word = 0;
-    if (wi * 32 + 32 <= O) {  // uniform: full channel tile
+    if (FULL || wi * 32 + 32 <= O) {  // uniform: full channel tile
 #pragma unroll
         for (int n = 0; n < 32; ++n) {
             // (the NaN test on the threshold's bits: wave-uniform, so it stays on the scalar unit)
@@ -181,12 +183,13 @@ __device__ __forceinline__ uint32_t inconv_threshold_word(const float* acc, cons
 // 8 int16), or 24 per group of 16 channels at 12 bits; channels past O are stored as 0, groups past O not at all.
 // Streaming stores: the tensor (77-103 MB for ResNet-18 at batch 256) is far larger than the caches and is read two
 // launches later.
+template <bool FULL>
 __device__ __forceinline__ void inconv_store_residual(const float* acc, int32_t* __restrict__ res, int fmt, size_t pix,
                                                       int wi, int O, int B, int b) {
     int r32[32];
 #pragma unroll
     for (int n = 0; n < 32; ++n) r32[n] = (int)acc[n];
-    if (wi * 32 + 32 > O) {  // uniform
+    if (!FULL && wi * 32 + 32 > O) {  // uniform
 #pragma unroll
         for (int n = 0; n < 32; ++n) r32[n] = wi * 32 + n < O ? r32[n] : 0;
     }
@@ -197,7 +200,7 @@ __device__ __forceinline__ void inconv_store_residual(const float* acc, int32_t*
         const size_t G = (size_t)((O + 15) / 16);
 #pragma unroll
         for (int g = 0; g < 2; ++g)
-            if (wi * 32 + 16 * g < O) {
+            if (FULL || wi * 32 + 16 * g < O) {
                 uint32_t d[6];
                 i12_pack8(&r32[16 * g], d[0], d[1], d[2]);
                 i12_pack8(&r32[16 * g + 8], d[3], d[4], d[5]);
@@ -210,7 +213,7 @@ __device__ __forceinline__ void inconv_store_residual(const float* acc, int32_t*
         const size_t g0 = (pix * ((O + 7) / 8) + wi * 4) * B + b;
 #pragma unroll
         for (int g = 0; g < 4; ++g)
-            if (wi * 32 + 8 * g < O)
+            if (FULL || wi * 32 + 8 * g < O)
                 __builtin_nontemporal_store(v4i_t{(r32[8 * g] & 0xffff) | (r32[8 * g + 1] << 16),
                                                   (r32[8 * g + 2] & 0xffff) | (r32[8 * g + 3] << 16),
                                                   (r32[8 * g + 4] & 0xffff) | (r32[8 * g + 5] << 16),
@@ -220,7 +223,7 @@ __device__ __forceinline__ void inconv_store_residual(const float* acc, int32_t*
         const size_t g0 = (pix * ((O + 3) / 4) + wi * 8) * B + b;
 #pragma unroll
         for (int g = 0; g < 8; ++g)
-            if (wi * 32 + 4 * g < O)
+            if (FULL || wi * 32 + 4 * g < O)
                 __builtin_nontemporal_store(v4i_t{r32[4 * g], r32[4 * g + 1], r32[4 * g + 2], r32[4 * g + 3]},
                                             dst + g0 + (size_t)g * B);
     }
@@ -238,8 +241,9 @@ __device__ __forceinline__ void inconv_store_residual(const float* acc, int32_t*
 // POOLED: blockIdx selects a row of the POOLED output; the workgroup runs the pool_h convolution rows
 // of it one after the other and ORs their words (kernel.cuh:646-664); with pool_w = 2 the two columns of
 // a wave are one window.  pool_w is 1 or 2 (the host checks), no residual is saved.
-// ALLIN (ROWS): the host found every staging pass of every lane inside the 192 segments and the batch a
-// multiple of 64, so no pass is tested (and none of those tests' invariants is computed or kept).
+// ALLIN (ROWS): the host found every staging pass of every lane inside the 192 segments, the batch a multiple of 64
+// and the output channels a multiple of 64, so no pass, image or channel is tested (and none of those tests'
+// invariants is computed or kept).
 template <int NST, bool ROWS, bool POOLED, bool ALLIN>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS && NST <= 16 ? 4 : 3))) void inconv_tiled_kernel(
     const InConvParams p, const float* __restrict__ in, const uint4* __restrict__ masks,
@@ -399,7 +403,7 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS &
             }
         }
 
-        if (work && b < p.B && wi < p.ow) {
+        if (work && (ALLIN || (b < p.B && wi < p.ow))) {
             // The stores' addresses are worked out here, after the tap loops: formed ahead of them (the compiler hoists
             // what does not depend on the loops) they were live across the whole kernel and were spilled.
             // (the lane index comes from the hardware's lane count here, not from a register kept since the start)
@@ -409,18 +413,18 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS &
                 if (px == 1 && !xb_ok) continue;
                 const float* acc = px == 0 ? acca : accb;
                 const size_t pix = (size_t)yc * p.PW + xa + px;
-                const uint32_t word = inconv_threshold_word(acc, bn, wi, p.O);
+                const uint32_t word = inconv_threshold_word<ALLIN>(acc, bn, wi, p.O);
                 if constexpr (POOLED) {
                     pooled[px] |= word;
                     continue;
                 }
                 out[(pix * p.ow + wi) * p.B + b] = word;
-                if (res != nullptr) inconv_store_residual(acc, res, p.res_fmt, pix, wi, p.O, p.B, b);
+                if (res != nullptr) inconv_store_residual<ALLIN>(acc, res, p.res_fmt, pix, wi, p.O, p.B, b);
             }
         }
       }
       if constexpr (POOLED) {
-          if (work && b < p.B && wi < p.ow) {
+          if (work && (ALLIN || (b < p.B && wi < p.ow))) {
               if (p.pool_w == 2) {
                   out[(((size_t)y * p.OW + xa / 2) * p.ow + wi) * p.B + b] = pooled[0] | (xb_ok ? pooled[1] : 0u);
               } else {
@@ -518,9 +522,9 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) v
                 if (px == 1 && !xb_ok) continue;
                 const float* acc = px == 0 ? acca : accb;
                 const size_t pix = (size_t)y * p.PW + xa + px;
-                const uint32_t word = inconv_threshold_word(acc, bn, wi, p.O);
+                const uint32_t word = inconv_threshold_word<false>(acc, bn, wi, p.O);
                 out[(pix * p.ow + wi) * p.B + b] = word;
-                if (res != nullptr) inconv_store_residual(acc, res, p.res_fmt, pix, wi, p.O, p.B, b);
+                if (res != nullptr) inconv_store_residual<false>(acc, res, p.res_fmt, pix, wi, p.O, p.B, b);
             }
         }
     }
@@ -755,7 +759,7 @@ static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name
             const int passes = (3 * 64 + 4 * rpw - 1) / (4 * rpw);
             const int nst = passes <= 4 ? 4 : (passes <= 8 ? 8 : (passes <= 16 ? 16 : 24));
             snprintf(name_buf, name_len, "inconv_tiled_kernel<%d, true, %s, %s>", nst, pooled ? "true" : "false",
-                     nst * 4 * rpw == 3 * 64 && p.B % 64 == 0 ? "true" : "false");
+                     nst * 4 * rpw == 3 * 64 && p.B % 64 == 0 && p.O % 64 == 0 ? "true" : "false");
         } else {
             snprintf(name_buf, name_len, "inconv_tiled_kernel<%d, false, %s, false>",
                      (3 * 64 * ncols + kThreads - 1) / kThreads <= 15 ? 15 : 24, pooled ? "true" : "false");
@@ -782,7 +786,7 @@ static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name
             constexpr int NST = decltype(nst_tag)::value;
             constexpr bool ROWS = decltype(rows_tag)::value;
             if constexpr (ROWS) {
-                if (NST * 4 * rpw == 3 * 64 && p.B % 64 == 0) {
+                if (NST * 4 * rpw == 3 * 64 && p.B % 64 == 0 && p.O % 64 == 0) {
                     if (pooled) return launch(inconv_tiled_kernel<NST, true, true, true>);
                     return launch(inconv_tiled_kernel<NST, true, false, true>);
                 }
