@@ -129,21 +129,26 @@ __device__ __forceinline__ void add_indexed8x2(float* a, float* b, v8f ca, v8f c
 // the workgroup of row r does.  Dealt in natural order the two start almost together and the row has left the XCD's
 // L2 by the time it is needed again; dealt k rows apart the later start of row r + 1 makes the two requests meet
 // (fetched bytes of ResNet-18's first layer at batch 256: 286 -> 214 MB).
-__device__ __forceinline__ bool inconv_workgroup_position(int block, int b_tiles, int x_groups, int y_phases, int row_il,
-                                                          int rows_total, int& bt, int& xg, int& y) {
+// In that order the grid is (8 slots, column groups per slot, rows): the workgroup's linear number, which the
+// hardware deals to the XCDs, is slot + 8 (column group + groups per slot x row), and nothing has to be divided
+// (b_tiles is a power of two there; row / row_g by the host's multiplier).  Every instruction of this kernel's set-up
+// is paid 12544 times per launch on an instruction-issue-bound kernel.
+__device__ __forceinline__ bool inconv_workgroup_position(int b_tiles, int x_groups, int y_phases, int row_il,
+                                                          int rows_total, int row_g, unsigned row_g_magic, int& bt,
+                                                          int& xg, int& y) {
     if (y_phases > 0) {
-        const int slot = block & 7, j = block >> 3;
-        const int xg_per = (x_groups + y_phases - 1) / y_phases;
-        bt = slot % b_tiles;
-        xg = (slot / b_tiles) * xg_per + j % xg_per;
-        y = j / xg_per;
+        const int slot = (int)blockIdx.x, xg_per = (int)gridDim.y;
+        bt = slot & (b_tiles - 1);
+        xg = (slot >> __builtin_ctz((unsigned)b_tiles)) * xg_per + (int)blockIdx.y;
+        y = (int)blockIdx.z;
         if (row_il > 1) {
-            const int G = (rows_total + row_il - 1) / row_il;
-            y = (y % G) * row_il + y / G;
+            const int q = (int)__umulhi((unsigned)y, row_g_magic);  // y / row_g
+            y = (y - q * row_g) * row_il + q;
             if (y >= rows_total) return false;
         }
         return xg < x_groups;
     }
+    const int block = (int)blockIdx.x;
     bt = block % b_tiles;
     xg = (block / b_tiles) % x_groups;
     y = block / (b_tiles * x_groups);
@@ -248,14 +253,14 @@ template <int NST, bool ROWS, bool POOLED, bool ALLIN>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS && NST <= 16 ? 4 : 3))) void inconv_tiled_kernel(
     const InConvParams p, const float* __restrict__ in, const uint4* __restrict__ masks,
     const float* __restrict__ bn, uint32_t* __restrict__ out, int32_t* __restrict__ res, int b_tiles,
-    int x_groups, int y_phases, int div_magic, int rpw, int row_il, int rows_total) {
+    int x_groups, int y_phases, int div_magic, int rpw, int row_il, int rows_total, int row_g, unsigned row_g_magic) {
     __shared__ float tile[3 * kMaxCols * kLB];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     int bt, xg, y;
-    if (!inconv_workgroup_position((int)blockIdx.x, b_tiles, x_groups, y_phases, row_il, rows_total, bt, xg, y))
+    if (!inconv_workgroup_position(b_tiles, x_groups, y_phases, row_il, rows_total, row_g, row_g_magic, bt, xg, y))
         return;  // whole workgroup: grid padding
     const int x0 = xg * kXT;
     const int pp = wave & 1;    // which pair of the workgroup's four columns
@@ -447,14 +452,14 @@ constexpr int kDirectAhead = 3;  // taps requested ahead of their use
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(4))) void inconv_direct_kernel(
     const InConvParams p, const float* __restrict__ in, const uint4* __restrict__ masks,
     const float* __restrict__ bn, uint32_t* __restrict__ out, int32_t* __restrict__ res, int b_tiles,
-    int x_groups, int y_phases, int row_il, int Wp, unsigned in_bytes) {
+    int x_groups, int y_phases, int row_il, int Wp, unsigned in_bytes, int row_g, unsigned row_g_magic) {
     const int rows_total = p.PH;
     typedef float v3f __attribute__((ext_vector_type(3)));
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     int bt, xg, y;
-    if (!inconv_workgroup_position((int)blockIdx.x, b_tiles, x_groups, y_phases, row_il, rows_total, bt, xg, y)) return;
+    if (!inconv_workgroup_position(b_tiles, x_groups, y_phases, row_il, rows_total, row_g, row_g_magic, bt, xg, y)) return;
     const int pp = wave & 1, chh = wave >> 1;
     const int xa = xg * kXT + 2 * pp;
     const bool xa_ok = xa < p.PW, xb_ok = xa + 1 < p.PW;  // uniform
@@ -644,6 +649,10 @@ static int inconv_segments_per_wave(int ncols) {
 struct InConvOrder {
     int b_tiles, x_groups, y_phases, row_il;
     long long blocks;
+    dim3 grid;             // (8, column groups per slot, rows) in the XCD-aware order, else (blocks)
+    int row_g;             // rows per interleave group (row_il > 1)
+    unsigned row_g_magic;  // y / row_g == umulhi(y, row_g_magic) for every row of the grid
+    bool ok;               // the grid fits the launch limits and the multiplier is exact
 };
 static InConvOrder inconv_order(const InConvParams& p, bool pooled, int rows_out) {
     InConvOrder o;
@@ -666,8 +675,20 @@ static InConvOrder inconv_order(const InConvParams& p, bool pooled, int rows_out
         if (il_env < 0 && o.row_il < 4) o.row_il = 0;  // (little to gain where rows already start close to the right lag)
     }
     const int rows_grid = o.row_il > 1 ? (rows_out + o.row_il - 1) / o.row_il * o.row_il : rows_out;
-    o.blocks = o.y_phases > 0 ? 8LL * ((o.x_groups + o.y_phases - 1) / o.y_phases) * rows_grid
-                              : (long long)o.b_tiles * o.x_groups * rows_out;
+    const int xg_per = o.y_phases > 0 ? (o.x_groups + o.y_phases - 1) / o.y_phases : 0;
+    o.blocks = o.y_phases > 0 ? 8LL * xg_per * rows_grid : (long long)o.b_tiles * o.x_groups * rows_out;
+    o.row_g = o.row_il > 1 ? (rows_out + o.row_il - 1) / o.row_il : 1;
+    o.row_g_magic = o.row_g > 1 ? 0xffffffffu / (unsigned)o.row_g + 1u : 0u;
+    o.ok = o.blocks <= 0x7fffffffLL;
+    if (o.y_phases > 0) {
+        o.ok = o.ok && xg_per <= 65535 && rows_grid <= 65535;
+        o.grid = dim3(8u, (unsigned)std::max(1, xg_per), (unsigned)std::max(1, rows_grid));
+        if (o.row_il > 1 && o.ok)
+            for (int y = 0; y < rows_grid; ++y)
+                o.ok = o.ok && (int)(((unsigned long long)(unsigned)y * o.row_g_magic) >> 32) == y / o.row_g;
+    } else {
+        o.grid = dim3((unsigned)std::max(1LL, o.blocks));
+    }
     return o;
 }
 
@@ -740,10 +761,10 @@ static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name
             return TCBNN_OK;
         }
         const InConvOrder o = inconv_order(p, false, p.PH);
-        TCBNN_REQUIRE(o.blocks <= 0x7fffffffLL, "inconv128: grid too large");
-        hipLaunchKernelGGL(inconv_direct_kernel, dim3((unsigned)o.blocks), dim3(kThreads), 0, (hipStream_t)stream, p,
+        TCBNN_REQUIRE(o.ok, "inconv128: grid too large");
+        hipLaunchKernelGGL(inconv_direct_kernel, o.grid, dim3(kThreads), 0, (hipStream_t)stream, p,
                            p.in, p.masks, p.bn, p.out, p.res, o.b_tiles, o.x_groups, o.y_phases, o.row_il, (int)Wp,
-                           (unsigned)in_bytes);
+                           (unsigned)in_bytes, o.row_g, o.row_g_magic);
         TCBNN_LAUNCH_CHECK("inconv_direct_kernel");
         return TCBNN_OK;
     }
@@ -774,13 +795,13 @@ static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name
             TCBNN_REQUIRE((int)(((unsigned)e * (unsigned)div_magic) >> 16) == e / ncols,
                           "inconv128: internal error (division constant)");
         const InConvOrder o = inconv_order(p, pooled, rows_out);
-        TCBNN_REQUIRE(o.blocks <= 0x7fffffffLL, "inconv128: grid too large");
+        TCBNN_REQUIRE(o.ok, "inconv128: grid too large");
         // staging scheme (see the kernel and inconv_segments_per_wave; ncols <= kMaxCols = 32)
         const int rpw = inconv_segments_per_wave(ncols);
         auto launch = [&](auto kernel) {
-            hipLaunchKernelGGL(kernel, dim3((unsigned)o.blocks), dim3(kThreads), 0, (hipStream_t)stream, p, p.in,
+            hipLaunchKernelGGL(kernel, o.grid, dim3(kThreads), 0, (hipStream_t)stream, p, p.in,
                                p.masks, p.bn, p.out, p.res, o.b_tiles, o.x_groups, o.y_phases, div_magic, rpw, o.row_il,
-                               rows_out);
+                               rows_out, o.row_g, o.row_g_magic);
         };
         auto launch_nst = [&](auto nst_tag, auto rows_tag) {
             constexpr int NST = decltype(nst_tag)::value;
