@@ -389,10 +389,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS &
             __syncthreads();
             if (r + 1 < r_hi) fetch_row(r + 1);
             if (!work) continue;
-            for (int s = 0; s < p.S; ++s) {
+            // sign patterns of a tap's 32 channels, one per word (wide scalar loads); the pointer moves on by one tap
+            // (formed anew per tap it was seven scalar instructions, a 64-bit multiplication among them)
+            const uint32_t* __restrict__ ptap = pats + (size_t)(r * p.S) * p.opad + wi * 32;
+            for (int s = 0; s < p.S; ++s, ptap += p.opad) {
                 const int cola = 2 * pp * p.stride_w + s, colb = cola + p.stride_w;
-                // sign patterns of this tap's 32 channels, one per word (wide scalar loads)
-                const u16v* pw = reinterpret_cast<const u16v*>(pats + (size_t)(r * p.S + s) * p.opad + wi * 32);
+                const u16v* pw = reinterpret_cast<const u16v*>(ptap);
                 const u16v i0 = pw[0], i1 = pw[1];
                 // the three channels of a column are kLB floats apart: one address per pixel, constant offsets
                 const float* ta = tile + cola * 3 * kLB + lane;
