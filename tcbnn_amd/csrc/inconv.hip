@@ -253,7 +253,10 @@ template <int NST, bool ROWS, bool POOLED, bool ALLIN>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS && NST <= 16 ? 4 : 3))) void inconv_tiled_kernel(
     const InConvParams p, const float* __restrict__ in, const uint4* __restrict__ masks,
     const float* __restrict__ bn, uint32_t* __restrict__ out, int32_t* __restrict__ res, int b_tiles,
-    int x_groups, int y_phases, int div_magic, int rpw, int row_il, int rows_total, int row_g, unsigned row_g_magic) {
+    int x_groups, int y_phases, int div_magic, int rpw_arg, int row_il, int rows_total, int row_g, unsigned row_g_magic) {
+    // (ALLIN: NST passes of 4 rpw segments are exactly the 192 segments, so rpw is a constant of the instantiation and
+    // the staging's LDS offsets are immediates)
+    const int rpw = ALLIN ? 48 / NST : rpw_arg;
     __shared__ float tile[3 * kMaxCols * kLB];
 
     const int tid = threadIdx.x;
