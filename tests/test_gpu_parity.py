@@ -481,6 +481,40 @@ def test_conv128_saved_residual_as_window_maximum(gpu, variant, b, h, cin, cout,
     prod.release()
 
 
+@pytest.mark.parametrize("b,h,w,cin,cout,in_fmt", [(40, 6, 10, 64, 64, 2), (16, 8, 4, 128, 128, 1),
+                                                   (64, 2, 14, 256, 256, 1), (8, 12, 2, 64, 128, 2)])
+def test_conv128_window_maximum_on_frames_that_are_not_square(gpu, b, h, w, cin, cout, in_fmt):
+    """The window walk of the producer and the pooled injection of the reader on frames with different heights and
+    widths (a transposed row / column count anywhere would mix up pixels)."""
+    r = rng(b + 13 * h + 29 * w + cin)
+    x, f = rm.pm1(r, (b, h, w, cin)), rm.pm1(r, (3, 3, cin, cout))
+    bn = r.normal(0, 20, cout).astype(np.float32)
+    src = r.integers(-300, 301, size=(h, w, b, cout)).astype(np.int32)
+    x2, f2 = rm.pm1(r, (b, h // 2, w // 2, cout)), rm.pm1(r, (3, 3, cout, cout))
+    bn2 = r.normal(0, 40, cout).astype(np.float32)
+    want_p, res_p = orc.conv128(orc.pack_conv_input_nhwc(x), orc.pack_conv_filter(f), bn, cin, cout, 3, 3,
+                                save_residual=True, inject_residual=True, residual_channels=cout, res_in=src)
+    want_c, res_c = orc.conv128(orc.pack_conv_input_nhwc(x2), orc.pack_conv_filter(f2), bn2, cout, cout, 3, 3,
+                                save_residual=True, inject_residual=True, residual_channels=cout // 2,
+                                residual_pool=True, res_in=res_p)
+    prod = gpu.Conv128LayerParam("P", h, w, 3, 3, cin, cout, b, 1, 1, True, 1, 1, False, True, True, cout, False)
+    prod.initialize(gpu.ArrayWeights([f, bn]), gpuops.pack_conv_input(x), _residual_source(src, in_fmt))
+    cons = gpu.Conv128LayerParam("C", h // 2, w // 2, 3, 3, cout, cout, b, 1, 1, True, 1, 1, False, True, True, cout // 2,
+                                 True)
+    cons.initialize(gpu.ArrayWeights([f2, bn2]), gpuops.pack_conv_input(x2), prod.get_output_residual_gpu())
+    assert ", 2, true>" in prod.kernel_name()
+    prod.forward()
+    cons.forward()
+    got, pooled = prod.download_saved_residual()
+    assert pooled
+    np.testing.assert_array_equal(got, _window_maximum(res_p))
+    np.testing.assert_array_equal(prod.download_packed(), want_p)
+    np.testing.assert_array_equal(cons.download_packed(), want_c)
+    np.testing.assert_array_equal(cons.download_saved_residual()[0], res_c)
+    cons.release()
+    prod.release()
+
+
 def test_saved_residual_stays_full_for_other_readers(gpu):
     """The 2x2 maximum alone is stored only while every hand-out of the tensor went to a pooling Conv128 reader."""
     r = rng(31)
