@@ -57,6 +57,7 @@ enum EpilogueMode : int {
 struct BgemmParams {
     const uint32_t* act;  // [H][W][cw][B]
     const uint32_t* wgt;  // [npad32][taps*cw]
+    int wgt_lane_copy;    // wgt is a fully connected layer's buffer: the copy in lane order follows the rows
     int H, W, B, cw;      // input geometry, words per (pixel, image)
     int R, S, stride_h, stride_w, pad_h, pad_w;
     int PH, PW;           // conv output size before pooling

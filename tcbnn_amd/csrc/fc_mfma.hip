@@ -188,6 +188,8 @@ __global__ __launch_bounds__(64 * kMaxWaves) void fc_mfma_f4_kernel(
 }  // namespace
 
 bool fc_mfma_applicable(const BgemmParams& p) {
+    // (a 1 x 1 convolution on a 1 x 1 frame has this shape too, but its filter buffer holds no copy in lane order)
+    if (!p.wgt_lane_copy) return false;
     if (p.PH * p.PW != 1 || p.R * p.S != 1 || p.res_in != nullptr || p.res_out != nullptr) return false;
     if (p.mode != EPI_THRESH && p.mode != EPI_AFFINE) return false;
     if (p.cw % 4 != 0 || p.k_tap > 32 * p.cw) return false;

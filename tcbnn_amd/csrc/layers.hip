@@ -99,6 +99,7 @@ static BgemmParams fc_problem(const uint32_t* input, const uint32_t* weight, int
     memset(&p, 0, sizeof(p));
     p.act = input;
     p.wgt = weight;
+    p.wgt_lane_copy = 1;  // (tcbnn_pack_fc_weight wrote it)
     p.H = p.W = 1;
     p.B = batch;
     p.cw = kw128(k);

@@ -556,6 +556,27 @@ def test_saved_residual_stays_full_for_other_readers(gpu):
         p.release()
 
 
+@pytest.mark.parametrize("variant", VARIANTS)
+@pytest.mark.parametrize("b,cin,cout,R,ahead_fc", [(8, 512, 128, 1, True), (40, 128, 64, 1, False), (33, 256, 96, 1, True),
+                                                   (8, 1024, 256, 1, False), (8, 128, 64, 3, True)])
+def test_conv128_on_a_one_pixel_frame(gpu, variant, b, cin, cout, R, ahead_fc):
+    """A convolution whose frame is one pixel has the shape of a fully connected layer (one output pixel, and one
+    tap with a 1x1 filter), but its filter buffer is a convolution's: it holds the sign-bit rows only, not the copy in
+    lane order that the fully connected kernel of the FP4 engine reads."""
+    r = rng(b + cin + cout + R)
+    x, f = rm.pm1(r, (b, 1, 1, cin)), rm.pm1(r, (R, R, cin, cout))
+    bn = r.normal(0, np.sqrt(cin) * 0.5, cout).astype(np.float32)
+    want, _ = orc.conv128(orc.pack_conv_input_nhwc(x), orc.pack_conv_filter(f), bn, cin, cout, R, R, 1, True, 1, ahead_fc)
+    layer = gpu.Conv128LayerParam("C", 1, 1, R, R, cin, cout, b, 1, 1, True, 1, 1, ahead_fc, variant=_variant(gpu, variant))
+    layer.initialize(gpu.ArrayWeights([f, bn]), gpuops.pack_conv_input(x))
+    assert "fc_mfma" not in layer.kernel_name()
+    layer.output_gpu.fill(0xCD)
+    layer.forward()
+    gpuops.sync()
+    np.testing.assert_array_equal(layer.download_packed(), want)
+    layer.release()
+
+
 def test_conv128_random_shapes(gpu):
     """Seeded random bit-convolution layers: non-square frames of 1-14 pixels, 3x3 mostly (also 1x1 / 3x5 / 5x5 ...),
     strides, pools, FC-ready outputs, every residual mode with random storage formats, channel limits that cut through
