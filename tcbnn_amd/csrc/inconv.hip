@@ -249,7 +249,14 @@ __device__ __forceinline__ void inconv_store_residual(const float* acc, int32_t*
 // ALLIN (ROWS): the host found every staging pass of every lane inside the 192 segments, the batch a multiple of 64
 // and the output channels a multiple of 64, so no pass, image or channel is tested (and none of those tests'
 // invariants is computed or kept).
-template <int NST, bool ROWS, bool POOLED, bool ALLIN>
+// DLDS (ALLIN): the row segments go from memory straight into LDS (buffer loads with the LDS flag: a wave's 64 lanes
+// fill 64 consecutive words at a wave-uniform LDS address), into one of two buffers in turn: no staging registers, no
+// LDS write instructions, and one barrier per filter row instead of two.  A lane's place in the 64 words is its
+// segment times a fixed stride (kSegStride, odd) plus its column, so the layout is [image][channel][kSegStride]: the
+// three channels of a tap are constant offsets apart and the 64 images of a wave's tap read fall into 64 different
+// banks (3 kSegStride is odd).  The host selects it when a segment fits the stride.
+constexpr int inconv_seg_stride(int nst) { return nst == 4 ? 5 : (nst == 8 ? 9 : (nst == 16 ? 21 : 31)); }
+template <int NST, bool ROWS, bool POOLED, bool ALLIN, bool DLDS = false>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS && NST <= 16 ? 4 : 3))) void inconv_tiled_kernel(
     const InConvParams p, const float* __restrict__ in, const uint4* __restrict__ masks,
     const float* __restrict__ bn, uint32_t* __restrict__ out, int32_t* __restrict__ res, int b_tiles,
@@ -257,7 +264,10 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS &
     // (ALLIN: NST passes of 4 rpw segments are exactly the 192 segments, so rpw is a constant of the instantiation and
     // the staging's LDS offsets are immediates)
     const int rpw = ALLIN ? 48 / NST : rpw_arg;
-    __shared__ float tile[3 * kMaxCols * kLB];
+    static_assert(!DLDS || (ALLIN && ROWS), "direct-to-LDS staging is a variant of the full-tile row staging");
+    constexpr int kSegStride = inconv_seg_stride(NST);
+    constexpr int kBufWords = 3 * 64 * kSegStride;  // DLDS: one buffer = 192 segments
+    __shared__ float tile[DLDS ? 2 * kBufWords : 3 * kMaxCols * kLB];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -305,11 +315,12 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS &
         float stg[NST];
         // ROWS scheme: per-lane constants
         const int rp = 4 * rpw;                      // segments per pass of the workgroup
-        const int sub = lane / ncols;                // segment of the wave's rpw this lane reads
-        const int scol = lane - sub * ncols;         // column in the segment
+        const int sub = DLDS ? lane / kSegStride : lane / ncols;  // segment of the wave's rpw this lane reads
+        const int scol = lane - sub * (DLDS ? kSegStride : ncols);  // column in the segment
         const int seg0 = wave * rpw + sub;           // segment (image * 3 + channel) in pass 0
         const int sax = ax_base + scol;
-        const bool lane_ok = sub < rpw && sax >= 0 && sax < p.W;  // constant over passes and rows
+        const bool lane_used = sub < rpw && scol < ncols;  // DLDS: the lane has a word of the segment at all
+        const bool lane_ok = sub < rpw && sax >= 0 && sax < p.W && (!DLDS || scol < ncols);  // constant over passes and rows
         // Buffer addressing: descriptor = this workgroup's 64 images, per-lane byte offset (one
         // constant), wave-uniform scalar offset per (row, pass).  A lane outside the frame carries an
         // offset beyond the descriptor's range: the hardware returns 0 for it without touching memory.
@@ -362,6 +373,20 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS &
                 }
             }
         };
+        // DLDS: the same requests with LDS as their destination: pass k of this wave fills the 64 words of its rpw
+        // segments in buffer `sel` (lanes without a word are switched off; columns outside the frame arrive as zeros).
+        auto fetch_row_lds = [&](int r, int sel) {
+            typedef __attribute__((address_space(3))) void* lds_ptr_t;
+            const unsigned row_bytes = (unsigned)(ay0 + r) * (unsigned)p.W * 4u;       // uniform
+            const unsigned pass_bytes = (unsigned)rp * (unsigned)plane * 4u;           // uniform
+            float* dst = tile + sel * kBufWords + wave * (48 / NST) * kSegStride;
+            if (lane_used) {
+#pragma unroll
+                for (int k = 0; k < NST; ++k)
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lds_ptr_t)(dst + k * 4 * (48 / NST) * kSegStride), 4,
+                                                             (int)voff, (int)(row_bytes + k * pass_bytes), 0, 0);
+            }
+        };
         auto store_row = [&]() {
             if constexpr (ROWS) {
                 if (sub < rpw) {
@@ -385,12 +410,26 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS &
             }
         };
 
-        if (r_lo < r_hi) fetch_row(r_lo);
+        if constexpr (DLDS) {
+            // (a slower wave may still be reading the previous row loop's last buffer)
+            if (g > 0 || py > 0) __syncthreads();
+            if (r_lo < r_hi) fetch_row_lds(r_lo, 0);
+        } else {
+            if (r_lo < r_hi) fetch_row(r_lo);
+        }
         for (int r = r_lo; r < r_hi; ++r) {
-            __syncthreads();
-            store_row();
-            __syncthreads();
-            if (r + 1 < r_hi) fetch_row(r + 1);
+            if constexpr (DLDS) {
+                // this wave's words of row r have arrived; after the barrier everybody's have, and everybody has left
+                // row r - 1, whose buffer the requests for row r + 1 overwrite
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                __syncthreads();
+                if (r + 1 < r_hi) fetch_row_lds(r + 1, (r + 1 - r_lo) & 1);
+            } else {
+                __syncthreads();
+                store_row();
+                __syncthreads();
+                if (r + 1 < r_hi) fetch_row(r + 1);
+            }
             if (!work) continue;
             // sign patterns of a tap's 32 channels, one per word (wide scalar loads); the pointer moves on by one tap
             // (formed anew per tap it was seven scalar instructions, a 64-bit multiplication among them)
@@ -400,10 +439,13 @@ __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS &
                 const u16v* pw = reinterpret_cast<const u16v*>(ptap);
                 const u16v i0 = pw[0], i1 = pw[1];
                 // the three channels of a column are kLB floats apart: one address per pixel, constant offsets
-                const float* ta = tile + cola * 3 * kLB + lane;
-                const float* tb = tile + colb * 3 * kLB + lane;
-                const v8f ca = sign_combos(ta[0], ta[kLB], ta[2 * kLB]);
-                const v8f cb = sign_combos(tb[0], tb[kLB], tb[2 * kLB]);
+                // (DLDS: [image][channel][kSegStride] in the row's buffer)
+                constexpr int kChan = DLDS ? kSegStride : kLB;
+                const float* ta = DLDS ? tile + ((r - r_lo) & 1) * kBufWords + lane * 3 * kSegStride + cola
+                                       : tile + cola * 3 * kLB + lane;
+                const float* tb = DLDS ? ta + p.stride_w : tile + colb * 3 * kLB + lane;
+                const v8f ca = sign_combos(ta[0], ta[kChan], ta[2 * kChan]);
+                const v8f cb = sign_combos(tb[0], tb[kChan], tb[2 * kChan]);
                 add_indexed8x2(&acca[0], &accb[0], ca, cb, i0[0], i0[1], i0[2], i0[3], i0[4], i0[5], i0[6], i0[7]);
                 add_indexed8x2(&acca[8], &accb[8], ca, cb, i0[8], i0[9], i0[10], i0[11], i0[12], i0[13], i0[14],
                                i0[15]);
@@ -784,10 +826,11 @@ static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name
         if (row_staging) {
             const int passes = (3 * 64 + 4 * rpw - 1) / (4 * rpw);
             const int nst = passes <= 4 ? 4 : (passes <= 8 ? 8 : (passes <= 16 ? 16 : 24));
-            snprintf(name_buf, name_len, "inconv_tiled_kernel<%d, true, %s, %s>", nst, pooled ? "true" : "false",
-                     nst * 4 * rpw == 3 * 64 && p.B % 64 == 0 && p.O % 64 == 0 ? "true" : "false");
+            const bool allin = nst * 4 * rpw == 3 * 64 && p.B % 64 == 0 && p.O % 64 == 0;
+            snprintf(name_buf, name_len, "inconv_tiled_kernel<%d, true, %s, %s, %s>", nst, pooled ? "true" : "false",
+                     allin ? "true" : "false", allin && ncols <= inconv_seg_stride(nst) ? "true" : "false");
         } else {
-            snprintf(name_buf, name_len, "inconv_tiled_kernel<%d, false, %s, false>",
+            snprintf(name_buf, name_len, "inconv_tiled_kernel<%d, false, %s, false, false>",
                      (3 * 64 * ncols + kThreads - 1) / kThreads <= 15 ? 15 : 24, pooled ? "true" : "false");
         }
         return TCBNN_OK;
@@ -813,6 +856,10 @@ static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name
             constexpr bool ROWS = decltype(rows_tag)::value;
             if constexpr (ROWS) {
                 if (NST * 4 * rpw == 3 * 64 && p.B % 64 == 0 && p.O % 64 == 0) {
+                    if (ncols <= inconv_seg_stride(NST)) {  // a segment fits the fixed stride: straight into LDS
+                        if (pooled) return launch(inconv_tiled_kernel<NST, true, true, true, true>);
+                        return launch(inconv_tiled_kernel<NST, true, false, true, true>);
+                    }
                     if (pooled) return launch(inconv_tiled_kernel<NST, true, true, true>);
                     return launch(inconv_tiled_kernel<NST, true, false, true>);
                 }
