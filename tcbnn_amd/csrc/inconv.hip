@@ -256,6 +256,10 @@ __device__ __forceinline__ void inconv_store_residual(const float* acc, int32_t*
 // three channels of a tap are constant offsets apart and the 64 images of a wave's tap read fall into 64 different
 // banks (3 kSegStride is odd).  The host selects it when a segment fits the stride.
 constexpr int inconv_seg_stride(int nst) { return nst == 4 ? 5 : (nst == 8 ? 9 : (nst == 16 ? 21 : 31)); }
+// Where it is used: 16 passes (segments of 11 to 21 columns: 7-wide filters at strides 2 to 4, three waves' worth of
+// segments per pass), where it measured 2-4 % faster than staging through registers.  With 8 passes (3x3 filters at
+// stride 1: three taps per row) it measured 3-5 % slower and with 24 (11-wide filters, three waves per SIMD) 20 %.
+constexpr bool inconv_straight_to_lds(int nst, int ncols) { return nst == 16 && ncols <= inconv_seg_stride(nst); }
 template <int NST, bool ROWS, bool POOLED, bool ALLIN, bool DLDS = false>
 __global__ __launch_bounds__(kThreads) __attribute__((amdgpu_waves_per_eu(ROWS && NST <= 16 ? 4 : 3))) void inconv_tiled_kernel(
     const InConvParams p, const float* __restrict__ in, const uint4* __restrict__ masks,
@@ -828,7 +832,7 @@ static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name
             const int nst = passes <= 4 ? 4 : (passes <= 8 ? 8 : (passes <= 16 ? 16 : 24));
             const bool allin = nst * 4 * rpw == 3 * 64 && p.B % 64 == 0 && p.O % 64 == 0;
             snprintf(name_buf, name_len, "inconv_tiled_kernel<%d, true, %s, %s, %s>", nst, pooled ? "true" : "false",
-                     allin ? "true" : "false", allin && ncols <= inconv_seg_stride(nst) ? "true" : "false");
+                     allin ? "true" : "false", allin && inconv_straight_to_lds(nst, ncols) ? "true" : "false");
         } else {
             snprintf(name_buf, name_len, "inconv_tiled_kernel<%d, false, %s, false, false>",
                      (3 * 64 * ncols + kThreads - 1) / kThreads <= 15 ? 15 : 24, pooled ? "true" : "false");
@@ -856,9 +860,11 @@ static int inconv128_run(const tcbnn_inconv128_desc* d, void* stream, char* name
             constexpr bool ROWS = decltype(rows_tag)::value;
             if constexpr (ROWS) {
                 if (NST * 4 * rpw == 3 * 64 && p.B % 64 == 0 && p.O % 64 == 0) {
-                    if (ncols <= inconv_seg_stride(NST)) {  // a segment fits the fixed stride: straight into LDS
-                        if (pooled) return launch(inconv_tiled_kernel<NST, true, true, true, true>);
-                        return launch(inconv_tiled_kernel<NST, true, false, true, true>);
+                    if constexpr (inconv_straight_to_lds(NST, 0)) {
+                        if (inconv_straight_to_lds(NST, ncols)) {
+                            if (pooled) return launch(inconv_tiled_kernel<NST, true, true, true, true>);
+                            return launch(inconv_tiled_kernel<NST, true, false, true, true>);
+                        }
                     }
                     if (pooled) return launch(inconv_tiled_kernel<NST, true, true, true>);
                     return launch(inconv_tiled_kernel<NST, true, false, true>);
